@@ -1,0 +1,116 @@
+/*
+ * natten_amd — C ABI of the MI355X (gfx950) fused neighborhood attention forward path.
+ *
+ * Every entry point takes plain device pointers and sizes (no framework types), launches on
+ * the HIP stream handle it is given (NULL = default stream), never synchronises and never
+ * allocates or frees device memory.  The caller owns all buffers.  Return value: 0 on
+ * success, non-zero on error; natten_amd_last_error() then returns a message (thread local).
+ *
+ * The entry points replace, one for one, the native functions the reference binds with
+ * pybind11 for this path (paths relative to the SHI-Labs/NATTEN tree):
+ *
+ *   natten_amd_fna_forward      <- blackwell_na{1,2,3}d_forward
+ *                                  csrc/include/natten/blackwell_fna.h:36-52, csrc/natten.cpp:39-160
+ *   natten_amd_token_permute    <- token_permute_{1,2,3}d   csrc/include/natten/token_permute.h:34-52
+ *   natten_amd_token_unpermute  <- token_unpermute_{1,2,3}d csrc/include/natten/token_permute.h:54-74
+ *   natten_amd_attention_forward<- blackwell_fmha_forward   csrc/include/natten/blackwell_fmha.h
+ *                                  (dense attention used for additional keys/values and for
+ *                                  kernel_size == input size; no variable-length batches)
+ *   natten_amd_merge_attentions <- the elementwise merge of src/natten/attn_merge.py:48-105
+ *                                  (the reference runs it as framework ops; here it is one kernel)
+ */
+#ifndef NATTEN_AMD_H_
+#define NATTEN_AMD_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Element types of Q/K/V (`dtype` arguments). */
+#define NATTEN_AMD_F16 0
+#define NATTEN_AMD_BF16 1
+#define NATTEN_AMD_F8E4M3 2 /* OCP e4m3fn inputs, bf16 output */
+#define NATTEN_AMD_F32 3    /* merge / permute payloads only */
+
+/* ABI version; bumped whenever a signature changes. */
+int natten_amd_abi_version(void);
+
+/* Message of the last failing call on this thread ("" if none). */
+const char* natten_amd_last_error(void);
+
+/*
+ * Fused neighborhood attention forward on token-permuted operands.
+ *
+ *   q   [batch, seqlen_q,  heads_q,  head_dim]   contiguous
+ *   k,v [batch, seqlen_kv, heads_kv, head_dim]   contiguous, heads_q % heads_kv == 0
+ *   out [batch, seqlen_q,  heads_q,  head_dim]   dtype of q (bf16 when q is e4m3)
+ *   lse [batch, seqlen_q,  heads_q]              float32, natural log of the sum of exp(scale*q.k)
+ *
+ * `batch` already includes the dilation groups (batch index = b * prod(dilation) + group,
+ * group decoded with dimension 0 fastest).  q_shape / kv_shape are the padded per-group token
+ * layouts the permuted sequences were built from (seqlen = product), qkv_shape the original
+ * token layout.  All shape-like arrays hold `na_dim` entries.  Tiles are multi-dimensional;
+ * their element counts must be a supported (Q tile, KV tile) pair, see
+ * natten_amd_fna_supported_tiles().  head_dim must be 32, 64 or 128.
+ * For e4m3 inputs q_scale*k_scale multiplies the logits' scale and v_scale the output
+ * (pass 1.0f otherwise).
+ */
+int natten_amd_fna_forward(const void* q, const void* k, const void* v, void* out, float* lse,
+                           int dtype, int na_dim, int batch, int seqlen_q, int seqlen_kv,
+                           int heads_q, int heads_kv, int head_dim, const int32_t* q_shape,
+                           const int32_t* kv_shape, const int32_t* qkv_shape,
+                           const int32_t* kernel_size, const int32_t* stride,
+                           const int32_t* dilation, const int32_t* is_causal,
+                           const int32_t* q_tile_shape, const int32_t* kv_tile_shape, float scale,
+                           float q_scale, float k_scale, float v_scale, void* stream);
+
+/*
+ * Supported tile sizes (tokens per tile).  Writes up to `capacity` pairs
+ * (q_tile_size, kv_tile_size) for the given dtype / head_dim and returns how many exist.
+ */
+int natten_amd_fna_supported_tiles(int dtype, int head_dim, int32_t* q_sizes, int32_t* kv_sizes,
+                                   int capacity);
+
+/*
+ * Dense attention forward (optional top-left causal mask) on unpermuted operands.
+ *   q [batch, seqlen_q, heads_q, head_dim], k/v [batch, seqlen_kv, heads_kv, head_dim],
+ *   out like q, lse [batch, seqlen_q, heads_q] float32.  Any seqlen >= 1.
+ */
+int natten_amd_attention_forward(const void* q, const void* k, const void* v, void* out,
+                                 float* lse, int dtype, int batch, int seqlen_q, int seqlen_kv,
+                                 int heads_q, int heads_kv, int head_dim, int is_causal,
+                                 float scale, void* stream);
+
+/*
+ * Token permute: src [batch, *token_layout, heads, head_dim] -> dst
+ * [batch * prod(dilation), prod(ceil(ceil(X/t)/d) * t), heads, head_dim]; padding rows are
+ * zero.  Payload is copied verbatim (`elem_bytes` bytes per element, any type).
+ */
+int natten_amd_token_permute(const void* src, void* dst, int elem_bytes, int na_dim, int batch,
+                             int heads, int head_dim, const int32_t* token_layout,
+                             const int32_t* tile_shape, const int32_t* dilation,
+                             int flip_tiled_dims, void* stream);
+
+/* Inverse of natten_amd_token_permute; padding rows of `src` are dropped. */
+int natten_amd_token_unpermute(const void* src, void* dst, int elem_bytes, int na_dim, int batch,
+                               int heads, int head_dim, const int32_t* token_layout,
+                               const int32_t* tile_shape, const int32_t* dilation,
+                               int flip_tiled_dims, void* stream);
+
+/*
+ * Merge two partial attentions over disjoint key sets of the same queries:
+ *   out = o0 - sigmoid(lse1 - lse0) * (o0 - o1),  lse = lse0 - logsigmoid(lse0 - lse1)
+ * o0/o1/out [rows, head_dim] of `dtype` (F16/BF16/F32), lse0/lse1/lse_out [rows] float32,
+ * rows = batch * seqlen * heads.  out may alias o0, lse_out may alias lse0.
+ */
+int natten_amd_merge_attentions(const void* o0, const float* lse0, const void* o1,
+                                const float* lse1, void* out, float* lse_out, int dtype,
+                                int64_t rows, int head_dim, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* NATTEN_AMD_H_ */

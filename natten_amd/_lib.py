@@ -1,0 +1,250 @@
+"""Loader and thin wrappers of the C-ABI library (libnatten_amd.so).
+
+Counterpart of the reference's op boundary, src/natten/_libnatten/__init__.py:26-113 and
+src/natten/_libnatten/torch_wrappers.py:657-716, :1373-1503: outputs are allocated here with
+torch and written by the native code on torch's current stream.  There is no fallback: when
+the library is missing every op raises ImportError (the reference's stubs do the same,
+src/natten/_libnatten/stubs.py:25-31).
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+from typing import Optional, Sequence, Tuple
+
+import torch
+from torch import Tensor
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libnatten_amd.so")
+
+ABI_VERSION = 1
+
+DTYPE_CODES = {
+    torch.float16: 0,
+    torch.bfloat16: 1,
+    torch.float8_e4m3fn: 2,
+    torch.float32: 3,
+}
+
+_lib = None
+_load_error: Optional[str] = None
+
+_SIGNATURES = {
+    "natten_amd_abi_version": (ctypes.c_int, []),
+    "natten_amd_last_error": (ctypes.c_char_p, []),
+    "natten_amd_fna_supported_tiles": (
+        ctypes.c_int,
+        [ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int],
+    ),
+    "natten_amd_fna_forward": (
+        ctypes.c_int,
+        [ctypes.c_void_p] * 5
+        + [ctypes.c_int] * 8
+        + [ctypes.c_void_p] * 9
+        + [ctypes.c_float] * 4
+        + [ctypes.c_void_p],
+    ),
+    "natten_amd_attention_forward": (
+        ctypes.c_int,
+        [ctypes.c_void_p] * 5 + [ctypes.c_int] * 8 + [ctypes.c_float, ctypes.c_void_p],
+    ),
+    "natten_amd_token_permute": (
+        ctypes.c_int,
+        [ctypes.c_void_p] * 2 + [ctypes.c_int] * 5 + [ctypes.c_void_p] * 3 + [ctypes.c_int, ctypes.c_void_p],
+    ),
+    "natten_amd_token_unpermute": (
+        ctypes.c_int,
+        [ctypes.c_void_p] * 2 + [ctypes.c_int] * 5 + [ctypes.c_void_p] * 3 + [ctypes.c_int, ctypes.c_void_p],
+    ),
+    "natten_amd_merge_attentions": (
+        ctypes.c_int,
+        [ctypes.c_void_p] * 6 + [ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_void_p],
+    ),
+}
+
+EXPORTED_SYMBOLS = tuple(_SIGNATURES)
+
+
+def _try_load():
+    global _lib, _load_error
+    if _lib is not None or _load_error is not None:
+        return
+    if not os.path.exists(LIB_PATH):
+        _load_error = (
+            f"natten_amd: native library not found at {LIB_PATH}. Build it with "
+            "`python -m natten_amd.build` (hipcc, --offload-arch=gfx950)."
+        )
+        return
+    try:
+        lib = ctypes.CDLL(LIB_PATH)
+        for name, (restype, argtypes) in _SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype = restype
+            fn.argtypes = argtypes
+        if lib.natten_amd_abi_version() != ABI_VERSION:
+            raise OSError(f"ABI version {lib.natten_amd_abi_version()} != expected {ABI_VERSION}")
+        _lib = lib
+    except (OSError, AttributeError) as e:  # pragma: no cover - depends on the build
+        _load_error = f"natten_amd: failed to load {LIB_PATH}: {e}"
+
+
+def has_lib() -> bool:
+    _try_load()
+    return _lib is not None
+
+
+def lib():
+    _try_load()
+    if _lib is None:
+        raise ImportError(_load_error)
+    return _lib
+
+
+def _i32(values: Sequence[int]):
+    return (ctypes.c_int32 * len(values))(*[int(v) for v in values])
+
+
+def _check(rc: int):
+    if rc != 0:
+        raise RuntimeError(lib().natten_amd_last_error().decode())
+
+
+def _stream(t: Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _require_gpu(*tensors: Tensor):
+    for t in tensors:
+        if not t.is_cuda:
+            raise RuntimeError("natten_amd native ops need tensors on the GPU device.")
+        if not t.is_contiguous():
+            raise RuntimeError("natten_amd native ops need contiguous tensors.")
+
+
+def supported_tile_sizes(dtype: torch.dtype, head_dim: int):
+    if dtype not in DTYPE_CODES:
+        return []
+    n = lib().natten_amd_fna_supported_tiles(DTYPE_CODES[dtype], head_dim, None, None, 0)
+    if n <= 0:
+        return []
+    q = (ctypes.c_int32 * n)()
+    kv = (ctypes.c_int32 * n)()
+    lib().natten_amd_fna_supported_tiles(DTYPE_CODES[dtype], head_dim, q, kv, n)
+    return [(int(a), int(b)) for a, b in zip(q, kv)]
+
+
+def fna_forward(
+    q: Tensor, k: Tensor, v: Tensor,
+    kernel_size, stride, dilation, is_causal, scale: float,
+    q_shape, kv_shape, qkv_shape, q_tile_shape, kv_tile_shape,
+    q_scale: float = 1.0, k_scale: float = 1.0, v_scale: float = 1.0,
+) -> Tuple[Tensor, Tensor]:
+    """Token-permuted q [B*G, SQ, H, D], k/v [B*G, SK, Hkv, D] -> (out, lse float32 [B*G, SQ, H])."""
+    L = lib()
+    _require_gpu(q, k, v)
+    if q.dtype not in (torch.float16, torch.bfloat16, torch.float8_e4m3fn):
+        raise NotImplementedError(f"natten_amd fna_forward does not support {q.dtype}.")
+    na_dim = len(kernel_size)
+    out_dtype = torch.bfloat16 if q.dtype == torch.float8_e4m3fn else q.dtype
+    out = torch.empty(q.shape, dtype=out_dtype, device=q.device)
+    lse = torch.empty(q.shape[:-1], dtype=torch.float32, device=q.device)
+    with torch.cuda.device(q.device):
+        rc = L.natten_amd_fna_forward(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
+            DTYPE_CODES[q.dtype], na_dim, q.shape[0], q.shape[1], k.shape[1], q.shape[2], k.shape[2], q.shape[3],
+            _i32(q_shape), _i32(kv_shape), _i32(qkv_shape), _i32(kernel_size), _i32(stride), _i32(dilation),
+            _i32([1 if c else 0 for c in is_causal]), _i32(q_tile_shape), _i32(kv_tile_shape),
+            float(scale), float(q_scale), float(k_scale), float(v_scale), _stream(q),
+        )
+    _check(rc)
+    return out, lse
+
+
+def attention_forward(q: Tensor, k: Tensor, v: Tensor, is_causal: bool, scale: float) -> Tuple[Tensor, Tensor]:
+    """Dense attention q [B, S, H, D], k/v [B, Skv, Hkv, D] -> (out, lse float32 [B, S, H])."""
+    L = lib()
+    _require_gpu(q, k, v)
+    if q.dtype not in (torch.float16, torch.bfloat16):
+        raise NotImplementedError(f"natten_amd attention_forward does not support {q.dtype}.")
+    out = torch.empty_like(q)
+    lse = torch.empty(q.shape[:-1], dtype=torch.float32, device=q.device)
+    with torch.cuda.device(q.device):
+        rc = L.natten_amd_attention_forward(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(), DTYPE_CODES[q.dtype],
+            q.shape[0], q.shape[1], k.shape[1], q.shape[2], k.shape[2], q.shape[3], 1 if is_causal else 0,
+            float(scale), _stream(q),
+        )
+    _check(rc)
+    return out, lse
+
+
+def _ceil_div(a: int, b: int) -> int:
+    return (a + b - 1) // b
+
+
+def token_permute(x: Tensor, tile_shape, dilation, flip_tiled_dims: bool) -> Tensor:
+    """[B, *X, H, Dh] -> [B * prod(dilation), prod(ceil(ceil(X/t)/d) * t), H, Dh], zero padded."""
+    L = lib()
+    _require_gpu(x)
+    na_dim = x.dim() - 3
+    layout = [int(s) for s in x.shape[1 : 1 + na_dim]]
+    post = [_ceil_div(_ceil_div(X, t), d) * t for X, t, d in zip(layout, tile_shape, dilation)]
+    groups = 1
+    seqlen = 1
+    for d, p in zip(dilation, post):
+        groups *= d
+        seqlen *= p
+    out = torch.empty((x.shape[0] * groups, seqlen, x.shape[-2], x.shape[-1]), dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        rc = L.natten_amd_token_permute(
+            x.data_ptr(), out.data_ptr(), x.element_size(), na_dim, x.shape[0], x.shape[-2], x.shape[-1],
+            _i32(layout), _i32(tile_shape), _i32(dilation), 1 if flip_tiled_dims else 0, _stream(x),
+        )
+    _check(rc)
+    return out
+
+
+def token_unpermute(y: Tensor, token_layout, tile_shape, dilation, flip_tiled_dims: bool) -> Tensor:
+    """Inverse of token_permute: [B*G, S', H, Dh] -> [B, *token_layout, H, Dh]."""
+    L = lib()
+    _require_gpu(y)
+    na_dim = len(token_layout)
+    groups = 1
+    seqlen = 1
+    for X, t, d in zip(token_layout, tile_shape, dilation):
+        groups *= d
+        seqlen *= _ceil_div(_ceil_div(X, t), d) * t
+    if y.dim() != 4 or y.shape[0] % groups != 0 or y.shape[1] != seqlen:
+        raise RuntimeError(
+            f"token_unpermute: tensor of shape {tuple(y.shape)} does not match token layout {tuple(token_layout)}, "
+            f"tile shape {tuple(tile_shape)}, dilation {tuple(dilation)} (expected [B*{groups}, {seqlen}, H, D])."
+        )
+    batch = y.shape[0] // groups
+    out = torch.empty((batch, *token_layout, y.shape[-2], y.shape[-1]), dtype=y.dtype, device=y.device)
+    with torch.cuda.device(y.device):
+        rc = L.natten_amd_token_unpermute(
+            y.data_ptr(), out.data_ptr(), y.element_size(), na_dim, batch, y.shape[-2], y.shape[-1],
+            _i32(token_layout), _i32(tile_shape), _i32(dilation), 1 if flip_tiled_dims else 0, _stream(y),
+        )
+    _check(rc)
+    return out
+
+
+def merge_two(o0: Tensor, lse0: Tensor, o1: Tensor, lse1: Tensor) -> Tuple[Tensor, Tensor]:
+    """Merge two partial attentions [B, S, H, D] with float32 LSE [B, S, H]."""
+    L = lib()
+    _require_gpu(o0, lse0, o1, lse1)
+    if o0.dtype not in (torch.float16, torch.bfloat16, torch.float32):
+        raise NotImplementedError(f"natten_amd merge does not support {o0.dtype}.")
+    out = torch.empty_like(o0)
+    lse = torch.empty_like(lse0)
+    rows = lse0.numel()
+    with torch.cuda.device(o0.device):
+        rc = L.natten_amd_merge_attentions(
+            o0.data_ptr(), lse0.data_ptr(), o1.data_ptr(), lse1.data_ptr(), out.data_ptr(), lse.data_ptr(),
+            DTYPE_CODES[o0.dtype], rows, o0.shape[-1], _stream(o0),
+        )
+    _check(rc)
+    return out, lse

@@ -1,0 +1,57 @@
+"""merge_attentions: combine partial attentions over disjoint key sets of the same queries.
+
+Same API and validation as the reference's src/natten/attn_merge.py:193-292; the arithmetic
+(:83-95) runs as one HIP kernel per pair.  `torch_compile` and `use_autograd_fix` are accepted
+for signature compatibility and ignored (forward only, nothing to compile)."""
+
+from __future__ import annotations
+
+from typing import List, Tuple
+
+from torch import Tensor
+
+from . import _lib
+
+
+def merge_attentions(
+    outputs: List[Tensor],
+    lse_tensors: List[Tensor],
+    torch_compile: bool = True,
+    use_autograd_fix: bool = True,
+) -> Tuple[Tensor, Tensor]:
+    if len(outputs) < 2:
+        raise ValueError("`merge_attentions` expects at least two tensors.")
+    if len(outputs) != len(lse_tensors):
+        raise ValueError(
+            "`merge_attentions` expected number of outputs and LSE tensors to match, "
+            f"got {len(outputs)=} != {len(lse_tensors)}."
+        )
+    shape = outputs[0].shape
+    for i, (output, lse) in enumerate(zip(outputs, lse_tensors)):
+        if output.dim() != 4:
+            raise ValueError(
+                f"Output tensors must be rank-4 tensors with (batch, seq, heads, dim), but got output {i} with "
+                f"rank={output.dim()}."
+            )
+        if output.shape != shape:
+            raise ValueError(f"Output tensors must match in shape, but got output {i} with shape={output.shape}.")
+        if lse.dim() != 3:
+            raise ValueError(
+                f"LSE tensors must be rank-3 tensors with (batch, seq, heads), but got LSE {i} with rank={lse.dim()}."
+            )
+        if lse.shape != shape[:3]:
+            raise ValueError(
+                f"LSE tensors must match outputs in shape except last dim ({shape=}), but got LSE {i} with "
+                f"shape={lse.shape}."
+            )
+    out_dtype = outputs[0].dtype
+    # more than two partials: keep the running result in float32 between pairwise merges
+    work = (lambda t: t.float().contiguous()) if len(outputs) > 2 else (lambda t: t.contiguous())
+    out = work(outputs[0])
+    lse = lse_tensors[0].float().contiguous()
+    for o, l in zip(outputs[1:], lse_tensors[1:]):
+        out, lse = _lib.merge_two(out, lse, work(o.to(outputs[0].dtype)), l.float().contiguous())
+    return out.to(out_dtype), lse
+
+
+__all__ = ["merge_attentions"]

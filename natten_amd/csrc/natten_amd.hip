@@ -1,0 +1,346 @@
+// C ABI of the MI355X fused neighborhood attention forward path (see include/natten_amd.h).
+// Host-side argument validation, kernel selection and launches; no framework types.
+
+#include "../../include/natten_amd.h"
+
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include <type_traits>
+
+#include "fna_fwd.hpp"
+#include "merge.hpp"
+#include "na_math.hpp"
+#include "tokperm.hpp"
+
+using namespace natten_amd;
+
+namespace {
+
+thread_local char g_error[512] = "";
+
+int fail(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+  return 1;
+}
+
+int check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail("%s: launch failed: %s", what, hipGetErrorString(e));
+  return 0;
+}
+
+int prod3(const int* x) { return x[0] * x[1] * x[2]; }
+
+struct TileConfig {
+  int q_tile, kv_tile;
+};
+
+// (Q tile, KV tile) sizes in tokens that have a kernel instance.
+const TileConfig kTileConfigs[] = {{128, 64}, {256, 64}, {128, 128}, {256, 128}, {64, 64}};
+constexpr int kNumTileConfigs = sizeof(kTileConfigs) / sizeof(kTileConfigs[0]);
+
+template <typename T, int D, int NWAVES, int MQ, int KVT>
+int launch_fna(const FnaParams& p, hipStream_t stream) {
+  constexpr int QT = NWAVES * MQ * 32;
+  constexpr int smem = FnaSmem<D, KVT>::BYTES;
+  auto kernel = fna_fwd_kernel<T, D, NWAVES, MQ, KVT>;
+  static bool configured = false;
+  if (smem > 64 * 1024 && !configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return fail("fna_forward: cannot reserve %d bytes of LDS: %s", smem, hipGetErrorString(e));
+    configured = true;
+  }
+  dim3 grid((p.seqlen_q + QT - 1) / QT, p.heads_q, p.batch);
+  hipLaunchKernelGGL(kernel, grid, dim3(NWAVES * 64), smem, stream, p);
+  return check_launch("fna_forward");
+}
+
+template <typename T, int D>
+int dispatch_tiles(const FnaParams& p, int qt, int kvt, hipStream_t stream) {
+  if (qt == 128 && kvt == 64) return launch_fna<T, D, 4, 1, 64>(p, stream);
+  if (qt == 256 && kvt == 64) return launch_fna<T, D, 4, 2, 64>(p, stream);
+  if (qt == 128 && kvt == 128) return launch_fna<T, D, 4, 1, 128>(p, stream);
+  if (qt == 256 && kvt == 128) return launch_fna<T, D, 4, 2, 128>(p, stream);
+  if (qt == 64 && kvt == 64) return launch_fna<T, D, 2, 1, 64>(p, stream);
+  return fail("fna_forward: no kernel for Q tile of %d and KV tile of %d tokens", qt, kvt);
+}
+
+template <typename T>
+int dispatch_head_dim(const FnaParams& p, int head_dim, int qt, int kvt, hipStream_t stream) {
+  switch (head_dim) {
+    case 32: return dispatch_tiles<T, 32>(p, qt, kvt, stream);
+    case 64: return dispatch_tiles<T, 64>(p, qt, kvt, stream);
+    case 128: return dispatch_tiles<T, 128>(p, qt, kvt, stream);
+  }
+  return fail("fna_forward: head_dim must be 32, 64 or 128, got %d", head_dim);
+}
+
+int dispatch_dtype(const FnaParams& p, int dtype, int head_dim, int qt, int kvt, hipStream_t stream) {
+  switch (dtype) {
+    case NATTEN_AMD_F16: return dispatch_head_dim<_Float16>(p, head_dim, qt, kvt, stream);
+    case NATTEN_AMD_BF16: return dispatch_head_dim<__bf16>(p, head_dim, qt, kvt, stream);
+  }
+  return fail("fna_forward: unsupported dtype code %d", dtype);
+}
+
+int check_common(const char* what, const void* q, const void* k, const void* v, const void* out, const float* lse,
+                 int batch, int seqlen_q, int seqlen_kv, int heads_q, int heads_kv, int head_dim) {
+  if (!q || !k || !v || !out || !lse) return fail("%s: null pointer argument", what);
+  if (batch < 1 || seqlen_q < 1 || seqlen_kv < 1 || heads_q < 1 || heads_kv < 1)
+    return fail("%s: batch, sequence lengths and head counts must be positive", what);
+  if (heads_q % heads_kv != 0)
+    return fail("%s: heads_kv (%d) must divide heads_q (%d)", what, heads_kv, heads_q);
+  if (head_dim != 32 && head_dim != 64 && head_dim != 128)
+    return fail("%s: head_dim must be 32, 64 or 128, got %d", what, head_dim);
+  if ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v) |
+       reinterpret_cast<uintptr_t>(out)) & 15)
+    return fail("%s: q, k, v and out must be 16-byte aligned", what);
+  if (heads_q > 65535 || batch > 65535) return fail("%s: heads_q and batch must be below 65536", what);
+  return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+int natten_amd_abi_version(void) { return 1; }
+
+const char* natten_amd_last_error(void) { return g_error; }
+
+int natten_amd_fna_supported_tiles(int dtype, int head_dim, int32_t* q_sizes, int32_t* kv_sizes, int capacity) {
+  if (dtype != NATTEN_AMD_F16 && dtype != NATTEN_AMD_BF16) return 0;
+  if (head_dim != 32 && head_dim != 64 && head_dim != 128) return 0;
+  for (int i = 0; i < kNumTileConfigs && i < capacity; ++i) {
+    if (q_sizes) q_sizes[i] = kTileConfigs[i].q_tile;
+    if (kv_sizes) kv_sizes[i] = kTileConfigs[i].kv_tile;
+  }
+  return kNumTileConfigs;
+}
+
+int natten_amd_fna_forward(const void* q, const void* k, const void* v, void* out, float* lse, int dtype, int na_dim,
+                           int batch, int seqlen_q, int seqlen_kv, int heads_q, int heads_kv, int head_dim,
+                           const int32_t* q_shape, const int32_t* kv_shape, const int32_t* qkv_shape,
+                           const int32_t* kernel_size, const int32_t* stride, const int32_t* dilation,
+                           const int32_t* is_causal, const int32_t* q_tile_shape, const int32_t* kv_tile_shape,
+                           float scale, float q_scale, float k_scale, float v_scale, void* stream) {
+  g_error[0] = 0;
+  if (na_dim < 1 || na_dim > 3) return fail("fna_forward: na_dim must be 1, 2 or 3, got %d", na_dim);
+  if (int rc = check_common("fna_forward", q, k, v, out, lse, batch, seqlen_q, seqlen_kv, heads_q, heads_kv, head_dim))
+    return rc;
+  if (!q_shape || !kv_shape || !qkv_shape || !kernel_size || !stride || !dilation || !is_causal || !q_tile_shape ||
+      !kv_tile_shape)
+    return fail("fna_forward: null shape argument");
+
+  FnaParams p;
+  memset(&p, 0, sizeof(p));
+  int qs[3] = {1, 1, 1}, ks[3] = {1, 1, 1};
+  p.num_groups = 1;
+  for (int a = 0; a < 3; ++a) {
+    const bool used = a < na_dim;
+    p.qkv_shape[a] = used ? qkv_shape[a] : 1;
+    p.ksize[a] = used ? kernel_size[a] : 1;
+    p.stride[a] = used ? stride[a] : 1;
+    p.dil[a] = used ? dilation[a] : 1;
+    p.causal[a] = used ? (is_causal[a] != 0) : 0;
+    p.q_tile[a] = used ? q_tile_shape[a] : 1;
+    p.kv_tile[a] = used ? kv_tile_shape[a] : 1;
+    qs[a] = used ? q_shape[a] : 1;
+    ks[a] = used ? kv_shape[a] : 1;
+    if (p.qkv_shape[a] < 1 || p.dil[a] < 1 || p.stride[a] < 1 || p.q_tile[a] < 1 || p.kv_tile[a] < 1 ||
+        (used && p.ksize[a] < 2))
+      return fail("fna_forward: invalid parameter along dimension %d", a);
+    if (p.ksize[a] * p.dil[a] > p.qkv_shape[a])
+      return fail("fna_forward: kernel_size * dilation exceeds the input along dimension %d (%d * %d > %d)", a,
+                  p.ksize[a], p.dil[a], p.qkv_shape[a]);
+    if (p.stride[a] > p.ksize[a])
+      return fail("fna_forward: stride exceeds kernel_size along dimension %d (%d > %d)", a, p.stride[a], p.ksize[a]);
+    if (qs[a] % p.q_tile[a] != 0 || ks[a] % p.kv_tile[a] != 0)
+      return fail("fna_forward: padded layouts must be multiples of the tile shapes (dimension %d)", a);
+    const int need = na_ceil_div(p.qkv_shape[a], p.dil[a]);
+    if (qs[a] < need || ks[a] < need)
+      return fail("fna_forward: q_shape / kv_shape smaller than the dilation group extent along dimension %d", a);
+    if (p.kv_tile[a] > 512) return fail("fna_forward: KV tile extent above 512 along dimension %d", a);
+    p.q_tiled[a] = qs[a] / p.q_tile[a];
+    p.kv_tiled[a] = ks[a] / p.kv_tile[a];
+    p.num_groups *= p.dil[a];
+  }
+  if (prod3(qs) != seqlen_q || prod3(ks) != seqlen_kv)
+    return fail("fna_forward: seqlen_q / seqlen_kv do not match q_shape / kv_shape (%d vs %d, %d vs %d)", prod3(qs),
+                seqlen_q, prod3(ks), seqlen_kv);
+  if (batch % p.num_groups != 0)
+    return fail("fna_forward: batch (%d) is not a multiple of the number of dilation groups (%d)", batch, p.num_groups);
+  p.q = q;
+  p.k = k;
+  p.v = v;
+  p.o = out;
+  p.lse = lse;
+  p.batch = batch;
+  p.heads_q = heads_q;
+  p.heads_kv = heads_kv;
+  p.seqlen_q = seqlen_q;
+  p.seqlen_kv = seqlen_kv;
+  p.scale = scale * q_scale * k_scale;
+  p.out_scale = v_scale;
+  return dispatch_dtype(p, dtype, head_dim, prod3(p.q_tile), prod3(p.kv_tile), static_cast<hipStream_t>(stream));
+}
+
+int natten_amd_attention_forward(const void* q, const void* k, const void* v, void* out, float* lse, int dtype,
+                                 int batch, int seqlen_q, int seqlen_kv, int heads_q, int heads_kv, int head_dim,
+                                 int is_causal, float scale, void* stream) {
+  g_error[0] = 0;
+  if (int rc = check_common("attention_forward", q, k, v, out, lse, batch, seqlen_q, seqlen_kv, heads_q, heads_kv,
+                            head_dim))
+    return rc;
+  // Dense attention is the 1-D neighborhood problem whose window is the whole key sequence:
+  // non-causal windows are [0, seqlen_kv), causal ones [0, min(i + 1, seqlen_kv)).
+  constexpr int QT = 128, KVT = 64;
+  FnaParams p;
+  memset(&p, 0, sizeof(p));
+  for (int a = 0; a < 3; ++a) {
+    p.qkv_shape[a] = p.ksize[a] = p.stride[a] = p.dil[a] = p.q_tile[a] = p.kv_tile[a] = p.q_tiled[a] = p.kv_tiled[a] = 1;
+  }
+  if (seqlen_kv < 2) {
+    // a one-key window is the unused-dimension case of the window arithmetic (k = 1)
+    p.ksize[0] = 1;
+  } else {
+    p.ksize[0] = seqlen_kv;
+  }
+  p.qkv_shape[0] = seqlen_kv;
+  p.causal[0] = is_causal != 0;
+  p.q_tile[0] = QT;
+  p.kv_tile[0] = KVT;
+  p.q_tiled[0] = na_ceil_div(seqlen_q, QT);
+  p.kv_tiled[0] = na_ceil_div(seqlen_kv, KVT);
+  p.num_groups = 1;
+  p.q = q;
+  p.k = k;
+  p.v = v;
+  p.o = out;
+  p.lse = lse;
+  p.batch = batch;
+  p.heads_q = heads_q;
+  p.heads_kv = heads_kv;
+  p.seqlen_q = seqlen_q;
+  p.seqlen_kv = seqlen_kv;
+  p.scale = scale;
+  p.out_scale = 1.f;
+  return dispatch_dtype(p, dtype, head_dim, QT, KVT, static_cast<hipStream_t>(stream));
+}
+
+static int tokperm_common(const char* what, bool unpermute, const void* src, void* dst, int elem_bytes, int na_dim,
+                          int batch, int heads, int head_dim, const int32_t* token_layout, const int32_t* tile_shape,
+                          const int32_t* dilation, int flip, void* stream) {
+  g_error[0] = 0;
+  if (!src || !dst) return fail("%s: null pointer argument", what);
+  if (na_dim < 1 || na_dim > 3) return fail("%s: na_dim must be 1, 2 or 3, got %d", what, na_dim);
+  if (elem_bytes != 1 && elem_bytes != 2 && elem_bytes != 4 && elem_bytes != 8)
+    return fail("%s: elem_bytes must be 1, 2, 4 or 8, got %d", what, elem_bytes);
+  if (batch < 1 || heads < 1 || head_dim < 1) return fail("%s: batch, heads and head_dim must be positive", what);
+  if (!token_layout || !tile_shape || !dilation) return fail("%s: null shape argument", what);
+  TokPermParams p;
+  memset(&p, 0, sizeof(p));
+  p.src = static_cast<const char*>(src);
+  p.dst = static_cast<char*>(dst);
+  p.na_dim = na_dim;
+  p.batch = batch;
+  p.num_groups = 1;
+  p.perm_len = 1;
+  p.orig_len = 1;
+  p.row_bytes = int64_t(heads) * head_dim * elem_bytes;
+  int R[3] = {1, 1, 1};
+  for (int a = 0; a < na_dim; ++a) {
+    if (token_layout[a] < 1 || tile_shape[a] < 1 || dilation[a] < 1)
+      return fail("%s: token_layout, tile_shape and dilation must be positive (dimension %d)", what, a);
+    p.layout[a] = token_layout[a];
+    p.tile[a] = tile_shape[a];
+    p.dil[a] = dilation[a];
+    R[a] = na_ceil_div(na_ceil_div(token_layout[a], tile_shape[a]), dilation[a]);
+    p.num_groups *= dilation[a];
+    p.perm_len *= int64_t(R[a]) * tile_shape[a];
+    p.orig_len *= token_layout[a];
+  }
+  for (int i = 0; i < na_dim; ++i) {
+    const int a = flip ? i : na_dim - 1 - i;  // slot i (fastest first) -> original dimension
+    p.t_dim[i] = a;
+    p.t_size[i] = p.tile[a];
+    p.r_size[i] = R[a];
+    p.g_size[i] = p.dil[a];
+  }
+  const uintptr_t align = reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst) | uintptr_t(p.row_bytes);
+  const int vec = (align % 16 == 0) ? 16 : (align % 4 == 0) ? 4 : (align % 2 == 0) ? 2 : 1;
+  const int64_t total = int64_t(batch) * p.num_groups * p.perm_len * (p.row_bytes / vec);
+  int64_t blocks = (total + 255) / 256;
+  const int64_t cap = 256 * 64;  // grid-stride beyond this many workgroups
+  if (blocks > cap) blocks = cap;
+  if (blocks < 1) blocks = 1;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+#define NA_TOKPERM_LAUNCH(VEC)                                                                    \
+  do {                                                                                            \
+    if (unpermute)                                                                                \
+      hipLaunchKernelGGL((tokperm_kernel<VEC, true>), dim3(unsigned(blocks)), dim3(256), 0, s, p);  \
+    else                                                                                          \
+      hipLaunchKernelGGL((tokperm_kernel<VEC, false>), dim3(unsigned(blocks)), dim3(256), 0, s, p); \
+  } while (0)
+  switch (vec) {
+    case 16: NA_TOKPERM_LAUNCH(16); break;
+    case 4: NA_TOKPERM_LAUNCH(4); break;
+    case 2: NA_TOKPERM_LAUNCH(2); break;
+    default: NA_TOKPERM_LAUNCH(1); break;
+  }
+#undef NA_TOKPERM_LAUNCH
+  return check_launch(what);
+}
+
+int natten_amd_token_permute(const void* src, void* dst, int elem_bytes, int na_dim, int batch, int heads,
+                             int head_dim, const int32_t* token_layout, const int32_t* tile_shape,
+                             const int32_t* dilation, int flip_tiled_dims, void* stream) {
+  return tokperm_common("token_permute", false, src, dst, elem_bytes, na_dim, batch, heads, head_dim, token_layout,
+                        tile_shape, dilation, flip_tiled_dims, stream);
+}
+
+int natten_amd_token_unpermute(const void* src, void* dst, int elem_bytes, int na_dim, int batch, int heads,
+                               int head_dim, const int32_t* token_layout, const int32_t* tile_shape,
+                               const int32_t* dilation, int flip_tiled_dims, void* stream) {
+  return tokperm_common("token_unpermute", true, src, dst, elem_bytes, na_dim, batch, heads, head_dim, token_layout,
+                        tile_shape, dilation, flip_tiled_dims, stream);
+}
+
+int natten_amd_merge_attentions(const void* o0, const float* lse0, const void* o1, const float* lse1, void* out,
+                                float* lse_out, int dtype, int64_t rows, int head_dim, void* stream) {
+  g_error[0] = 0;
+  if (!o0 || !lse0 || !o1 || !lse1 || !out || !lse_out) return fail("merge_attentions: null pointer argument");
+  if (rows < 1 || head_dim < 1) return fail("merge_attentions: rows and head_dim must be positive");
+  if (lse_out == lse0 || lse_out == lse1) return fail("merge_attentions: lse_out must not alias an input");
+  const int64_t total = rows * head_dim;
+  int64_t blocks = (total + 255) / 256;
+  if (blocks > 256 * 64) blocks = 256 * 64;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  switch (dtype) {
+    case NATTEN_AMD_F16:
+      hipLaunchKernelGGL(merge_kernel<_Float16>, dim3(unsigned(blocks)), dim3(256), 0, s,
+                         static_cast<const _Float16*>(o0), lse0, static_cast<const _Float16*>(o1), lse1,
+                         static_cast<_Float16*>(out), lse_out, rows, head_dim);
+      break;
+    case NATTEN_AMD_BF16:
+      hipLaunchKernelGGL(merge_kernel<__bf16>, dim3(unsigned(blocks)), dim3(256), 0, s, static_cast<const __bf16*>(o0),
+                         lse0, static_cast<const __bf16*>(o1), lse1, static_cast<__bf16*>(out), lse_out, rows,
+                         head_dim);
+      break;
+    case NATTEN_AMD_F32:
+      hipLaunchKernelGGL(merge_kernel<float>, dim3(unsigned(blocks)), dim3(256), 0, s, static_cast<const float*>(o0),
+                         lse0, static_cast<const float*>(o1), lse1, static_cast<float*>(out), lse_out, rows, head_dim);
+      break;
+    default:
+      return fail("merge_attentions: unsupported dtype code %d", dtype);
+  }
+  return check_launch("merge_attentions");
+}
+
+}  // extern "C"

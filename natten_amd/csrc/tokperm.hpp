@@ -1,0 +1,92 @@
+// Token permute / unpermute for gfx950: a coalesced row gather / scatter.
+//
+// Index map restated from SHI-Labs/NATTEN
+//   src/natten/token_permute/torch_impl.py:99-187 (view [B, (R, t, d) per dim, H, Dh], permute to
+//       [B, d..., R..., t..., H, Dh], dimension order reversed inside each kind when flipping)
+//   csrc/include/natten/cuda/tokperm/token_permute_kernel.cuh:40-163 (coordinate maps),
+//   :338-340 (padding is written as zero)
+// One kernel serves both directions: it walks the permuted index space, decodes the original
+// coordinate, and copies one token row (heads * head_dim elements, contiguous on both sides).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace natten_amd {
+
+struct TokPermParams {
+  const char* src;
+  char* dst;
+  int na_dim;
+  int batch;            // original batch
+  int num_groups;       // prod(dilation)
+  int64_t perm_len;     // tokens per (batch, group) in the permuted layout
+  int64_t orig_len;     // tokens per batch in the original layout
+  int64_t row_bytes;    // heads * head_dim * elem_bytes
+  // decode order, fastest first: the `na_dim` tile offsets, then the `na_dim` tile indices
+  int t_size[3], r_size[3], t_dim[3];  // t_dim[i]: which original dimension slot i refers to
+  int g_size[3];                       // dilation, fastest first, same slot -> dim mapping
+  int layout[3], tile[3], dil[3];      // by original dimension
+};
+
+// VEC = bytes moved per thread per step (16, 4, 2 or 1)
+template <int VEC, bool UNPERMUTE>
+__global__ void __launch_bounds__(256) tokperm_kernel(const TokPermParams p) {
+  const int64_t chunks_per_row = p.row_bytes / VEC;
+  const int64_t total = int64_t(p.batch) * p.num_groups * p.perm_len * chunks_per_row;
+  for (int64_t idx = int64_t(blockIdx.x) * 256 + threadIdx.x; idx < total; idx += int64_t(gridDim.x) * 256) {
+    const int64_t tok = idx / chunks_per_row;
+    const int64_t chunk = idx - tok * chunks_per_row;
+    const int64_t bgi = tok / p.perm_len;
+    int64_t pos = tok - bgi * p.perm_len;
+    const int b = int(bgi / p.num_groups);
+    int gl = int(bgi - int64_t(b) * p.num_groups);
+    int tau[3] = {0, 0, 0}, rr[3] = {0, 0, 0}, dl[3] = {0, 0, 0};
+#pragma unroll
+    for (int i = 0; i < 3; ++i)
+      if (i < p.na_dim) {
+        tau[p.t_dim[i]] = int(pos % p.t_size[i]);
+        pos /= p.t_size[i];
+      }
+#pragma unroll
+    for (int i = 0; i < 3; ++i)
+      if (i < p.na_dim) {
+        rr[p.t_dim[i]] = int(pos % p.r_size[i]);
+        pos /= p.r_size[i];
+        dl[p.t_dim[i]] = gl % p.g_size[i];
+        gl /= p.g_size[i];
+      }
+    bool inside = true;
+    int64_t lin = 0;
+#pragma unroll
+    for (int a = 0; a < 3; ++a)
+      if (a < p.na_dim) {
+        const int x = rr[a] * (p.tile[a] * p.dil[a]) + tau[a] * p.dil[a] + dl[a];
+        inside = inside && (x < p.layout[a]);
+        lin = lin * p.layout[a] + x;
+      }
+    const int64_t perm_off = tok * p.row_bytes + chunk * VEC;
+    const int64_t orig_off = (int64_t(b) * p.orig_len + lin) * p.row_bytes + chunk * VEC;
+    if constexpr (VEC == 16) {
+      typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+      if constexpr (UNPERMUTE) {
+        if (inside) *reinterpret_cast<u4*>(p.dst + orig_off) = *reinterpret_cast<const u4*>(p.src + perm_off);
+      } else {
+        u4 val = {0, 0, 0, 0};
+        if (inside) val = *reinterpret_cast<const u4*>(p.src + orig_off);
+        *reinterpret_cast<u4*>(p.dst + perm_off) = val;
+      }
+    } else {
+      using E = typename std::conditional<VEC == 4, uint32_t, typename std::conditional<VEC == 2, uint16_t, uint8_t>::type>::type;
+      if constexpr (UNPERMUTE) {
+        if (inside) *reinterpret_cast<E*>(p.dst + orig_off) = *reinterpret_cast<const E*>(p.src + perm_off);
+      } else {
+        E val = 0;
+        if (inside) val = *reinterpret_cast<const E*>(p.src + orig_off);
+        *reinterpret_cast<E*>(p.dst + perm_off) = val;
+      }
+    }
+  }
+}
+
+}  // namespace natten_amd

@@ -1,0 +1,40 @@
+"""Dense attention forward on MI355X (the callee for additional keys/values and for
+kernel_size == input size).  Counterpart of the forward half of the reference's
+src/natten/backends/blackwell_fmha.py; variable-length batches are not implemented."""
+
+from __future__ import annotations
+
+from typing import Optional, Tuple, Union
+
+import torch
+from torch import Tensor
+
+from . import _lib
+from .checks import fmha_tensor_checks
+from .fna import SUPPORTED_DTYPES, _pad_head_dim
+from .tile_config import padded_head_dim
+
+
+def amd_fmha(
+    query: Tensor, key: Tensor, value: Tensor, is_causal: bool = False, scale: Optional[float] = None,
+    return_lse: bool = False,
+) -> Union[Tensor, Tuple[Tensor, Tensor]]:
+    fmha_tensor_checks(query, key, value, must_match_head_dims=True)
+    if not query.is_cuda:
+        raise NotImplementedError(f"natten_amd runs on MI355X device tensors only; got a tensor on {query.device}.")
+    if query.dtype not in SUPPORTED_DTYPES:
+        raise NotImplementedError(f"natten_amd attention supports {SUPPORTED_DTYPES}, got {query.dtype}.")
+    head_dim = query.shape[-1]
+    if head_dim > 128 or head_dim % 8 != 0:
+        raise NotImplementedError(f"natten_amd attention supports head_dim <= 128, multiple of 8; got {head_dim}.")
+    if torch.is_grad_enabled() and (query.requires_grad or key.requires_grad or value.requires_grad):
+        raise NotImplementedError("natten_amd implements the forward pass only; call it under torch.no_grad().")
+    scale = scale or head_dim**-0.5
+    d_pad = padded_head_dim(head_dim)
+    q, k, v = (_pad_head_dim(t.contiguous(), d_pad).contiguous() for t in (query, key, value))
+    out, lse = _lib.attention_forward(q, k, v, bool(is_causal), scale)
+    if d_pad != head_dim:
+        out = out[..., :head_dim].contiguous()
+    if return_lse:
+        return out, lse
+    return out

@@ -1,0 +1,98 @@
+"""Driver of the MI355X fused neighborhood attention forward:
+token permute -> fused kernel -> token unpermute (output and LSE).
+
+Forward half of the reference's src/natten/backends/blackwell_fna.py:90-165 and :332-407.
+"""
+
+from __future__ import annotations
+
+from typing import Optional, Tuple, Union
+
+import torch
+from torch import Tensor
+
+from . import _lib
+from .checks import check_all_args, check_args_against_input, na_tensor_checks
+from .tile_config import check_fna_forward_config, padded_head_dim
+from .token_permute import token_permute_operation, token_unpermute_operation
+
+SUPPORTED_DTYPES = (torch.float16, torch.bfloat16)
+
+
+def can_run_amd_fna(query: Tensor, key: Tensor, value: Tensor, raise_error: bool = False) -> bool:
+    """MI355X capability check (counterpart of can_run_cutlass_blackwell_fna,
+    src/natten/backends/configs/checks.py:143-251)."""
+
+    def no(msg: str, exc=NotImplementedError) -> bool:
+        if raise_error:
+            raise exc(msg)
+        return False
+
+    if not query.is_cuda:
+        return no("natten_amd runs on MI355X device tensors only; got a tensor on " + str(query.device) + ".")
+    if not _lib.has_lib():
+        return no("natten_amd native library is not built (python -m natten_amd.build).", ImportError)
+    if query.dtype not in SUPPORTED_DTYPES:
+        return no(f"natten_amd FNA supports {SUPPORTED_DTYPES}, got {query.dtype}.")
+    if query.shape[-1] != value.shape[-1]:
+        return no("natten_amd FNA does not support different head dims for QK and V.", ValueError)
+    if query.shape[-1] > 128 or query.shape[-1] % 8 != 0:
+        return no(f"natten_amd FNA supports head_dim <= 128 that is a multiple of 8, got {query.shape[-1]}.")
+    if query.requires_grad or key.requires_grad or value.requires_grad:
+        if torch.is_grad_enabled():
+            return no("natten_amd implements the forward pass only; call it under torch.no_grad().")
+    return True
+
+
+def _pad_head_dim(x: Tensor, d_to: int) -> Tensor:
+    if x.shape[-1] == d_to:
+        return x
+    return torch.nn.functional.pad(x, (0, d_to - x.shape[-1]))
+
+
+def amd_fna_generic(
+    query: Tensor,
+    key: Tensor,
+    value: Tensor,
+    kernel_size,
+    stride=1,
+    dilation=1,
+    is_causal=False,
+    scale: Optional[float] = None,
+    q_tile_shape=None,
+    kv_tile_shape=None,
+    return_lse: bool = False,
+) -> Union[Tensor, Tuple[Tensor, Tensor]]:
+    na_tensor_checks(query, key, value, must_match_head_dims=True)
+    can_run_amd_fna(query, key, value, raise_error=True)
+    na_dim = query.dim() - 3
+    kernel_size, stride, dilation, is_causal = check_all_args(na_dim, kernel_size, stride, dilation, is_causal)
+    check_args_against_input(query, kernel_size, stride, dilation, is_causal)
+    q_tile_shape, kv_tile_shape = check_fna_forward_config(
+        query, kernel_size, stride, dilation, is_causal, q_tile_shape, kv_tile_shape
+    )
+    head_dim = query.shape[-1]
+    scale = scale or head_dim**-0.5
+    d_pad = padded_head_dim(head_dim)
+    if d_pad != head_dim:
+        # zero columns change neither q.k nor the first head_dim output columns
+        query, key, value = (_pad_head_dim(t, d_pad) for t in (query, key, value))
+
+    q_perm, qkv_shape, q_shape = token_permute_operation(query, q_tile_shape, dilation, flip_tiled_dims=True)
+    k_perm, _, kv_shape = token_permute_operation(key, kv_tile_shape, dilation, flip_tiled_dims=True)
+    v_perm, _, _ = token_permute_operation(value, kv_tile_shape, dilation, flip_tiled_dims=True)
+
+    out_perm, lse_perm = _lib.fna_forward(
+        q_perm, k_perm, v_perm, kernel_size, stride, dilation, is_causal, scale,
+        q_shape, kv_shape, qkv_shape, q_tile_shape, kv_tile_shape,
+    )
+
+    output = token_unpermute_operation(out_perm, qkv_shape, q_tile_shape, dilation, flip_tiled_dims=True)
+    lse = token_unpermute_operation(
+        lse_perm.unsqueeze(-1), qkv_shape, q_tile_shape, dilation, flip_tiled_dims=True
+    ).squeeze(-1)
+    if d_pad != head_dim:
+        output = output[..., :head_dim].contiguous()
+    if return_lse:
+        return output, lse
+    return output

@@ -1,0 +1,202 @@
+"""Public operations: attention, na1d, na2d, na3d.
+
+Mirrors the reference's src/natten/functional.py (attention :74-348,
+neighborhood_attention_generic :354-564, na1d/na2d/na3d :567-1151): same signatures, same
+argument rules and error classes, same self-attention fast path and additional-KV merge.
+There is one backend (the MI355X kernels); the reference's NVIDIA-only performance arguments are
+accepted and ignored, except `q_tile_shape` / `kv_tile_shape`, which select the kernel's tiles.
+"""
+
+from __future__ import annotations
+
+from typing import Dict, Optional, Tuple, Union
+
+import torch
+from torch import Tensor
+
+from .attn_merge import merge_attentions
+from .checks import (
+    additional_kv_tensor_checks,
+    check_all_args,
+    check_args_against_input,
+    is_self_attention,
+    na_tensor_checks,
+)
+from .fmha import amd_fmha
+from .fna import amd_fna_generic
+
+_BACKEND_FNA = "amd-fna"
+_BACKEND_FMHA = "amd-fmha"
+
+
+def attention(
+    query: Tensor,
+    key: Tensor,
+    value: Tensor,
+    is_causal: bool = False,
+    scale: Optional[float] = None,
+    # varlen parameters
+    seqlens_Q: Optional[Tensor] = None,
+    seqlens_KV: Optional[Tensor] = None,
+    cumulative_seqlen_Q: Optional[Tensor] = None,
+    cumulative_seqlen_KV: Optional[Tensor] = None,
+    max_seqlen_Q: Optional[int] = None,
+    max_seqlen_KV: Optional[int] = None,
+    # backend parameters
+    backend: Optional[str] = None,
+    q_tile_size: Optional[int] = None,
+    kv_tile_size: Optional[int] = None,
+    backward_q_tile_size: Optional[int] = None,
+    backward_kv_tile_size: Optional[int] = None,
+    backward_kv_splits: Optional[int] = None,
+    backward_use_pt_reduction: bool = False,
+    run_persistent_kernel: bool = True,
+    kernel_schedule=None,
+    torch_compile: bool = False,
+    return_lse: bool = False,
+) -> Union[Tensor, Tuple[Tensor, Tensor]]:
+    """Dot product attention on `[batch, seqlen, heads, head_dim]` tensors (heads last).
+
+    `is_causal` is top-left aligned.  Returns the output, and the float32 logsumexp
+    `[batch, seqlen, heads]` when `return_lse=True`.
+    """
+    if any(x is not None for x in (seqlens_Q, seqlens_KV, cumulative_seqlen_Q, cumulative_seqlen_KV)) or any(
+        x not in (None, 0) for x in (max_seqlen_Q, max_seqlen_KV)
+    ):
+        raise NotImplementedError("natten_amd does not implement variable-length attention.")
+    if backend not in (None, _BACKEND_FMHA):
+        raise NotImplementedError(f"Unrecognized attention backend {backend}; natten_amd provides '{_BACKEND_FMHA}'.")
+    return amd_fmha(query, key, value, is_causal=is_causal, scale=scale, return_lse=return_lse)
+
+
+def neighborhood_attention_generic(
+    query: Tensor,
+    key: Tensor,
+    value: Tensor,
+    kernel_size,
+    stride=1,
+    dilation=1,
+    is_causal=False,
+    scale: Optional[float] = None,
+    additional_keys: Optional[Tensor] = None,
+    additional_values: Optional[Tensor] = None,
+    attention_kwargs: Optional[Dict] = None,
+    # Perf-related args
+    backend: Optional[str] = None,
+    q_tile_shape=None,
+    kv_tile_shape=None,
+    backward_q_tile_shape=None,
+    backward_kv_tile_shape=None,
+    backward_kv_splits=None,
+    backward_use_pt_reduction: bool = False,
+    run_persistent_kernel: bool = True,
+    kernel_schedule=None,
+    torch_compile: bool = False,
+    return_lse: bool = False,
+) -> Union[Tensor, Tuple[Tensor, Tensor]]:
+    na_tensor_checks(query, key, value)
+    additional_kv_tensor_checks(query, key, value, additional_keys, additional_values)
+    na_dim = query.dim() - 3
+    kernel_size, stride, dilation, is_causal = check_all_args(na_dim, kernel_size, stride, dilation, is_causal)
+    check_args_against_input(query, kernel_size=kernel_size, stride=stride, dilation=dilation, is_causal=is_causal)
+    if backend not in (None, _BACKEND_FNA):
+        raise NotImplementedError(f"Unrecognized backend {backend}; natten_amd provides '{_BACKEND_FNA}'.")
+
+    has_additional_attention = additional_keys is not None and additional_values is not None
+    attn_kwargs = dict(attention_kwargs or {})
+    attn_kwargs.pop("torch_compile", None)
+
+    if is_self_attention(query, kernel_size=kernel_size, is_causal=is_causal,
+                         has_additional_attention=has_additional_attention):
+        # a window covering the whole input is plain attention over the flattened tokens
+        query_shape = query.shape
+        q = query.flatten(1, na_dim)
+        k = key.flatten(1, na_dim)
+        v = value.flatten(1, na_dim)
+        if has_additional_attention:
+            k = torch.cat([k, additional_keys], dim=1)
+            v = torch.cat([v, additional_values], dim=1)
+        out, lse = attention(q, k, v, is_causal=is_causal[0], scale=scale, return_lse=True, **attn_kwargs)
+        lse_shape = list(query_shape[:-1])
+        out = out.reshape(*lse_shape, v.shape[-1])
+        lse = lse.reshape(*lse_shape)
+        return (out, lse) if return_lse else out
+
+    scale = scale or query.shape[-1] ** -0.5
+    output, lse = amd_fna_generic(
+        query, key, value, kernel_size=kernel_size, stride=stride, dilation=dilation, is_causal=is_causal,
+        scale=scale, q_tile_shape=q_tile_shape, kv_tile_shape=kv_tile_shape, return_lse=True,
+    )
+
+    if has_additional_attention:
+        add_out, add_lse = attention(
+            query.flatten(1, na_dim), additional_keys, additional_values, is_causal=False, scale=scale,
+            return_lse=True, **attn_kwargs,
+        )
+        merged_out, merged_lse = merge_attentions(
+            [output.flatten(1, na_dim), add_out], [lse.flatten(1, na_dim), add_lse]
+        )
+        output = merged_out.reshape(output.shape)
+        lse = merged_lse.reshape(output.shape[:-1])
+
+    return (output, lse) if return_lse else output
+
+
+def _make_na(na_dim: int, name: str):
+    def op(
+        query: Tensor,
+        key: Tensor,
+        value: Tensor,
+        kernel_size,
+        stride=1,
+        dilation=1,
+        is_causal=False,
+        scale: Optional[float] = None,
+        additional_keys: Optional[Tensor] = None,
+        additional_values: Optional[Tensor] = None,
+        attention_kwargs: Optional[Dict] = None,
+        backend: Optional[str] = None,
+        q_tile_shape=None,
+        kv_tile_shape=None,
+        backward_q_tile_shape=None,
+        backward_kv_tile_shape=None,
+        backward_kv_splits=None,
+        backward_use_pt_reduction: bool = False,
+        run_persistent_kernel: bool = True,
+        kernel_schedule=None,
+        torch_compile: bool = False,
+        return_lse: bool = False,
+    ) -> Union[Tensor, Tuple[Tensor, Tensor]]:
+        if query.dim() != na_dim + 3:
+            raise ValueError(
+                f"{name} expects rank-{na_dim + 3} tensors [batch, {'*' if na_dim > 1 else ''}tokens, heads, head_dim], "
+                f"got rank {query.dim()}."
+            )
+        return neighborhood_attention_generic(
+            query=query, key=key, value=value, kernel_size=kernel_size, stride=stride, dilation=dilation,
+            is_causal=is_causal, scale=scale, additional_keys=additional_keys, additional_values=additional_values,
+            attention_kwargs=attention_kwargs, backend=backend, q_tile_shape=q_tile_shape,
+            kv_tile_shape=kv_tile_shape, backward_q_tile_shape=backward_q_tile_shape,
+            backward_kv_tile_shape=backward_kv_tile_shape, backward_kv_splits=backward_kv_splits,
+            backward_use_pt_reduction=backward_use_pt_reduction, run_persistent_kernel=run_persistent_kernel,
+            kernel_schedule=kernel_schedule, torch_compile=torch_compile, return_lse=return_lse,
+        )
+
+    op.__name__ = name
+    op.__qualname__ = name
+    op.__doc__ = (
+        f"{na_dim}-D neighborhood attention on heads-last tensors "
+        f"`[batch, {', '.join('XYZ'[:na_dim])}, heads, head_dim]`.\n\n"
+        "kernel_size, stride, dilation: int or tuple per dimension (kernel_size >= 2, stride <= kernel_size, "
+        "kernel_size * dilation <= input size); is_causal: bool or tuple.  additional_keys / additional_values "
+        "`[batch, seqlen, heads_kv, head_dim]` add context every query attends to.  Returns the output and, with "
+        "`return_lse=True`, the float32 logsumexp `[batch, *tokens, heads]`."
+    )
+    return op
+
+
+na1d = _make_na(1, "na1d")
+na2d = _make_na(2, "na2d")
+na3d = _make_na(3, "na3d")
+
+__all__ = ["attention", "na1d", "na2d", "na3d", "neighborhood_attention_generic"]

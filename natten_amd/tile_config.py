@@ -1,0 +1,132 @@
+"""Tile shapes of the MI355X FNA forward kernel.
+
+Plays the role of the reference's per-architecture tables and validators
+(src/natten/backends/configs/cutlass_blackwell/__init__.py:44-63, :90-102, :208-256): the
+kernel is instantiated for a few (Q tile, KV tile) token counts; a multi-dimensional tile
+shape is any factorisation of those counts.  The default picks, per problem, the
+factorisation that minimises the (query, key) pairs the kernel visits (padding and partially
+masked tiles included), which is separable per dimension and therefore cheap to search.
+"""
+
+from __future__ import annotations
+
+import functools
+import math
+from typing import List, Optional, Tuple
+
+import torch
+
+DimensionType = Tuple[int, ...]
+
+# (Q tile tokens, KV tile tokens) with a kernel instance; first entry = default.
+TILE_SIZES: List[Tuple[int, int]] = [(128, 64), (256, 64), (128, 128), (256, 128), (64, 64)]
+SUPPORTED_HEAD_DIMS = (32, 64, 128)
+
+
+def padded_head_dim(head_dim: int) -> int:
+    for d in SUPPORTED_HEAD_DIMS:
+        if head_dim <= d:
+            return d
+    raise NotImplementedError(f"natten_amd supports head_dim <= 128, got {head_dim}.")
+
+
+def _ceil_div(a: int, b: int) -> int:
+    return (a + b - 1) // b
+
+
+def _win(i: int, k: int, s: int, L: int, causal: bool) -> Tuple[int, int]:
+    wl, wr = k // 2, k // 2 + (k % 2 - 1)
+    if causal:
+        leader = min((i // s) * s + s - 1, L - 1)
+        return max(leader - wl - wr, 0), min(i + 1, L)
+    leader = min((i // s) * s + s // 2, L - 1)
+    st = max(leader - wl, 0) + ((L - wr - leader - 1) if leader + wr >= L else 0)
+    return st, st + k
+
+
+@functools.lru_cache(maxsize=4096)
+def _dim_cost(L: int, k: int, s: int, causal: bool, tq: int, tk: int) -> Tuple[int, int]:
+    """(visited pairs, fully-unmasked pairs) along one dimension of extent L for Q tile extent tq
+    and KV tile extent tk; the totals of a multi-dimensional problem are products of these."""
+    visited = full = 0
+    for q0 in range(0, _ceil_div(L, tq) * tq, tq):
+        st_f, en_f = _win(q0, k, s, L, causal)
+        st_l, en_l = _win(q0 + tq - 1, k, s, L, causal)
+        t0, t1 = st_f // tk, _ceil_div(en_l, tk)
+        visited += (t1 - t0) * tk * tq
+        for t in range(t0, t1):
+            if t * tk >= st_l and (t + 1) * tk <= en_f:
+                full += tk * tq
+    return visited, full
+
+
+def _factorisations(total: int, n: int) -> List[DimensionType]:
+    if n == 1:
+        return [(total,)]
+    out = []
+    f = 1
+    while f <= total:
+        if total % f == 0:
+            out += [(f,) + rest for rest in _factorisations(total // f, n - 1)]
+        f *= 2
+    return out
+
+
+@functools.lru_cache(maxsize=1024)
+def choose_tile_shapes(
+    token_layout: DimensionType, kernel_size: DimensionType, stride: DimensionType, dilation: DimensionType,
+    is_causal: Tuple[bool, ...], q_size: int, kv_size: int,
+) -> Tuple[DimensionType, DimensionType]:
+    n = len(token_layout)
+    ext = tuple(_ceil_div(x, d) for x, d in zip(token_layout, dilation))
+    best, best_cost = None, None
+    for qt in _factorisations(q_size, n):
+        for kt in _factorisations(kv_size, n):
+            visited = full = 1
+            for a in range(n):
+                v, f = _dim_cost(ext[a], kernel_size[a], stride[a], is_causal[a], qt[a], kt[a])
+                visited *= v
+                full *= f
+            cost = visited + 0.3 * (visited - full)
+            # ties: prefer tiles that are long in the last (memory-contiguous) dimensions
+            key = (cost, tuple(-x for x in reversed(qt)), tuple(-x for x in reversed(kt)))
+            if best_cost is None or key < best_cost:
+                best, best_cost = (qt, kt), key
+    assert best is not None
+    return best
+
+
+def check_fna_forward_config(
+    input_tensor: torch.Tensor, kernel_size: DimensionType, stride: DimensionType, dilation: DimensionType,
+    is_causal: Tuple[bool, ...], q_tile_shape: Optional[DimensionType] = None,
+    kv_tile_shape: Optional[DimensionType] = None,
+) -> Tuple[DimensionType, DimensionType]:
+    """Validate user tile shapes or choose defaults.  Raises ValueError for unsupported shapes."""
+    na_dim = input_tensor.dim() - 3
+    layout = tuple(int(x) for x in input_tensor.shape[1 : 1 + na_dim])
+    if (q_tile_shape is None) != (kv_tile_shape is None):
+        raise ValueError("`q_tile_shape` and `kv_tile_shape` must be given together or not at all.")
+    if q_tile_shape is None:
+        q_size, kv_size = TILE_SIZES[0]
+        return choose_tile_shapes(layout, tuple(kernel_size), tuple(stride), tuple(dilation), tuple(is_causal), q_size, kv_size)
+    from .checks import check_tile_shape
+
+    q_tile_shape = check_tile_shape(q_tile_shape, na_dim, "q_tile_shape")
+    kv_tile_shape = check_tile_shape(kv_tile_shape, na_dim, "kv_tile_shape")
+    sizes = (math.prod(q_tile_shape), math.prod(kv_tile_shape))
+    if sizes not in TILE_SIZES:
+        raise ValueError(
+            f"Unsupported tile shapes {q_tile_shape=}, {kv_tile_shape=} ({sizes[0]} x {sizes[1]} tokens); "
+            f"supported (Q tile, KV tile) token counts are {TILE_SIZES}."
+        )
+    return q_tile_shape, kv_tile_shape
+
+
+def get_all_tile_shapes(na_dim: int) -> List[Tuple[DimensionType, DimensionType]]:
+    """Every legal (q_tile_shape, kv_tile_shape) for an na_dim-dimensional problem."""
+    out = []
+    for q_size, kv_size in TILE_SIZES:
+        for qt in _factorisations(q_size, na_dim):
+            for kt in _factorisations(kv_size, na_dim):
+                out.append((qt, kt))
+    return out

@@ -1,0 +1,115 @@
+"""GPU parity: fused neighborhood attention forward through the public API (which goes through
+the C ABI), against the CPU oracle on the same seeded inputs.  Tolerance atol = rtol = 1e-2."""
+
+import itertools
+
+import numpy as np
+import pytest
+import torch
+
+import natten_amd
+from tests import problems
+from tests.gpu_utils import assert_close, make_qkv, oracle_full, to_np, tuplify
+
+pytestmark = pytest.mark.gpu
+
+NA = {1: natten_amd.na1d, 2: natten_amd.na2d, 3: natten_amd.na3d}
+
+
+def run_case(B, H, Hkv, D, shape, k, s, d, causal, dtype, q_tile=None, kv_tile=None, seed=0, std=1.0):
+    n = len(shape)
+    k, s, d, causal = (tuplify(x, n) for x in (k, s, d, causal))
+    q, kk, v = make_qkv(B, shape, H, Hkv, D, dtype, seed=seed, std=std)
+    with torch.no_grad():
+        out, lse = NA[n](q, kk, v, k, s, d, causal, q_tile_shape=q_tile, kv_tile_shape=kv_tile, return_lse=True)
+    torch.cuda.synchronize()
+    assert out.shape == q.shape and out.dtype == dtype
+    assert lse.shape == q.shape[:-1] and lse.dtype == torch.float32
+    ref_o, ref_l = oracle_full(q, kk, v, k, s, d, causal)
+    tag = f"{shape} k={k} s={s} d={d} c={causal} {dtype} tiles={q_tile},{kv_tile}"
+    assert_close("out " + tag, to_np(out), ref_o)
+    assert_close("lse " + tag, to_np(lse), ref_l)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_config1_shape_na1d(dtype):
+    # BASELINE config 1's problem (B=1, heads=2, L=256, D=32, k=7) on the GPU path
+    run_case(1, 2, 2, 32, (256,), 7, 1, 1, False, dtype)
+
+
+@pytest.mark.parametrize("dil", [(1, 1), (2, 2)])
+def test_config2_na2d_bf16(dil):
+    run_case(2, 8, 8, 64, (64, 64), (13, 13), (1, 1), dil, False, torch.bfloat16)
+
+
+@pytest.mark.parametrize("D", [32, 64, 128])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_head_dims_and_dtypes_2d(D, dtype):
+    run_case(1, 2, 2, D, (20, 24), (5, 7), (2, 1), (1, 2), (False, True), dtype)
+
+
+@pytest.mark.parametrize("sizes", [(128, 64), (256, 64), (128, 128), (256, 128), (64, 64)])
+def test_every_tile_size_3d(sizes):
+    qt = {128: (2, 8, 8), 256: (4, 8, 8), 64: (1, 8, 8)}[sizes[0]]
+    kt = {64: (1, 8, 8), 128: (2, 8, 8)}[sizes[1]]
+    run_case(1, 2, 1, 64, (9, 16, 24), (4, 8, 8), (1, 8, 4), 1, (True, False, False), torch.bfloat16, qt, kt)
+
+
+def test_reference_1d_problems():
+    for i, (B, H, Hkv, D, shape, k, s, d) in enumerate(problems.NA_1D):
+        for causal in (False, True):
+            run_case(B, H, Hkv, D, shape, k, s, d, (causal,), torch.float16, seed=i)
+
+
+def test_reference_2d_problems():
+    for i, (B, H, Hkv, D, shape, k, s, d) in enumerate(problems.NA_2D):
+        for causal in itertools.product([False, True], repeat=2):
+            run_case(B, H, Hkv, D, shape, k, s, d, causal, torch.bfloat16, seed=i)
+
+
+def test_reference_3d_problems():
+    for i, (B, H, Hkv, D, shape, k, s, d) in enumerate(problems.NA_3D):
+        if int(np.prod(shape)) > 40000:
+            continue  # covered by sampled checks in test_gpu_configs.py
+        for causal in [(False, False, False), (True, False, True), (True, True, True)]:
+            run_case(B, H, Hkv, D, shape, k, s, d, causal, torch.bfloat16, seed=i)
+
+
+def test_random_sweep():
+    rng = np.random.default_rng(2024)
+    done = 0
+    while done < 40:
+        n = int(rng.integers(1, 4))
+        shape = tuple(int(rng.integers(4, {1: 300, 2: 40, 3: 14}[n])) for _ in range(n))
+        d = tuple(int(rng.integers(1, max(2, x // 4 + 1))) for x in shape)
+        if any(x // dd < 2 for x, dd in zip(shape, d)):
+            continue
+        k = tuple(int(rng.integers(2, x // dd + 1)) for x, dd in zip(shape, d))
+        s = tuple(int(rng.integers(1, kk + 1)) for kk in k)
+        causal = tuple(bool(rng.integers(0, 2)) for _ in range(n))
+        Hkv = int(rng.choice([1, 2]))
+        H = Hkv * int(rng.choice([1, 2]))
+        D = int(rng.choice([32, 64, 128]))
+        dtype = [torch.bfloat16, torch.float16][done % 2]
+        tiles = natten_amd.get_all_tile_shapes(n)
+        qt, kt = tiles[int(rng.integers(0, len(tiles)))]
+        run_case(1, H, Hkv, D, shape, k, s, d, causal, dtype, qt, kt, seed=done)
+        done += 1
+
+
+def test_argument_errors():
+    q = torch.randn(1, 16, 16, 2, 32, dtype=torch.bfloat16).cuda()
+    with pytest.raises(ValueError):
+        natten_amd.na2d(q, q, q, kernel_size=1)
+    with pytest.raises(ValueError):
+        natten_amd.na2d(q, q, q, kernel_size=(3, 3), stride=(4, 1))
+    with pytest.raises(ValueError):
+        natten_amd.na2d(q, q, q, kernel_size=(9, 9), dilation=(2, 2))
+    with pytest.raises(ValueError):
+        natten_amd.na1d(q, q, q, kernel_size=3)
+    with pytest.raises(ValueError):
+        natten_amd.na2d(q, q, q, kernel_size=3, q_tile_shape=(3, 5), kv_tile_shape=(8, 8))
+    with pytest.raises(NotImplementedError):
+        natten_amd.na2d(q.float(), q.float(), q.float(), kernel_size=3)
+    with pytest.raises(NotImplementedError):
+        natten_amd.na2d(q.cpu(), q.cpu(), q.cpu(), kernel_size=3)

@@ -1,0 +1,112 @@
+"""Host-side checks that need no GPU: the C-ABI library loads and exports every symbol the
+header declares, argument validation raises the reference's exception classes, tile choice."""
+
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+import natten_amd
+from natten_amd import _lib, checks, tile_config
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "natten_amd.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(natten_amd_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = _declared_symbols()
+    assert len(names) >= 8
+    assert os.path.exists(_lib.LIB_PATH), "libnatten_amd.so is not built (python -m natten_amd.build)"
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in include/natten_amd.h but not exported"
+    assert sorted(_lib.EXPORTED_SYMBOLS) == names
+    assert lib.natten_amd_abi_version() == _lib.ABI_VERSION
+
+
+def test_supported_tiles_query_matches_python_table():
+    for dt in (torch.float16, torch.bfloat16):
+        for d in (32, 64, 128):
+            assert _lib.supported_tile_sizes(dt, d) == tile_config.TILE_SIZES
+    assert _lib.supported_tile_sizes(torch.float16, 48) == []
+
+
+def test_argument_normalisation_and_errors():
+    assert checks.check_all_args(2, 3, None, None, None) == ((3, 3), (1, 1), (1, 1), (False, False))
+    assert checks.check_all_args(3, (3, 4, 5), 2, (1, 2, 3), (True, False, True)) == (
+        (3, 4, 5), (2, 2, 2), (1, 2, 3), (True, False, True))
+    for bad in (1, (3,), (3, 1), 3.0, "3"):
+        with pytest.raises(ValueError):
+            checks.check_kernel_size_arg(2, bad)
+    with pytest.raises(ValueError):
+        checks.check_stride_arg(2, 0)
+    with pytest.raises(ValueError):
+        checks.check_dilation_arg(1, (1, 1))
+    with pytest.raises(ValueError):
+        checks.check_causal_arg(2, (True,))
+    with pytest.raises(ValueError):
+        checks.check_causal_arg(2, 1)
+
+
+def test_tensor_checks():
+    q = torch.zeros(1, 8, 8, 4, 16)
+    checks.na_tensor_checks(q, q, q)
+    with pytest.raises(ValueError):
+        checks.na_tensor_checks(q, q[:, :4], q)  # token layout mismatch
+    with pytest.raises(ValueError):
+        checks.na_tensor_checks(q, q[..., :3, :], q)  # K and V heads differ
+    with pytest.raises(ValueError):
+        checks.na_tensor_checks(q, q[..., :3, :], q[..., :3, :])  # 3 does not divide 4
+    checks.na_tensor_checks(q, q[..., :2, :], q[..., :2, :])  # GQA
+    with pytest.raises(ValueError):
+        checks.na_tensor_checks(q, q.half(), q)
+    with pytest.raises(ValueError):
+        checks.na_tensor_checks(q[0], q[0], q[0])  # rank 4 is fine, rank 3 is not
+        checks.na_tensor_checks(q[0, 0], q[0, 0], q[0, 0])
+    with pytest.raises(ValueError):
+        checks.check_args_against_input(q, (5, 5), (1, 1), (2, 2), (False, False))
+    with pytest.raises(ValueError):
+        checks.check_args_against_input(q, (3, 3), (4, 1), (1, 1), (False, False))
+    with pytest.raises(ValueError):
+        checks.additional_kv_tensor_checks(q, q, q, torch.zeros(1, 5, 4, 16), None)
+
+
+def test_is_self_attention_rules():
+    q1 = torch.zeros(1, 16, 2, 8)
+    assert checks.is_self_attention(q1, (16,), (True,), False)  # 1-D full window, causal or not
+    assert not checks.is_self_attention(q1, (16,), (True,), True)
+    assert checks.is_self_attention(q1, (16,), (False,), True)
+    q2 = torch.zeros(1, 8, 6, 2, 8)
+    assert checks.is_self_attention(q2, (8, 6), (False, False), False)
+    assert not checks.is_self_attention(q2, (8, 6), (True, False), False)
+    assert not checks.is_self_attention(q2, (8, 5), (False, False), False)
+
+
+def test_tile_choice_prefers_block_aligned_tiles():
+    qt, kt = tile_config.choose_tile_shapes(
+        (30, 48, 80), (18, 24, 24), (1, 8, 8), (1, 1, 1), (True, False, False), 128, 64)
+    assert qt == (2, 8, 8) and kt == (1, 8, 8)
+    q = torch.zeros(1, 16, 16, 1, 32)
+    with pytest.raises(ValueError):
+        tile_config.check_fna_forward_config(q, (3, 3), (1, 1), (1, 1), (False, False), (16, 8), None)
+    with pytest.raises(ValueError):
+        tile_config.check_fna_forward_config(q, (3, 3), (1, 1), (1, 1), (False, False), (10, 10), (8, 8))
+    assert tile_config.check_fna_forward_config(q, (3, 3), (1, 1), (1, 1), (False, False), (16, 8), (8, 8)) == (
+        (16, 8), (8, 8))
+
+
+def test_cpu_tensors_are_rejected_not_emulated():
+    q = torch.zeros(1, 16, 16, 1, 32, dtype=torch.bfloat16)
+    with pytest.raises(NotImplementedError):
+        natten_amd.na2d(q, q, q, kernel_size=3)
+    with pytest.raises(NotImplementedError):
+        natten_amd.attention(q.flatten(1, 2), q.flatten(1, 2), q.flatten(1, 2))
+    with pytest.raises(RuntimeError):
+        natten_amd.token_permute_operation(q, (4, 4))
