@@ -1,0 +1,238 @@
+"""Benchmark of the MI355X neighborhood attention forward path.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c4|c3|c2|c2d]
+
+One step = one na3d/na2d forward (token permute of Q/K/V, fused kernel, unpermute of O and LSE)
+on inputs already resident in HBM.  Prints ONE JSON line: whole-path throughput in effective
+NA TFLOP/s (4 * B * H * D * sum_q |window(q)| per step), the fused kernel's roofline figures from
+HIP-event timing of kernel-only launches, and a CPU baseline (the C oracle on a bounded sample
+of the same workload's queries, timed on this box's host cores).
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_TFLOPS = {"bf16": 2500.0, "fp16": 2500.0}  # MI355X dense MFMA peak
+
+WORKLOADS = {
+    # name: (B, H, layout, D, kernel, stride, dilation, causal, dtype, std)
+    "c4": (1, 24, (30, 48, 80), 128, (18, 24, 24), (1, 8, 8), (1, 1, 1), (True, False, False), "bf16", 1.0),
+    "c3": (1, 16, (128, 128), 128, (32, 32), (16, 16), (1, 1), (False, False), "fp16", 0.5),
+    "c2": (2, 8, (64, 64), 64, (13, 13), (1, 1), (1, 1), (False, False), "bf16", 1.0),
+    "c2d": (2, 8, (64, 64), 64, (13, 13), (1, 1), (2, 2), (False, False), "bf16", 1.0),
+}
+WORKLOAD_NAMES = {
+    "c4": "na3d bf16 B=1 H=24 30x48x80 D=128 k=(18,24,24) s=(1,8,8) causal=(T,F,F) +LSE",
+    "c3": "na2d fp16 B=1 H=16 128x128 D=128 k=(32,32) s=(16,16)",
+    "c2": "na2d bf16 B=2 H=8 64x64 D=64 k=(13,13)",
+    "c2d": "na2d bf16 B=2 H=8 64x64 D=64 k=(13,13) d=(2,2)",
+}
+
+
+def count_attended(layout, k, s, d, c):
+    # closed-form sum over queries of window sizes (product of per-dimension sums)
+    def win(i, kk, ss, L, causal):
+        wl, wr = kk // 2, kk // 2 + (kk % 2 - 1)
+        if causal:
+            leader = min((i // ss) * ss + ss - 1, L - 1)
+            return min(i + 1, L) - max(leader - wl - wr, 0)
+        return kk
+
+    total = 1
+    for X, kk, ss, dd, cc in zip(layout, k, s, d, c):
+        acc = 0
+        for g in range(dd):
+            L = X // dd + 1 - ((g + (dd - X % dd)) // dd)
+            acc += sum(win(i, kk, ss, L, cc) for i in range(L))
+        total *= acc
+    return total
+
+
+def cpu_baseline(q, k, v, kernel, stride, dilation, causal, out_gpu, lse_gpu, seconds_target=15.0):
+    """C oracle on a bounded sample of this workload's queries, all heads, host cores."""
+    import numpy as np
+
+    from oracle import c_oracle
+
+    B = q.shape[0]
+    n = q.dim() - 3
+    N = 1
+    for x in q.shape[1 : 1 + n]:
+        N *= int(x)
+    H, D = q.shape[-2], q.shape[-1]
+    threads = min(16, os.cpu_count() or 1)
+    qn, kn, vn = (t.float().cpu().numpy() for t in (q, k, v))
+    rng = np.random.default_rng(0)
+    # calibrate on a few queries, then size the sample for ~seconds_target of wall time
+    probe = rng.integers(0, N, size=threads)
+    t0 = time.perf_counter()
+    c_oracle.na_rows(qn, kn, vn, kernel, stride, dilation, causal, None, np.zeros_like(probe), probe, threads)
+    dt = max(time.perf_counter() - t0, 1e-4)
+    nq = int(max(threads, min(N * B, threads * seconds_target / dt)))
+    tok = rng.integers(0, N, size=nq)
+    bat = rng.integers(0, B, size=nq)
+    t0 = time.perf_counter()
+    ref_o, ref_l, visited = c_oracle.na_rows(qn, kn, vn, kernel, stride, dilation, causal, None, bat, tok, threads)
+    dt = time.perf_counter() - t0
+    flops = 4.0 * D * visited
+    got_o = out_gpu.reshape(B, N, H, D)[torch_idx(bat), torch_idx(tok)].float().cpu().numpy()
+    got_l = lse_gpu.reshape(B, N, H)[torch_idx(bat), torch_idx(tok)].float().cpu().numpy()
+    err_o = float(np.abs(got_o - ref_o).max())
+    err_l = float(np.abs(got_l - ref_l).max())
+    ok = bool(((np.abs(got_o - ref_o) <= 1e-2 + 1e-2 * np.abs(ref_o)).all())
+              and ((np.abs(got_l - ref_l) <= 1e-2 + 1e-2 * np.abs(ref_l)).all()))
+    return {
+        "value": flops / dt / 1e12,
+        "unit": "TFLOP/s",
+        "cores": threads,
+        "kind": "port",
+        "sample": f"C oracle (float64), {nq} random queries x {H} heads of this workload, {dt:.1f} s wall",
+        "parity_on_sample": {"ok": ok, "max_abs_err_out": err_o, "max_abs_err_lse": err_l, "atol_rtol": 1e-2},
+    }
+
+
+def torch_idx(a):
+    import torch
+
+    return torch.as_tensor(a, dtype=torch.long)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS))
+    ap.add_argument("--q-tile", type=str, default=None, help="comma separated, e.g. 2,8,8")
+    ap.add_argument("--kv-tile", type=str, default=None)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU; --gpus above 1 is not supported (no multi-GPU path).",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    import natten_amd
+    from natten_amd import _lib
+    from natten_amd.tile_config import check_fna_forward_config
+
+    _lib.lib()  # no fallback: fail here when the HIP library is missing
+    dev = torch.device("cuda:0")
+    B, H, layout, D, kernel, stride, dilation, causal, dt_name, std = WORKLOADS[args.workload]
+    dtype = {"bf16": torch.bfloat16, "fp16": torch.float16}[dt_name]
+    n = len(layout)
+    gen = torch.Generator().manual_seed(0)
+    q, k, v = ((torch.randn((B, *layout, H, D), generator=gen) * std).to(dtype).to(dev) for _ in range(3))
+    na = {1: natten_amd.na1d, 2: natten_amd.na2d, 3: natten_amd.na3d}[n]
+    q_tile = tuple(int(x) for x in args.q_tile.split(",")) if args.q_tile else None
+    kv_tile = tuple(int(x) for x in args.kv_tile.split(",")) if args.kv_tile else None
+    q_tile, kv_tile = check_fna_forward_config(q, kernel, stride, dilation, causal, q_tile, kv_tile)
+
+    def step():
+        return na(q, k, v, kernel, stride, dilation, causal, q_tile_shape=q_tile, kv_tile_shape=kv_tile,
+                  return_lse=True)
+
+    with torch.no_grad():
+        for _ in range(args.warmup):
+            out, lse = step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            out, lse = step()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    flops = 4.0 * B * H * D * count_attended(layout, kernel, stride, dilation, causal)
+    tflops_e2e = flops / (ms_per_step * 1e-3) / 1e12
+
+    # ---- kernel-only timings with HIP events on the launch stream ----------------------------
+    from natten_amd.token_permute import token_permute_operation, token_unpermute_operation
+
+    with torch.no_grad():
+        qp, qkv_shape, q_shape = token_permute_operation(q, q_tile, dilation)
+        kp, _, kv_shape = token_permute_operation(k, kv_tile, dilation)
+        vp, _, _ = token_permute_operation(v, kv_tile, dilation)
+        scale = D**-0.5
+
+        def kern():
+            return _lib.fna_forward(qp, kp, vp, kernel, stride, dilation, causal, scale, q_shape, kv_shape,
+                                    qkv_shape, q_tile, kv_tile)
+
+        def timed(fn, iters):
+            for _ in range(3):
+                fn()
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            e0.record()
+            for _ in range(iters):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) / iters
+
+        kernel_ms = timed(kern, args.steps)
+        op, lp = kern()
+        perm_ms = timed(lambda: token_permute_operation(q, q_tile, dilation), args.steps)
+        unperm_ms = timed(lambda: token_unpermute_operation(op, qkv_shape, q_tile, dilation), args.steps)
+    q_bytes = q.numel() * q.element_size()
+    achieved = flops / (kernel_ms * 1e-3) / 1e12
+    peak = PEAK_TFLOPS[dt_name]
+    dense_flops = 4.0 * B * H * D * float(q.numel() // (B * H * D)) ** 2
+
+    result = {
+        "metric": "FNA fwd ms + effective TFLOP/s (% MFMA peak), na3d bf16 D=128, 1 GPU",
+        "value": tflops_e2e,
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": dt_name,
+        "data": "synthetic",
+        "config": {
+            "workload": WORKLOAD_NAMES[args.workload],
+            "q_tile_shape": list(q_tile),
+            "kv_tile_shape": list(kv_tile),
+            "path": "token permute (Q,K,V) + fused FNA kernel + token unpermute (O, LSE)",
+        },
+        "na_flop_per_step": flops,
+        "dense_over_na_flop": dense_flops / flops,
+        "kernel_ms": kernel_ms,
+        "token_permute": {
+            "permute_q_ms": perm_ms,
+            "unpermute_o_ms": unperm_ms,
+            "permute_GBps": 2 * q_bytes / (perm_ms * 1e-3) / 1e9,
+            "unpermute_GBps": 2 * q_bytes / (unperm_ms * 1e-3) / 1e9,
+        },
+        "roofline": {
+            "kernel": "fna_fwd_kernel",
+            "bound": "mfma",
+            "achieved": achieved,
+            "peak": peak,
+            "unit": "TFLOP/s",
+            "frac": achieved / peak,
+            "traffic": None,
+        },
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(q, k, v, kernel, stride, dilation, causal, out, lse)
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()
