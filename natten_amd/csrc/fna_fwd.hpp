@@ -1,17 +1,27 @@
-// Fused neighborhood attention forward for gfx950 (MI355X): one workgroup per Q tile of one
-// (batch*dilation-group, head); K/V tiles staged in LDS; S^T = K Q^T and O^T = V^T P^T on
-// 32x32x16 MFMA so that every lane owns exactly one query row (row max / row sum are per-lane
-// scalars plus one exchange between the two half-waves).
+// Fused neighborhood attention forward for gfx950 (MI355X).
+//
+// One workgroup = one Q tile of one (batch*dilation-group, head).  K/V tiles stream through a
+// double-buffered LDS ring filled by asynchronous global->LDS loads; S^T = K Q^T and
+// O^T = V^T P^T run on 32x32x16 MFMA so that every lane owns exactly one query row: row max
+// and row sum are per-lane scalars plus one exchange between the two half-waves.  The softmax
+// keeps a stale row maximum and rescales the accumulators only when a row's maximum grew by
+// more than 2^8 (exact: the final normalisation uses the same maximum).
 //
 // The structure it restates (not the code): SHI-Labs/NATTEN
 //   csrc/include/natten/cuda/fna_blackwell/collective/fna_fusion.hpp:315-347 (KV tile box per Q tile)
 //   csrc/include/natten/cuda/fna_blackwell/collective/fna_fusion.hpp:384-436 (element mask)
 //   csrc/include/natten/cuda/fna_blackwell/collective/sm100_fna_fwd_mainloop_tma_warpspecialized.hpp:618-861,
 //   :1314-1327 (online softmax in the exp2 domain, O / rowsum, LSE = ln(rowsum) + scale * rowmax)
+// Differences by design: KV tiles of the box are visited with dimension 0 slowest (the
+// reference visits dimension 0 fastest) and workgroups are laid out so that the Q tiles
+// resident on one XCD share their KV tiles in that XCD's L2; every (Q tile, KV tile) pair is
+// classified per tile (fully inside all windows -> no mask) instead of once per launch.
 #pragma once
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+
+#include <type_traits>
 
 #include "na_math.hpp"
 
@@ -30,19 +40,27 @@ struct FnaParams {
   int ksize[3], stride[3], dil[3], causal[3];
   int q_tile[3], kv_tile[3];
   int q_tiled[3], kv_tiled[3];  // tiles per dimension of the padded per-group layouts
-  float scale;                  // softmax scale (dequantisation scales of q and k folded in)
-  float out_scale;              // dequantisation scale of v
+  int num_q_tiles;              // q_tiled[0] * q_tiled[1] * q_tiled[2]
+  // workgroup layout: consecutive `wg_group` Q tiles (dimension 0 slowest) of one (batch, head)
+  // form a group; groups are dealt round-robin to the 8 XCDs
+  int wg_group, groups_per_bh, total_groups;
+  float scale;      // softmax scale (dequantisation scales of q and k folded in)
+  float out_scale;  // dequantisation scale of v
 };
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
-typedef float f32x4_t __attribute__((ext_vector_type(4)));
 typedef short s16x4_t __attribute__((ext_vector_type(4)));
 typedef short s16x8_t __attribute__((ext_vector_type(8)));
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
 #define NA_LDS __attribute__((address_space(3)))
+#define NA_GLOBAL __attribute__((address_space(1)))
+
+constexpr int kNumXcd = 8;
 
 template <typename T>
 struct Mma;
@@ -50,16 +68,27 @@ struct Mma;
 template <>
 struct Mma<__bf16> {
   using vec8 = bf16x8_t;
+  using vec2 = bf16x2_t;
   static __device__ __forceinline__ f32x16_t run(vec8 a, vec8 b, f32x16_t c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+  // c + a.x + a.y
+  static __device__ __forceinline__ float add2(vec2 a, float c) {
+    const vec2 one = {static_cast<__bf16>(1.0f), static_cast<__bf16>(1.0f)};
+    return __builtin_amdgcn_fdot2_f32_bf16(a, one, c, false);
   }
 };
 
 template <>
 struct Mma<_Float16> {
   using vec8 = f16x8_t;
+  using vec2 = f16x2_t;
   static __device__ __forceinline__ f32x16_t run(vec8 a, vec8 b, f32x16_t c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ float add2(vec2 a, float c) {
+    const vec2 one = {static_cast<_Float16>(1.0f), static_cast<_Float16>(1.0f)};
+    return __builtin_amdgcn_fdot2(a, one, c, false);
   }
 };
 
@@ -73,57 +102,118 @@ static __device__ __forceinline__ s16x4_t lds_read_tr16(const char* p) {
 #pragma clang diagnostic pop
 }
 
+// Asynchronous 16-byte-per-lane copy global -> LDS: lane i's 16 bytes land at lds_base + 16*i
+// (lds_base must be wave-uniform).  Completion is tracked by the vector memory counter.
+static __device__ __forceinline__ void async_copy16(const void* gptr, char* lds_base) {
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Wold-style-cast"
+  __builtin_amdgcn_global_load_lds((const NA_GLOBAL void*)(gptr), (NA_LDS void*)(lds_base), 16, 0, 0);
+#pragma clang diagnostic pop
+}
+
+// s_waitcnt vmcnt(N) only (expcnt / lgkmcnt left at their maxima), gfx9 encoding
+template <int N>
+static __device__ __forceinline__ void wait_vmcnt() {
+  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+  __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 0xF) | ((N >> 4) << 14));
+}
+
 static __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 constexpr uint32_t kGuardBits = (1u << 9) | (1u << 19) | (1u << 29);
+// a row's running maximum may lag the true one by up to this many powers of two
+constexpr float kLazyRescaleLog2 = 8.0f;
 
+// LDS layout of one K or V tile: KVT rows of D 16-bit elements, unpadded, with the 16-byte
+// chunks of each row XOR-swizzled so that the MFMA operand reads are bank-conflict free:
+//   K: chunk c of row r lives in slot c ^ ((r / RPL) % CPR)            (b128 reads down a column of rows)
+//   V: chunk c of row r lives in slot c ^ (2 * ((r / RPL) % (CPR/2)))  (transpose reads of 4 rows x 32 bytes)
+// CPR = chunks per row, RPL = rows per 256 bytes.
 template <int D, int KVT>
 struct FnaSmem {
-  static constexpr int KROW = D * 2 + 16;  // bytes per K row (padding breaks bank conflicts of b128 reads)
-  static constexpr int VROW = D * 2 + 32;  // bytes per V row (padding for the transpose reads)
-  static constexpr int BYTES = KVT * (KROW + VROW) + KVT * 4;
+  static constexpr int ROWB = D * 2;
+  static constexpr int CPR = D / 8;
+  static constexpr int RPL = (16 / CPR) > 0 ? (16 / CPR) : 1;
+  static constexpr int TILE_BYTES = KVT * ROWB;
+  static constexpr int STAGES = 2;
+  static constexpr int BYTES = STAGES * 2 * TILE_BYTES + KVT * 4;  // static LDS of the kernel
+  static __host__ __device__ constexpr int k_slot(int r, int c) { return c ^ ((r / RPL) % CPR); }
+  static __host__ __device__ constexpr int v_slot(int r, int c) { return c ^ (2 * ((r / RPL) % (CPR / 2))); }
 };
 
+// Register budget: one query block per wave is meant to run two workgroups per CU (two waves per
+// SIMD, 256 registers each) so that one wave's softmax overlaps the other's MFMA work.
 template <typename T, int D, int NWAVES, int MQ, int KVT>
-__global__ void __launch_bounds__(NWAVES * 64) fna_fwd_kernel(const FnaParams p) {
+__global__ void __launch_bounds__(NWAVES * 64) __attribute__((amdgpu_waves_per_eu(MQ == 1 ? 2 : 1)))
+fna_fwd_kernel(const FnaParams p) {
   constexpr int NT = NWAVES * 64;
   constexpr int QT = NWAVES * MQ * 32;
   constexpr int KSTEPS = D / 16;
   constexpr int DB = D / 32;
   constexpr int NSB = KVT / 32;
-  constexpr int KROW = FnaSmem<D, KVT>::KROW;
-  constexpr int VROW = FnaSmem<D, KVT>::VROW;
+  using L = FnaSmem<D, KVT>;
+  constexpr int ROWB = L::ROWB;
+  constexpr int CPR = L::CPR;
+  constexpr int TILE_BYTES = L::TILE_BYTES;
+  constexpr int PER = (KVT * CPR) / NT;  // async copies per thread per operand per tile
+  static_assert((KVT * CPR) % NT == 0, "tile does not split evenly over the workgroup");
   using M = Mma<T>;
   using vec8 = typename M::vec8;
+  using vec2 = typename M::vec2;
 
-  extern __shared__ __attribute__((aligned(16))) char smem[];
-  char* sK = smem;
-  char* sV = smem + KVT * KROW;
-  uint32_t* sTab = reinterpret_cast<uint32_t*>(smem + KVT * (KROW + VROW));
+  // One LDS object per stage and operand: distinct objects let the compiler see that the
+  // asynchronous fill of one stage does not alias the operand reads of the other, so those
+  // reads do not wait for the fill.
+  __shared__ __attribute__((aligned(1024))) char sK0[TILE_BYTES];
+  __shared__ __attribute__((aligned(1024))) char sV0[TILE_BYTES];
+  __shared__ __attribute__((aligned(1024))) char sK1[TILE_BYTES];
+  __shared__ __attribute__((aligned(1024))) char sV1[TILE_BYTES];
+  __shared__ __attribute__((aligned(16))) uint32_t sTab[KVT];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int l32 = lane & 31;
   const int g = lane >> 5;
-  const int qtile_idx = blockIdx.x;
-  const int head = blockIdx.y;
-  const int bg = blockIdx.z;
+
+  // ---- workgroup id -> (batch*group, head, Q tile); groups of Q tiles are dealt to XCDs ------
+  int bg, head, qtile_rm;
+  {
+    const int pid = blockIdx.x;
+    const int xcd = pid % kNumXcd;
+    const int local = pid / kNumXcd;
+    const int group = (local / p.wg_group) * kNumXcd + xcd;
+    const int within = local % p.wg_group;
+    if (group >= p.total_groups) return;
+    const int bh = group / p.groups_per_bh;
+    qtile_rm = (group % p.groups_per_bh) * p.wg_group + within;
+    if (qtile_rm >= p.num_q_tiles) return;
+    bg = bh / p.heads_q;
+    head = bh % p.heads_q;
+  }
   const int head_kv = head / (p.heads_q / p.heads_kv);
 
   // ---- workgroup-uniform setup: dilation group, Q tile origin, KV tile box -------------------
+  // qtile_rm enumerates Q tiles with dimension 0 slowest; causal dimension 0 is walked from
+  // the far end so that the Q tiles with the longest KV loops start first.
   int extent[3], q_first[3], box_tile0[3], box_n[3], full_lo[3], full_hi[3];
+  int qtile_idx;  // position of the tile in the permuted sequence (dimension 0 fastest)
   {
     int gl = bg % p.num_groups;
-    int t = qtile_idx;
+    int tc[3];
+    int t = qtile_rm;
+    tc[2] = t % p.q_tiled[2];
+    t /= p.q_tiled[2];
+    tc[1] = t % p.q_tiled[1];
+    tc[0] = t / p.q_tiled[1];
+    if (p.causal[0]) tc[0] = p.q_tiled[0] - 1 - tc[0];
+    qtile_idx = tc[0] + p.q_tiled[0] * (tc[1] + p.q_tiled[1] * tc[2]);
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
       const int gi = gl % p.dil[a];
       gl /= p.dil[a];
       extent[a] = na_group_extent(p.qkv_shape[a], p.dil[a], gi);
-      const int tc = t % p.q_tiled[a];
-      t /= p.q_tiled[a];
-      q_first[a] = tc * p.q_tile[a];
+      q_first[a] = tc[a] * p.q_tile[a];
       const int qf = q_first[a], ql = qf + p.q_tile[a] - 1;
       const bool c = p.causal[a] != 0;
       const int st_f = na_window_start(qf, p.ksize[a], p.stride[a], extent[a], c);
@@ -148,14 +238,58 @@ __global__ void __launch_bounds__(NWAVES * 64) fna_fwd_kernel(const FnaParams p)
     sTab[i] = uint32_t(t0) | (uint32_t(t1) << 10) | (uint32_t(r) << 20);
   }
 
-  // ---- per-lane setup: this lane's query rows, their windows, Q fragments ---------------------
-  int wst[MQ][3], wen[MQ][3];
-  vec8 qf[MQ][KSTEPS];
   const int64_t q_row_stride = int64_t(p.heads_q) * D;
   const int64_t kv_row_stride = int64_t(p.heads_kv) * D;
   const T* qbase = reinterpret_cast<const T*>(p.q) + int64_t(bg) * p.seqlen_q * q_row_stride + int64_t(head) * D;
   const T* kbase = reinterpret_cast<const T*>(p.k) + int64_t(bg) * p.seqlen_kv * kv_row_stride + int64_t(head_kv) * D;
   const T* vbase = reinterpret_cast<const T*>(p.v) + int64_t(bg) * p.seqlen_kv * kv_row_stride + int64_t(head_kv) * D;
+
+  // ---- async tile loads: thread-constant part of the addressing ------------------------------
+  // copy i of this thread fills LDS chunk position P = i*NT + tid (row P / CPR, slot P % CPR)
+  int ld_row[PER], ld_kcol[PER], ld_vcol[PER];
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    const int P = i * NT + tid;
+    ld_row[i] = P / CPR;
+    const int slot = P % CPR;
+    ld_kcol[i] = L::k_slot(ld_row[i], slot) * 8;  // XOR swizzles are involutions
+    ld_vcol[i] = L::v_slot(ld_row[i], slot) * 8;
+  }
+  auto issue_tile_loads = [&](int kv_row0, auto stage_tag) {
+    char* sK = decltype(stage_tag)::value ? sK1 : sK0;
+    char* sV = decltype(stage_tag)::value ? sV1 : sV0;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      // rows past the end of the sequence are masked; read a valid row instead of zero filling
+      const int grow = na_min(kv_row0 + ld_row[i], p.seqlen_kv - 1);
+      const int wave_chunk0 = (i * NT + wave * 64) * 16;
+      async_copy16(kbase + int64_t(grow) * kv_row_stride + ld_kcol[i], sK + wave_chunk0);
+      async_copy16(vbase + int64_t(grow) * kv_row_stride + ld_vcol[i], sV + wave_chunk0);
+    }
+  };
+
+  // KV tile iteration state: dimension 2 fastest, dimension 0 slowest
+  int itc[3] = {0, 0, 0};
+  auto tile_row0 = [&]() {
+    return ((box_tile0[0] + itc[0]) + p.kv_tiled[0] * ((box_tile0[1] + itc[1]) + p.kv_tiled[1] * (box_tile0[2] + itc[2]))) * KVT;
+  };
+  auto advance = [&]() {
+    if (++itc[2] == box_n[2]) {
+      itc[2] = 0;
+      if (++itc[1] == box_n[1]) {
+        itc[1] = 0;
+        ++itc[0];
+      }
+    }
+  };
+
+  using Stage0 = std::integral_constant<int, 0>;
+  using Stage1 = std::integral_constant<int, 1>;
+  issue_tile_loads(tile_row0(), Stage0{});
+
+  // ---- per-lane setup: this lane's query rows, their windows, Q fragments ---------------------
+  int wst[MQ][3], wen[MQ][3];
+  vec8 qf[MQ][KSTEPS];
 #pragma unroll
   for (int mb = 0; mb < MQ; ++mb) {
     int r = (wave * MQ + mb) * 32 + l32;
@@ -190,9 +324,20 @@ __global__ void __launch_bounds__(NWAVES * 64) fna_fwd_kernel(const FnaParams p)
   }
   const float c_log2 = p.scale * 1.4426950408889634f;
 
-  // ---- main loop over the KV tile box (dimension 0 fastest) ----------------------------------
-  int itc[3] = {0, 0, 0};
-  for (int it = 0; it < total_tiles; ++it) {
+  // lane-constant LDS read offsets
+  int k_off[KSTEPS];  // K operand: row l32 (+32*sb), chunk 2*ks+g
+#pragma unroll
+  for (int ks = 0; ks < KSTEPS; ++ks) k_off[ks] = l32 * ROWB + L::k_slot(l32, ks * 2 + g) * 16;
+  // V operand: transpose read of rows (4g + e) [+8], 4 columns at 16*(l32/16) + 4*j4 of a 32-column block
+  const int l16 = lane & 15;
+  const int v_e = l16 >> 2, v_j4 = l16 & 3;
+  const int v_row = 4 * g + v_e;
+  const int v_chunk = (l32 >> 4) * 2 + (v_j4 >> 1);  // 16-byte chunk inside the 64-byte column block
+  const int v_sub = (v_j4 & 1) * 8;
+
+  // ---- main loop over the KV tile box (unrolled by the two LDS stages) -------------------------
+  auto process_tile = [&](auto stage_tag, int it) {
+    constexpr int stage = decltype(stage_tag)::value;
     int origin[3];
     bool full = true;
 #pragma unroll
@@ -200,38 +345,14 @@ __global__ void __launch_bounds__(NWAVES * 64) fna_fwd_kernel(const FnaParams p)
       origin[a] = (box_tile0[a] + itc[a]) * p.kv_tile[a];
       full = full && (origin[a] >= full_lo[a]) && (origin[a] + p.kv_tile[a] <= full_hi[a]);
     }
-    const int kv_lin = (box_tile0[0] + itc[0]) +
-                       p.kv_tiled[0] * ((box_tile0[1] + itc[1]) + p.kv_tiled[1] * (box_tile0[2] + itc[2]));
-    const int kv_row0 = kv_lin * KVT;
+    advance();
 
-    __syncthreads();  // everyone is done reading the previous tile (and sTab is written)
-    {
-      constexpr int CPR = D / 8;  // 16-byte chunks per row
-      constexpr int PER = (KVT * CPR) / NT;
-      static_assert((KVT * CPR) % NT == 0, "tile does not split evenly over the workgroup");
-      u32x4_t kreg[PER], vreg[PER];
-#pragma unroll
-      for (int i = 0; i < PER; ++i) {
-        const int c = i * NT + tid;
-        const int row = c / CPR, col = c % CPR;
-        const int grow = kv_row0 + row;
-        if (grow < p.seqlen_kv) {
-          kreg[i] = *reinterpret_cast<const u32x4_t*>(kbase + int64_t(grow) * kv_row_stride + col * 8);
-          vreg[i] = *reinterpret_cast<const u32x4_t*>(vbase + int64_t(grow) * kv_row_stride + col * 8);
-        } else {
-          kreg[i] = u32x4_t{0, 0, 0, 0};
-          vreg[i] = u32x4_t{0, 0, 0, 0};
-        }
-      }
-#pragma unroll
-      for (int i = 0; i < PER; ++i) {
-        const int c = i * NT + tid;
-        const int row = c / CPR, col = c % CPR;
-        *reinterpret_cast<u32x4_t*>(sK + row * KROW + col * 16) = kreg[i];
-        *reinterpret_cast<u32x4_t*>(sV + row * VROW + col * 16) = vreg[i];
-      }
-    }
-    __syncthreads();
+    wait_vmcnt<0>();   // this thread's copies of tile `it` have landed
+    __syncthreads();   // ... and everyone's; everyone is also done reading the other stage
+    if (it + 1 < total_tiles) issue_tile_loads(tile_row0(), std::integral_constant<int, stage ^ 1>{});
+
+    const char* sK = stage ? sK1 : sK0;
+    const char* sV = stage ? sV1 : sV0;
 
     // S^T = K Q^T : lane owns query row l32 (per q block) and 16 key rows per 32-key sub-block
     f32x16_t S[MQ][NSB];
@@ -241,12 +362,14 @@ __global__ void __launch_bounds__(NWAVES * 64) fna_fwd_kernel(const FnaParams p)
       for (int mb = 0; mb < MQ; ++mb)
 #pragma unroll
         for (int r = 0; r < 16; ++r) S[mb][sb][r] = 0.f;
+      // rows sb*32 + l32: (sb*32) is a multiple of 16 rows, so the swizzle term is unchanged
+      vec8 kf[KSTEPS];
 #pragma unroll
-      for (int ks = 0; ks < KSTEPS; ++ks) {
-        const vec8 kf = *reinterpret_cast<const vec8*>(sK + (sb * 32 + l32) * KROW + (ks * 2 + g) * 16);
+      for (int ks = 0; ks < KSTEPS; ++ks) kf[ks] = *reinterpret_cast<const vec8*>(sK + sb * 32 * ROWB + k_off[ks]);
 #pragma unroll
-        for (int mb = 0; mb < MQ; ++mb) S[mb][sb] = M::run(kf, qf[mb][ks], S[mb][sb]);
-      }
+      for (int ks = 0; ks < KSTEPS; ++ks)
+#pragma unroll
+        for (int mb = 0; mb < MQ; ++mb) S[mb][sb] = M::run(kf[ks], qf[mb][ks], S[mb][sb]);
     }
 
     vec8 pf[MQ][NSB][2];
@@ -281,11 +404,20 @@ __global__ void __launch_bounds__(NWAVES * 64) fna_fwd_kernel(const FnaParams p)
 #pragma unroll
         for (int r = 0; r < 16; ++r) mx = fmaxf(mx, S[mb][sb][r]);
       mx = fmaxf(mx, __shfl_xor(mx, 32));
-      const float m_new = fmaxf(m_run[mb], mx);
-      const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-      const float alpha = fast_exp2((m_run[mb] - m_use) * c_log2);
-      const float msc = m_use * c_log2;
-      m_run[mb] = m_new;
+      // rescale only when some row of this wave outgrew its (stale) maximum by more than 2^8
+      const bool grow = (mx - m_run[mb]) * c_log2 > kLazyRescaleLog2;  // also true while m_run == -inf and mx finite
+      if (__any(grow)) {
+        const float m_new = fmaxf(m_run[mb], mx);
+        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+        const float alpha = fast_exp2((m_run[mb] - m_use) * c_log2);  // m_run == -inf -> 0
+        m_run[mb] = m_new;
+        l_run[mb] *= alpha;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[mb][db][r] *= alpha;
+      }
+      const float msc = ((m_run[mb] == -INFINITY) ? 0.f : m_run[mb]) * c_log2;
       float psum = 0.f;
 #pragma unroll
       for (int sb = 0; sb < NSB; ++sb)
@@ -293,50 +425,43 @@ __global__ void __launch_bounds__(NWAVES * 64) fna_fwd_kernel(const FnaParams p)
         for (int h = 0; h < 2; ++h) {
           vec8 pv;
 #pragma unroll
-          for (int i = 0; i < 8; ++i) {
-            const float pe = fast_exp2(S[mb][sb][8 * h + i] * c_log2 - msc);
-            psum += pe;
-            pv[i] = static_cast<T>(pe);
+          for (int i = 0; i < 8; i += 2) {
+            vec2 p2;
+            p2[0] = static_cast<T>(fast_exp2(S[mb][sb][8 * h + i] * c_log2 - msc));
+            p2[1] = static_cast<T>(fast_exp2(S[mb][sb][8 * h + i + 1] * c_log2 - msc));
+            psum = M::add2(p2, psum);  // sums the rounded probabilities, the ones P V uses
+            pv[i] = p2[0];
+            pv[i + 1] = p2[1];
           }
           pf[mb][sb][h] = pv;
         }
-      l_run[mb] = l_run[mb] * alpha + psum;
-#pragma unroll
-      for (int db = 0; db < DB; ++db)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[mb][db][r] *= alpha;
+      l_run[mb] += psum;
     }
 
     // O^T += V^T P^T : the k-slot order of the P fragment (rows 4g..4g+3 and 8+4g..8+4g+3 of
     // each 16-key half) is matched by two transpose reads of V.
-    {
-      const int l16 = lane & 15;
-      const int e = l16 >> 2, j4 = l16 & 3;
-      const int colb = ((l32 >> 4) * 16 + 4 * j4) * 2;
 #pragma unroll
-      for (int sb = 0; sb < NSB; ++sb)
+    for (int sb = 0; sb < NSB; ++sb)
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-          const char* vrow = sV + (sb * 32 + h * 16 + 4 * g + e) * VROW + colb;
+      for (int h = 0; h < 2; ++h) {
+        const int r0 = sb * 32 + h * 16 + v_row;  // r0 + 8 shares (r0 / RPL) % (CPR/2) only when RPL >= 16; recompute
+        const char* row_lo = sV + r0 * ROWB + v_sub;
+        const char* row_hi = sV + (r0 + 8) * ROWB + v_sub;
 #pragma unroll
-          for (int db = 0; db < DB; ++db) {
-            const s16x4_t lo = lds_read_tr16(vrow + db * 64);
-            const s16x4_t hi = lds_read_tr16(vrow + db * 64 + 8 * VROW);
-            const s16x8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-            const vec8 vf = __builtin_bit_cast(vec8, both);
+        for (int db = 0; db < DB; ++db) {
+          const int c = db * 4 + v_chunk;
+          const s16x4_t lo = lds_read_tr16(row_lo + L::v_slot(r0, c) * 16);
+          const s16x4_t hi = lds_read_tr16(row_hi + L::v_slot(r0 + 8, c) * 16);
+          const s16x8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+          const vec8 vf = __builtin_bit_cast(vec8, both);
 #pragma unroll
-            for (int mb = 0; mb < MQ; ++mb) acc[mb][db] = M::run(vf, pf[mb][sb][h], acc[mb][db]);
-          }
+          for (int mb = 0; mb < MQ; ++mb) acc[mb][db] = M::run(vf, pf[mb][sb][h], acc[mb][db]);
         }
-    }
-
-    if (++itc[0] == box_n[0]) {
-      itc[0] = 0;
-      if (++itc[1] == box_n[1]) {
-        itc[1] = 0;
-        ++itc[2];
       }
-    }
+  };
+  for (int it = 0; it < total_tiles; it += 2) {
+    process_tile(Stage0{}, it);
+    if (it + 1 < total_tiles) process_tile(Stage1{}, it + 1);
   }
 
   // ---- epilogue: O = acc / rowsum, LSE = ln(rowsum) + scale * rowmax -------------------------

@@ -37,6 +37,20 @@ int check_launch(const char* what) {
 
 int prod3(const int* x) { return x[0] * x[1] * x[2]; }
 
+// Workgroup layout: Q tiles are enumerated with dimension 0 slowest; a group is a run of about
+// as many consecutive Q tiles as one XCD keeps resident (32 CUs x 2 workgroups), made of whole
+// dimension-0 slabs when possible, so that the tiles resident on an XCD overlap in their KV boxes.
+void set_wg_layout(FnaParams& p) {
+  p.num_q_tiles = p.q_tiled[0] * p.q_tiled[1] * p.q_tiled[2];
+  const int slab = p.q_tiled[1] * p.q_tiled[2];
+  int rows = (64 + slab / 2) / slab;
+  if (rows < 1) rows = 1;
+  if (rows > p.q_tiled[0]) rows = p.q_tiled[0];
+  p.wg_group = slab * rows;
+  p.groups_per_bh = (p.num_q_tiles + p.wg_group - 1) / p.wg_group;
+  p.total_groups = p.batch * p.heads_q * p.groups_per_bh;
+}
+
 struct TileConfig {
   int q_tile, kv_tile;
 };
@@ -48,17 +62,11 @@ constexpr int kNumTileConfigs = sizeof(kTileConfigs) / sizeof(kTileConfigs[0]);
 template <typename T, int D, int NWAVES, int MQ, int KVT>
 int launch_fna(const FnaParams& p, hipStream_t stream) {
   constexpr int QT = NWAVES * MQ * 32;
-  constexpr int smem = FnaSmem<D, KVT>::BYTES;
   auto kernel = fna_fwd_kernel<T, D, NWAVES, MQ, KVT>;
-  static bool configured = false;
-  if (smem > 64 * 1024 && !configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-    if (e != hipSuccess) return fail("fna_forward: cannot reserve %d bytes of LDS: %s", smem, hipGetErrorString(e));
-    configured = true;
-  }
-  dim3 grid((p.seqlen_q + QT - 1) / QT, p.heads_q, p.batch);
-  hipLaunchKernelGGL(kernel, grid, dim3(NWAVES * 64), smem, stream, p);
+  if ((p.seqlen_q + QT - 1) / QT != p.num_q_tiles) return fail("fna_forward: internal tile count mismatch");
+  const long long wgs = (long long)((p.total_groups + kNumXcd - 1) / kNumXcd) * kNumXcd * p.wg_group;
+  if (wgs > 0x7fffffffLL) return fail("fna_forward: problem needs more than 2^31 workgroups");
+  hipLaunchKernelGGL(kernel, dim3((unsigned)wgs), dim3(NWAVES * 64), 0, stream, p);
   return check_launch("fna_forward");
 }
 
@@ -102,7 +110,6 @@ int check_common(const char* what, const void* q, const void* k, const void* v, 
   if ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v) |
        reinterpret_cast<uintptr_t>(out)) & 15)
     return fail("%s: q, k, v and out must be 16-byte aligned", what);
-  if (heads_q > 65535 || batch > 65535) return fail("%s: heads_q and batch must be below 65536", what);
   return 0;
 }
 
@@ -188,6 +195,7 @@ int natten_amd_fna_forward(const void* q, const void* k, const void* v, void* ou
   p.seqlen_kv = seqlen_kv;
   p.scale = scale * q_scale * k_scale;
   p.out_scale = v_scale;
+  set_wg_layout(p);
   return dispatch_dtype(p, dtype, head_dim, prod3(p.q_tile), prod3(p.kv_tile), static_cast<hipStream_t>(stream));
 }
 
@@ -231,6 +239,7 @@ int natten_amd_attention_forward(const void* q, const void* k, const void* v, vo
   p.seqlen_kv = seqlen_kv;
   p.scale = scale;
   p.out_scale = 1.f;
+  set_wg_layout(p);
   return dispatch_dtype(p, dtype, head_dim, QT, KVT, static_cast<hipStream_t>(stream));
 }
 
