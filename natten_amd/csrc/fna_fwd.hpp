@@ -118,7 +118,21 @@ static __device__ __forceinline__ void wait_vmcnt() {
   __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 0xF) | ((N >> 4) << 14));
 }
 
+#ifdef NA_X_NOEXP
+static __device__ __forceinline__ float fast_exp2(float x) { return x; }
+#else
 static __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+#endif
+
+// max of x over the lane pair (l, l ^ 32): v_permlane32_swap exchanges the upper half of its
+// first register with the lower half of its second, after which every lane holds both values
+// of its pair.  Written as inline assembly (with the wait states the instruction needs around
+// it) because the two-result builtin is miscompiled when both inputs are the same value.
+static __device__ __forceinline__ float cross_half_max(float x) {
+  float a = x, b = x;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+  return fmaxf(fmaxf(a, b), x);
+}
 
 constexpr uint32_t kGuardBits = (1u << 9) | (1u << 19) | (1u << 29);
 // a row's running maximum may lag the true one by up to this many powers of two
@@ -144,7 +158,7 @@ struct FnaSmem {
 // Register budget: one query block per wave is meant to run two workgroups per CU (two waves per
 // SIMD, 256 registers each) so that one wave's softmax overlaps the other's MFMA work.
 template <typename T, int D, int NWAVES, int MQ, int KVT>
-__global__ void __launch_bounds__(NWAVES * 64) __attribute__((amdgpu_waves_per_eu(MQ == 1 ? 2 : 1)))
+__global__ void __launch_bounds__(NWAVES * 64) __attribute__((amdgpu_waves_per_eu(MQ == 1 ? 2 : 1, MQ == 1 ? 2 : 1)))
 fna_fwd_kernel(const FnaParams p) {
   constexpr int NT = NWAVES * 64;
   constexpr int QT = NWAVES * MQ * 32;
@@ -155,8 +169,9 @@ fna_fwd_kernel(const FnaParams p) {
   constexpr int ROWB = L::ROWB;
   constexpr int CPR = L::CPR;
   constexpr int TILE_BYTES = L::TILE_BYTES;
-  constexpr int PER = (KVT * CPR) / NT;  // async copies per thread per operand per tile
-  static_assert((KVT * CPR) % NT == 0, "tile does not split evenly over the workgroup");
+  constexpr int CHUNKS = KVT * CPR;             // 16-byte chunks per operand tile
+  constexpr int PER = (CHUNKS + NT - 1) / NT;   // async copies per thread per operand per tile
+  static_assert(CHUNKS % 64 == 0, "a tile must be a whole number of wave-wide copies");
   using M = Mma<T>;
   using vec8 = typename M::vec8;
   using vec2 = typename M::vec2;
@@ -172,7 +187,7 @@ fna_fwd_kernel(const FnaParams p) {
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform by construction
   const int l32 = lane & 31;
   const int g = lane >> 5;
 
@@ -244,36 +259,61 @@ fna_fwd_kernel(const FnaParams p) {
   const T* kbase = reinterpret_cast<const T*>(p.k) + int64_t(bg) * p.seqlen_kv * kv_row_stride + int64_t(head_kv) * D;
   const T* vbase = reinterpret_cast<const T*>(p.v) + int64_t(bg) * p.seqlen_kv * kv_row_stride + int64_t(head_kv) * D;
 
-  // ---- async tile loads: thread-constant part of the addressing ------------------------------
-  // copy i of this thread fills LDS chunk position P = i*NT + tid (row P / CPR, slot P % CPR)
-  int ld_row[PER], ld_kcol[PER], ld_vcol[PER];
+  // ---- async tile loads -------------------------------------------------------------------------
+  // Copy i of this thread fills LDS chunk position P = i*NT + tid (row P / CPR, slot P % CPR).
+  // Its global address is a per-tile uniform base (first row of the tile) plus a byte offset
+  // that never changes for the thread, so a tile load costs no vector address arithmetic.
+  int ld_row[PER];
+  uint32_t ld_koff[PER], ld_voff[PER];
 #pragma unroll
   for (int i = 0; i < PER; ++i) {
     const int P = i * NT + tid;
     ld_row[i] = P / CPR;
     const int slot = P % CPR;
-    ld_kcol[i] = L::k_slot(ld_row[i], slot) * 8;  // XOR swizzles are involutions
-    ld_vcol[i] = L::v_slot(ld_row[i], slot) * 8;
+    // XOR swizzles are involutions: slot -> source chunk uses the same function
+    ld_koff[i] = uint32_t(ld_row[i]) * uint32_t(kv_row_stride * 2) + uint32_t(L::k_slot(ld_row[i], slot) * 16);
+    ld_voff[i] = uint32_t(ld_row[i]) * uint32_t(kv_row_stride * 2) + uint32_t(L::v_slot(ld_row[i], slot) * 16);
   }
-  auto issue_tile_loads = [&](int kv_row0, auto stage_tag) {
-    char* sK = decltype(stage_tag)::value ? sK1 : sK0;
-    char* sV = decltype(stage_tag)::value ? sV1 : sV0;
+  auto issue_tile_load = [&](const T* base, const uint32_t (&off)[PER], char* dst, int kv_row0) {
+#ifdef NA_X_SAMETILE
+    kv_row0 = (kv_row0 % (8 * KVT));
+#endif
+    const char* tile_base = reinterpret_cast<const char*>(base) + int64_t(kv_row0) * kv_row_stride * 2;
+    if (kv_row0 + KVT <= p.seqlen_kv) {
 #pragma unroll
-    for (int i = 0; i < PER; ++i) {
-      // rows past the end of the sequence are masked; read a valid row instead of zero filling
-      const int grow = na_min(kv_row0 + ld_row[i], p.seqlen_kv - 1);
-      const int wave_chunk0 = (i * NT + wave * 64) * 16;
-      async_copy16(kbase + int64_t(grow) * kv_row_stride + ld_kcol[i], sK + wave_chunk0);
-      async_copy16(vbase + int64_t(grow) * kv_row_stride + ld_vcol[i], sV + wave_chunk0);
+      for (int i = 0; i < PER; ++i)
+        if (i * NT + wave * 64 < CHUNKS) async_copy16(tile_base + off[i], dst + (i * NT + wave * 64) * 16);
+    } else {
+      // last, partial tile of an unpadded sequence: rows past the end are masked anyway; read the
+      // last valid row instead so that no out-of-bounds address is formed
+#pragma unroll
+      for (int i = 0; i < PER; ++i) {
+        if (i * NT + wave * 64 >= CHUNKS) continue;
+        const int grow = na_min(kv_row0 + ld_row[i], p.seqlen_kv - 1);
+        const uint32_t in_row = off[i] - uint32_t(ld_row[i]) * uint32_t(kv_row_stride * 2);
+        async_copy16(reinterpret_cast<const char*>(base) + int64_t(grow) * kv_row_stride * 2 + in_row,
+                     dst + (i * NT + wave * 64) * 16);
+      }
     }
   };
 
-  // KV tile iteration state: dimension 2 fastest, dimension 0 slowest
-  int itc[3] = {0, 0, 0};
-  auto tile_row0 = [&]() {
-    return ((box_tile0[0] + itc[0]) + p.kv_tiled[0] * ((box_tile0[1] + itc[1]) + p.kv_tiled[1] * (box_tile0[2] + itc[2]))) * KVT;
+  // KV tile stream: dimension 2 fastest, dimension 0 slowest.  The load stream runs up to two
+  // tiles ahead of the softmax, so tile descriptors are produced in order and handed down.
+  struct TileInfo {
+    int row0;       // first row of the tile in the permuted KV sequence
+    int origin[3];  // coordinate of its first token
+    bool full;      // every key of the tile is attended by every query of this Q tile
   };
-  auto advance = [&]() {
+  int itc[3] = {0, 0, 0};
+  auto next_tile = [&]() {
+    TileInfo t;
+    t.full = true;
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+      t.origin[a] = (box_tile0[a] + itc[a]) * p.kv_tile[a];
+      t.full = t.full && (t.origin[a] >= full_lo[a]) && (t.origin[a] + p.kv_tile[a] <= full_hi[a]);
+    }
+    t.row0 = ((box_tile0[0] + itc[0]) + p.kv_tiled[0] * ((box_tile0[1] + itc[1]) + p.kv_tiled[1] * (box_tile0[2] + itc[2]))) * KVT;
     if (++itc[2] == box_n[2]) {
       itc[2] = 0;
       if (++itc[1] == box_n[1]) {
@@ -281,11 +321,14 @@ fna_fwd_kernel(const FnaParams p) {
         ++itc[0];
       }
     }
+    return t;
   };
 
   using Stage0 = std::integral_constant<int, 0>;
   using Stage1 = std::integral_constant<int, 1>;
-  issue_tile_loads(tile_row0(), Stage0{});
+  TileInfo cur = next_tile();  // tile 0
+  issue_tile_load(kbase, ld_koff, sK0, cur.row0);
+  issue_tile_load(vbase, ld_voff, sV0, cur.row0);
 
   // ---- per-lane setup: this lane's query rows, their windows, Q fragments ---------------------
   int wst[MQ][3], wen[MQ][3];
@@ -335,27 +378,8 @@ fna_fwd_kernel(const FnaParams p) {
   const int v_chunk = (l32 >> 4) * 2 + (v_j4 >> 1);  // 16-byte chunk inside the 64-byte column block
   const int v_sub = (v_j4 & 1) * 8;
 
-  // ---- main loop over the KV tile box (unrolled by the two LDS stages) -------------------------
-  auto process_tile = [&](auto stage_tag, int it) {
-    constexpr int stage = decltype(stage_tag)::value;
-    int origin[3];
-    bool full = true;
-#pragma unroll
-    for (int a = 0; a < 3; ++a) {
-      origin[a] = (box_tile0[a] + itc[a]) * p.kv_tile[a];
-      full = full && (origin[a] >= full_lo[a]) && (origin[a] + p.kv_tile[a] <= full_hi[a]);
-    }
-    advance();
-
-    wait_vmcnt<0>();   // this thread's copies of tile `it` have landed
-    __syncthreads();   // ... and everyone's; everyone is also done reading the other stage
-    if (it + 1 < total_tiles) issue_tile_loads(tile_row0(), std::integral_constant<int, stage ^ 1>{});
-
-    const char* sK = stage ? sK1 : sK0;
-    const char* sV = stage ? sV1 : sV0;
-
-    // S^T = K Q^T : lane owns query row l32 (per q block) and 16 key rows per 32-key sub-block
-    f32x16_t S[MQ][NSB];
+  // S^T = K Q^T of one tile: lane owns query row l32 (per q block) and 16 key rows per 32-key sub-block
+  auto qk_tile = [&](const char* sK, f32x16_t (&S)[MQ][NSB]) {
 #pragma unroll
     for (int sb = 0; sb < NSB; ++sb) {
 #pragma unroll
@@ -363,38 +387,82 @@ fna_fwd_kernel(const FnaParams p) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) S[mb][sb][r] = 0.f;
       // rows sb*32 + l32: (sb*32) is a multiple of 16 rows, so the swizzle term is unchanged
-      vec8 kf[KSTEPS];
 #pragma unroll
-      for (int ks = 0; ks < KSTEPS; ++ks) kf[ks] = *reinterpret_cast<const vec8*>(sK + sb * 32 * ROWB + k_off[ks]);
+      for (int ks = 0; ks < KSTEPS; ++ks) {
+        const vec8 kf = *reinterpret_cast<const vec8*>(sK + sb * 32 * ROWB + k_off[ks]);
 #pragma unroll
-      for (int ks = 0; ks < KSTEPS; ++ks)
-#pragma unroll
-        for (int mb = 0; mb < MQ; ++mb) S[mb][sb] = M::run(kf[ks], qf[mb][ks], S[mb][sb]);
+        for (int mb = 0; mb < MQ; ++mb) S[mb][sb] = M::run(kf, qf[mb][ks], S[mb][sb]);
+      }
     }
+  };
 
-    vec8 pf[MQ][NSB][2];
+  // ---- software pipeline --------------------------------------------------------------------
+  // Iteration j computes S(j+1) = K(j+1) Q^T on the matrix cores while the vector units run the
+  // softmax of S(j); then O += P(j) V(j).  At its top, K(j+2) and V(j+1) are put in flight.
+  // LDS: K(j) and V(j) live in stage j % 2.
+  TileInfo nxt = next_tile();  // tile 1 (a descriptor past the box is never used for loads)
+  wait_vmcnt<0>();
+  __syncthreads();  // K(0), V(0) and the coordinate table are in LDS
+  if (1 < total_tiles) issue_tile_load(kbase, ld_koff, sK1, nxt.row0);
+  f32x16_t S_cur[MQ][NSB];
+  qk_tile(sK0, S_cur);
+
+#ifdef NA_X_TIMING
+  unsigned long long tacc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  unsigned long long tlast = __builtin_amdgcn_s_memtime();
+#define NA_TICK1(k) { unsigned long long tn = __builtin_amdgcn_s_memtime(); tacc[k] += tn - tlast; tlast = tn; }
+#else
+#define NA_TICK1(k)
+#endif
+  auto iteration = [&](auto stage_tag, int j) {
+    constexpr int st = decltype(stage_tag)::value;
+    char* sK_cur = st ? sK1 : sK0;  // held K(j): free, receives K(j+2)
+    char* sK_nxt = st ? sK0 : sK1;  // holds K(j+1)
+    char* sV_cur = st ? sV1 : sV0;  // holds V(j)
+    char* sV_nxt = st ? sV0 : sV1;  // held V(j-1): free, receives V(j+1)
+
+    NA_TICK1(5)
+#ifndef NA_X_NOWAIT
+    wait_vmcnt<0>();   // this thread's copies of K(j+1) and V(j) have landed
+#endif
+    NA_TICK1(0)
+#ifndef NA_X_NOBAR
+    __syncthreads();   // ... and everyone's; everyone is done reading K(j) and V(j-1)
+#endif
+    NA_TICK1(1)
+    const TileInfo t2 = next_tile();
+#ifndef NA_X_NOLOAD
+    if (j + 2 < total_tiles) issue_tile_load(kbase, ld_koff, sK_cur, t2.row0);
+#ifndef NA_X_NOVLOAD
+    if (j + 1 < total_tiles) issue_tile_load(vbase, ld_voff, sV_nxt, nxt.row0);
+#endif
+#endif
+
+    NA_TICK1(2)
+    // -- softmax, part 1: mask, row maximum, (rare) rescale -----------------------------------
+    float msc[MQ];
 #pragma unroll
     for (int mb = 0; mb < MQ; ++mb) {
-      if (!full) {
+      if (!cur.full) {
         // window of this lane's query relative to the tile origin, clamped to the tile
         uint32_t addc = 0, subc = 0;
 #pragma unroll
         for (int a = 0; a < 3; ++a) {
-          const int lo = na_min(na_max(wst[mb][a] - origin[a], 0), p.kv_tile[a]);
-          const int hi = na_min(na_max(wen[mb][a] - origin[a], 0), p.kv_tile[a]);
+          const int lo = na_min(na_max(wst[mb][a] - cur.origin[a], 0), p.kv_tile[a]);
+          const int hi = na_min(na_max(wen[mb][a] - cur.origin[a], 0), p.kv_tile[a]);
           addc |= uint32_t(512 - lo) << (10 * a);
           subc |= uint32_t(511 + hi) << (10 * a);
         }
 #pragma unroll
         for (int sb = 0; sb < NSB; ++sb)
 #pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            const u32x4_t tc4 = *reinterpret_cast<const u32x4_t*>(&sTab[sb * 32 + 8 * j + 4 * g]);
+          for (int jj = 0; jj < 4; ++jj) {
+            const u32x4_t tc4 = *reinterpret_cast<const u32x4_t*>(&sTab[sb * 32 + 8 * jj + 4 * g]);
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
               const uint32_t tp = tc4[i];
               const uint32_t ok = (tp + addc) & (subc - tp) & kGuardBits;
-              S[mb][sb][4 * j + i] = (ok == kGuardBits) ? S[mb][sb][4 * j + i] : -INFINITY;
+              S_cur[mb][sb][4 * jj + i] = (ok == kGuardBits) ? S_cur[mb][sb][4 * jj + i] : -INFINITY;
             }
           }
       }
@@ -402,7 +470,7 @@ fna_fwd_kernel(const FnaParams p) {
 #pragma unroll
       for (int sb = 0; sb < NSB; ++sb)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, S[mb][sb][r]);
+        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, S_cur[mb][sb][r]);
       mx = fmaxf(mx, __shfl_xor(mx, 32));
       // rescale only when some row of this wave outgrew its (stale) maximum by more than 2^8
       const bool grow = (mx - m_run[mb]) * c_log2 > kLazyRescaleLog2;  // also true while m_run == -inf and mx finite
@@ -417,7 +485,20 @@ fna_fwd_kernel(const FnaParams p) {
 #pragma unroll
           for (int r = 0; r < 16; ++r) acc[mb][db][r] *= alpha;
       }
-      const float msc = ((m_run[mb] == -INFINITY) ? 0.f : m_run[mb]) * c_log2;
+      msc[mb] = ((m_run[mb] == -INFINITY) ? 0.f : m_run[mb]) * c_log2;
+    }
+
+    NA_TICK1(3)
+    // -- S(j+1) on the matrix cores, exponentials of S(j) on the vector units ------------------
+    f32x16_t S_nxt[MQ][NSB];
+#ifndef NA_X_NOQK
+    qk_tile(sK_nxt, S_nxt);
+#else
+    for (int mb = 0; mb < MQ; ++mb) for (int sb = 0; sb < NSB; ++sb) S_nxt[mb][sb] = S_cur[mb][sb] + 1.0f;
+#endif
+    vec8 pf[MQ][NSB][2];
+#pragma unroll
+    for (int mb = 0; mb < MQ; ++mb) {
       float psum = 0.f;
 #pragma unroll
       for (int sb = 0; sb < NSB; ++sb)
@@ -427,8 +508,8 @@ fna_fwd_kernel(const FnaParams p) {
 #pragma unroll
           for (int i = 0; i < 8; i += 2) {
             vec2 p2;
-            p2[0] = static_cast<T>(fast_exp2(S[mb][sb][8 * h + i] * c_log2 - msc));
-            p2[1] = static_cast<T>(fast_exp2(S[mb][sb][8 * h + i + 1] * c_log2 - msc));
+            p2[0] = static_cast<T>(fast_exp2(S_cur[mb][sb][8 * h + i] * c_log2 - msc[mb]));
+            p2[1] = static_cast<T>(fast_exp2(S_cur[mb][sb][8 * h + i + 1] * c_log2 - msc[mb]));
             psum = M::add2(p2, psum);  // sums the rounded probabilities, the ones P V uses
             pv[i] = p2[0];
             pv[i + 1] = p2[1];
@@ -438,15 +519,16 @@ fna_fwd_kernel(const FnaParams p) {
       l_run[mb] += psum;
     }
 
-    // O^T += V^T P^T : the k-slot order of the P fragment (rows 4g..4g+3 and 8+4g..8+4g+3 of
+    NA_TICK1(4)
+    // -- O^T += V^T P^T : the k-slot order of the P fragment (rows 4g..4g+3 and 8+4g..8+4g+3 of
     // each 16-key half) is matched by two transpose reads of V.
 #pragma unroll
     for (int sb = 0; sb < NSB; ++sb)
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
-        const int r0 = sb * 32 + h * 16 + v_row;  // r0 + 8 shares (r0 / RPL) % (CPR/2) only when RPL >= 16; recompute
-        const char* row_lo = sV + r0 * ROWB + v_sub;
-        const char* row_hi = sV + (r0 + 8) * ROWB + v_sub;
+        const int r0 = sb * 32 + h * 16 + v_row;
+        const char* row_lo = sV_cur + r0 * ROWB + v_sub;
+        const char* row_hi = sV_cur + (r0 + 8) * ROWB + v_sub;
 #pragma unroll
         for (int db = 0; db < DB; ++db) {
           const int c = db * 4 + v_chunk;
@@ -455,14 +537,30 @@ fna_fwd_kernel(const FnaParams p) {
           const s16x8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
           const vec8 vf = __builtin_bit_cast(vec8, both);
 #pragma unroll
+#ifndef NA_X_NOPV
           for (int mb = 0; mb < MQ; ++mb) acc[mb][db] = M::run(vf, pf[mb][sb][h], acc[mb][db]);
+#else
+          for (int mb = 0; mb < MQ; ++mb) acc[mb][db][0] += float(vf[0]) * float(pf[mb][sb][h][0]);
+#endif
         }
       }
+
+#pragma unroll
+    for (int mb = 0; mb < MQ; ++mb)
+#pragma unroll
+      for (int sb = 0; sb < NSB; ++sb) S_cur[mb][sb] = S_nxt[mb][sb];
+    cur = nxt;
+    nxt = t2;
   };
-  for (int it = 0; it < total_tiles; it += 2) {
-    process_tile(Stage0{}, it);
-    if (it + 1 < total_tiles) process_tile(Stage1{}, it + 1);
+  for (int j = 0; j < total_tiles; j += 2) {
+    iteration(Stage0{}, j);
+    if (j + 1 < total_tiles) iteration(Stage1{}, j + 1);
   }
+#ifdef NA_X_TIMING
+  if ((blockIdx.x == 4000 || blockIdx.x == 15001) && lane == 0)
+    printf("blk %d wave %d tiles %d | vmwait %llu barrier %llu issue %llu part1 %llu qk+exp %llu pv %llu\n", blockIdx.x, wave, total_tiles,
+           tacc[0] / total_tiles, tacc[1] / total_tiles, tacc[2] / total_tiles, tacc[3] / total_tiles, tacc[4] / total_tiles, tacc[5] / total_tiles);
+#endif
 
   // ---- epilogue: O = acc / rowsum, LSE = ln(rowsum) + scale * rowmax -------------------------
   T* obase = reinterpret_cast<T*>(p.o) + int64_t(bg) * p.seqlen_q * q_row_stride + int64_t(head) * D;

@@ -6,11 +6,13 @@
 #include <hip/hip_runtime.h>
 #include <stdarg.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include <type_traits>
 
 #include "fna_fwd.hpp"
+#include "fna_fwd_pp.hpp"
 #include "merge.hpp"
 #include "na_math.hpp"
 #include "tokperm.hpp"
@@ -40,15 +42,37 @@ int prod3(const int* x) { return x[0] * x[1] * x[2]; }
 // Workgroup layout: Q tiles are enumerated with dimension 0 slowest; a group is a run of about
 // as many consecutive Q tiles as one XCD keeps resident (32 CUs x 2 workgroups), made of whole
 // dimension-0 slabs when possible, so that the tiles resident on an XCD overlap in their KV boxes.
-void set_wg_layout(FnaParams& p) {
+// `tiles_per_wg` Q tiles share a workgroup (consecutive tiles of the enumeration) and an XCD keeps
+// about 64 Q tiles resident either way (32 CUs x 2 single-tile workgroups or x 1 two-tile workgroup).
+void set_wg_layout(FnaParams& p, int tiles_per_wg) {
   p.num_q_tiles = p.q_tiled[0] * p.q_tiled[1] * p.q_tiled[2];
   const int slab = p.q_tiled[1] * p.q_tiled[2];
   int rows = (64 + slab / 2) / slab;
   if (rows < 1) rows = 1;
   if (rows > p.q_tiled[0]) rows = p.q_tiled[0];
-  p.wg_group = slab * rows;
-  p.groups_per_bh = (p.num_q_tiles + p.wg_group - 1) / p.wg_group;
+  const int units = (p.num_q_tiles + tiles_per_wg - 1) / tiles_per_wg;
+  p.wg_group = (slab * rows + tiles_per_wg - 1) / tiles_per_wg;
+  if (p.wg_group > units) p.wg_group = units;
+  p.groups_per_bh = (units + p.wg_group - 1) / p.wg_group;
   p.total_groups = p.batch * p.heads_q * p.groups_per_bh;
+}
+
+// Schedule choice for 128 x 64 tiles: the two-group kernel needs enough Q tiles to fill the
+// chip with half as many workgroups.  NATTEN_AMD_FNA_SCHEDULE=single|pingpong overrides.
+bool use_pingpong(const FnaParams& p) {
+  const char* e = getenv("NATTEN_AMD_FNA_SCHEDULE");
+  if (e && !strcmp(e, "single")) return false;
+  if (e && !strcmp(e, "pingpong")) return true;
+  return false;
+}
+
+template <typename T, int D, int KVT>
+int launch_fna_pp(FnaParams p, hipStream_t stream) {
+  set_wg_layout(p, 2);
+  const long long wgs = (long long)((p.total_groups + kNumXcd - 1) / kNumXcd) * kNumXcd * p.wg_group;
+  if (wgs > 0x7fffffffLL) return fail("fna_forward: problem needs more than 2^31 workgroups");
+  hipLaunchKernelGGL((fna_fwd_pp_kernel<T, D, KVT>), dim3((unsigned)wgs), dim3(512), 0, stream, p);
+  return check_launch("fna_forward");
 }
 
 struct TileConfig {
@@ -72,8 +96,11 @@ int launch_fna(const FnaParams& p, hipStream_t stream) {
 
 template <typename T, int D>
 int dispatch_tiles(const FnaParams& p, int qt, int kvt, hipStream_t stream) {
-  if (qt == 128 && kvt == 64) return launch_fna<T, D, 4, 1, 64>(p, stream);
-  if (qt == 256 && kvt == 64) return launch_fna<T, D, 4, 2, 64>(p, stream);
+  if (qt == 128 && kvt == 64) {
+    if (use_pingpong(p)) return launch_fna_pp<T, D, 64>(p, stream);
+    return launch_fna<T, D, 4, 1, 64>(p, stream);
+  }
+  if (qt == 256 && kvt == 64) return launch_fna<T, D, 8, 1, 64>(p, stream);
   if (qt == 128 && kvt == 128) return launch_fna<T, D, 4, 1, 128>(p, stream);
   if (qt == 256 && kvt == 128) return launch_fna<T, D, 4, 2, 128>(p, stream);
   if (qt == 64 && kvt == 64) return launch_fna<T, D, 2, 1, 64>(p, stream);
@@ -195,7 +222,7 @@ int natten_amd_fna_forward(const void* q, const void* k, const void* v, void* ou
   p.seqlen_kv = seqlen_kv;
   p.scale = scale * q_scale * k_scale;
   p.out_scale = v_scale;
-  set_wg_layout(p);
+  set_wg_layout(p, 1);
   return dispatch_dtype(p, dtype, head_dim, prod3(p.q_tile), prod3(p.kv_tile), static_cast<hipStream_t>(stream));
 }
 
@@ -239,7 +266,7 @@ int natten_amd_attention_forward(const void* q, const void* k, const void* v, vo
   p.seqlen_kv = seqlen_kv;
   p.scale = scale;
   p.out_scale = 1.f;
-  set_wg_layout(p);
+  set_wg_layout(p, 1);
   return dispatch_dtype(p, dtype, head_dim, QT, KVT, static_cast<hipStream_t>(stream));
 }
 
