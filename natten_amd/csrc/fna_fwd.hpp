@@ -102,12 +102,26 @@ static __device__ __forceinline__ s16x4_t lds_read_tr16(const char* p) {
 #pragma clang diagnostic pop
 }
 
-// Asynchronous 16-byte-per-lane copy global -> LDS: lane i's 16 bytes land at lds_base + 16*i
-// (lds_base must be wave-uniform).  Completion is tracked by the vector memory counter.
-static __device__ __forceinline__ void async_copy16(const void* gptr, char* lds_base) {
+// Asynchronous 16-byte-per-lane copy global -> LDS, written as inline assembly so that the
+// compiler does not see an LDS write in flight (it would otherwise make every later LDS read
+// wait for the copy): lane i's 16 bytes from `base + voff (+ IMM)` land at LDS address
+// `lds_addr + IMM + 16 * i`.  Completion is tracked by the vector memory counter; ordering
+// against LDS reads of the same bytes is the caller's business (workgroup barriers).
+template <int IMM>
+static __device__ __forceinline__ void async_copy16_asm(const void* base, uint32_t voff, uint32_t lds_addr) {
+  asm volatile(
+      "s_mov_b32 m0, %0\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dwordx4 %1, %2 offset:%3"
+      :
+      : "s"(lds_addr), "v"(voff), "s"(base), "n"(IMM)
+      : "memory", "m0");
+}
+
+static __device__ __forceinline__ uint32_t lds_address(const void* p) {
 #pragma clang diagnostic push
 #pragma clang diagnostic ignored "-Wold-style-cast"
-  __builtin_amdgcn_global_load_lds((const NA_GLOBAL void*)(gptr), (NA_LDS void*)(lds_base), 16, 0, 0);
+  return (uint32_t)(uintptr_t)((NA_LDS const char*)(p));
 #pragma clang diagnostic pop
 }
 
@@ -118,11 +132,7 @@ static __device__ __forceinline__ void wait_vmcnt() {
   __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 0xF) | ((N >> 4) << 14));
 }
 
-#ifdef NA_X_NOEXP
-static __device__ __forceinline__ float fast_exp2(float x) { return x; }
-#else
 static __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
-#endif
 
 // max of x over the lane pair (l, l ^ 32): v_permlane32_swap exchanges the upper half of its
 // first register with the lower half of its second, after which every lane holds both values
@@ -267,34 +277,45 @@ fna_fwd_kernel(const FnaParams p) {
   uint32_t ld_koff[PER], ld_voff[PER];
 #pragma unroll
   for (int i = 0; i < PER; ++i) {
-    const int P = i * NT + tid;
+    // copy i of wave w fills LDS chunks (w*PER + i)*64 .. +63; up to four copies share one M0
+    // value through the instruction's immediate offset, which the hardware adds to the global
+    // address as well, hence the compensation
+    const int P = (wave * PER + i) * 64 + lane;
     ld_row[i] = P / CPR;
     const int slot = P % CPR;
+    const uint32_t imm = uint32_t(i % 4) * 1024u;
     // XOR swizzles are involutions: slot -> source chunk uses the same function
-    ld_koff[i] = uint32_t(ld_row[i]) * uint32_t(kv_row_stride * 2) + uint32_t(L::k_slot(ld_row[i], slot) * 16);
-    ld_voff[i] = uint32_t(ld_row[i]) * uint32_t(kv_row_stride * 2) + uint32_t(L::v_slot(ld_row[i], slot) * 16);
+    ld_koff[i] = uint32_t(ld_row[i]) * uint32_t(kv_row_stride * 2) + uint32_t(L::k_slot(ld_row[i], slot) * 16) - imm;
+    ld_voff[i] = uint32_t(ld_row[i]) * uint32_t(kv_row_stride * 2) + uint32_t(L::v_slot(ld_row[i], slot) * 16) - imm;
   }
   auto issue_tile_load = [&](const T* base, const uint32_t (&off)[PER], char* dst, int kv_row0) {
-#ifdef NA_X_SAMETILE
-    kv_row0 = (kv_row0 % (8 * KVT));
-#endif
     const char* tile_base = reinterpret_cast<const char*>(base) + int64_t(kv_row0) * kv_row_stride * 2;
-    if (kv_row0 + KVT <= p.seqlen_kv) {
-#pragma unroll
-      for (int i = 0; i < PER; ++i)
-        if (i * NT + wave * 64 < CHUNKS) async_copy16(tile_base + off[i], dst + (i * NT + wave * 64) * 16);
-    } else {
-      // last, partial tile of an unpadded sequence: rows past the end are masked anyway; read the
-      // last valid row instead so that no out-of-bounds address is formed
-#pragma unroll
-      for (int i = 0; i < PER; ++i) {
-        if (i * NT + wave * 64 >= CHUNKS) continue;
-        const int grow = na_min(kv_row0 + ld_row[i], p.seqlen_kv - 1);
-        const uint32_t in_row = off[i] - uint32_t(ld_row[i]) * uint32_t(kv_row_stride * 2);
-        async_copy16(reinterpret_cast<const char*>(base) + int64_t(grow) * kv_row_stride * 2 + in_row,
-                     dst + (i * NT + wave * 64) * 16);
+    const uint32_t lds0 = lds_address(dst) + uint32_t(wave * PER * 1024);
+    const bool inside = kv_row0 + KVT <= p.seqlen_kv;
+    auto one = [&](auto i_tag) {
+      constexpr int I = decltype(i_tag)::value;
+      if constexpr (I < PER) {
+        if ((wave * PER + I) * 64 < CHUNKS) {
+          uint32_t voff = off[I];
+          if (!inside) {
+            // last, partial tile of an unpadded sequence: rows past the end are masked; read the
+            // last valid row instead so that no out-of-bounds address is formed
+            const int over = na_max(kv_row0 + ld_row[I] - (p.seqlen_kv - 1), 0);
+            voff -= uint32_t(over) * uint32_t(kv_row_stride * 2);
+          }
+          async_copy16_asm<(I % 4) * 1024>(tile_base, voff, lds0 + uint32_t((I / 4) * 4096));
+        }
       }
-    }
+    };
+    one(std::integral_constant<int, 0>{});
+    one(std::integral_constant<int, 1>{});
+    one(std::integral_constant<int, 2>{});
+    one(std::integral_constant<int, 3>{});
+    one(std::integral_constant<int, 4>{});
+    one(std::integral_constant<int, 5>{});
+    one(std::integral_constant<int, 6>{});
+    one(std::integral_constant<int, 7>{});
+    static_assert(PER <= 8, "tile copy is written for at most eight copies per thread");
   };
 
   // KV tile stream: dimension 2 fastest, dimension 0 slowest.  The load stream runs up to two
@@ -407,13 +428,6 @@ fna_fwd_kernel(const FnaParams p) {
   f32x16_t S_cur[MQ][NSB];
   qk_tile(sK0, S_cur);
 
-#ifdef NA_X_TIMING
-  unsigned long long tacc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-  unsigned long long tlast = __builtin_amdgcn_s_memtime();
-#define NA_TICK1(k) { unsigned long long tn = __builtin_amdgcn_s_memtime(); tacc[k] += tn - tlast; tlast = tn; }
-#else
-#define NA_TICK1(k)
-#endif
   auto iteration = [&](auto stage_tag, int j) {
     constexpr int st = decltype(stage_tag)::value;
     char* sK_cur = st ? sK1 : sK0;  // held K(j): free, receives K(j+2)
@@ -421,24 +435,12 @@ fna_fwd_kernel(const FnaParams p) {
     char* sV_cur = st ? sV1 : sV0;  // holds V(j)
     char* sV_nxt = st ? sV0 : sV1;  // held V(j-1): free, receives V(j+1)
 
-    NA_TICK1(5)
-#ifndef NA_X_NOWAIT
     wait_vmcnt<0>();   // this thread's copies of K(j+1) and V(j) have landed
-#endif
-    NA_TICK1(0)
-#ifndef NA_X_NOBAR
     __syncthreads();   // ... and everyone's; everyone is done reading K(j) and V(j-1)
-#endif
-    NA_TICK1(1)
     const TileInfo t2 = next_tile();
-#ifndef NA_X_NOLOAD
     if (j + 2 < total_tiles) issue_tile_load(kbase, ld_koff, sK_cur, t2.row0);
-#ifndef NA_X_NOVLOAD
     if (j + 1 < total_tiles) issue_tile_load(vbase, ld_voff, sV_nxt, nxt.row0);
-#endif
-#endif
 
-    NA_TICK1(2)
     // -- softmax, part 1: mask, row maximum, (rare) rescale -----------------------------------
     float msc[MQ];
 #pragma unroll
@@ -471,7 +473,7 @@ fna_fwd_kernel(const FnaParams p) {
       for (int sb = 0; sb < NSB; ++sb)
 #pragma unroll
         for (int r = 0; r < 16; ++r) mx = fmaxf(mx, S_cur[mb][sb][r]);
-      mx = fmaxf(mx, __shfl_xor(mx, 32));
+      mx = cross_half_max(mx);
       // rescale only when some row of this wave outgrew its (stale) maximum by more than 2^8
       const bool grow = (mx - m_run[mb]) * c_log2 > kLazyRescaleLog2;  // also true while m_run == -inf and mx finite
       if (__any(grow)) {
@@ -488,14 +490,9 @@ fna_fwd_kernel(const FnaParams p) {
       msc[mb] = ((m_run[mb] == -INFINITY) ? 0.f : m_run[mb]) * c_log2;
     }
 
-    NA_TICK1(3)
     // -- S(j+1) on the matrix cores, exponentials of S(j) on the vector units ------------------
     f32x16_t S_nxt[MQ][NSB];
-#ifndef NA_X_NOQK
     qk_tile(sK_nxt, S_nxt);
-#else
-    for (int mb = 0; mb < MQ; ++mb) for (int sb = 0; sb < NSB; ++sb) S_nxt[mb][sb] = S_cur[mb][sb] + 1.0f;
-#endif
     vec8 pf[MQ][NSB][2];
 #pragma unroll
     for (int mb = 0; mb < MQ; ++mb) {
@@ -519,7 +516,6 @@ fna_fwd_kernel(const FnaParams p) {
       l_run[mb] += psum;
     }
 
-    NA_TICK1(4)
     // -- O^T += V^T P^T : the k-slot order of the P fragment (rows 4g..4g+3 and 8+4g..8+4g+3 of
     // each 16-key half) is matched by two transpose reads of V.
 #pragma unroll
@@ -537,11 +533,7 @@ fna_fwd_kernel(const FnaParams p) {
           const s16x8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
           const vec8 vf = __builtin_bit_cast(vec8, both);
 #pragma unroll
-#ifndef NA_X_NOPV
           for (int mb = 0; mb < MQ; ++mb) acc[mb][db] = M::run(vf, pf[mb][sb][h], acc[mb][db]);
-#else
-          for (int mb = 0; mb < MQ; ++mb) acc[mb][db][0] += float(vf[0]) * float(pf[mb][sb][h][0]);
-#endif
         }
       }
 
@@ -556,11 +548,6 @@ fna_fwd_kernel(const FnaParams p) {
     iteration(Stage0{}, j);
     if (j + 1 < total_tiles) iteration(Stage1{}, j + 1);
   }
-#ifdef NA_X_TIMING
-  if ((blockIdx.x == 4000 || blockIdx.x == 15001) && lane == 0)
-    printf("blk %d wave %d tiles %d | vmwait %llu barrier %llu issue %llu part1 %llu qk+exp %llu pv %llu\n", blockIdx.x, wave, total_tiles,
-           tacc[0] / total_tiles, tacc[1] / total_tiles, tacc[2] / total_tiles, tacc[3] / total_tiles, tacc[4] / total_tiles, tacc[5] / total_tiles);
-#endif
 
   // ---- epilogue: O = acc / rowsum, LSE = ln(rowsum) + scale * rowmax -------------------------
   T* obase = reinterpret_cast<T*>(p.o) + int64_t(bg) * p.seqlen_q * q_row_stride + int64_t(head) * D;

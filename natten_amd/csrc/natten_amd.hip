@@ -12,7 +12,6 @@
 #include <type_traits>
 
 #include "fna_fwd.hpp"
-#include "fna_fwd_pp.hpp"
 #include "merge.hpp"
 #include "na_math.hpp"
 #include "tokperm.hpp"
@@ -44,7 +43,7 @@ int prod3(const int* x) { return x[0] * x[1] * x[2]; }
 // dimension-0 slabs when possible, so that the tiles resident on an XCD overlap in their KV boxes.
 // `tiles_per_wg` Q tiles share a workgroup (consecutive tiles of the enumeration) and an XCD keeps
 // about 64 Q tiles resident either way (32 CUs x 2 single-tile workgroups or x 1 two-tile workgroup).
-void set_wg_layout(FnaParams& p, int tiles_per_wg) {
+void set_wg_layout(FnaParams& p, int tiles_per_wg = 1) {
   p.num_q_tiles = p.q_tiled[0] * p.q_tiled[1] * p.q_tiled[2];
   const int slab = p.q_tiled[1] * p.q_tiled[2];
   int rows = (64 + slab / 2) / slab;
@@ -57,30 +56,12 @@ void set_wg_layout(FnaParams& p, int tiles_per_wg) {
   p.total_groups = p.batch * p.heads_q * p.groups_per_bh;
 }
 
-// Schedule choice for 128 x 64 tiles: the two-group kernel needs enough Q tiles to fill the
-// chip with half as many workgroups.  NATTEN_AMD_FNA_SCHEDULE=single|pingpong overrides.
-bool use_pingpong(const FnaParams& p) {
-  const char* e = getenv("NATTEN_AMD_FNA_SCHEDULE");
-  if (e && !strcmp(e, "single")) return false;
-  if (e && !strcmp(e, "pingpong")) return true;
-  return false;
-}
-
-template <typename T, int D, int KVT>
-int launch_fna_pp(FnaParams p, hipStream_t stream) {
-  set_wg_layout(p, 2);
-  const long long wgs = (long long)((p.total_groups + kNumXcd - 1) / kNumXcd) * kNumXcd * p.wg_group;
-  if (wgs > 0x7fffffffLL) return fail("fna_forward: problem needs more than 2^31 workgroups");
-  hipLaunchKernelGGL((fna_fwd_pp_kernel<T, D, KVT>), dim3((unsigned)wgs), dim3(512), 0, stream, p);
-  return check_launch("fna_forward");
-}
-
 struct TileConfig {
   int q_tile, kv_tile;
 };
 
 // (Q tile, KV tile) sizes in tokens that have a kernel instance.
-const TileConfig kTileConfigs[] = {{128, 64}, {256, 64}, {128, 128}, {256, 128}, {64, 64}};
+const TileConfig kTileConfigs[] = {{128, 64}, {256, 64}, {128, 128}, {64, 64}};
 constexpr int kNumTileConfigs = sizeof(kTileConfigs) / sizeof(kTileConfigs[0]);
 
 template <typename T, int D, int NWAVES, int MQ, int KVT>
@@ -96,13 +77,9 @@ int launch_fna(const FnaParams& p, hipStream_t stream) {
 
 template <typename T, int D>
 int dispatch_tiles(const FnaParams& p, int qt, int kvt, hipStream_t stream) {
-  if (qt == 128 && kvt == 64) {
-    if (use_pingpong(p)) return launch_fna_pp<T, D, 64>(p, stream);
-    return launch_fna<T, D, 4, 1, 64>(p, stream);
-  }
+  if (qt == 128 && kvt == 64) return launch_fna<T, D, 4, 1, 64>(p, stream);
   if (qt == 256 && kvt == 64) return launch_fna<T, D, 8, 1, 64>(p, stream);
   if (qt == 128 && kvt == 128) return launch_fna<T, D, 4, 1, 128>(p, stream);
-  if (qt == 256 && kvt == 128) return launch_fna<T, D, 4, 2, 128>(p, stream);
   if (qt == 64 && kvt == 64) return launch_fna<T, D, 2, 1, 64>(p, stream);
   return fail("fna_forward: no kernel for Q tile of %d and KV tile of %d tokens", qt, kvt);
 }
