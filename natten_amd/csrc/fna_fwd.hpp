@@ -278,15 +278,13 @@ fna_fwd_kernel(const FnaParams p) {
 #pragma unroll
   for (int i = 0; i < PER; ++i) {
     // copy i of wave w fills LDS chunks (w*PER + i)*64 .. +63; up to four copies share one M0
-    // value through the instruction's immediate offset, which the hardware adds to the global
-    // address as well, hence the compensation
+    // value through the instruction's immediate offset
     const int P = (wave * PER + i) * 64 + lane;
     ld_row[i] = P / CPR;
     const int slot = P % CPR;
-    const uint32_t imm = uint32_t(i % 4) * 1024u;
     // XOR swizzles are involutions: slot -> source chunk uses the same function
-    ld_koff[i] = uint32_t(ld_row[i]) * uint32_t(kv_row_stride * 2) + uint32_t(L::k_slot(ld_row[i], slot) * 16) - imm;
-    ld_voff[i] = uint32_t(ld_row[i]) * uint32_t(kv_row_stride * 2) + uint32_t(L::v_slot(ld_row[i], slot) * 16) - imm;
+    ld_koff[i] = uint32_t(ld_row[i]) * uint32_t(kv_row_stride * 2) + uint32_t(L::k_slot(ld_row[i], slot) * 16);
+    ld_voff[i] = uint32_t(ld_row[i]) * uint32_t(kv_row_stride * 2) + uint32_t(L::v_slot(ld_row[i], slot) * 16);
   }
   auto issue_tile_load = [&](const T* base, const uint32_t (&off)[PER], char* dst, int kv_row0) {
     const char* tile_base = reinterpret_cast<const char*>(base) + int64_t(kv_row0) * kv_row_stride * 2;
@@ -303,7 +301,9 @@ fna_fwd_kernel(const FnaParams p) {
             const int over = na_max(kv_row0 + ld_row[I] - (p.seqlen_kv - 1), 0);
             voff -= uint32_t(over) * uint32_t(kv_row_stride * 2);
           }
-          async_copy16_asm<(I % 4) * 1024>(tile_base, voff, lds0 + uint32_t((I / 4) * 4096));
+          // the hardware adds the immediate to the global address too: take it off the uniform
+          // base (the per-lane offset stays a small non-negative number)
+          async_copy16_asm<(I % 4) * 1024>(tile_base - (I % 4) * 1024, voff, lds0 + uint32_t((I / 4) * 4096));
         }
       }
     };
