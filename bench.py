@@ -30,6 +30,13 @@ WORKLOADS = {
     "c2": (2, 8, (64, 64), 64, (13, 13), (1, 1), (1, 1), (False, False), "bf16", 1.0),
     "c2d": (2, 8, (64, 64), 64, (13, 13), (1, 1), (2, 2), (False, False), "bf16", 1.0),
 }
+# HBM-side traffic of one fused-kernel launch, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# and calibrated on the permute kernel (a copy of known size); see profiles/fna_fwd_c4_na3d_bf16.md.
+# Keyed by (workload, q_tile_shape, kv_tile_shape); other combinations report null.
+MEASURED_TRAFFIC_BYTES = {
+    ("c4", (2, 8, 8), (1, 8, 8)): 2.77e10,
+}
+
 WORKLOAD_NAMES = {
     "c4": "na3d bf16 B=1 H=24 30x48x80 D=128 k=(18,24,24) s=(1,8,8) causal=(T,F,F) +LSE",
     "c3": "na2d fp16 B=1 H=16 128x128 D=128 k=(32,32) s=(16,16)",
@@ -226,7 +233,8 @@ def main():
             "peak": peak,
             "unit": "TFLOP/s",
             "frac": achieved / peak,
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, tuple(q_tile), tuple(kv_tile))),
+            "algorithmic_bytes": 4 * q_bytes + lse.numel() * 4,
         },
     }
     if not args.no_cpu_baseline:

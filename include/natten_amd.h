@@ -103,7 +103,8 @@ int natten_amd_token_unpermute(const void* src, void* dst, int elem_bytes, int n
  * Merge two partial attentions over disjoint key sets of the same queries:
  *   out = o0 - sigmoid(lse1 - lse0) * (o0 - o1),  lse = lse0 - logsigmoid(lse0 - lse1)
  * o0/o1/out [rows, head_dim] of `dtype` (F16/BF16/F32), lse0/lse1/lse_out [rows] float32,
- * rows = batch * seqlen * heads.  out may alias o0, lse_out may alias lse0.
+ * rows = batch * seqlen * heads.  out may alias o0; lse_out must not alias lse0 or lse1
+ * (several lanes of a row read both while one writes the result; aliasing is rejected).
  */
 int natten_amd_merge_attentions(const void* o0, const float* lse0, const void* o1,
                                 const float* lse1, void* out, float* lse_out, int dtype,
