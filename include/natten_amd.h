@@ -12,6 +12,7 @@
  *   natten_amd_fna_forward      <- blackwell_na{1,2,3}d_forward
  *                                  csrc/include/natten/blackwell_fna.h:36-52, csrc/natten.cpp:39-160
  *   natten_amd_token_permute    <- token_permute_{1,2,3}d   csrc/include/natten/token_permute.h:34-52
+ *   natten_amd_token_permute_widen <- the same, for e4m3 / e5m2 operands (writes bf16)
  *   natten_amd_token_unpermute  <- token_unpermute_{1,2,3}d csrc/include/natten/token_permute.h:54-74
  *   natten_amd_attention_forward<- blackwell_fmha_forward   csrc/include/natten/blackwell_fmha.h
  *                                  (dense attention used for additional keys/values and for
@@ -31,8 +32,9 @@ extern "C" {
 /* Element types of Q/K/V (`dtype` arguments). */
 #define NATTEN_AMD_F16 0
 #define NATTEN_AMD_BF16 1
-#define NATTEN_AMD_F8E4M3 2 /* OCP e4m3fn inputs, bf16 output */
-#define NATTEN_AMD_F32 3    /* merge / permute payloads only */
+#define NATTEN_AMD_F8E4M3 2 /* OCP e4m3fn: source type of natten_amd_token_permute_widen only */
+#define NATTEN_AMD_F32 3    /* merge payloads only */
+#define NATTEN_AMD_F8E5M2 4 /* OCP e5m2: source type of natten_amd_token_permute_widen only */
 
 /* ABI version; bumped whenever a signature changes. */
 int natten_amd_abi_version(void);
@@ -45,7 +47,7 @@ const char* natten_amd_last_error(void);
  *
  *   q   [batch, seqlen_q,  heads_q,  head_dim]   contiguous
  *   k,v [batch, seqlen_kv, heads_kv, head_dim]   contiguous, heads_q % heads_kv == 0
- *   out [batch, seqlen_q,  heads_q,  head_dim]   dtype of q (bf16 when q is e4m3)
+ *   out [batch, seqlen_q,  heads_q,  head_dim]   dtype of q
  *   lse [batch, seqlen_q,  heads_q]              float32, natural log of the sum of exp(scale*q.k)
  *
  * `batch` already includes the dilation groups (batch index = b * prod(dilation) + group,
@@ -53,9 +55,15 @@ const char* natten_amd_last_error(void);
  * layouts the permuted sequences were built from (seqlen = product), qkv_shape the original
  * token layout.  All shape-like arrays hold `na_dim` entries.  Tiles are multi-dimensional;
  * their element counts must be a supported (Q tile, KV tile) pair, see
- * natten_amd_fna_supported_tiles().  head_dim must be 32, 64 or 128.
- * For e4m3 inputs q_scale*k_scale multiplies the logits' scale and v_scale the output
- * (pass 1.0f otherwise).
+ * natten_amd_fna_supported_tiles().  head_dim must be 32, 64 or 128.  dtype is F16 or BF16.
+ *
+ * q_scale [heads_q], k_scale [heads_kv], v_scale [heads_kv] are optional device arrays of
+ * per-head dequantisation scales (NULL = 1): logits are scale * q_scale[h] * k_scale[hkv] * q.k,
+ * the output is multiplied by v_scale[hkv], and lse is the log-sum-exp of those logits.
+ * Quantised 8-bit float operands (the reference passes e4m3 / e5m2 tensors to this same entry
+ * point, csrc/src/blackwell_fna_forward.cu:81-222) are served in two steps: widen them to bf16
+ * while permuting with natten_amd_token_permute_widen (exact), then call this function with
+ * dtype BF16 and the scales.  Passing an 8-bit dtype code here is an error.
  */
 int natten_amd_fna_forward(const void* q, const void* k, const void* v, void* out, float* lse,
                            int dtype, int na_dim, int batch, int seqlen_q, int seqlen_kv,
@@ -64,7 +72,8 @@ int natten_amd_fna_forward(const void* q, const void* k, const void* v, void* ou
                            const int32_t* kernel_size, const int32_t* stride,
                            const int32_t* dilation, const int32_t* is_causal,
                            const int32_t* q_tile_shape, const int32_t* kv_tile_shape, float scale,
-                           float q_scale, float k_scale, float v_scale, void* stream);
+                           const float* q_scale, const float* k_scale, const float* v_scale,
+                           void* stream);
 
 /*
  * Supported tile sizes (tokens per tile).  Writes up to `capacity` pairs
@@ -77,11 +86,13 @@ int natten_amd_fna_supported_tiles(int dtype, int head_dim, int32_t* q_sizes, in
  * Dense attention forward (optional top-left causal mask) on unpermuted operands.
  *   q [batch, seqlen_q, heads_q, head_dim], k/v [batch, seqlen_kv, heads_kv, head_dim],
  *   out like q, lse [batch, seqlen_q, heads_q] float32.  Any seqlen >= 1.
+ * q_scale / k_scale / v_scale as in natten_amd_fna_forward.
  */
 int natten_amd_attention_forward(const void* q, const void* k, const void* v, void* out,
                                  float* lse, int dtype, int batch, int seqlen_q, int seqlen_kv,
                                  int heads_q, int heads_kv, int head_dim, int is_causal,
-                                 float scale, void* stream);
+                                 float scale, const float* q_scale, const float* k_scale,
+                                 const float* v_scale, void* stream);
 
 /*
  * Token permute: src [batch, *token_layout, heads, head_dim] -> dst
@@ -92,6 +103,20 @@ int natten_amd_token_permute(const void* src, void* dst, int elem_bytes, int na_
                              int heads, int head_dim, const int32_t* token_layout,
                              const int32_t* tile_shape, const int32_t* dilation,
                              int flip_tiled_dims, void* stream);
+
+/*
+ * Token permute of an 8-bit float tensor (src_dtype F8E4M3 or F8E5M2) that writes bf16: same
+ * index map as natten_amd_token_permute, every element converted exactly (all e4m3 / e5m2
+ * values are bf16 values; NaN stays NaN).  heads * head_dim must be a multiple of 8.
+ * With token_layout = {seqlen}, tile_shape = {1}, dilation = {1} it is a plain widening copy.
+ * The reference permutes the 8-bit payload verbatim (csrc/include/natten/token_permute.h:34-52)
+ * and multiplies in 8 bits; here the operands are widened on the permute's HBM pass and the
+ * products are taken in bf16.
+ */
+int natten_amd_token_permute_widen(const void* src, void* dst, int src_dtype, int na_dim,
+                                   int batch, int heads, int head_dim,
+                                   const int32_t* token_layout, const int32_t* tile_shape,
+                                   const int32_t* dilation, int flip_tiled_dims, void* stream);
 
 /* Inverse of natten_amd_token_permute; padding rows of `src` are dropped. */
 int natten_amd_token_unpermute(const void* src, void* dst, int elem_bytes, int na_dim, int batch,

@@ -19,14 +19,16 @@ from torch import Tensor
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libnatten_amd.so")
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 DTYPE_CODES = {
     torch.float16: 0,
     torch.bfloat16: 1,
     torch.float8_e4m3fn: 2,
     torch.float32: 3,
+    torch.float8_e5m2: 4,
 }
+FP8_DTYPES = (torch.float8_e4m3fn, torch.float8_e5m2)
 
 _lib = None
 _load_error: Optional[str] = None
@@ -43,12 +45,16 @@ _SIGNATURES = {
         [ctypes.c_void_p] * 5
         + [ctypes.c_int] * 8
         + [ctypes.c_void_p] * 9
-        + [ctypes.c_float] * 4
-        + [ctypes.c_void_p],
+        + [ctypes.c_float]
+        + [ctypes.c_void_p] * 4,
     ),
     "natten_amd_attention_forward": (
         ctypes.c_int,
-        [ctypes.c_void_p] * 5 + [ctypes.c_int] * 8 + [ctypes.c_float, ctypes.c_void_p],
+        [ctypes.c_void_p] * 5 + [ctypes.c_int] * 8 + [ctypes.c_float] + [ctypes.c_void_p] * 4,
+    ),
+    "natten_amd_token_permute_widen": (
+        ctypes.c_int,
+        [ctypes.c_void_p] * 2 + [ctypes.c_int] * 5 + [ctypes.c_void_p] * 3 + [ctypes.c_int, ctypes.c_void_p],
     ),
     "natten_amd_token_permute": (
         ctypes.c_int,
@@ -135,20 +141,35 @@ def supported_tile_sizes(dtype: torch.dtype, head_dim: int):
     return [(int(a), int(b)) for a, b in zip(q, kv)]
 
 
+def _scale_ptrs(q: Tensor, k: Tensor, q_scale, k_scale, v_scale):
+    """Device pointers (or None) of the per-head scale arrays, after checking shape/dtype/device."""
+    ptrs = []
+    for name, s, heads in (("q_scale", q_scale, q.shape[2]), ("k_scale", k_scale, k.shape[2]), ("v_scale", v_scale, k.shape[2])):
+        if s is None:
+            ptrs.append(None)
+            continue
+        if s.dtype != torch.float32 or s.device != q.device or not s.is_contiguous() or tuple(s.shape) != (heads,):
+            raise ValueError(f"{name} must be a contiguous float32 tensor of shape ({heads},) on {q.device}.")
+        ptrs.append(s.data_ptr())
+    return ptrs
+
+
 def fna_forward(
     q: Tensor, k: Tensor, v: Tensor,
     kernel_size, stride, dilation, is_causal, scale: float,
     q_shape, kv_shape, qkv_shape, q_tile_shape, kv_tile_shape,
-    q_scale: float = 1.0, k_scale: float = 1.0, v_scale: float = 1.0,
+    q_scale: Optional[Tensor] = None, k_scale: Optional[Tensor] = None, v_scale: Optional[Tensor] = None,
 ) -> Tuple[Tensor, Tensor]:
-    """Token-permuted q [B*G, SQ, H, D], k/v [B*G, SK, Hkv, D] -> (out, lse float32 [B*G, SQ, H])."""
+    """Token-permuted q [B*G, SQ, H, D], k/v [B*G, SK, Hkv, D] -> (out, lse float32 [B*G, SQ, H]).
+
+    q_scale [H], k_scale / v_scale [Hkv]: optional float32 per-head dequantisation scales."""
     L = lib()
     _require_gpu(q, k, v)
-    if q.dtype not in (torch.float16, torch.bfloat16, torch.float8_e4m3fn):
+    if q.dtype not in (torch.float16, torch.bfloat16):
         raise NotImplementedError(f"natten_amd fna_forward does not support {q.dtype}.")
     na_dim = len(kernel_size)
-    out_dtype = torch.bfloat16 if q.dtype == torch.float8_e4m3fn else q.dtype
-    out = torch.empty(q.shape, dtype=out_dtype, device=q.device)
+    scales = _scale_ptrs(q, k, q_scale, k_scale, v_scale)
+    out = torch.empty_like(q)
     lse = torch.empty(q.shape[:-1], dtype=torch.float32, device=q.device)
     with torch.cuda.device(q.device):
         rc = L.natten_amd_fna_forward(
@@ -156,25 +177,29 @@ def fna_forward(
             DTYPE_CODES[q.dtype], na_dim, q.shape[0], q.shape[1], k.shape[1], q.shape[2], k.shape[2], q.shape[3],
             _i32(q_shape), _i32(kv_shape), _i32(qkv_shape), _i32(kernel_size), _i32(stride), _i32(dilation),
             _i32([1 if c else 0 for c in is_causal]), _i32(q_tile_shape), _i32(kv_tile_shape),
-            float(scale), float(q_scale), float(k_scale), float(v_scale), _stream(q),
+            float(scale), *scales, _stream(q),
         )
     _check(rc)
     return out, lse
 
 
-def attention_forward(q: Tensor, k: Tensor, v: Tensor, is_causal: bool, scale: float) -> Tuple[Tensor, Tensor]:
+def attention_forward(
+    q: Tensor, k: Tensor, v: Tensor, is_causal: bool, scale: float,
+    q_scale: Optional[Tensor] = None, k_scale: Optional[Tensor] = None, v_scale: Optional[Tensor] = None,
+) -> Tuple[Tensor, Tensor]:
     """Dense attention q [B, S, H, D], k/v [B, Skv, Hkv, D] -> (out, lse float32 [B, S, H])."""
     L = lib()
     _require_gpu(q, k, v)
     if q.dtype not in (torch.float16, torch.bfloat16):
         raise NotImplementedError(f"natten_amd attention_forward does not support {q.dtype}.")
+    scales = _scale_ptrs(q, k, q_scale, k_scale, v_scale)
     out = torch.empty_like(q)
     lse = torch.empty(q.shape[:-1], dtype=torch.float32, device=q.device)
     with torch.cuda.device(q.device):
         rc = L.natten_amd_attention_forward(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(), DTYPE_CODES[q.dtype],
             q.shape[0], q.shape[1], k.shape[1], q.shape[2], k.shape[2], q.shape[3], 1 if is_causal else 0,
-            float(scale), _stream(q),
+            float(scale), *scales, _stream(q),
         )
     _check(rc)
     return out, lse
@@ -184,10 +209,14 @@ def _ceil_div(a: int, b: int) -> int:
     return (a + b - 1) // b
 
 
-def token_permute(x: Tensor, tile_shape, dilation, flip_tiled_dims: bool) -> Tensor:
-    """[B, *X, H, Dh] -> [B * prod(dilation), prod(ceil(ceil(X/t)/d) * t), H, Dh], zero padded."""
+def token_permute(x: Tensor, tile_shape, dilation, flip_tiled_dims: bool, widen: bool = False) -> Tensor:
+    """[B, *X, H, Dh] -> [B * prod(dilation), prod(ceil(ceil(X/t)/d) * t), H, Dh], zero padded.
+
+    widen=True (8-bit float input only) writes the exact bf16 values instead of the raw bytes."""
     L = lib()
     _require_gpu(x)
+    if widen and x.dtype not in FP8_DTYPES:
+        raise ValueError(f"token_permute(widen=True) needs an 8-bit float tensor, got {x.dtype}.")
     na_dim = x.dim() - 3
     layout = [int(s) for s in x.shape[1 : 1 + na_dim]]
     post = [_ceil_div(_ceil_div(X, t), d) * t for X, t, d in zip(layout, tile_shape, dilation)]
@@ -196,7 +225,16 @@ def token_permute(x: Tensor, tile_shape, dilation, flip_tiled_dims: bool) -> Ten
     for d, p in zip(dilation, post):
         groups *= d
         seqlen *= p
-    out = torch.empty((x.shape[0] * groups, seqlen, x.shape[-2], x.shape[-1]), dtype=x.dtype, device=x.device)
+    out_dtype = torch.bfloat16 if widen else x.dtype
+    out = torch.empty((x.shape[0] * groups, seqlen, x.shape[-2], x.shape[-1]), dtype=out_dtype, device=x.device)
+    if widen:
+        with torch.cuda.device(x.device):
+            rc = L.natten_amd_token_permute_widen(
+                x.data_ptr(), out.data_ptr(), DTYPE_CODES[x.dtype], na_dim, x.shape[0], x.shape[-2], x.shape[-1],
+                _i32(layout), _i32(tile_shape), _i32(dilation), 1 if flip_tiled_dims else 0, _stream(x),
+            )
+        _check(rc)
+        return out
     with torch.cuda.device(x.device):
         rc = L.natten_amd_token_permute(
             x.data_ptr(), out.data_ptr(), x.element_size(), na_dim, x.shape[0], x.shape[-2], x.shape[-1],

@@ -44,8 +44,12 @@ struct FnaParams {
   // workgroup layout: consecutive `wg_group` Q tiles (dimension 0 slowest) of one (batch, head)
   // form a group; groups are dealt round-robin to the 8 XCDs
   int wg_group, groups_per_bh, total_groups;
-  float scale;      // softmax scale (dequantisation scales of q and k folded in)
-  float out_scale;  // dequantisation scale of v
+  float scale;  // softmax scale
+  // optional per-head dequantisation scales (device arrays or null): logits are multiplied by
+  // q_scale[head] * k_scale[head_kv], the output by v_scale[head_kv]
+  const float* q_scale;  // [heads_q]
+  const float* k_scale;  // [heads_kv]
+  const float* v_scale;  // [heads_kv]
 };
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
@@ -386,7 +390,11 @@ fna_fwd_kernel(const FnaParams p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[mb][db][r] = 0.f;
   }
-  const float c_log2 = p.scale * 1.4426950408889634f;
+  float sm_scale = p.scale, out_scale = 1.f;
+  if (p.q_scale) sm_scale *= p.q_scale[head];
+  if (p.k_scale) sm_scale *= p.k_scale[head_kv];
+  if (p.v_scale) out_scale = p.v_scale[head_kv];
+  const float c_log2 = sm_scale * 1.4426950408889634f;
 
   // lane-constant LDS read offsets
   int k_off[KSTEPS];  // K operand: row l32 (+32*sb), chunk 2*ks+g
@@ -554,7 +562,7 @@ fna_fwd_kernel(const FnaParams p) {
 #pragma unroll
   for (int mb = 0; mb < MQ; ++mb) {
     const float l = l_run[mb] + __shfl_xor(l_run[mb], 32);
-    const float inv = (l > 0.f) ? p.out_scale / l : 0.f;
+    const float inv = (l > 0.f) ? out_scale / l : 0.f;
     const int row = qtile_idx * QT + (wave * MQ + mb) * 32 + l32;
     if (row < p.seqlen_q) {
       T* orow = obase + int64_t(row) * q_row_stride;
@@ -569,7 +577,7 @@ fna_fwd_kernel(const FnaParams p) {
           *reinterpret_cast<tx4*>(orow + db * 32 + 8 * j + 4 * g) = o4;
         }
       if (g == 0) {
-        const float lse = (l > 0.f) ? (m_run[mb] * p.scale + __logf(l)) : -INFINITY;
+        const float lse = (l > 0.f) ? (m_run[mb] * sm_scale + __logf(l)) : -INFINITY;
         p.lse[(int64_t(bg) * p.seqlen_q + row) * p.heads_q + head] = lse;
       }
     }

@@ -99,6 +99,9 @@ int dispatch_dtype(const FnaParams& p, int dtype, int head_dim, int qt, int kvt,
     case NATTEN_AMD_F16: return dispatch_head_dim<_Float16>(p, head_dim, qt, kvt, stream);
     case NATTEN_AMD_BF16: return dispatch_head_dim<__bf16>(p, head_dim, qt, kvt, stream);
   }
+  if (dtype == NATTEN_AMD_F8E4M3 || dtype == NATTEN_AMD_F8E5M2)
+    return fail("8-bit float operands are widened by natten_amd_token_permute_widen; pass the bf16 result and "
+                "the dequantisation scales here");
   return fail("fna_forward: unsupported dtype code %d", dtype);
 }
 
@@ -121,7 +124,7 @@ int check_common(const char* what, const void* q, const void* k, const void* v, 
 
 extern "C" {
 
-int natten_amd_abi_version(void) { return 1; }
+int natten_amd_abi_version(void) { return 2; }
 
 const char* natten_amd_last_error(void) { return g_error; }
 
@@ -140,7 +143,8 @@ int natten_amd_fna_forward(const void* q, const void* k, const void* v, void* ou
                            const int32_t* q_shape, const int32_t* kv_shape, const int32_t* qkv_shape,
                            const int32_t* kernel_size, const int32_t* stride, const int32_t* dilation,
                            const int32_t* is_causal, const int32_t* q_tile_shape, const int32_t* kv_tile_shape,
-                           float scale, float q_scale, float k_scale, float v_scale, void* stream) {
+                           float scale, const float* q_scale, const float* k_scale, const float* v_scale,
+                           void* stream) {
   g_error[0] = 0;
   if (na_dim < 1 || na_dim > 3) return fail("fna_forward: na_dim must be 1, 2 or 3, got %d", na_dim);
   if (int rc = check_common("fna_forward", q, k, v, out, lse, batch, seqlen_q, seqlen_kv, heads_q, heads_kv, head_dim))
@@ -197,15 +201,18 @@ int natten_amd_fna_forward(const void* q, const void* k, const void* v, void* ou
   p.heads_kv = heads_kv;
   p.seqlen_q = seqlen_q;
   p.seqlen_kv = seqlen_kv;
-  p.scale = scale * q_scale * k_scale;
-  p.out_scale = v_scale;
+  p.scale = scale;
+  p.q_scale = q_scale;
+  p.k_scale = k_scale;
+  p.v_scale = v_scale;
   set_wg_layout(p, 1);
   return dispatch_dtype(p, dtype, head_dim, prod3(p.q_tile), prod3(p.kv_tile), static_cast<hipStream_t>(stream));
 }
 
 int natten_amd_attention_forward(const void* q, const void* k, const void* v, void* out, float* lse, int dtype,
                                  int batch, int seqlen_q, int seqlen_kv, int heads_q, int heads_kv, int head_dim,
-                                 int is_causal, float scale, void* stream) {
+                                 int is_causal, float scale, const float* q_scale, const float* k_scale,
+                                 const float* v_scale, void* stream) {
   g_error[0] = 0;
   if (int rc = check_common("attention_forward", q, k, v, out, lse, batch, seqlen_q, seqlen_kv, heads_q, heads_kv,
                             head_dim))
@@ -242,12 +249,15 @@ int natten_amd_attention_forward(const void* q, const void* k, const void* v, vo
   p.seqlen_q = seqlen_q;
   p.seqlen_kv = seqlen_kv;
   p.scale = scale;
-  p.out_scale = 1.f;
+  p.q_scale = q_scale;
+  p.k_scale = k_scale;
+  p.v_scale = v_scale;
   set_wg_layout(p, 1);
   return dispatch_dtype(p, dtype, head_dim, QT, KVT, static_cast<hipStream_t>(stream));
 }
 
-static int tokperm_common(const char* what, bool unpermute, const void* src, void* dst, int elem_bytes, int na_dim,
+// widen: 0 = copy the payload, NATTEN_AMD_F8E4M3 / NATTEN_AMD_F8E5M2 = 8-bit float source, bf16 destination
+static int tokperm_common(const char* what, bool unpermute, int widen, const void* src, void* dst, int elem_bytes, int na_dim,
                           int batch, int heads, int head_dim, const int32_t* token_layout, const int32_t* tile_shape,
                           const int32_t* dilation, int flip, void* stream) {
   g_error[0] = 0;
@@ -287,7 +297,11 @@ static int tokperm_common(const char* what, bool unpermute, const void* src, voi
     p.g_size[i] = p.dil[a];
   }
   const uintptr_t align = reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst) | uintptr_t(p.row_bytes);
-  const int vec = (align % 16 == 0) ? 16 : (align % 4 == 0) ? 4 : (align % 2 == 0) ? 2 : 1;
+  if (widen) {
+    if (p.row_bytes % 8 != 0 || reinterpret_cast<uintptr_t>(src) % 8 != 0 || reinterpret_cast<uintptr_t>(dst) % 16 != 0)
+      return fail("%s: heads * head_dim must be a multiple of 8, src 8-byte and dst 16-byte aligned", what);
+  }
+  const int vec = widen ? 8 : (align % 16 == 0) ? 16 : (align % 4 == 0) ? 4 : (align % 2 == 0) ? 2 : 1;
   const int64_t total = int64_t(batch) * p.num_groups * p.perm_len * (p.row_bytes / vec);
   int64_t blocks = (total + 255) / 256;
   const int64_t cap = 256 * 64;  // grid-stride beyond this many workgroups
@@ -301,6 +315,13 @@ static int tokperm_common(const char* what, bool unpermute, const void* src, voi
     else                                                                                          \
       hipLaunchKernelGGL((tokperm_kernel<VEC, false>), dim3(unsigned(blocks)), dim3(256), 0, s, p); \
   } while (0)
+  if (widen == NATTEN_AMD_F8E5M2) {
+    hipLaunchKernelGGL((tokperm_widen_kernel<true>), dim3(unsigned(blocks)), dim3(256), 0, s, p);
+    return check_launch(what);
+  } else if (widen) {
+    hipLaunchKernelGGL((tokperm_widen_kernel<false>), dim3(unsigned(blocks)), dim3(256), 0, s, p);
+    return check_launch(what);
+  }
   switch (vec) {
     case 16: NA_TOKPERM_LAUNCH(16); break;
     case 4: NA_TOKPERM_LAUNCH(4); break;
@@ -314,15 +335,26 @@ static int tokperm_common(const char* what, bool unpermute, const void* src, voi
 int natten_amd_token_permute(const void* src, void* dst, int elem_bytes, int na_dim, int batch, int heads,
                              int head_dim, const int32_t* token_layout, const int32_t* tile_shape,
                              const int32_t* dilation, int flip_tiled_dims, void* stream) {
-  return tokperm_common("token_permute", false, src, dst, elem_bytes, na_dim, batch, heads, head_dim, token_layout,
+  return tokperm_common("token_permute", false, 0, src, dst, elem_bytes, na_dim, batch, heads, head_dim, token_layout,
                         tile_shape, dilation, flip_tiled_dims, stream);
 }
 
 int natten_amd_token_unpermute(const void* src, void* dst, int elem_bytes, int na_dim, int batch, int heads,
                                int head_dim, const int32_t* token_layout, const int32_t* tile_shape,
                                const int32_t* dilation, int flip_tiled_dims, void* stream) {
-  return tokperm_common("token_unpermute", true, src, dst, elem_bytes, na_dim, batch, heads, head_dim, token_layout,
+  return tokperm_common("token_unpermute", true, 0, src, dst, elem_bytes, na_dim, batch, heads, head_dim, token_layout,
                         tile_shape, dilation, flip_tiled_dims, stream);
+}
+
+int natten_amd_token_permute_widen(const void* src, void* dst, int src_dtype, int na_dim, int batch, int heads,
+                                   int head_dim, const int32_t* token_layout, const int32_t* tile_shape,
+                                   const int32_t* dilation, int flip_tiled_dims, void* stream) {
+  if (src_dtype != NATTEN_AMD_F8E4M3 && src_dtype != NATTEN_AMD_F8E5M2) {
+    g_error[0] = 0;
+    return fail("token_permute_widen: src_dtype must be an 8-bit float code, got %d", src_dtype);
+  }
+  return tokperm_common("token_permute_widen", false, src_dtype, src, dst, 1, na_dim, batch, heads, head_dim,
+                        token_layout, tile_shape, dilation, flip_tiled_dims, stream);
 }
 
 int natten_amd_merge_attentions(const void* o0, const float* lse0, const void* o1, const float* lse1, void* out,

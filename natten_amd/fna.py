@@ -16,7 +16,36 @@ from .checks import check_all_args, check_args_against_input, na_tensor_checks
 from .tile_config import check_fna_forward_config, padded_head_dim
 from .token_permute import token_permute_operation, token_unpermute_operation
 
-SUPPORTED_DTYPES = (torch.float16, torch.bfloat16)
+SUPPORTED_DTYPES = (torch.float16, torch.bfloat16, torch.float8_e4m3fn, torch.float8_e5m2)
+FP8_DTYPES = _lib.FP8_DTYPES
+
+
+def is_fp8(dtype: torch.dtype) -> bool:
+    return dtype in FP8_DTYPES
+
+
+def resolve_scale(scale, heads: int, device, name: str) -> Optional[Tensor]:
+    """Per-head dequantisation scale as a float32 tensor [heads] (or None): accepts None, a
+    number, a one-element tensor or a tensor with one entry per head."""
+    if scale is None:
+        return None
+    if not isinstance(scale, Tensor):
+        return torch.full((heads,), float(scale), dtype=torch.float32, device=device)
+    s = scale.detach().to(device=device, dtype=torch.float32).reshape(-1)
+    if s.numel() == 1:
+        return s.expand(heads).contiguous()
+    if s.numel() != heads:
+        raise ValueError(f"{name} must have one entry or one entry per head ({heads}), got {tuple(scale.shape)}.")
+    return s.contiguous()
+
+
+def pad_head_dim(x: Tensor, d_to: int) -> Tensor:
+    """Zero-pads the last dimension (8-bit floats through their bytes: 0x00 is +0)."""
+    if x.shape[-1] == d_to:
+        return x
+    if is_fp8(x.dtype):
+        return torch.nn.functional.pad(x.view(torch.uint8), (0, d_to - x.shape[-1])).view(x.dtype)
+    return torch.nn.functional.pad(x, (0, d_to - x.shape[-1]))
 
 
 def can_run_amd_fna(query: Tensor, key: Tensor, value: Tensor, raise_error: bool = False) -> bool:
@@ -38,16 +67,15 @@ def can_run_amd_fna(query: Tensor, key: Tensor, value: Tensor, raise_error: bool
         return no("natten_amd FNA does not support different head dims for QK and V.", ValueError)
     if query.shape[-1] > 128 or query.shape[-1] % 8 != 0:
         return no(f"natten_amd FNA supports head_dim <= 128 that is a multiple of 8, got {query.shape[-1]}.")
+    if is_fp8(query.dtype) and query.shape[-1] % 16 != 0:
+        return no(f"natten_amd FNA needs head dims that are multiples of 16 for 8-bit floats, got {query.shape[-1]}.")
     if query.requires_grad or key.requires_grad or value.requires_grad:
         if torch.is_grad_enabled():
             return no("natten_amd implements the forward pass only; call it under torch.no_grad().")
     return True
 
 
-def _pad_head_dim(x: Tensor, d_to: int) -> Tensor:
-    if x.shape[-1] == d_to:
-        return x
-    return torch.nn.functional.pad(x, (0, d_to - x.shape[-1]))
+_pad_head_dim = pad_head_dim
 
 
 def amd_fna_generic(
@@ -62,7 +90,14 @@ def amd_fna_generic(
     q_tile_shape=None,
     kv_tile_shape=None,
     return_lse: bool = False,
+    q_scale=None,
+    k_scale=None,
+    v_scale=None,
+    out_dtype: Optional[torch.dtype] = None,
 ) -> Union[Tensor, Tuple[Tensor, Tensor]]:
+    """8-bit float operands (e4m3fn / e5m2) are widened to bf16 (exactly) by the token permute and
+    multiplied in bf16; `q_scale`, `k_scale`, `v_scale` (number or per-head tensor) are their
+    dequantisation scales.  `out_dtype` defaults to the dtype of `query`, as in the reference."""
     na_tensor_checks(query, key, value, must_match_head_dims=True)
     can_run_amd_fna(query, key, value, raise_error=True)
     na_dim = query.dim() - 3
@@ -78,13 +113,20 @@ def amd_fna_generic(
         # zero columns change neither q.k nor the first head_dim output columns
         query, key, value = (_pad_head_dim(t, d_pad) for t in (query, key, value))
 
-    q_perm, qkv_shape, q_shape = token_permute_operation(query, q_tile_shape, dilation, flip_tiled_dims=True)
-    k_perm, _, kv_shape = token_permute_operation(key, kv_tile_shape, dilation, flip_tiled_dims=True)
-    v_perm, _, _ = token_permute_operation(value, kv_tile_shape, dilation, flip_tiled_dims=True)
+    in_dtype = query.dtype
+    widen = is_fp8(in_dtype)
+    q_scale = resolve_scale(q_scale, query.shape[-2], query.device, "q_scale")
+    k_scale = resolve_scale(k_scale, key.shape[-2], query.device, "k_scale")
+    v_scale = resolve_scale(v_scale, key.shape[-2], query.device, "v_scale")
+
+    q_perm, qkv_shape, q_shape = token_permute_operation(query, q_tile_shape, dilation, flip_tiled_dims=True, widen=widen)
+    k_perm, _, kv_shape = token_permute_operation(key, kv_tile_shape, dilation, flip_tiled_dims=True, widen=widen)
+    v_perm, _, _ = token_permute_operation(value, kv_tile_shape, dilation, flip_tiled_dims=True, widen=widen)
 
     out_perm, lse_perm = _lib.fna_forward(
         q_perm, k_perm, v_perm, kernel_size, stride, dilation, is_causal, scale,
         q_shape, kv_shape, qkv_shape, q_tile_shape, kv_tile_shape,
+        q_scale=q_scale, k_scale=k_scale, v_scale=v_scale,
     )
 
     output = token_unpermute_operation(out_perm, qkv_shape, q_tile_shape, dilation, flip_tiled_dims=True)
@@ -93,6 +135,9 @@ def amd_fna_generic(
     ).squeeze(-1)
     if d_pad != head_dim:
         output = output[..., :head_dim].contiguous()
+    out_dtype = out_dtype or in_dtype
+    if output.dtype != out_dtype:
+        output = output.to(out_dtype)
     if return_lse:
         return output, lse
     return output

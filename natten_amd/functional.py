@@ -23,7 +23,7 @@ from .checks import (
     na_tensor_checks,
 )
 from .fmha import amd_fmha
-from .fna import amd_fna_generic
+from .fna import amd_fna_generic, is_fp8
 
 _BACKEND_FNA = "amd-fna"
 _BACKEND_FMHA = "amd-fmha"
@@ -54,11 +54,18 @@ def attention(
     kernel_schedule=None,
     torch_compile: bool = False,
     return_lse: bool = False,
+    # quantised (8-bit float) operands; not in the reference
+    q_scale=None,
+    k_scale=None,
+    v_scale=None,
+    out_dtype: Optional[torch.dtype] = None,
 ) -> Union[Tensor, Tuple[Tensor, Tensor]]:
     """Dot product attention on `[batch, seqlen, heads, head_dim]` tensors (heads last).
 
     `is_causal` is top-left aligned.  Returns the output, and the float32 logsumexp
-    `[batch, seqlen, heads]` when `return_lse=True`.
+    `[batch, seqlen, heads]` when `return_lse=True`.  For e4m3 / e5m2 operands `q_scale`, `k_scale`,
+    `v_scale` (number or per-head tensor) are the dequantisation scales and `out_dtype` the
+    result type (default: the operands' type, as in the reference).
     """
     if any(x is not None for x in (seqlens_Q, seqlens_KV, cumulative_seqlen_Q, cumulative_seqlen_KV)) or any(
         x not in (None, 0) for x in (max_seqlen_Q, max_seqlen_KV)
@@ -66,7 +73,10 @@ def attention(
         raise NotImplementedError("natten_amd does not implement variable-length attention.")
     if backend not in (None, _BACKEND_FMHA):
         raise NotImplementedError(f"Unrecognized attention backend {backend}; natten_amd provides '{_BACKEND_FMHA}'.")
-    return amd_fmha(query, key, value, is_causal=is_causal, scale=scale, return_lse=return_lse)
+    return amd_fmha(
+        query, key, value, is_causal=is_causal, scale=scale, return_lse=return_lse,
+        q_scale=q_scale, k_scale=k_scale, v_scale=v_scale, out_dtype=out_dtype,
+    )
 
 
 def neighborhood_attention_generic(
@@ -93,6 +103,10 @@ def neighborhood_attention_generic(
     kernel_schedule=None,
     torch_compile: bool = False,
     return_lse: bool = False,
+    q_scale=None,
+    k_scale=None,
+    v_scale=None,
+    out_dtype: Optional[torch.dtype] = None,
 ) -> Union[Tensor, Tuple[Tensor, Tensor]]:
     na_tensor_checks(query, key, value)
     additional_kv_tensor_checks(query, key, value, additional_keys, additional_values)
@@ -116,27 +130,36 @@ def neighborhood_attention_generic(
         if has_additional_attention:
             k = torch.cat([k, additional_keys], dim=1)
             v = torch.cat([v, additional_values], dim=1)
-        out, lse = attention(q, k, v, is_causal=is_causal[0], scale=scale, return_lse=True, **attn_kwargs)
+        out, lse = attention(
+            q, k, v, is_causal=is_causal[0], scale=scale, return_lse=True,
+            q_scale=q_scale, k_scale=k_scale, v_scale=v_scale, out_dtype=out_dtype, **attn_kwargs,
+        )
         lse_shape = list(query_shape[:-1])
         out = out.reshape(*lse_shape, v.shape[-1])
         lse = lse.reshape(*lse_shape)
         return (out, lse) if return_lse else out
 
     scale = scale or query.shape[-1] ** -0.5
+    final_dtype = out_dtype or query.dtype
+    # 8-bit float operands: partial results stay in bf16 until after the merge
+    work_dtype = torch.bfloat16 if is_fp8(query.dtype) else final_dtype
     output, lse = amd_fna_generic(
         query, key, value, kernel_size=kernel_size, stride=stride, dilation=dilation, is_causal=is_causal,
         scale=scale, q_tile_shape=q_tile_shape, kv_tile_shape=kv_tile_shape, return_lse=True,
+        q_scale=q_scale, k_scale=k_scale, v_scale=v_scale,
+        out_dtype=work_dtype if has_additional_attention else final_dtype,
     )
 
     if has_additional_attention:
+        # the additional keys / values share the dequantisation scales of key / value
         add_out, add_lse = attention(
             query.flatten(1, na_dim), additional_keys, additional_values, is_causal=False, scale=scale,
-            return_lse=True, **attn_kwargs,
+            return_lse=True, q_scale=q_scale, k_scale=k_scale, v_scale=v_scale, out_dtype=work_dtype, **attn_kwargs,
         )
         merged_out, merged_lse = merge_attentions(
             [output.flatten(1, na_dim), add_out], [lse.flatten(1, na_dim), add_lse]
         )
-        output = merged_out.reshape(output.shape)
+        output = merged_out.reshape(output.shape).to(final_dtype)
         lse = merged_lse.reshape(output.shape[:-1])
 
     return (output, lse) if return_lse else output
@@ -166,6 +189,10 @@ def _make_na(na_dim: int, name: str):
         kernel_schedule=None,
         torch_compile: bool = False,
         return_lse: bool = False,
+        q_scale=None,
+        k_scale=None,
+        v_scale=None,
+        out_dtype: Optional[torch.dtype] = None,
     ) -> Union[Tensor, Tuple[Tensor, Tensor]]:
         if query.dim() != na_dim + 3:
             raise ValueError(
@@ -180,6 +207,7 @@ def _make_na(na_dim: int, name: str):
             backward_kv_tile_shape=backward_kv_tile_shape, backward_kv_splits=backward_kv_splits,
             backward_use_pt_reduction=backward_use_pt_reduction, run_persistent_kernel=run_persistent_kernel,
             kernel_schedule=kernel_schedule, torch_compile=torch_compile, return_lse=return_lse,
+            q_scale=q_scale, k_scale=k_scale, v_scale=v_scale, out_dtype=out_dtype,
         )
 
     op.__name__ = name
@@ -190,7 +218,9 @@ def _make_na(na_dim: int, name: str):
         "kernel_size, stride, dilation: int or tuple per dimension (kernel_size >= 2, stride <= kernel_size, "
         "kernel_size * dilation <= input size); is_causal: bool or tuple.  additional_keys / additional_values "
         "`[batch, seqlen, heads_kv, head_dim]` add context every query attends to.  Returns the output and, with "
-        "`return_lse=True`, the float32 logsumexp `[batch, *tokens, heads]`."
+        "`return_lse=True`, the float32 logsumexp `[batch, *tokens, heads]`.  For e4m3 / e5m2 operands `q_scale`, "
+        "`k_scale`, `v_scale` (number or per-head tensor) are the dequantisation scales and `out_dtype` the result "
+        "type (default: the operands' type)."
     )
     return op
 

@@ -35,7 +35,9 @@ def token_permute_operation(
     tile_shape: DimensionType,
     dilation: Optional[DimensionType] = None,
     flip_tiled_dims: bool = True,
+    widen: bool = False,
 ) -> Tuple[Tensor, DimensionType, DimensionType]:
+    """`widen=True` (8-bit float input): the permuted tensor holds the same values in bf16."""
     if tensor.dim() not in (4, 5, 6):
         raise ValueError(
             f"Expected 4D, 5D, or 6D tensor (corresponding to NA1D, 2D, 3D), got {tensor.dim()}D input."
@@ -47,7 +49,7 @@ def token_permute_operation(
     tensor = tensor.contiguous()
     token_layout = tuple(int(x) for x in tensor.shape[1 : 1 + na_dim])
     post = tuple(_ceil_div(_ceil_div(x, t), d) * t for x, t, d in zip(token_layout, tile_shape, dilation_))
-    out = _lib.token_permute(tensor, tile_shape, dilation_, flip_tiled_dims)
+    out = _lib.token_permute(tensor, tile_shape, dilation_, flip_tiled_dims, widen=widen)
     return out, token_layout, post
 
 

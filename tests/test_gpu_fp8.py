@@ -1,0 +1,160 @@
+"""GPU parity for quantised 8-bit float operands (e4m3fn / e5m2 with per-head scales).
+
+The widening token permute must be bit-exact (every 8-bit float value is a bf16 value); the
+attention results are compared with the float64 oracle evaluated on the DEQUANTISED inputs.
+Tolerance: atol = rtol = 1e-2, the same as for bf16 operands, because the operands enter the
+bf16 matrix instructions exactly and only P and the output are rounded to bf16.  (The reference
+rounds P to 8 bits and tests with atol 0.5 for e4m3, tests/test_blackwell_fna.py:107.)"""
+
+import numpy as np
+import pytest
+import torch
+
+import natten_amd
+from natten_amd import _lib
+from oracle import c_oracle
+from oracle import na_oracle as O
+from tests.gpu_utils import assert_close, to_np
+
+pytestmark = pytest.mark.gpu
+
+E4M3_MAX = 448.0
+E5M2_MAX = 57344.0
+
+
+def quantise_per_head(x, dtype):
+    """Per-head absmax scaling into the 8-bit range: returns (x8, scale[H]) with x ~ x8 * scale."""
+    fmax = E4M3_MAX if dtype == torch.float8_e4m3fn else E5M2_MAX
+    red = tuple(i for i in range(x.dim()) if i != x.dim() - 2)
+    scale = x.abs().amax(dim=red).float() / fmax
+    x8 = (x / scale.view(*([1] * (x.dim() - 2)), -1, 1)).to(dtype)
+    return x8, scale
+
+
+def dequantise(x8, scale):
+    return x8.float() * scale.view(*([1] * (x8.dim() - 2)), -1, 1)
+
+
+@pytest.mark.parametrize("dtype", [torch.float8_e4m3fn, torch.float8_e5m2])
+def test_widen_all_byte_values_bit_exact(dtype):
+    # every byte value, laid out as [B=1, S=32, H=1, D=8]
+    raw = torch.arange(256, dtype=torch.uint8, device="cuda").reshape(1, 32, 1, 8)
+    x = raw.view(dtype)
+    got = _lib.token_permute(x, (1,), (1,), True, widen=True)
+    ref = x.to(torch.bfloat16)
+    assert got.dtype == torch.bfloat16 and got.shape == ref.shape
+    nan = torch.isnan(ref)
+    assert torch.equal(torch.isnan(got), nan)
+    assert torch.equal(got.view(torch.int16)[~nan], ref.view(torch.int16)[~nan])
+
+
+@pytest.mark.parametrize(
+    "shape,tile,dil",
+    [((37,), (8,), (1,)), ((19, 23), (4, 8), (2, 3)), ((5, 9, 11), (2, 4, 4), (1, 2, 2)), ((16, 16), (8, 8), (1, 1))],
+)
+def test_widen_permute_matches_oracle(shape, tile, dil):
+    gen = torch.Generator().manual_seed(3)
+    x = torch.randn((2, *shape, 3, 16), generator=gen).to(torch.float8_e4m3fn).cuda()
+    got = _lib.token_permute(x, tile, dil, True, widen=True)
+    ref, _, _ = O.token_permute(to_np(x), tile, dil, flip=True)
+    assert got.dtype == torch.bfloat16
+    assert np.array_equal(to_np(got), ref)
+    # and the plain permute of the same tensor carries the bytes verbatim
+    raw = _lib.token_permute(x, tile, dil, True)
+    assert raw.dtype == x.dtype
+    assert np.array_equal(to_np(raw), ref)
+
+
+def _sampled(qd, kd, vd, out, lse, kernel, stride, dilation, causal, n_samples, seed):
+    B = qd.shape[0]
+    n = qd.dim() - 3
+    N = int(np.prod(qd.shape[1 : 1 + n]))
+    H, D = qd.shape[-2], qd.shape[-1]
+    rng = np.random.default_rng(seed)
+    tok = rng.integers(0, N, size=n_samples)
+    tok[:2] = (0, N - 1)
+    bat = rng.integers(0, B, size=n_samples)
+    ref_o, ref_l, _ = c_oracle.na_rows(to_np(qd), to_np(kd), to_np(vd), kernel, stride, dilation, causal, None, bat,
+                                       tok, threads=8)
+    ti, bi = torch.as_tensor(tok), torch.as_tensor(bat)
+    assert_close("sampled out", to_np(out.reshape(B, N, H, D)[bi, ti]), ref_o)
+    assert_close("sampled lse", to_np(lse.reshape(B, N, H)[bi, ti]), ref_l)
+
+
+def test_config5_e4m3_full_size_sampled():
+    # na3d e4m3, B=1, heads 16, 16x64x64, D=128, kernel (8,16,16), stride (4,8,8), dilation (1,2,2)
+    gen = torch.Generator().manual_seed(0)
+    shape, H, D = (16, 64, 64), 16, 128
+    q, k, v = (torch.randn((1, *shape, H, D), generator=gen).cuda() for _ in range(3))
+    (q8, sq), (k8, sk), (v8, sv) = (quantise_per_head(t, torch.float8_e4m3fn) for t in (q, k, v))
+    args = ((8, 16, 16), (4, 8, 8), (1, 2, 2))
+    with torch.no_grad():
+        out, lse = natten_amd.na3d(q8, k8, v8, *args, return_lse=True, q_scale=sq, k_scale=sk, v_scale=sv,
+                                   out_dtype=torch.bfloat16)
+    assert out.dtype == torch.bfloat16 and lse.dtype == torch.float32
+    qd, kd, vd = dequantise(q8, sq), dequantise(k8, sk), dequantise(v8, sv)
+    _sampled(qd, kd, vd, out, lse, *args, (False, False, False), n_samples=96, seed=5)
+    assert torch.isfinite(out).all() and torch.isfinite(lse).all()
+    # doubling v_scale doubles the output bit-exactly and leaves LSE alone
+    with torch.no_grad():
+        out2, lse2 = natten_amd.na3d(q8, k8, v8, *args, return_lse=True, q_scale=sq, k_scale=sk, v_scale=sv * 2,
+                                     out_dtype=torch.bfloat16)
+    assert torch.equal(out2, out * 2) and torch.equal(lse2, lse)
+
+
+@pytest.mark.parametrize("dtype", [torch.float8_e4m3fn, torch.float8_e5m2])
+@pytest.mark.parametrize("causal", [False, True])
+def test_small_fp8_problems_match_oracle(dtype, causal):
+    gen = torch.Generator().manual_seed(11)
+    B, shape, H, Hkv, D = 2, (14, 20), 4, 2, 48
+    q = torch.randn((B, *shape, H, D), generator=gen).cuda()
+    k = torch.randn((B, *shape, Hkv, D), generator=gen).cuda()
+    v = torch.randn((B, *shape, Hkv, D), generator=gen).cuda()
+    (q8, sq), (k8, sk), (v8, sv) = (quantise_per_head(t, dtype) for t in (q, k, v))
+    kernel, stride, dil, cz = (5, 6), (2, 3), (2, 1), (causal, False)
+    with torch.no_grad():
+        out, lse = natten_amd.na2d(q8, k8, v8, kernel, stride, dil, cz, return_lse=True, q_scale=sq, k_scale=sk,
+                                   v_scale=sv, out_dtype=torch.bfloat16)
+    qd, kd, vd = dequantise(q8, sq), dequantise(k8, sk), dequantise(v8, sv)
+    ref_o, ref_l = c_oracle.na_forward(to_np(qd), to_np(kd), to_np(vd), kernel, stride, dil, cz, None)
+    assert_close("out", to_np(out), ref_o)
+    assert_close("lse", to_np(lse), ref_l)
+
+
+def test_fp8_default_output_dtype_and_unit_scales():
+    # without scales and out_dtype the call behaves like the reference: 8-bit result
+    gen = torch.Generator().manual_seed(2)
+    q, k, v = ((torch.randn((1, 40, 2, 32), generator=gen) * 0.5).to(torch.float8_e4m3fn).cuda() for _ in range(3))
+    with torch.no_grad():
+        out, lse = natten_amd.na1d(q, k, v, 9, return_lse=True)
+    assert out.dtype == torch.float8_e4m3fn
+    ref_o, ref_l = c_oracle.na_forward(to_np(q), to_np(k), to_np(v), (9,), (1,), (1,), (False,), None)
+    # the result is rounded to e4m3 (3 mantissa bits: relative step 2^-3, half of it as error)
+    assert_close("out", to_np(out), ref_o, atol=2e-2, rtol=2.0**-4)
+    assert_close("lse", to_np(lse), ref_l)
+
+
+def test_fp8_dense_attention_and_additional_kv():
+    gen = torch.Generator().manual_seed(4)
+    B, L, H, D = 1, 70, 2, 64
+    q, k, v = (torch.randn((B, L, H, D), generator=gen).cuda() for _ in range(3))
+    ak, av = (torch.randn((B, 13, H, D), generator=gen).cuda() for _ in range(2))
+    (q8, sq), (k8, sk), (v8, sv) = (quantise_per_head(t, torch.float8_e4m3fn) for t in (q, k, v))
+    # the additional tensors share the scales of key / value
+    ak8 = (ak / sk.view(1, 1, -1, 1)).clamp(-E4M3_MAX, E4M3_MAX).to(torch.float8_e4m3fn)
+    av8 = (av / sv.view(1, 1, -1, 1)).clamp(-E4M3_MAX, E4M3_MAX).to(torch.float8_e4m3fn)
+    qd, kd, vd = dequantise(q8, sq), dequantise(k8, sk), dequantise(v8, sv)
+    akd, avd = dequantise(ak8, sk), dequantise(av8, sv)
+    with torch.no_grad():
+        out, lse = natten_amd.attention(q8, k8, v8, return_lse=True, q_scale=sq, k_scale=sk, v_scale=sv,
+                                        out_dtype=torch.bfloat16)
+    ref_o, ref_l = O.attention_forward(to_np(qd), to_np(kd), to_np(vd))
+    assert_close("dense out", to_np(out), ref_o)
+    assert_close("dense lse", to_np(lse), ref_l)
+    with torch.no_grad():
+        out, lse = natten_amd.na1d(q8, k8, v8, 7, additional_keys=ak8, additional_values=av8, return_lse=True,
+                                   q_scale=sq, k_scale=sk, v_scale=sv, out_dtype=torch.bfloat16)
+    ref_o, ref_l = O.na_forward(to_np(qd), to_np(kd), to_np(vd), (7,), additional_keys=to_np(akd),
+                                additional_values=to_np(avd))
+    assert_close("na + additional out", to_np(out), ref_o)
+    assert_close("na + additional lse", to_np(lse), ref_l)
