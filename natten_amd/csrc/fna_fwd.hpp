@@ -22,6 +22,7 @@
 #include <stdint.h>
 
 #include <type_traits>
+#include <utility>
 
 #include "na_math.hpp"
 
@@ -136,6 +137,21 @@ static __device__ __forceinline__ void wait_vmcnt() {
   __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 0xF) | ((N >> 4) << 14));
 }
 
+// calls f(std::integral_constant<int, LO + i>{}) for i = 0 .. N-1, in order
+template <int LO, typename F, int... Is>
+static __device__ __forceinline__ void for_range_impl(F&& f, std::integer_sequence<int, Is...>) {
+  (f(std::integral_constant<int, LO + Is>{}), ...);
+}
+template <int LO, int N, typename F>
+static __device__ __forceinline__ void for_range(F&& f) {
+  for_range_impl<LO>(f, std::make_integer_sequence<int, N>{});
+}
+
+// Keeps the computation of x at this point of the instruction stream: the empty statement
+// is a use the compiler can neither remove nor move into a later basic block.
+static __device__ __forceinline__ void pin(float& x) { asm volatile("" : "+v"(x)); }
+static __device__ __forceinline__ void pin(uint32_t& x) { asm volatile("" : "+v"(x)); }
+
 static __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 // max of x over the lane pair (l, l ^ 32): v_permlane32_swap exchanges the upper half of its
@@ -169,13 +185,14 @@ struct FnaSmem {
   static __host__ __device__ constexpr int v_slot(int r, int c) { return c ^ (2 * ((r / RPL) % (CPR / 2))); }
 };
 
-// Register budget: one query block per wave is meant to run two workgroups per CU (two waves per
-// SIMD, 256 registers each) so that one wave's softmax overlaps the other's MFMA work.
-template <typename T, int D, int NWAVES, int MQ, int KVT>
-__global__ void __launch_bounds__(NWAVES * 64) __attribute__((amdgpu_waves_per_eu(MQ == 1 ? 2 : 1, MQ == 1 ? 2 : 1)))
+// One 32-row query block per wave; two waves per SIMD (256 registers each).
+// RAGGED: seqlen_kv is not a multiple of KVT (dense attention on unpadded sequences); the tile
+// copies then clamp their rows and are issued at the top of an iteration instead of one per slot.
+template <typename T, int D, int NWAVES, bool RAGGED, int KVT>
+__global__ void __launch_bounds__(NWAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 fna_fwd_kernel(const FnaParams p) {
   constexpr int NT = NWAVES * 64;
-  constexpr int QT = NWAVES * MQ * 32;
+  constexpr int QT = NWAVES * 32;
   constexpr int KSTEPS = D / 16;
   constexpr int DB = D / 32;
   constexpr int NSB = KVT / 32;
@@ -290,36 +307,51 @@ fna_fwd_kernel(const FnaParams p) {
     ld_koff[i] = uint32_t(ld_row[i]) * uint32_t(kv_row_stride * 2) + uint32_t(L::k_slot(ld_row[i], slot) * 16);
     ld_voff[i] = uint32_t(ld_row[i]) * uint32_t(kv_row_stride * 2) + uint32_t(L::v_slot(ld_row[i], slot) * 16);
   }
-  auto issue_tile_load = [&](const T* base, const uint32_t (&off)[PER], char* dst, int kv_row0) {
-    const char* tile_base = reinterpret_cast<const char*>(base) + int64_t(kv_row0) * kv_row_stride * 2;
-    const uint32_t lds0 = lds_address(dst) + uint32_t(wave * PER * 1024);
-    const bool inside = kv_row0 + KVT <= p.seqlen_kv;
-    auto one = [&](auto i_tag) {
-      constexpr int I = decltype(i_tag)::value;
-      if constexpr (I < PER) {
-        if ((wave * PER + I) * 64 < CHUNKS) {
-          uint32_t voff = off[I];
-          if (!inside) {
-            // last, partial tile of an unpadded sequence: rows past the end are masked; read the
-            // last valid row instead so that no out-of-bounds address is formed
-            const int over = na_max(kv_row0 + ld_row[I] - (p.seqlen_kv - 1), 0);
-            voff -= uint32_t(over) * uint32_t(kv_row_stride * 2);
-          }
-          // the hardware adds the immediate to the global address too: take it off the uniform
-          // base (the per-lane offset stays a small non-negative number)
-          async_copy16_asm<(I % 4) * 1024>(tile_base - (I % 4) * 1024, voff, lds0 + uint32_t((I / 4) * 4096));
+  // One operand tile in flight: uniform source base, LDS destination of this wave's share.
+  struct TileCopy {
+    const char* src;  // first row of the tile (this head)
+    uint32_t lds0;    // LDS byte address of this wave's first chunk
+    int row0;
+    bool inside;      // the whole tile lies inside the sequence
+  };
+  auto make_copy = [&](const T* base, char* dst, int kv_row0) {
+    TileCopy c;
+    c.src = reinterpret_cast<const char*>(base) + int64_t(kv_row0) * kv_row_stride * 2;
+    c.lds0 = lds_address(dst) + uint32_t(wave * PER * 1024);
+    c.row0 = kv_row0;
+    c.inside = kv_row0 + KVT <= p.seqlen_kv;
+    return c;
+  };
+  // issues copy I (0 <= I < PER) of a tile
+  // (known_inside: the caller guarantees that the tile lies inside the sequence)
+  auto copy_one = [&](auto i_tag, auto known_inside, const TileCopy& c, const uint32_t (&off)[PER]) {
+    constexpr int I = decltype(i_tag)::value;
+    if constexpr (I < PER) {
+      if (CHUNKS % (NT * PER) == 0 || (wave * PER + I) * 64 < CHUNKS) {
+        uint32_t voff = off[I];
+        if (!decltype(known_inside)::value && !c.inside) {
+          // last, partial tile of an unpadded sequence: rows past the end are masked; read the
+          // last valid row instead so that no out-of-bounds address is formed
+          const int over = na_max(c.row0 + ld_row[I] - (p.seqlen_kv - 1), 0);
+          voff -= uint32_t(over) * uint32_t(kv_row_stride * 2);
         }
+        // the hardware adds the immediate to the global address too: take it off the uniform
+        // base (the per-lane offset stays a small non-negative number)
+        async_copy16_asm<(I % 4) * 1024>(c.src - (I % 4) * 1024, voff, c.lds0 + uint32_t((I / 4) * 4096));
       }
-    };
-    one(std::integral_constant<int, 0>{});
-    one(std::integral_constant<int, 1>{});
-    one(std::integral_constant<int, 2>{});
-    one(std::integral_constant<int, 3>{});
-    one(std::integral_constant<int, 4>{});
-    one(std::integral_constant<int, 5>{});
-    one(std::integral_constant<int, 6>{});
-    one(std::integral_constant<int, 7>{});
-    static_assert(PER <= 8, "tile copy is written for at most eight copies per thread");
+    }
+  };
+  static_assert(PER <= 8, "tile copy is written for at most eight copies per thread");
+  auto issue_tile_load = [&](const T* base, const uint32_t (&off)[PER], char* dst, int kv_row0) {
+    const TileCopy c = make_copy(base, dst, kv_row0);
+    copy_one(std::integral_constant<int, 0>{}, std::false_type{}, c, off);
+    copy_one(std::integral_constant<int, 1>{}, std::false_type{}, c, off);
+    copy_one(std::integral_constant<int, 2>{}, std::false_type{}, c, off);
+    copy_one(std::integral_constant<int, 3>{}, std::false_type{}, c, off);
+    copy_one(std::integral_constant<int, 4>{}, std::false_type{}, c, off);
+    copy_one(std::integral_constant<int, 5>{}, std::false_type{}, c, off);
+    copy_one(std::integral_constant<int, 6>{}, std::false_type{}, c, off);
+    copy_one(std::integral_constant<int, 7>{}, std::false_type{}, c, off);
   };
 
   // KV tile stream: dimension 2 fastest, dimension 0 slowest.  The load stream runs up to two
@@ -355,12 +387,11 @@ fna_fwd_kernel(const FnaParams p) {
   issue_tile_load(kbase, ld_koff, sK0, cur.row0);
   issue_tile_load(vbase, ld_voff, sV0, cur.row0);
 
-  // ---- per-lane setup: this lane's query rows, their windows, Q fragments ---------------------
-  int wst[MQ][3], wen[MQ][3];
-  vec8 qf[MQ][KSTEPS];
-#pragma unroll
-  for (int mb = 0; mb < MQ; ++mb) {
-    int r = (wave * MQ + mb) * 32 + l32;
+  // ---- per-lane setup: this lane's query row, its window, Q fragments ------------------------
+  int wst[3], wen[3];
+  vec8 qf[KSTEPS];
+  {
+    int r = wave * 32 + l32;
     const int row = qtile_idx * QT + r;
     int off[3];
     off[0] = r % p.q_tile[0];
@@ -370,26 +401,21 @@ fna_fwd_kernel(const FnaParams p) {
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
       const int c = q_first[a] + off[a];
-      wst[mb][a] = na_window_start(c, p.ksize[a], p.stride[a], extent[a], p.causal[a] != 0);
-      wen[mb][a] = na_window_end(c, wst[mb][a], p.ksize[a], extent[a], p.causal[a] != 0);
+      wst[a] = na_window_start(c, p.ksize[a], p.stride[a], extent[a], p.causal[a] != 0);
+      wen[a] = na_window_end(c, wst[a], p.ksize[a], extent[a], p.causal[a] != 0);
     }
     const int row_c = na_min(row, p.seqlen_q - 1);
     const T* qrow = qbase + int64_t(row_c) * q_row_stride + g * 8;
 #pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) qf[mb][ks] = *reinterpret_cast<const vec8*>(qrow + ks * 16);
+    for (int ks = 0; ks < KSTEPS; ++ks) qf[ks] = *reinterpret_cast<const vec8*>(qrow + ks * 16);
   }
 
-  f32x16_t acc[MQ][DB];
-  float m_run[MQ], l_run[MQ];
+  f32x16_t acc[DB];
+  float m_run = -INFINITY, l_run = 0.f;
 #pragma unroll
-  for (int mb = 0; mb < MQ; ++mb) {
-    m_run[mb] = -INFINITY;
-    l_run[mb] = 0.f;
+  for (int db = 0; db < DB; ++db)
 #pragma unroll
-    for (int db = 0; db < DB; ++db)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[mb][db][r] = 0.f;
-  }
+    for (int r = 0; r < 16; ++r) acc[db][r] = 0.f;
   float sm_scale = p.scale, out_scale = 1.f;
   if (p.q_scale) sm_scale *= p.q_scale[head];
   if (p.k_scale) sm_scale *= p.k_scale[head_kv];
@@ -407,37 +433,127 @@ fna_fwd_kernel(const FnaParams p) {
   const int v_chunk = (l32 >> 4) * 2 + (v_j4 >> 1);  // 16-byte chunk inside the 64-byte column block
   const int v_sub = (v_j4 & 1) * 8;
 
-  // S^T = K Q^T of one tile: lane owns query row l32 (per q block) and 16 key rows per 32-key sub-block
-  auto qk_tile = [&](const char* sK, f32x16_t (&S)[MQ][NSB]) {
+  // ---- building blocks ---------------------------------------------------------------------------
+  // The lane owns query row l32 of its wave and, per 32-key sub-block, the 16 key rows
+  // 8*(r/4) + 4*g + r%4.  One "slot" below is one MFMA plus the vector work that is to run in
+  // its shadow; slots are fenced so that the compiler keeps that interleaving (a 32x32x16 MFMA
+  // occupies the matrix pipe for 32 cycles but only one issue cycle, and up to six ordinary
+  // vector instructions of the same wave issue behind it for free).
+  constexpr int N_QK = NSB * KSTEPS;   // MFMAs of S^T = K Q^T
+  constexpr int N_PV = NSB * 2 * DB;   // MFMAs of O^T += V^T P^T
+  constexpr int N_UNITS = NSB * 8;     // pairs of probabilities
+  constexpr int UNITS_G1 = N_UNITS * 3 / 4;  // pairs exponentiated in the shadow of the QK MFMAs
+  constexpr int PF_K = 2, PF_V = 2;    // operand fragments read ahead of their MFMA
+  static_assert(NSB % 2 == 0 && N_QK > PF_K && N_PV > PF_V, "tile too small for the schedule");
+
+  // QK slot s multiplies k-step s % KSTEPS of sub-block s / KSTEPS (a sub-block's logits only
+  // occupy registers once its first slot is reached)
+  auto k_frag = [&](const char* sK, int s) {
+    return *reinterpret_cast<const vec8*>(sK + (s / KSTEPS) * 32 * ROWB + k_off[s % KSTEPS]);
+  };
+  // PV slot t: sub-block t / (2*DB), 16-key half (t / DB) % 2, 32-column block t % DB
+  auto v_frag = [&](const char* sV, int t) {
+    const int r0 = (t / (2 * DB)) * 32 + ((t / DB) % 2) * 16 + v_row;
+    const int c = (t % DB) * 4 + v_chunk;
+    const s16x4_t lo = lds_read_tr16(sV + r0 * ROWB + v_sub + L::v_slot(r0, c) * 16);
+    const s16x4_t hi = lds_read_tr16(sV + (r0 + 8) * ROWB + v_sub + L::v_slot(r0 + 8, c) * 16);
+    return __builtin_bit_cast(vec8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+  };
+
+  f32x16_t S_a[NSB], S_b[NSB];  // logits of the current / coming tile, swapping roles every iteration
+  vec8 pf[NSB][2];
+  float msc = 0.f;              // running maximum in the exp2 domain (0 while it is -inf)
+  float psum0 = 0.f, psum1 = 0.f;
+
+  // probabilities 2u, 2u+1 of the current tile: exp2(c*s - c*m), summed in float, rounded to T
+  auto exp_unit = [&](const f32x16_t (&S_cur)[NSB], int u) {
+    const int sb = u / 8, r = 2 * (u % 8);
+    const float e0 = fast_exp2(S_cur[sb][r] * c_log2 - msc);
+    const float e1 = fast_exp2(S_cur[sb][r + 1] * c_log2 - msc);
+    psum0 += e0;
+    psum1 += e1;
+    vec2 p2 = {static_cast<T>(e0), static_cast<T>(e1)};
+    uint32_t bits = __builtin_bit_cast(uint32_t, p2);
+    pin(bits);
+    p2 = __builtin_bit_cast(vec2, bits);
+    pf[sb][r / 8][r % 8] = p2[0];
+    pf[sb][r / 8][r % 8 + 1] = p2[1];
+  };
+
+  // element mask of a PARTIAL tile
+  auto apply_mask = [&](f32x16_t (&S)[NSB], const int (&origin)[3]) {
+    // window of this lane's query relative to the tile origin, clamped to the tile
+    uint32_t addc = 0, subc = 0;
 #pragma unroll
-    for (int sb = 0; sb < NSB; ++sb) {
-#pragma unroll
-      for (int mb = 0; mb < MQ; ++mb)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) S[mb][sb][r] = 0.f;
-      // rows sb*32 + l32: (sb*32) is a multiple of 16 rows, so the swizzle term is unchanged
-#pragma unroll
-      for (int ks = 0; ks < KSTEPS; ++ks) {
-        const vec8 kf = *reinterpret_cast<const vec8*>(sK + sb * 32 * ROWB + k_off[ks]);
-#pragma unroll
-        for (int mb = 0; mb < MQ; ++mb) S[mb][sb] = M::run(kf, qf[mb][ks], S[mb][sb]);
-      }
+    for (int a = 0; a < 3; ++a) {
+      const int lo = na_min(na_max(wst[a] - origin[a], 0), p.kv_tile[a]);
+      const int hi = na_min(na_max(wen[a] - origin[a], 0), p.kv_tile[a]);
+      addc |= uint32_t(512 - lo) << (10 * a);
+      subc |= uint32_t(511 + hi) << (10 * a);
     }
+#pragma unroll
+    for (int sb = 0; sb < NSB; ++sb)
+#pragma unroll
+      for (int jj = 0; jj < 4; ++jj) {
+        const u32x4_t tc4 = *reinterpret_cast<const u32x4_t*>(&sTab[sb * 32 + 8 * jj + 4 * g]);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const uint32_t tp = tc4[i];
+          const uint32_t ok = (tp + addc) & (subc - tp) & kGuardBits;
+          S[sb][4 * jj + i] = (ok == kGuardBits) ? S[sb][4 * jj + i] : -INFINITY;
+        }
+      }
+  };
+
+  // adopts the maximum `mx` of the lane's half row of the coming tile: the running maximum is
+  // only moved (and O, the row sum rescaled) when some row of the wave outgrew it by 2^8
+  auto update_max = [&](float mx) {
+    mx = cross_half_max(mx);
+    const bool grow = (mx - m_run) * c_log2 > kLazyRescaleLog2;  // also true while m_run == -inf and mx finite
+    if (__any(grow)) {
+      const float m_new = fmaxf(m_run, mx);
+      const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+      const float alpha = fast_exp2((m_run - m_use) * c_log2);  // m_run == -inf -> 0
+      m_run = m_new;
+      l_run *= alpha;
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[db][r] *= alpha;
+    }
+    msc = ((m_run == -INFINITY) ? 0.f : m_run) * c_log2;
   };
 
   // ---- software pipeline --------------------------------------------------------------------
-  // Iteration j computes S(j+1) = K(j+1) Q^T on the matrix cores while the vector units run the
-  // softmax of S(j); then O += P(j) V(j).  At its top, K(j+2) and V(j+1) are put in flight.
+  // Iteration j: (G1) S(j+1) = K(j+1) Q^T with three quarters of the exponentials of S(j) and
+  // the asynchronous copies of K(j+2), V(j+1) in its shadow; (G2) first half of O += P(j) V(j)
+  // with the remaining exponentials; (G3) second half with the row maximum of S(j+1).
   // LDS: K(j) and V(j) live in stage j % 2.
-  TileInfo nxt = next_tile();  // tile 1 (a descriptor past the box is never used for loads)
+  TileInfo nxt = next_tile();  // tile 1 (a descriptor past the box is never used)
   wait_vmcnt<0>();
   __syncthreads();  // K(0), V(0) and the coordinate table are in LDS
   if (1 < total_tiles) issue_tile_load(kbase, ld_koff, sK1, nxt.row0);
-  f32x16_t S_cur[MQ][NSB];
-  qk_tile(sK0, S_cur);
+  {
+#pragma unroll
+    for (int sb = 0; sb < NSB; ++sb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) S_a[sb][r] = 0.f;
+#pragma unroll
+    for (int s = 0; s < N_QK; ++s) S_a[s / KSTEPS] = M::run(k_frag(sK0, s), qf[s % KSTEPS], S_a[s / KSTEPS]);
+    if (!cur.full) apply_mask(S_a, cur.origin);
+    float mx = -INFINITY;
+#pragma unroll
+    for (int sb = 0; sb < NSB; ++sb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, S_a[sb][r]);
+    update_max(mx);
+  }
 
   auto iteration = [&](auto stage_tag, int j) {
     constexpr int st = decltype(stage_tag)::value;
+    constexpr bool SPREAD = !RAGGED;
+    f32x16_t (&S_cur)[NSB] = st ? S_b : S_a;
+    f32x16_t (&S_nxt)[NSB] = st ? S_a : S_b;
     char* sK_cur = st ? sK1 : sK0;  // held K(j): free, receives K(j+2)
     char* sK_nxt = st ? sK0 : sK1;  // holds K(j+1)
     char* sV_cur = st ? sV1 : sV0;  // holds V(j)
@@ -446,109 +562,101 @@ fna_fwd_kernel(const FnaParams p) {
     wait_vmcnt<0>();   // this thread's copies of K(j+1) and V(j) have landed
     __syncthreads();   // ... and everyone's; everyone is done reading K(j) and V(j-1)
     const TileInfo t2 = next_tile();
-    if (j + 2 < total_tiles) issue_tile_load(kbase, ld_koff, sK_cur, t2.row0);
-    if (j + 1 < total_tiles) issue_tile_load(vbase, ld_voff, sV_nxt, nxt.row0);
+    // Past the end of the box the spread copies re-read the current tile into the free stage
+    // (never used), which keeps the slots below free of control flow.
+    const TileCopy ck = make_copy(kbase, sK_cur, (j + 2 < total_tiles) ? t2.row0 : cur.row0);
+    const TileCopy cv = make_copy(vbase, sV_nxt, (j + 1 < total_tiles) ? nxt.row0 : cur.row0);
+    if constexpr (!SPREAD) {
+      if (j + 2 < total_tiles) issue_tile_load(kbase, ld_koff, sK_cur, t2.row0);
+      if (j + 1 < total_tiles) issue_tile_load(vbase, ld_voff, sV_nxt, nxt.row0);
+    }
 
-    // -- softmax, part 1: mask, row maximum, (rare) rescale -----------------------------------
-    float msc[MQ];
+    // -- G1 ------------------------------------------------------------------------------------
+    vec8 kf[N_QK];
 #pragma unroll
-    for (int mb = 0; mb < MQ; ++mb) {
-      if (!cur.full) {
-        // window of this lane's query relative to the tile origin, clamped to the tile
-        uint32_t addc = 0, subc = 0;
+    for (int s = 0; s < PF_K; ++s) kf[s] = k_frag(sK_nxt, s);
+    psum0 = 0.f;
+    psum1 = 0.f;
+    auto g1_slot = [&](auto s_tag) {
+      constexpr int s = decltype(s_tag)::value;
+      if constexpr (s + PF_K < N_QK) kf[s + PF_K] = k_frag(sK_nxt, s + PF_K);
+      if constexpr (s % KSTEPS == 0) {
+        f32x16_t zero;
 #pragma unroll
-        for (int a = 0; a < 3; ++a) {
-          const int lo = na_min(na_max(wst[mb][a] - cur.origin[a], 0), p.kv_tile[a]);
-          const int hi = na_min(na_max(wen[mb][a] - cur.origin[a], 0), p.kv_tile[a]);
-          addc |= uint32_t(512 - lo) << (10 * a);
-          subc |= uint32_t(511 + hi) << (10 * a);
+        for (int r = 0; r < 16; ++r) zero[r] = 0.f;
+        S_nxt[s / KSTEPS] = M::run(kf[s], qf[s % KSTEPS], zero);
+      } else {
+        S_nxt[s / KSTEPS] = M::run(kf[s], qf[s % KSTEPS], S_nxt[s / KSTEPS]);
+      }
+      constexpr int u_lo = (s * UNITS_G1) / N_QK, u_hi = ((s + 1) * UNITS_G1) / N_QK;
+#pragma unroll
+      for (int u = u_lo; u < u_hi; ++u) exp_unit(S_cur, u);
+      if constexpr (u_hi > u_lo) {
+        pin(psum0);
+        pin(psum1);
+      }
+      if constexpr (SPREAD) {
+        // 2 * PER copies spread over the first half of the slots, K first
+        constexpr int c_lo = (s * 2 * PER * 2) / N_QK, c_hi = ((s + 1) * 2 * PER * 2) / N_QK;
+        for_range<c_lo, c_hi - c_lo>([&](auto c_tag) {
+          constexpr int c = decltype(c_tag)::value;
+          if constexpr (c < PER) copy_one(std::integral_constant<int, c>{}, std::true_type{}, ck, ld_koff);
+          else if constexpr (c < 2 * PER) copy_one(std::integral_constant<int, c - PER>{}, std::true_type{}, cv, ld_voff);
+        });
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    for_range<0, N_QK>(g1_slot);
+
+    // -- G2 / G3 -------------------------------------------------------------------------------
+    vec8 vf[N_PV];
+#pragma unroll
+    for (int t = 0; t < PF_V; ++t) vf[t] = v_frag(sV_cur, t);
+    float mx0 = -INFINITY, mx1 = -INFINITY;
+    auto pv_slot = [&](auto t_tag) {
+      constexpr int t = decltype(t_tag)::value;
+      if constexpr (t + PF_V < N_PV) vf[t + PF_V] = v_frag(sV_cur, t + PF_V);
+      acc[t % DB] = M::run(vf[t], pf[t / (2 * DB)][(t / DB) % 2], acc[t % DB]);
+      if constexpr (t < N_PV / 2) {
+        constexpr int u_lo = UNITS_G1 + (t * (N_UNITS - UNITS_G1)) / (N_PV / 2);
+        constexpr int u_hi = UNITS_G1 + ((t + 1) * (N_UNITS - UNITS_G1)) / (N_PV / 2);
+#pragma unroll
+        for (int u = u_lo; u < u_hi; ++u) exp_unit(S_cur, u);
+        if constexpr (u_hi > u_lo) {
+          pin(psum0);
+          pin(psum1);
         }
+      } else {
+        // row maximum of the coming tile (as if unmasked), NSB * 16 values over N_PV / 2 slots
+        constexpr int t3 = t - N_PV / 2;
+        constexpr int e_lo = (t3 * NSB * 16) / (N_PV / 2), e_hi = ((t3 + 1) * NSB * 16) / (N_PV / 2);
+#pragma unroll
+        for (int e = e_lo; e < e_hi; ++e) {
+          if (e % 2 == 0) mx0 = fmaxf(mx0, S_nxt[e / 16][e % 16]);
+          else mx1 = fmaxf(mx1, S_nxt[e / 16][e % 16]);
+        }
+        if constexpr (e_hi > e_lo) {
+          pin(mx0);
+          pin(mx1);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    for_range<0, N_PV>(pv_slot);
+    l_run += psum0 + psum1;
+
+    if (j + 1 < total_tiles) {
+      float mx = fmaxf(mx0, mx1);
+      if (!nxt.full) {
+        apply_mask(S_nxt, nxt.origin);
+        mx = -INFINITY;
 #pragma unroll
         for (int sb = 0; sb < NSB; ++sb)
 #pragma unroll
-          for (int jj = 0; jj < 4; ++jj) {
-            const u32x4_t tc4 = *reinterpret_cast<const u32x4_t*>(&sTab[sb * 32 + 8 * jj + 4 * g]);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-              const uint32_t tp = tc4[i];
-              const uint32_t ok = (tp + addc) & (subc - tp) & kGuardBits;
-              S_cur[mb][sb][4 * jj + i] = (ok == kGuardBits) ? S_cur[mb][sb][4 * jj + i] : -INFINITY;
-            }
-          }
+          for (int r = 0; r < 16; ++r) mx = fmaxf(mx, S_nxt[sb][r]);
       }
-      float mx = -INFINITY;
-#pragma unroll
-      for (int sb = 0; sb < NSB; ++sb)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, S_cur[mb][sb][r]);
-      mx = cross_half_max(mx);
-      // rescale only when some row of this wave outgrew its (stale) maximum by more than 2^8
-      const bool grow = (mx - m_run[mb]) * c_log2 > kLazyRescaleLog2;  // also true while m_run == -inf and mx finite
-      if (__any(grow)) {
-        const float m_new = fmaxf(m_run[mb], mx);
-        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-        const float alpha = fast_exp2((m_run[mb] - m_use) * c_log2);  // m_run == -inf -> 0
-        m_run[mb] = m_new;
-        l_run[mb] *= alpha;
-#pragma unroll
-        for (int db = 0; db < DB; ++db)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) acc[mb][db][r] *= alpha;
-      }
-      msc[mb] = ((m_run[mb] == -INFINITY) ? 0.f : m_run[mb]) * c_log2;
+      update_max(mx);
     }
-
-    // -- S(j+1) on the matrix cores, exponentials of S(j) on the vector units ------------------
-    f32x16_t S_nxt[MQ][NSB];
-    qk_tile(sK_nxt, S_nxt);
-    vec8 pf[MQ][NSB][2];
-#pragma unroll
-    for (int mb = 0; mb < MQ; ++mb) {
-      float psum = 0.f;
-#pragma unroll
-      for (int sb = 0; sb < NSB; ++sb)
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-          vec8 pv;
-#pragma unroll
-          for (int i = 0; i < 8; i += 2) {
-            vec2 p2;
-            p2[0] = static_cast<T>(fast_exp2(S_cur[mb][sb][8 * h + i] * c_log2 - msc[mb]));
-            p2[1] = static_cast<T>(fast_exp2(S_cur[mb][sb][8 * h + i + 1] * c_log2 - msc[mb]));
-            psum = M::add2(p2, psum);  // sums the rounded probabilities, the ones P V uses
-            pv[i] = p2[0];
-            pv[i + 1] = p2[1];
-          }
-          pf[mb][sb][h] = pv;
-        }
-      l_run[mb] += psum;
-    }
-
-    // -- O^T += V^T P^T : the k-slot order of the P fragment (rows 4g..4g+3 and 8+4g..8+4g+3 of
-    // each 16-key half) is matched by two transpose reads of V.
-#pragma unroll
-    for (int sb = 0; sb < NSB; ++sb)
-#pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        const int r0 = sb * 32 + h * 16 + v_row;
-        const char* row_lo = sV_cur + r0 * ROWB + v_sub;
-        const char* row_hi = sV_cur + (r0 + 8) * ROWB + v_sub;
-#pragma unroll
-        for (int db = 0; db < DB; ++db) {
-          const int c = db * 4 + v_chunk;
-          const s16x4_t lo = lds_read_tr16(row_lo + L::v_slot(r0, c) * 16);
-          const s16x4_t hi = lds_read_tr16(row_hi + L::v_slot(r0 + 8, c) * 16);
-          const s16x8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-          const vec8 vf = __builtin_bit_cast(vec8, both);
-#pragma unroll
-          for (int mb = 0; mb < MQ; ++mb) acc[mb][db] = M::run(vf, pf[mb][sb][h], acc[mb][db]);
-        }
-      }
-
-#pragma unroll
-    for (int mb = 0; mb < MQ; ++mb)
-#pragma unroll
-      for (int sb = 0; sb < NSB; ++sb) S_cur[mb][sb] = S_nxt[mb][sb];
     cur = nxt;
     nxt = t2;
   };
@@ -556,14 +664,14 @@ fna_fwd_kernel(const FnaParams p) {
     iteration(Stage0{}, j);
     if (j + 1 < total_tiles) iteration(Stage1{}, j + 1);
   }
+  wait_vmcnt<0>();  // the last iterations' copies into the unused stage must land before the LDS is released
 
   // ---- epilogue: O = acc / rowsum, LSE = ln(rowsum) + scale * rowmax -------------------------
   T* obase = reinterpret_cast<T*>(p.o) + int64_t(bg) * p.seqlen_q * q_row_stride + int64_t(head) * D;
-#pragma unroll
-  for (int mb = 0; mb < MQ; ++mb) {
-    const float l = l_run[mb] + __shfl_xor(l_run[mb], 32);
+  {
+    const float l = l_run + __shfl_xor(l_run, 32);
     const float inv = (l > 0.f) ? out_scale / l : 0.f;
-    const int row = qtile_idx * QT + (wave * MQ + mb) * 32 + l32;
+    const int row = qtile_idx * QT + wave * 32 + l32;
     if (row < p.seqlen_q) {
       T* orow = obase + int64_t(row) * q_row_stride;
 #pragma unroll
@@ -573,11 +681,11 @@ fna_fwd_kernel(const FnaParams p) {
           typedef T tx4 __attribute__((ext_vector_type(4)));
           tx4 o4;
 #pragma unroll
-          for (int i = 0; i < 4; ++i) o4[i] = static_cast<T>(acc[mb][db][4 * j + i] * inv);
+          for (int i = 0; i < 4; ++i) o4[i] = static_cast<T>(acc[db][4 * j + i] * inv);
           *reinterpret_cast<tx4*>(orow + db * 32 + 8 * j + 4 * g) = o4;
         }
       if (g == 0) {
-        const float lse = (l > 0.f) ? (m_run[mb] * sm_scale + __logf(l)) : -INFINITY;
+        const float lse = (l > 0.f) ? (m_run * sm_scale + __logf(l)) : -INFINITY;
         p.lse[(int64_t(bg) * p.seqlen_q + row) * p.heads_q + head] = lse;
       }
     }
