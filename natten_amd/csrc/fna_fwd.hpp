@@ -114,6 +114,13 @@ static __device__ __forceinline__ s16x4_t lds_read_tr16(const char* p) {
 // against LDS reads of the same bytes is the caller's business (workgroup barriers).
 template <int IMM>
 static __device__ __forceinline__ void async_copy16_asm(const void* base, uint32_t voff, uint32_t lds_addr) {
+  // base and lds_addr are wave-uniform by construction; say so, so that they are always
+  // handed over in scalar registers
+  const uint64_t b = reinterpret_cast<uint64_t>(base);
+  const uint64_t ub = (uint64_t(uint32_t(__builtin_amdgcn_readfirstlane(int(b >> 32)))) << 32) |
+                      uint32_t(__builtin_amdgcn_readfirstlane(int(uint32_t(b))));
+  base = reinterpret_cast<const void*>(ub);
+  lds_addr = uint32_t(__builtin_amdgcn_readfirstlane(int(lds_addr)));
   asm volatile(
       "s_mov_b32 m0, %0\n\t"
       "s_nop 0\n\t"
@@ -185,14 +192,16 @@ struct FnaSmem {
   static __host__ __device__ constexpr int v_slot(int r, int c) { return c ^ (2 * ((r / RPL) % (CPR / 2))); }
 };
 
-// One 32-row query block per wave; two waves per SIMD (256 registers each).
+// MQ 32-row query blocks per wave.  MQ = 1 runs two waves per SIMD (256 registers each);
+// MQ = 2 one wave per SIMD (512 registers: accumulators and Q fragments can sit in the
+// accumulation registers) and reads every K / V fragment from LDS once for two MFMAs.
 // RAGGED: seqlen_kv is not a multiple of KVT (dense attention on unpadded sequences); the tile
 // copies then clamp their rows and are issued at the top of an iteration instead of one per slot.
-template <typename T, int D, int NWAVES, bool RAGGED, int KVT>
-__global__ void __launch_bounds__(NWAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
+template <typename T, int D, int NWAVES, int MQ, bool RAGGED, int KVT>
+__global__ void __launch_bounds__(NWAVES * 64) __attribute__((amdgpu_waves_per_eu(MQ == 1 ? 2 : 1, MQ == 1 ? 2 : 1)))
 fna_fwd_kernel(const FnaParams p) {
   constexpr int NT = NWAVES * 64;
-  constexpr int QT = NWAVES * 32;
+  constexpr int QT = NWAVES * MQ * 32;
   constexpr int KSTEPS = D / 16;
   constexpr int DB = D / 32;
   constexpr int NSB = KVT / 32;
@@ -291,21 +300,30 @@ fna_fwd_kernel(const FnaParams p) {
   const T* vbase = reinterpret_cast<const T*>(p.v) + int64_t(bg) * p.seqlen_kv * kv_row_stride + int64_t(head_kv) * D;
 
   // ---- async tile loads -------------------------------------------------------------------------
-  // Copy i of this thread fills LDS chunk position P = i*NT + tid (row P / CPR, slot P % CPR).
-  // Its global address is a per-tile uniform base (first row of the tile) plus a byte offset
-  // that never changes for the thread, so a tile load costs no vector address arithmetic.
-  int ld_row[PER];
-  uint32_t ld_koff[PER], ld_voff[PER];
+  // Copy i of wave w fills LDS chunks (w*PER + i)*64 .. +63 of the tile (chunk P: row P / CPR,
+  // slot P % CPR).  Its global address is a per-tile uniform base (first row of the tile) plus
+  // a byte offset that never changes for the thread, so a tile load costs no vector address
+  // arithmetic.  Up to four copies share one M0 value through the instruction's immediate
+  // offset (which the hardware adds to the LDS and to the global address alike: it is taken off
+  // the per-lane offset again), and copy i + 4 lies a whole number of swizzle periods (16 rows
+  // or more) below copy i, so it reuses that copy's per-lane offset on a shifted base.
+  constexpr int NOFF = PER < 4 ? PER : 4;
+  constexpr int ROWS_PER_4 = 256 / CPR;  // rows between copy i and copy i + 4
+  int ld_row[NOFF];
+  uint32_t ld_koff[NOFF], ld_voff[NOFF];
 #pragma unroll
-  for (int i = 0; i < PER; ++i) {
-    // copy i of wave w fills LDS chunks (w*PER + i)*64 .. +63; up to four copies share one M0
-    // value through the instruction's immediate offset
+  for (int i = 0; i < NOFF; ++i) {
     const int P = (wave * PER + i) * 64 + lane;
     ld_row[i] = P / CPR;
     const int slot = P % CPR;
     // XOR swizzles are involutions: slot -> source chunk uses the same function
     ld_koff[i] = uint32_t(ld_row[i]) * uint32_t(kv_row_stride * 2) + uint32_t(L::k_slot(ld_row[i], slot) * 16);
     ld_voff[i] = uint32_t(ld_row[i]) * uint32_t(kv_row_stride * 2) + uint32_t(L::v_slot(ld_row[i], slot) * 16);
+    if constexpr (!RAGGED) {
+      // never negative: copy i starts at least 64 * i / CPR rows of at least 16 * CPR bytes into the tile
+      ld_koff[i] -= uint32_t(i * 1024);
+      ld_voff[i] -= uint32_t(i * 1024);
+    }
   }
   // One operand tile in flight: uniform source base, LDS destination of this wave's share.
   struct TileCopy {
@@ -316,6 +334,7 @@ fna_fwd_kernel(const FnaParams p) {
   };
   auto make_copy = [&](const T* base, char* dst, int kv_row0) {
     TileCopy c;
+    kv_row0 = __builtin_amdgcn_readfirstlane(kv_row0);  // uniform by construction; keeps the base in scalar registers
     c.src = reinterpret_cast<const char*>(base) + int64_t(kv_row0) * kv_row_stride * 2;
     c.lds0 = lds_address(dst) + uint32_t(wave * PER * 1024);
     c.row0 = kv_row0;
@@ -323,35 +342,39 @@ fna_fwd_kernel(const FnaParams p) {
     return c;
   };
   // issues copy I (0 <= I < PER) of a tile
-  // (known_inside: the caller guarantees that the tile lies inside the sequence)
-  auto copy_one = [&](auto i_tag, auto known_inside, const TileCopy& c, const uint32_t (&off)[PER]) {
+  auto copy_one = [&](auto i_tag, const TileCopy& c, const uint32_t (&off)[NOFF]) {
     constexpr int I = decltype(i_tag)::value;
     if constexpr (I < PER) {
       if (CHUNKS % (NT * PER) == 0 || (wave * PER + I) * 64 < CHUNKS) {
-        uint32_t voff = off[I];
-        if (!decltype(known_inside)::value && !c.inside) {
-          // last, partial tile of an unpadded sequence: rows past the end are masked; read the
-          // last valid row instead so that no out-of-bounds address is formed
-          const int over = na_max(c.row0 + ld_row[I] - (p.seqlen_kv - 1), 0);
-          voff -= uint32_t(over) * uint32_t(kv_row_stride * 2);
+        constexpr int IMM = (I % 4) * 1024;
+        const char* src = c.src + int64_t(I / 4) * ROWS_PER_4 * (kv_row_stride * 2);
+        uint32_t voff = off[I % 4];
+        if constexpr (RAGGED) {
+          if (!c.inside) {
+            // last, partial tile of an unpadded sequence: rows past the end are masked; read the
+            // last valid row instead so that no out-of-bounds address is formed
+            const int over = na_max(c.row0 + ld_row[I % 4] + (I / 4) * ROWS_PER_4 - (p.seqlen_kv - 1), 0);
+            voff -= uint32_t(over) * uint32_t(kv_row_stride * 2);
+          }
+          // the clamped per-lane offset may be smaller than the immediate: take the immediate
+          // off the uniform base instead
+          src -= IMM;
         }
-        // the hardware adds the immediate to the global address too: take it off the uniform
-        // base (the per-lane offset stays a small non-negative number)
-        async_copy16_asm<(I % 4) * 1024>(c.src - (I % 4) * 1024, voff, c.lds0 + uint32_t((I / 4) * 4096));
+        async_copy16_asm<IMM>(src, voff, c.lds0 + uint32_t((I / 4) * 4096));
       }
     }
   };
   static_assert(PER <= 8, "tile copy is written for at most eight copies per thread");
-  auto issue_tile_load = [&](const T* base, const uint32_t (&off)[PER], char* dst, int kv_row0) {
+  auto issue_tile_load = [&](const T* base, const uint32_t (&off)[NOFF], char* dst, int kv_row0) {
     const TileCopy c = make_copy(base, dst, kv_row0);
-    copy_one(std::integral_constant<int, 0>{}, std::false_type{}, c, off);
-    copy_one(std::integral_constant<int, 1>{}, std::false_type{}, c, off);
-    copy_one(std::integral_constant<int, 2>{}, std::false_type{}, c, off);
-    copy_one(std::integral_constant<int, 3>{}, std::false_type{}, c, off);
-    copy_one(std::integral_constant<int, 4>{}, std::false_type{}, c, off);
-    copy_one(std::integral_constant<int, 5>{}, std::false_type{}, c, off);
-    copy_one(std::integral_constant<int, 6>{}, std::false_type{}, c, off);
-    copy_one(std::integral_constant<int, 7>{}, std::false_type{}, c, off);
+    copy_one(std::integral_constant<int, 0>{}, c, off);
+    copy_one(std::integral_constant<int, 1>{}, c, off);
+    copy_one(std::integral_constant<int, 2>{}, c, off);
+    copy_one(std::integral_constant<int, 3>{}, c, off);
+    copy_one(std::integral_constant<int, 4>{}, c, off);
+    copy_one(std::integral_constant<int, 5>{}, c, off);
+    copy_one(std::integral_constant<int, 6>{}, c, off);
+    copy_one(std::integral_constant<int, 7>{}, c, off);
   };
 
   // KV tile stream: dimension 2 fastest, dimension 0 slowest.  The load stream runs up to two
@@ -387,11 +410,12 @@ fna_fwd_kernel(const FnaParams p) {
   issue_tile_load(kbase, ld_koff, sK0, cur.row0);
   issue_tile_load(vbase, ld_voff, sV0, cur.row0);
 
-  // ---- per-lane setup: this lane's query row, its window, Q fragments ------------------------
-  int wst[3], wen[3];
-  vec8 qf[KSTEPS];
-  {
-    int r = wave * 32 + l32;
+  // ---- per-lane setup: this lane's query rows, their windows, Q fragments ---------------------
+  int wst[MQ][3], wen[MQ][3];
+  vec8 qf[MQ][KSTEPS];
+#pragma unroll
+  for (int mb = 0; mb < MQ; ++mb) {
+    int r = (wave * MQ + mb) * 32 + l32;
     const int row = qtile_idx * QT + r;
     int off[3];
     off[0] = r % p.q_tile[0];
@@ -401,21 +425,26 @@ fna_fwd_kernel(const FnaParams p) {
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
       const int c = q_first[a] + off[a];
-      wst[a] = na_window_start(c, p.ksize[a], p.stride[a], extent[a], p.causal[a] != 0);
-      wen[a] = na_window_end(c, wst[a], p.ksize[a], extent[a], p.causal[a] != 0);
+      wst[mb][a] = na_window_start(c, p.ksize[a], p.stride[a], extent[a], p.causal[a] != 0);
+      wen[mb][a] = na_window_end(c, wst[mb][a], p.ksize[a], extent[a], p.causal[a] != 0);
     }
     const int row_c = na_min(row, p.seqlen_q - 1);
     const T* qrow = qbase + int64_t(row_c) * q_row_stride + g * 8;
 #pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) qf[ks] = *reinterpret_cast<const vec8*>(qrow + ks * 16);
+    for (int ks = 0; ks < KSTEPS; ++ks) qf[mb][ks] = *reinterpret_cast<const vec8*>(qrow + ks * 16);
   }
 
-  f32x16_t acc[DB];
-  float m_run = -INFINITY, l_run = 0.f;
+  f32x16_t acc[MQ][DB];
+  float m_run[MQ], l_run[MQ];
 #pragma unroll
-  for (int db = 0; db < DB; ++db)
+  for (int mb = 0; mb < MQ; ++mb) {
+    m_run[mb] = -INFINITY;
+    l_run[mb] = 0.f;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) acc[db][r] = 0.f;
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[mb][db][r] = 0.f;
+  }
   float sm_scale = p.scale, out_scale = 1.f;
   if (p.q_scale) sm_scale *= p.q_scale[head];
   if (p.k_scale) sm_scale *= p.k_scale[head_kv];
@@ -434,16 +463,15 @@ fna_fwd_kernel(const FnaParams p) {
   const int v_sub = (v_j4 & 1) * 8;
 
   // ---- building blocks ---------------------------------------------------------------------------
-  // The lane owns query row l32 of its wave and, per 32-key sub-block, the 16 key rows
-  // 8*(r/4) + 4*g + r%4.  One "slot" below is one MFMA plus the vector work that is to run in
-  // its shadow; slots are fenced so that the compiler keeps that interleaving (a 32x32x16 MFMA
-  // occupies the matrix pipe for 32 cycles but only one issue cycle, and up to six ordinary
-  // vector instructions of the same wave issue behind it for free).
-  constexpr int N_QK = NSB * KSTEPS;   // MFMAs of S^T = K Q^T
-  constexpr int N_PV = NSB * 2 * DB;   // MFMAs of O^T += V^T P^T
-  constexpr int N_UNITS = NSB * 8;     // pairs of probabilities
-  constexpr int UNITS_G1 = N_UNITS * 3 / 4;  // pairs exponentiated in the shadow of the QK MFMAs
-  constexpr int PF_K = 2, PF_V = 2;    // operand fragments read ahead of their MFMA
+  // The lane owns query row l32 of each of its wave's MQ row blocks and, per 32-key sub-block,
+  // the 16 key rows 8*(r/4) + 4*g + r%4.  One "slot" below is one operand fragment read from
+  // LDS, the MQ MFMAs that use it, and the vector work that is to run in their shadow; slots are
+  // fenced so that the compiler keeps that interleaving (a 32x32x16 MFMA occupies the matrix pipe
+  // for 32 cycles but only one issue cycle, and up to six ordinary vector instructions of the
+  // same wave issue behind it for free).
+  constexpr int N_QK = NSB * KSTEPS;        // slots of S^T = K Q^T
+  constexpr int N_PV = NSB * 2 * DB;        // slots of O^T += V^T P^T
+  constexpr int PF_K = 2, PF_V = 2;         // operand fragments read ahead of their MFMAs
   static_assert(NSB % 2 == 0 && N_QK > PF_K && N_PV > PF_V, "tile too small for the schedule");
 
   // QK slot s multiplies k-step s % KSTEPS of sub-block s / KSTEPS (a sub-block's logits only
@@ -460,34 +488,49 @@ fna_fwd_kernel(const FnaParams p) {
     return __builtin_bit_cast(vec8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
   };
 
-  f32x16_t S_a[NSB], S_b[NSB];  // logits of the current / coming tile, swapping roles every iteration
-  vec8 pf[NSB][2];
-  float msc = 0.f;              // running maximum in the exp2 domain (0 while it is -inf)
-  float psum0 = 0.f, psum1 = 0.f;
+  f32x16_t S_a[MQ][NSB], S_b[MQ][NSB];  // logits of the current / coming tile, swapping roles every iteration
+  vec8 pf[MQ][NSB][2];
+  float msc[MQ];                // running maxima in the exp2 domain (0 while -inf)
+  float psum[MQ][2];
 
-  // probabilities 2u, 2u+1 of the current tile: exp2(c*s - c*m), summed in float, rounded to T
-  auto exp_unit = [&](const f32x16_t (&S_cur)[NSB], int u) {
-    const int sb = u / 8, r = 2 * (u % 8);
-    const float e0 = fast_exp2(S_cur[sb][r] * c_log2 - msc);
-    const float e1 = fast_exp2(S_cur[sb][r + 1] * c_log2 - msc);
-    psum0 += e0;
-    psum1 += e1;
-    vec2 p2 = {static_cast<T>(e0), static_cast<T>(e1)};
-    uint32_t bits = __builtin_bit_cast(uint32_t, p2);
-    pin(bits);
-    p2 = __builtin_bit_cast(vec2, bits);
-    pf[sb][r / 8][r % 8] = p2[0];
-    pf[sb][r / 8][r % 8 + 1] = p2[1];
+  // Element e of the current tile's probabilities: row block e % MQ, logit v = e / MQ of the lane
+  // (sub-block v / 16, register v % 16): exp2(c*s - c*m), summed in float; every second
+  // element of a row block rounds its pair to T.
+  float held[MQ];
+  auto exp_elem = [&](const f32x16_t (&S_cur)[MQ][NSB], int e) {
+    const int mb = e % MQ, v = e / MQ;
+    const int sb = v / 16, r = v % 16;
+    float x = fast_exp2(S_cur[mb][sb][r] * c_log2 - msc[mb]);
+    psum[mb][r & 1] += x;
+    if (r % 2 == 0) {
+      pin(x);
+      held[mb] = x;
+    } else {
+      vec2 p2 = {static_cast<T>(held[mb]), static_cast<T>(x)};
+      uint32_t bits = __builtin_bit_cast(uint32_t, p2);
+      pin(bits);
+      p2 = __builtin_bit_cast(vec2, bits);
+      pf[mb][sb][r / 8][r % 8 - 1] = p2[0];
+      pf[mb][sb][r / 8][r % 8] = p2[1];
+    }
+  };
+  // Elements are spread evenly over the slots that precede the last 16-key block of O += P V
+  // (whose P fragment is the last to be completed): cumulative count after global slot x.
+  constexpr int N_ELEMS = MQ * NSB * 16;
+  constexpr int EXP_SLOTS = N_QK + N_PV - DB;
+  auto elems_done = [](int x) constexpr {
+    const int n = (N_ELEMS * (x + 1) + EXP_SLOTS - 1) / EXP_SLOTS;
+    return x < 0 ? 0 : (n > N_ELEMS ? N_ELEMS : n);
   };
 
-  // element mask of a PARTIAL tile
-  auto apply_mask = [&](f32x16_t (&S)[NSB], const int (&origin)[3]) {
+  // element mask of a PARTIAL tile for row block mb
+  auto apply_mask = [&](f32x16_t (&S)[NSB], const int (&ws)[3], const int (&we)[3], const int (&origin)[3]) {
     // window of this lane's query relative to the tile origin, clamped to the tile
     uint32_t addc = 0, subc = 0;
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
-      const int lo = na_min(na_max(wst[a] - origin[a], 0), p.kv_tile[a]);
-      const int hi = na_min(na_max(wen[a] - origin[a], 0), p.kv_tile[a]);
+      const int lo = na_min(na_max(ws[a] - origin[a], 0), p.kv_tile[a]);
+      const int hi = na_min(na_max(we[a] - origin[a], 0), p.kv_tile[a]);
       addc |= uint32_t(512 - lo) << (10 * a);
       subc |= uint32_t(511 + hi) << (10 * a);
     }
@@ -507,27 +550,43 @@ fna_fwd_kernel(const FnaParams p) {
 
   // adopts the maximum `mx` of the lane's half row of the coming tile: the running maximum is
   // only moved (and O, the row sum rescaled) when some row of the wave outgrew it by 2^8
-  auto update_max = [&](float mx) {
+  auto update_max = [&](int mb, float mx) {
     mx = cross_half_max(mx);
-    const bool grow = (mx - m_run) * c_log2 > kLazyRescaleLog2;  // also true while m_run == -inf and mx finite
+    const bool grow = (mx - m_run[mb]) * c_log2 > kLazyRescaleLog2;  // also true while m_run == -inf and mx finite
     if (__any(grow)) {
-      const float m_new = fmaxf(m_run, mx);
+      const float m_new = fmaxf(m_run[mb], mx);
       const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-      const float alpha = fast_exp2((m_run - m_use) * c_log2);  // m_run == -inf -> 0
-      m_run = m_new;
-      l_run *= alpha;
+      const float alpha = fast_exp2((m_run[mb] - m_use) * c_log2);  // m_run == -inf -> 0
+      m_run[mb] = m_new;
+      l_run[mb] *= alpha;
 #pragma unroll
       for (int db = 0; db < DB; ++db)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) acc[db][r] *= alpha;
+        for (int r = 0; r < 16; ++r) acc[mb][db][r] *= alpha;
     }
-    msc = ((m_run == -INFINITY) ? 0.f : m_run) * c_log2;
+    msc[mb] = ((m_run[mb] == -INFINITY) ? 0.f : m_run[mb]) * c_log2;
+  };
+  // masks (PARTIAL tiles) and maxima of a whole tile of logits, outside the slots
+  auto finish_logits = [&](f32x16_t (&S)[MQ][NSB], const bool t_full, const int (&t_origin)[3], bool have_max, const float (&mx_in)[MQ]) {
+#pragma unroll
+    for (int mb = 0; mb < MQ; ++mb) {
+      float mx = mx_in[mb];
+      if (!t_full || !have_max) {
+        if (!t_full) apply_mask(S[mb], wst[mb], wen[mb], t_origin);
+        mx = -INFINITY;
+#pragma unroll
+        for (int sb = 0; sb < NSB; ++sb)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) mx = fmaxf(mx, S[mb][sb][r]);
+      }
+      update_max(mb, mx);
+    }
   };
 
   // ---- software pipeline --------------------------------------------------------------------
-  // Iteration j: (G1) S(j+1) = K(j+1) Q^T with three quarters of the exponentials of S(j) and
-  // the asynchronous copies of K(j+2), V(j+1) in its shadow; (G2) first half of O += P(j) V(j)
-  // with the remaining exponentials; (G3) second half with the row maximum of S(j+1).
+  // Iteration j: (G1) the slots of S(j+1) = K(j+1) Q^T, with the asynchronous copies of K(j+2)
+  // and V(j+1); (G2, G3) the slots of O += P(j) V(j), the second half with the row maxima of
+  // S(j+1).  The exponentials of S(j) are spread evenly over all of them.
   // LDS: K(j) and V(j) live in stage j % 2.
   TileInfo nxt = next_tile();  // tile 1 (a descriptor past the box is never used)
   wait_vmcnt<0>();
@@ -535,25 +594,26 @@ fna_fwd_kernel(const FnaParams p) {
   if (1 < total_tiles) issue_tile_load(kbase, ld_koff, sK1, nxt.row0);
   {
 #pragma unroll
-    for (int sb = 0; sb < NSB; ++sb)
+    for (int mb = 0; mb < MQ; ++mb)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) S_a[sb][r] = 0.f;
+      for (int sb = 0; sb < NSB; ++sb)
 #pragma unroll
-    for (int s = 0; s < N_QK; ++s) S_a[s / KSTEPS] = M::run(k_frag(sK0, s), qf[s % KSTEPS], S_a[s / KSTEPS]);
-    if (!cur.full) apply_mask(S_a, cur.origin);
-    float mx = -INFINITY;
+        for (int r = 0; r < 16; ++r) S_a[mb][sb][r] = 0.f;
 #pragma unroll
-    for (int sb = 0; sb < NSB; ++sb)
+    for (int s = 0; s < N_QK; ++s) {
+      const vec8 kf = k_frag(sK0, s);
 #pragma unroll
-      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, S_a[sb][r]);
-    update_max(mx);
+      for (int mb = 0; mb < MQ; ++mb) S_a[mb][s / KSTEPS] = M::run(kf, qf[mb][s % KSTEPS], S_a[mb][s / KSTEPS]);
+    }
+    const float none[MQ] = {};
+    finish_logits(S_a, cur.full, cur.origin, false, none);
   }
 
   auto iteration = [&](auto stage_tag, int j) {
     constexpr int st = decltype(stage_tag)::value;
     constexpr bool SPREAD = !RAGGED;
-    f32x16_t (&S_cur)[NSB] = st ? S_b : S_a;
-    f32x16_t (&S_nxt)[NSB] = st ? S_a : S_b;
+    f32x16_t (&S_cur)[MQ][NSB] = st ? S_b : S_a;
+    f32x16_t (&S_nxt)[MQ][NSB] = st ? S_a : S_b;
     char* sK_cur = st ? sK1 : sK0;  // held K(j): free, receives K(j+2)
     char* sK_nxt = st ? sK0 : sK1;  // holds K(j+1)
     char* sV_cur = st ? sV1 : sV0;  // holds V(j)
@@ -575,33 +635,39 @@ fna_fwd_kernel(const FnaParams p) {
     vec8 kf[N_QK];
 #pragma unroll
     for (int s = 0; s < PF_K; ++s) kf[s] = k_frag(sK_nxt, s);
-    psum0 = 0.f;
-    psum1 = 0.f;
+#pragma unroll
+    for (int mb = 0; mb < MQ; ++mb) psum[mb][0] = psum[mb][1] = 0.f;
     auto g1_slot = [&](auto s_tag) {
       constexpr int s = decltype(s_tag)::value;
       if constexpr (s + PF_K < N_QK) kf[s + PF_K] = k_frag(sK_nxt, s + PF_K);
-      if constexpr (s % KSTEPS == 0) {
-        f32x16_t zero;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) zero[r] = 0.f;
-        S_nxt[s / KSTEPS] = M::run(kf[s], qf[s % KSTEPS], zero);
-      } else {
-        S_nxt[s / KSTEPS] = M::run(kf[s], qf[s % KSTEPS], S_nxt[s / KSTEPS]);
+      for (int mb = 0; mb < MQ; ++mb) {
+        if constexpr (s % KSTEPS == 0) {
+          f32x16_t zero;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) zero[r] = 0.f;
+          S_nxt[mb][s / KSTEPS] = M::run(kf[s], qf[mb][s % KSTEPS], zero);
+        } else {
+          S_nxt[mb][s / KSTEPS] = M::run(kf[s], qf[mb][s % KSTEPS], S_nxt[mb][s / KSTEPS]);
+        }
       }
-      constexpr int u_lo = (s * UNITS_G1) / N_QK, u_hi = ((s + 1) * UNITS_G1) / N_QK;
+      constexpr int e_lo = elems_done(s - 1), e_hi = elems_done(s);
 #pragma unroll
-      for (int u = u_lo; u < u_hi; ++u) exp_unit(S_cur, u);
-      if constexpr (u_hi > u_lo) {
-        pin(psum0);
-        pin(psum1);
+      for (int e = e_lo; e < e_hi; ++e) exp_elem(S_cur, e);
+      if constexpr (e_hi > e_lo) {
+#pragma unroll
+        for (int mb = 0; mb < MQ; ++mb) {
+          pin(psum[mb][0]);
+          pin(psum[mb][1]);
+        }
       }
       if constexpr (SPREAD) {
         // 2 * PER copies spread over the first half of the slots, K first
         constexpr int c_lo = (s * 2 * PER * 2) / N_QK, c_hi = ((s + 1) * 2 * PER * 2) / N_QK;
         for_range<c_lo, c_hi - c_lo>([&](auto c_tag) {
           constexpr int c = decltype(c_tag)::value;
-          if constexpr (c < PER) copy_one(std::integral_constant<int, c>{}, std::true_type{}, ck, ld_koff);
-          else if constexpr (c < 2 * PER) copy_one(std::integral_constant<int, c - PER>{}, std::true_type{}, cv, ld_voff);
+          if constexpr (c < PER) copy_one(std::integral_constant<int, c>{}, ck, ld_koff);
+          else if constexpr (c < 2 * PER) copy_one(std::integral_constant<int, c - PER>{}, cv, ld_voff);
         });
       }
       __builtin_amdgcn_sched_barrier(0);
@@ -612,50 +678,56 @@ fna_fwd_kernel(const FnaParams p) {
     vec8 vf[N_PV];
 #pragma unroll
     for (int t = 0; t < PF_V; ++t) vf[t] = v_frag(sV_cur, t);
-    float mx0 = -INFINITY, mx1 = -INFINITY;
+    float mx[MQ][2];
+#pragma unroll
+    for (int mb = 0; mb < MQ; ++mb) mx[mb][0] = mx[mb][1] = -INFINITY;
     auto pv_slot = [&](auto t_tag) {
       constexpr int t = decltype(t_tag)::value;
       if constexpr (t + PF_V < N_PV) vf[t + PF_V] = v_frag(sV_cur, t + PF_V);
-      acc[t % DB] = M::run(vf[t], pf[t / (2 * DB)][(t / DB) % 2], acc[t % DB]);
-      if constexpr (t < N_PV / 2) {
-        constexpr int u_lo = UNITS_G1 + (t * (N_UNITS - UNITS_G1)) / (N_PV / 2);
-        constexpr int u_hi = UNITS_G1 + ((t + 1) * (N_UNITS - UNITS_G1)) / (N_PV / 2);
 #pragma unroll
-        for (int u = u_lo; u < u_hi; ++u) exp_unit(S_cur, u);
-        if constexpr (u_hi > u_lo) {
-          pin(psum0);
-          pin(psum1);
+      for (int mb = 0; mb < MQ; ++mb)
+        acc[mb][t % DB] = M::run(vf[t], pf[mb][t / (2 * DB)][(t / DB) % 2], acc[mb][t % DB]);
+      // the P fragment of this slot's 16-key block is complete
+      static_assert(elems_done(N_QK + (t / DB) * DB - 1) >= MQ * 8 * (t / DB + 1), "exponentials scheduled too late");
+      constexpr int x_lo = elems_done(N_QK + t - 1), x_hi = elems_done(N_QK + t);
+#pragma unroll
+      for (int e = x_lo; e < x_hi; ++e) exp_elem(S_cur, e);
+      if constexpr (x_hi > x_lo) {
+#pragma unroll
+        for (int mb = 0; mb < MQ; ++mb) {
+          pin(psum[mb][0]);
+          pin(psum[mb][1]);
         }
-      } else {
-        // row maximum of the coming tile (as if unmasked), NSB * 16 values over N_PV / 2 slots
+      }
+      if constexpr (t >= N_PV / 2) {
+        // row maxima of the coming tile (as if unmasked), MQ * NSB * 16 values over N_PV / 2 slots
         constexpr int t3 = t - N_PV / 2;
-        constexpr int e_lo = (t3 * NSB * 16) / (N_PV / 2), e_hi = ((t3 + 1) * NSB * 16) / (N_PV / 2);
+        constexpr int NV = MQ * NSB * 16;
+        constexpr int e_lo = (t3 * NV) / (N_PV / 2), e_hi = ((t3 + 1) * NV) / (N_PV / 2);
 #pragma unroll
         for (int e = e_lo; e < e_hi; ++e) {
-          if (e % 2 == 0) mx0 = fmaxf(mx0, S_nxt[e / 16][e % 16]);
-          else mx1 = fmaxf(mx1, S_nxt[e / 16][e % 16]);
+          const int mb = e / (NSB * 16), i = e % (NSB * 16);
+          mx[mb][i % 2] = fmaxf(mx[mb][i % 2], S_nxt[mb][i / 16][i % 16]);
         }
         if constexpr (e_hi > e_lo) {
-          pin(mx0);
-          pin(mx1);
+#pragma unroll
+          for (int mb = 0; mb < MQ; ++mb) {
+            pin(mx[mb][0]);
+            pin(mx[mb][1]);
+          }
         }
       }
       __builtin_amdgcn_sched_barrier(0);
     };
     for_range<0, N_PV>(pv_slot);
-    l_run += psum0 + psum1;
+#pragma unroll
+    for (int mb = 0; mb < MQ; ++mb) l_run[mb] += psum[mb][0] + psum[mb][1];
 
     if (j + 1 < total_tiles) {
-      float mx = fmaxf(mx0, mx1);
-      if (!nxt.full) {
-        apply_mask(S_nxt, nxt.origin);
-        mx = -INFINITY;
+      float mxs[MQ];
 #pragma unroll
-        for (int sb = 0; sb < NSB; ++sb)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) mx = fmaxf(mx, S_nxt[sb][r]);
-      }
-      update_max(mx);
+      for (int mb = 0; mb < MQ; ++mb) mxs[mb] = fmaxf(mx[mb][0], mx[mb][1]);
+      finish_logits(S_nxt, nxt.full, nxt.origin, true, mxs);
     }
     cur = nxt;
     nxt = t2;
@@ -668,10 +740,11 @@ fna_fwd_kernel(const FnaParams p) {
 
   // ---- epilogue: O = acc / rowsum, LSE = ln(rowsum) + scale * rowmax -------------------------
   T* obase = reinterpret_cast<T*>(p.o) + int64_t(bg) * p.seqlen_q * q_row_stride + int64_t(head) * D;
-  {
-    const float l = l_run + __shfl_xor(l_run, 32);
+#pragma unroll
+  for (int mb = 0; mb < MQ; ++mb) {
+    const float l = l_run[mb] + __shfl_xor(l_run[mb], 32);
     const float inv = (l > 0.f) ? out_scale / l : 0.f;
-    const int row = qtile_idx * QT + wave * 32 + l32;
+    const int row = qtile_idx * QT + (wave * MQ + mb) * 32 + l32;
     if (row < p.seqlen_q) {
       T* orow = obase + int64_t(row) * q_row_stride;
 #pragma unroll
@@ -681,11 +754,11 @@ fna_fwd_kernel(const FnaParams p) {
           typedef T tx4 __attribute__((ext_vector_type(4)));
           tx4 o4;
 #pragma unroll
-          for (int i = 0; i < 4; ++i) o4[i] = static_cast<T>(acc[db][4 * j + i] * inv);
+          for (int i = 0; i < 4; ++i) o4[i] = static_cast<T>(acc[mb][db][4 * j + i] * inv);
           *reinterpret_cast<tx4*>(orow + db * 32 + 8 * j + 4 * g) = o4;
         }
       if (g == 0) {
-        const float lse = (l > 0.f) ? (m_run * sm_scale + __logf(l)) : -INFINITY;
+        const float lse = (l > 0.f) ? (m_run[mb] * sm_scale + __logf(l)) : -INFINITY;
         p.lse[(int64_t(bg) * p.seqlen_q + row) * p.heads_q + head] = lse;
       }
     }

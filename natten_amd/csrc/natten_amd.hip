@@ -61,13 +61,13 @@ struct TileConfig {
 };
 
 // (Q tile, KV tile) sizes in tokens that have a kernel instance.
-const TileConfig kTileConfigs[] = {{128, 64}, {256, 64}, {128, 128}, {64, 64}};
+const TileConfig kTileConfigs[] = {{128, 64}, {256, 64}, {64, 64}};
 constexpr int kNumTileConfigs = sizeof(kTileConfigs) / sizeof(kTileConfigs[0]);
 
-template <typename T, int D, int NWAVES, bool RAGGED, int KVT>
+template <typename T, int D, int NWAVES, int MQ, bool RAGGED, int KVT>
 int launch_fna(const FnaParams& p, hipStream_t stream) {
-  constexpr int QT = NWAVES * 32;
-  auto kernel = fna_fwd_kernel<T, D, NWAVES, RAGGED, KVT>;
+  constexpr int QT = NWAVES * MQ * 32;
+  auto kernel = fna_fwd_kernel<T, D, NWAVES, MQ, RAGGED, KVT>;
   if ((p.seqlen_q + QT - 1) / QT != p.num_q_tiles) return fail("fna_forward: internal tile count mismatch");
   const long long wgs = (long long)((p.total_groups + kNumXcd - 1) / kNumXcd) * kNumXcd * p.wg_group;
   if (wgs > 0x7fffffffLL) return fail("fna_forward: problem needs more than 2^31 workgroups");
@@ -79,13 +79,12 @@ template <typename T, int D>
 int dispatch_tiles(const FnaParams& p, int qt, int kvt, hipStream_t stream) {
   if (p.seqlen_kv % kvt != 0) {
     // key sequences that end inside a tile: dense attention on unpadded sequences only
-    if (qt == 128 && kvt == 64) return launch_fna<T, D, 4, true, 64>(p, stream);
+    if (qt == 128 && kvt == 64) return launch_fna<T, D, 4, 1, true, 64>(p, stream);
     return fail("fna_forward: seqlen_kv (%d) must be a multiple of the KV tile (%d tokens)", p.seqlen_kv, kvt);
   }
-  if (qt == 128 && kvt == 64) return launch_fna<T, D, 4, false, 64>(p, stream);
-  if (qt == 256 && kvt == 64) return launch_fna<T, D, 8, false, 64>(p, stream);
-  if (qt == 128 && kvt == 128) return launch_fna<T, D, 4, false, 128>(p, stream);
-  if (qt == 64 && kvt == 64) return launch_fna<T, D, 2, false, 64>(p, stream);
+  if (qt == 128 && kvt == 64) return launch_fna<T, D, 4, 1, false, 64>(p, stream);
+  if (qt == 256 && kvt == 64) return launch_fna<T, D, 8, 1, false, 64>(p, stream);
+  if (qt == 64 && kvt == 64) return launch_fna<T, D, 2, 1, false, 64>(p, stream);
   return fail("fna_forward: no kernel for Q tile of %d and KV tile of %d tokens", qt, kvt);
 }
 

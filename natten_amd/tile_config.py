@@ -19,7 +19,7 @@ import torch
 DimensionType = Tuple[int, ...]
 
 # (Q tile tokens, KV tile tokens) with a kernel instance; first entry = default.
-TILE_SIZES: List[Tuple[int, int]] = [(128, 64), (256, 64), (128, 128), (64, 64)]
+TILE_SIZES: List[Tuple[int, int]] = [(128, 64), (256, 64), (64, 64)]
 SUPPORTED_HEAD_DIMS = (32, 64, 128)
 
 

@@ -48,7 +48,7 @@ def test_head_dims_and_dtypes_2d(D, dtype):
     run_case(1, 2, 2, D, (20, 24), (5, 7), (2, 1), (1, 2), (False, True), dtype)
 
 
-@pytest.mark.parametrize("sizes", [(128, 64), (256, 64), (128, 128), (64, 64)])
+@pytest.mark.parametrize("sizes", [(128, 64), (256, 64), (64, 64)])
 def test_every_tile_size_3d(sizes):
     qt = {128: (2, 8, 8), 256: (4, 8, 8), 64: (1, 8, 8)}[sizes[0]]
     kt = {64: (1, 8, 8), 128: (2, 8, 8)}[sizes[1]]
