@@ -251,7 +251,7 @@ fna_fwd_kernel(const FnaParams p) {
   // ---- workgroup-uniform setup: dilation group, Q tile origin, KV tile box -------------------
   // qtile_rm enumerates Q tiles with dimension 0 slowest; causal dimension 0 is walked from
   // the far end so that the Q tiles with the longest KV loops start first.
-  int extent[3], q_first[3], box_tile0[3], box_n[3], full_lo[3], full_hi[3];
+  int extent[3], q_first[3], box_tile0[3], box_n[3];
   int qtile_idx;  // position of the tile in the permuted sequence (dimension 0 fastest)
   {
     int gl = bg % p.num_groups;
@@ -272,16 +272,56 @@ fna_fwd_kernel(const FnaParams p) {
       const int qf = q_first[a], ql = qf + p.q_tile[a] - 1;
       const bool c = p.causal[a] != 0;
       const int st_f = na_window_start(qf, p.ksize[a], p.stride[a], extent[a], c);
-      const int en_f = na_window_end(qf, st_f, p.ksize[a], extent[a], c);
       const int st_l = na_window_start(ql, p.ksize[a], p.stride[a], extent[a], c);
       const int en_l = na_window_end(ql, st_l, p.ksize[a], extent[a], c);
       box_tile0[a] = st_f / p.kv_tile[a];
       box_n[a] = na_ceil_div(en_l, p.kv_tile[a]) - box_tile0[a];
-      full_lo[a] = st_l;  // intersection of the tile's windows: [start(last), end(first))
-      full_hi[a] = en_f;
     }
   }
   const int total_tiles = box_n[0] * box_n[1] * box_n[2];
+
+  // ---- this wave's share of the Q tile ------------------------------------------------------------
+  // Lanes take the tile's tokens in row-major order (dimension 0 slowest), MQ * 32 consecutive
+  // ones per wave, so that a wave covers a compact box of queries; the token's row inside the
+  // permuted tile (dimension 0 fastest) follows from its coordinates.  Window starts and ends
+  // are monotone in the query coordinate, hence over the wave's bounding box the union of the
+  // windows is [start(min), end(max)) and their intersection [start(max), end(min)) per
+  // dimension: a KV tile outside the union is skipped by this wave, one inside the
+  // intersection needs no mask.
+  int wave_lo[3], wave_hi[3], wave_full_lo[3], wave_full_hi[3];
+  {
+    const int i0 = wave * (MQ * 32), i1 = i0 + MQ * 32 - 1;
+    const int t12 = p.q_tile[1] * p.q_tile[2];
+    int f[3], l[3];
+    f[0] = i0 / t12;
+    f[1] = (i0 / p.q_tile[2]) % p.q_tile[1];
+    f[2] = i0 % p.q_tile[2];
+    l[0] = i1 / t12;
+    l[1] = (i1 / p.q_tile[2]) % p.q_tile[1];
+    l[2] = i1 % p.q_tile[2];
+    if (f[0] != l[0]) {
+      f[1] = 0;
+      l[1] = p.q_tile[1] - 1;
+    }
+    if (f[0] != l[0] || f[1] != l[1]) {
+      f[2] = 0;
+      l[2] = p.q_tile[2] - 1;
+    }
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+      // rows past the end of an unpadded sequence (dense attention) are clamped like the loads
+      const int qmin = q_first[a] + f[a], qmax = q_first[a] + na_min(l[a], p.q_tile[a] - 1);
+      const bool c = p.causal[a] != 0;
+      const int st_min = na_window_start(qmin, p.ksize[a], p.stride[a], extent[a], c);
+      const int en_min = na_window_end(qmin, st_min, p.ksize[a], extent[a], c);
+      const int st_max = na_window_start(qmax, p.ksize[a], p.stride[a], extent[a], c);
+      const int en_max = na_window_end(qmax, st_max, p.ksize[a], extent[a], c);
+      wave_lo[a] = st_min;
+      wave_hi[a] = en_max;
+      wave_full_lo[a] = st_max;
+      wave_full_hi[a] = en_min;
+    }
+  }
 
   // in-tile coordinates of every KV position, packed in 10-bit fields
   for (int i = tid; i < KVT; i += NT) {
@@ -382,16 +422,20 @@ fna_fwd_kernel(const FnaParams p) {
   struct TileInfo {
     int row0;       // first row of the tile in the permuted KV sequence
     int origin[3];  // coordinate of its first token
-    bool full;      // every key of the tile is attended by every query of this Q tile
+    bool full;      // every key of the tile is attended by every query of this wave
+    bool skip;      // no key of the tile is attended by any query of this wave
   };
   int itc[3] = {0, 0, 0};
   auto next_tile = [&]() {
     TileInfo t;
     t.full = true;
+    t.skip = false;
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
       t.origin[a] = (box_tile0[a] + itc[a]) * p.kv_tile[a];
-      t.full = t.full && (t.origin[a] >= full_lo[a]) && (t.origin[a] + p.kv_tile[a] <= full_hi[a]);
+      const int end = t.origin[a] + p.kv_tile[a];
+      t.full = t.full && (t.origin[a] >= wave_full_lo[a]) && (end <= wave_full_hi[a]);
+      t.skip = t.skip || (end <= wave_lo[a]) || (t.origin[a] >= wave_hi[a]);
     }
     t.row0 = ((box_tile0[0] + itc[0]) + p.kv_tiled[0] * ((box_tile0[1] + itc[1]) + p.kv_tiled[1] * (box_tile0[2] + itc[2]))) * KVT;
     if (++itc[2] == box_n[2]) {
@@ -412,16 +456,18 @@ fna_fwd_kernel(const FnaParams p) {
 
   // ---- per-lane setup: this lane's query rows, their windows, Q fragments ---------------------
   int wst[MQ][3], wen[MQ][3];
+  int tile_row[MQ];  // this lane's row inside the permuted Q tile, per row block
   vec8 qf[MQ][KSTEPS];
 #pragma unroll
   for (int mb = 0; mb < MQ; ++mb) {
-    int r = (wave * MQ + mb) * 32 + l32;
-    const int row = qtile_idx * QT + r;
+    int r = (wave * MQ + mb) * 32 + l32;  // row-major index inside the tile
     int off[3];
-    off[0] = r % p.q_tile[0];
-    r /= p.q_tile[0];
+    off[2] = r % p.q_tile[2];
+    r /= p.q_tile[2];
     off[1] = r % p.q_tile[1];
-    off[2] = r / p.q_tile[1];
+    off[0] = r / p.q_tile[1];
+    tile_row[mb] = off[0] + p.q_tile[0] * (off[1] + p.q_tile[1] * off[2]);
+    const int row = qtile_idx * QT + tile_row[mb];
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
       const int c = q_first[a] + off[a];
@@ -567,11 +613,18 @@ fna_fwd_kernel(const FnaParams p) {
     msc[mb] = ((m_run[mb] == -INFINITY) ? 0.f : m_run[mb]) * c_log2;
   };
   // masks (PARTIAL tiles) and maxima of a whole tile of logits, outside the slots
-  auto finish_logits = [&](f32x16_t (&S)[MQ][NSB], const bool t_full, const int (&t_origin)[3], bool have_max, const float (&mx_in)[MQ]) {
+  auto finish_logits = [&](f32x16_t (&S)[MQ][NSB], const bool t_full, const bool t_skip, const int (&t_origin)[3], bool have_max, const float (&mx_in)[MQ]) {
 #pragma unroll
     for (int mb = 0; mb < MQ; ++mb) {
       float mx = mx_in[mb];
-      if (!t_full || !have_max) {
+      if (t_skip) {
+        // none of this wave's queries attends the tile: every logit is masked
+        mx = -INFINITY;
+#pragma unroll
+        for (int sb = 0; sb < NSB; ++sb)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) S[mb][sb][r] = -INFINITY;
+      } else if (!t_full || !have_max) {
         if (!t_full) apply_mask(S[mb], wst[mb], wen[mb], t_origin);
         mx = -INFINITY;
 #pragma unroll
@@ -592,6 +645,8 @@ fna_fwd_kernel(const FnaParams p) {
   wait_vmcnt<0>();
   __syncthreads();  // K(0), V(0) and the coordinate table are in LDS
   if (1 < total_tiles) issue_tile_load(kbase, ld_koff, sK1, nxt.row0);
+#pragma unroll
+  for (int mb = 0; mb < MQ; ++mb) msc[mb] = 0.f;
   {
 #pragma unroll
     for (int mb = 0; mb < MQ; ++mb)
@@ -606,11 +661,14 @@ fna_fwd_kernel(const FnaParams p) {
       for (int mb = 0; mb < MQ; ++mb) S_a[mb][s / KSTEPS] = M::run(kf, qf[mb][s % KSTEPS], S_a[mb][s / KSTEPS]);
     }
     const float none[MQ] = {};
-    finish_logits(S_a, cur.full, cur.origin, false, none);
+    finish_logits(S_a, cur.full, cur.skip, cur.origin, false, none);
   }
 
-  auto iteration = [&](auto stage_tag, int j) {
+  // CUR / NXT: this wave attends keys of tile j / tile j + 1; an inactive tile only takes part
+  // in the copies and the barrier.
+  auto iteration = [&](auto stage_tag, auto cur_tag, auto nxt_tag, int j) __attribute__((always_inline)) {
     constexpr int st = decltype(stage_tag)::value;
+    constexpr bool CUR = decltype(cur_tag)::value, NXT = decltype(nxt_tag)::value;
     constexpr bool SPREAD = !RAGGED;
     f32x16_t (&S_cur)[MQ][NSB] = st ? S_b : S_a;
     f32x16_t (&S_nxt)[MQ][NSB] = st ? S_a : S_b;
@@ -633,28 +691,32 @@ fna_fwd_kernel(const FnaParams p) {
 
     // -- G1 ------------------------------------------------------------------------------------
     vec8 kf[N_QK];
+    if constexpr (NXT) {
 #pragma unroll
-    for (int s = 0; s < PF_K; ++s) kf[s] = k_frag(sK_nxt, s);
+      for (int s = 0; s < PF_K; ++s) kf[s] = k_frag(sK_nxt, s);
+    }
 #pragma unroll
     for (int mb = 0; mb < MQ; ++mb) psum[mb][0] = psum[mb][1] = 0.f;
-    auto g1_slot = [&](auto s_tag) {
+    auto g1_slot = [&](auto s_tag) __attribute__((always_inline)) {
       constexpr int s = decltype(s_tag)::value;
-      if constexpr (s + PF_K < N_QK) kf[s + PF_K] = k_frag(sK_nxt, s + PF_K);
+      if constexpr (NXT) {
+        if constexpr (s + PF_K < N_QK) kf[s + PF_K] = k_frag(sK_nxt, s + PF_K);
 #pragma unroll
-      for (int mb = 0; mb < MQ; ++mb) {
-        if constexpr (s % KSTEPS == 0) {
-          f32x16_t zero;
+        for (int mb = 0; mb < MQ; ++mb) {
+          if constexpr (s % KSTEPS == 0) {
+            f32x16_t zero;
 #pragma unroll
-          for (int r = 0; r < 16; ++r) zero[r] = 0.f;
-          S_nxt[mb][s / KSTEPS] = M::run(kf[s], qf[mb][s % KSTEPS], zero);
-        } else {
-          S_nxt[mb][s / KSTEPS] = M::run(kf[s], qf[mb][s % KSTEPS], S_nxt[mb][s / KSTEPS]);
+            for (int r = 0; r < 16; ++r) zero[r] = 0.f;
+            S_nxt[mb][s / KSTEPS] = M::run(kf[s], qf[mb][s % KSTEPS], zero);
+          } else {
+            S_nxt[mb][s / KSTEPS] = M::run(kf[s], qf[mb][s % KSTEPS], S_nxt[mb][s / KSTEPS]);
+          }
         }
       }
       constexpr int e_lo = elems_done(s - 1), e_hi = elems_done(s);
+      if constexpr (CUR && e_hi > e_lo) {
 #pragma unroll
-      for (int e = e_lo; e < e_hi; ++e) exp_elem(S_cur, e);
-      if constexpr (e_hi > e_lo) {
+        for (int e = e_lo; e < e_hi; ++e) exp_elem(S_cur, e);
 #pragma unroll
         for (int mb = 0; mb < MQ; ++mb) {
           pin(psum[mb][0]);
@@ -676,30 +738,34 @@ fna_fwd_kernel(const FnaParams p) {
 
     // -- G2 / G3 -------------------------------------------------------------------------------
     vec8 vf[N_PV];
+    if constexpr (CUR) {
 #pragma unroll
-    for (int t = 0; t < PF_V; ++t) vf[t] = v_frag(sV_cur, t);
+      for (int t = 0; t < PF_V; ++t) vf[t] = v_frag(sV_cur, t);
+    }
     float mx[MQ][2];
 #pragma unroll
     for (int mb = 0; mb < MQ; ++mb) mx[mb][0] = mx[mb][1] = -INFINITY;
-    auto pv_slot = [&](auto t_tag) {
+    auto pv_slot = [&](auto t_tag) __attribute__((always_inline)) {
       constexpr int t = decltype(t_tag)::value;
-      if constexpr (t + PF_V < N_PV) vf[t + PF_V] = v_frag(sV_cur, t + PF_V);
-#pragma unroll
-      for (int mb = 0; mb < MQ; ++mb)
-        acc[mb][t % DB] = M::run(vf[t], pf[mb][t / (2 * DB)][(t / DB) % 2], acc[mb][t % DB]);
       // the P fragment of this slot's 16-key block is complete
       static_assert(elems_done(N_QK + (t / DB) * DB - 1) >= MQ * 8 * (t / DB + 1), "exponentials scheduled too late");
       constexpr int x_lo = elems_done(N_QK + t - 1), x_hi = elems_done(N_QK + t);
+      if constexpr (CUR) {
+        if constexpr (t + PF_V < N_PV) vf[t + PF_V] = v_frag(sV_cur, t + PF_V);
 #pragma unroll
-      for (int e = x_lo; e < x_hi; ++e) exp_elem(S_cur, e);
-      if constexpr (x_hi > x_lo) {
+        for (int mb = 0; mb < MQ; ++mb)
+          acc[mb][t % DB] = M::run(vf[t], pf[mb][t / (2 * DB)][(t / DB) % 2], acc[mb][t % DB]);
+        if constexpr (x_hi > x_lo) {
 #pragma unroll
-        for (int mb = 0; mb < MQ; ++mb) {
-          pin(psum[mb][0]);
-          pin(psum[mb][1]);
+          for (int e = x_lo; e < x_hi; ++e) exp_elem(S_cur, e);
+#pragma unroll
+          for (int mb = 0; mb < MQ; ++mb) {
+            pin(psum[mb][0]);
+            pin(psum[mb][1]);
+          }
         }
       }
-      if constexpr (t >= N_PV / 2) {
+      if constexpr (NXT && t >= N_PV / 2) {
         // row maxima of the coming tile (as if unmasked), MQ * NSB * 16 values over N_PV / 2 slots
         constexpr int t3 = t - N_PV / 2;
         constexpr int NV = MQ * NSB * 16;
@@ -719,22 +785,27 @@ fna_fwd_kernel(const FnaParams p) {
       }
       __builtin_amdgcn_sched_barrier(0);
     };
-    for_range<0, N_PV>(pv_slot);
+    if constexpr (CUR || NXT) for_range<0, N_PV>(pv_slot);
+    if constexpr (CUR) {
 #pragma unroll
-    for (int mb = 0; mb < MQ; ++mb) l_run[mb] += psum[mb][0] + psum[mb][1];
+      for (int mb = 0; mb < MQ; ++mb) l_run[mb] += psum[mb][0] + psum[mb][1];
+    }
 
-    if (j + 1 < total_tiles) {
+    if (NXT && j + 1 < total_tiles) {
       float mxs[MQ];
 #pragma unroll
       for (int mb = 0; mb < MQ; ++mb) mxs[mb] = fmaxf(mx[mb][0], mx[mb][1]);
-      finish_logits(S_nxt, nxt.full, nxt.origin, true, mxs);
+      finish_logits(S_nxt, nxt.full, nxt.skip, nxt.origin, true, mxs);
     }
     cur = nxt;
     nxt = t2;
   };
+  // A tile this wave has no use for (skip) is still multiplied and then masked entirely:
+  // choosing the CUR / NXT variants per iteration at run time costs more registers than the
+  // kernel has (the compiler no longer keeps the logits of both stages in place).
   for (int j = 0; j < total_tiles; j += 2) {
-    iteration(Stage0{}, j);
-    if (j + 1 < total_tiles) iteration(Stage1{}, j + 1);
+    iteration(Stage0{}, std::true_type{}, std::true_type{}, j);
+    if (j + 1 < total_tiles) iteration(Stage1{}, std::true_type{}, std::true_type{}, j + 1);
   }
   wait_vmcnt<0>();  // the last iterations' copies into the unused stage must land before the LDS is released
 
@@ -744,7 +815,7 @@ fna_fwd_kernel(const FnaParams p) {
   for (int mb = 0; mb < MQ; ++mb) {
     const float l = l_run[mb] + __shfl_xor(l_run[mb], 32);
     const float inv = (l > 0.f) ? out_scale / l : 0.f;
-    const int row = qtile_idx * QT + (wave * MQ + mb) * 32 + l32;
+    const int row = qtile_idx * QT + tile_row[mb];
     if (row < p.seqlen_q) {
       T* orow = obase + int64_t(row) * q_row_stride;
 #pragma unroll
