@@ -34,7 +34,7 @@ WORKLOADS = {
 # and calibrated on the permute kernel (a copy of known size); see profiles/fna_fwd_c4_na3d_bf16.md.
 # Keyed by (workload, q_tile_shape, kv_tile_shape); other combinations report null.
 MEASURED_TRAFFIC_BYTES = {
-    ("c4", (2, 8, 8), (1, 8, 8)): 2.77e10,
+    ("c4", (2, 8, 8), (1, 8, 8)): 2.84e10,
 }
 
 WORKLOAD_NAMES = {
@@ -122,6 +122,7 @@ def main():
     ap.add_argument("--q-tile", type=str, default=None, help="comma separated, e.g. 2,8,8")
     ap.add_argument("--kv-tile", type=str, default=None)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-mfma-probe", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU; --gpus above 1 is not supported (no multi-GPU path).",
@@ -237,6 +238,16 @@ def main():
             "algorithmic_bytes": 4 * q_bytes + lse.numel() * 4,
         },
     }
+    if not args.no_mfma_probe:
+        # context for roofline.frac: what the matrix cores sustain on random operands under the
+        # chip's power limit (the published peak assumes the maximum clock)
+        rnd_tflops, rnd_ghz = _lib.mfma_probe(random_operands=True)
+        const_tflops, const_ghz = _lib.mfma_probe(random_operands=False)
+        result["mfma_probe"] = {
+            "instruction": "v_mfma_f32_32x32x16_bf16, one wave per SIMD, nothing else",
+            "random_operands": {"TFLOP/s": rnd_tflops, "shader_clock_GHz": rnd_ghz},
+            "constant_operands": {"TFLOP/s": const_tflops, "shader_clock_GHz": const_ghz},
+        }
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(q, k, v, kernel, stride, dilation, causal, out, lse)
     print(json.dumps(result), flush=True)

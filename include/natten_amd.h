@@ -135,6 +135,20 @@ int natten_amd_merge_attentions(const void* o0, const float* lse0, const void* o
                                 const float* lse1, void* out, float* lse_out, int dtype,
                                 int64_t rows, int head_dim, void* stream);
 
+/*
+ * Diagnostic without a counterpart in the reference: sustained rate of the bf16 matrix
+ * instruction the fused kernel is built on.  256 workgroups of 256 threads (one wave per SIMD
+ * of an MI355X) each run `iters` x 16 v_mfma_f32_32x32x16_bf16 (interleaved with `fma_per_mfma`
+ * = 0 or 4 independent v_fma_f32 each) on operands read once from `operands`.
+ *   operands: 256 * 256 * 128 bytes of bf16 values (random values show the rate the power
+ *             limit allows; constant ones the rate at the highest clock)
+ *   sink:     256 * 256 floats, written
+ *   clocks:   2 * 256 uint64, written: per workgroup, shader cycles and 100 MHz ticks spent
+ * Work per launch: 256 * 4 * iters * 16 * 32768 FLOP; time it on the stream.
+ */
+int natten_amd_mfma_probe(const void* operands, float* sink, uint64_t* clocks, int iters,
+                          int fma_per_mfma, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

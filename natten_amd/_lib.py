@@ -56,6 +56,10 @@ _SIGNATURES = {
         ctypes.c_int,
         [ctypes.c_void_p] * 2 + [ctypes.c_int] * 5 + [ctypes.c_void_p] * 3 + [ctypes.c_int, ctypes.c_void_p],
     ),
+    "natten_amd_mfma_probe": (
+        ctypes.c_int,
+        [ctypes.c_void_p] * 3 + [ctypes.c_int] * 2 + [ctypes.c_void_p],
+    ),
     "natten_amd_token_permute": (
         ctypes.c_int,
         [ctypes.c_void_p] * 2 + [ctypes.c_int] * 5 + [ctypes.c_void_p] * 3 + [ctypes.c_int, ctypes.c_void_p],
@@ -286,3 +290,35 @@ def merge_two(o0: Tensor, lse0: Tensor, o1: Tensor, lse1: Tensor) -> Tuple[Tenso
         )
     _check(rc)
     return out, lse
+
+
+def mfma_probe(random_operands: bool = True, iters: int = 20000, fma_per_mfma: int = 0, device="cuda:0"):
+    """Sustained bf16 MFMA rate of the device: returns (TFLOP/s, shader clock in GHz)."""
+    L = lib()
+    dev = torch.device(device)
+    n = 256 * 256 * 64  # bf16 values
+    if random_operands:
+        gen = torch.Generator().manual_seed(0)
+        ops = torch.randn(n, generator=gen).to(torch.bfloat16).to(dev)
+    else:
+        ops = torch.full((n,), 0.25, dtype=torch.bfloat16, device=dev)
+    sink = torch.empty(256 * 256, dtype=torch.float32, device=dev)
+    clocks = torch.zeros(2 * 256, dtype=torch.int64, device=dev)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+
+    def launch(k):
+        with torch.cuda.device(dev):
+            _check(L.natten_amd_mfma_probe(ops.data_ptr(), sink.data_ptr(), clocks.data_ptr(), k, fma_per_mfma,
+                                           torch.cuda.current_stream(dev).cuda_stream))
+
+    launch(max(iters // 20, 1))
+    torch.cuda.synchronize(dev)
+    e0.record()
+    launch(iters)
+    e1.record()
+    torch.cuda.synchronize(dev)
+    ms = e0.elapsed_time(e1)
+    c = clocks.cpu().view(256, 2).double()
+    ghz = float(c[:, 0].sum() / (c[:, 1].sum() * 10.0))
+    flops = 256.0 * 4 * iters * 16 * 32768
+    return flops / ms / 1e9, ghz

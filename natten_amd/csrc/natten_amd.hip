@@ -13,6 +13,7 @@
 
 #include "fna_fwd.hpp"
 #include "merge.hpp"
+#include "mfma_probe.hpp"
 #include "na_math.hpp"
 #include "tokperm.hpp"
 
@@ -390,6 +391,26 @@ int natten_amd_merge_attentions(const void* o0, const float* lse0, const void* o
       return fail("merge_attentions: unsupported dtype code %d", dtype);
   }
   return check_launch("merge_attentions");
+}
+
+int natten_amd_mfma_probe(const void* operands, float* sink, uint64_t* clocks, int iters, int fma_per_mfma,
+                          void* stream) {
+  g_error[0] = 0;
+  if (!operands || !sink || !clocks) return fail("mfma_probe: null pointer argument");
+  if (iters < 1) return fail("mfma_probe: iters must be positive");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  unsigned long long* c = reinterpret_cast<unsigned long long*>(clocks);
+  switch (fma_per_mfma) {
+    case 0:
+      hipLaunchKernelGGL(mfma_probe_kernel<0>, dim3(kProbeBlocks), dim3(kProbeThreads), 0, s, operands, sink, c, iters);
+      break;
+    case 4:
+      hipLaunchKernelGGL(mfma_probe_kernel<4>, dim3(kProbeBlocks), dim3(kProbeThreads), 0, s, operands, sink, c, iters);
+      break;
+    default:
+      return fail("mfma_probe: fma_per_mfma must be 0 or 4, got %d", fma_per_mfma);
+  }
+  return check_launch("mfma_probe");
 }
 
 }  // extern "C"
