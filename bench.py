@@ -2,8 +2,9 @@
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c4|c3|c2|c2d]
 
-One step = one na3d/na2d forward (token permute of Q/K/V, fused kernel, unpermute of O and LSE)
-on inputs already resident in HBM.  Prints ONE JSON line: whole-path throughput in effective
+One step = one na3d/na2d forward through the public API on inputs already resident in HBM:
+a single launch that gathers its tiles from the original tensors when the problem allows it
+(all benchmark workloads do), else token permute of Q/K/V, kernel, unpermute of O and LSE.  Prints ONE JSON line: whole-path throughput in effective
 NA TFLOP/s (4 * B * H * D * sum_q |window(q)| per step), the fused kernel's roofline figures from
 HIP-event timing of kernel-only launches, and a CPU baseline (the C oracle on a bounded sample
 of the same workload's queries, timed on this box's host cores).
@@ -173,9 +174,17 @@ def main():
         vp, _, _ = token_permute_operation(v, kv_tile, dilation)
         scale = D**-0.5
 
-        def kern():
+        fused = _lib.fused_layout_supported(layout, dilation, kv_tile)
+
+        def kern_permuted():
             return _lib.fna_forward(qp, kp, vp, kernel, stride, dilation, causal, scale, q_shape, kv_shape,
                                     qkv_shape, q_tile, kv_tile)
+
+        def kern():
+            # the launch the step above makes
+            if fused:
+                return _lib.fna_forward_fused(q, k, v, kernel, stride, dilation, causal, scale, q_tile, kv_tile)
+            return kern_permuted()
 
         def timed(fn, iters):
             for _ in range(3):
@@ -191,7 +200,8 @@ def main():
             return e0.elapsed_time(e1) / iters
 
         kernel_ms = timed(kern, args.steps)
-        op, lp = kern()
+        kernel_permuted_ms = timed(kern_permuted, args.steps)
+        op, lp = kern_permuted()
         perm_ms = timed(lambda: token_permute_operation(q, q_tile, dilation), args.steps)
         unperm_ms = timed(lambda: token_unpermute_operation(op, qkv_shape, q_tile, dilation), args.steps)
     q_bytes = q.numel() * q.element_size()
@@ -216,11 +226,13 @@ def main():
             "workload": WORKLOAD_NAMES[args.workload],
             "q_tile_shape": list(q_tile),
             "kv_tile_shape": list(kv_tile),
-            "path": "token permute (Q,K,V) + fused FNA kernel + token unpermute (O, LSE)",
+            "path": ("one launch: fused FNA kernel gathering tiles from the original tensors" if fused else
+                     "token permute (Q,K,V) + fused FNA kernel + token unpermute (O, LSE)"),
         },
         "na_flop_per_step": flops,
         "dense_over_na_flop": dense_flops / flops,
         "kernel_ms": kernel_ms,
+        "kernel_on_permuted_operands_ms": kernel_permuted_ms,
         "token_permute": {
             "permute_q_ms": perm_ms,
             "unpermute_o_ms": unperm_ms,

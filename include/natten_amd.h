@@ -11,6 +11,8 @@
  *
  *   natten_amd_fna_forward      <- blackwell_na{1,2,3}d_forward
  *                                  csrc/include/natten/blackwell_fna.h:36-52, csrc/natten.cpp:39-160
+ *   natten_amd_fna_forward_fused<- the reference driver's permute + kernel + unpermute sequence,
+ *                                  src/natten/backends/blackwell_fna.py:99-164, in one launch
  *   natten_amd_token_permute    <- token_permute_{1,2,3}d   csrc/include/natten/token_permute.h:34-52
  *   natten_amd_token_permute_widen <- the same, for e4m3 / e5m2 operands (writes bf16)
  *   natten_amd_token_unpermute  <- token_unpermute_{1,2,3}d csrc/include/natten/token_permute.h:54-74
@@ -74,6 +76,26 @@ int natten_amd_fna_forward(const void* q, const void* k, const void* v, void* ou
                            const int32_t* q_tile_shape, const int32_t* kv_tile_shape, float scale,
                            const float* q_scale, const float* k_scale, const float* v_scale,
                            void* stream);
+
+/*
+ * The same function in one launch on the ORIGINAL tensors: q [batch, *qkv_shape, heads_q,
+ * head_dim], k / v [batch, *qkv_shape, heads_kv, head_dim], out like q, lse [batch, *qkv_shape,
+ * heads_q].  The kernel gathers the rows of each tile from the input and scatters its results,
+ * so the three token permutes and two unpermutes around natten_amd_fna_forward (what the
+ * reference's driver runs as separate operations, src/natten/backends/blackwell_fna.py:99-164)
+ * disappear; results are bit-identical to the permuted path with the same tile shapes.
+ * Requires qkv_shape[a] to be a multiple of dilation[a] * kv_tile_shape[a] in every dimension
+ * (no KV tile may reach past the input); returns an error otherwise, and the caller uses the
+ * permuted path.  dtype, tiles, head_dim and scales as in natten_amd_fna_forward.
+ */
+int natten_amd_fna_forward_fused(const void* q, const void* k, const void* v, void* out,
+                                 float* lse, int dtype, int na_dim, int batch, int heads_q,
+                                 int heads_kv, int head_dim, const int32_t* qkv_shape,
+                                 const int32_t* kernel_size, const int32_t* stride,
+                                 const int32_t* dilation, const int32_t* is_causal,
+                                 const int32_t* q_tile_shape, const int32_t* kv_tile_shape,
+                                 float scale, const float* q_scale, const float* k_scale,
+                                 const float* v_scale, void* stream);
 
 /*
  * Supported tile sizes (tokens per tile).  Writes up to `capacity` pairs

@@ -48,6 +48,10 @@ _SIGNATURES = {
         + [ctypes.c_float]
         + [ctypes.c_void_p] * 4,
     ),
+    "natten_amd_fna_forward_fused": (
+        ctypes.c_int,
+        [ctypes.c_void_p] * 5 + [ctypes.c_int] * 6 + [ctypes.c_void_p] * 7 + [ctypes.c_float] + [ctypes.c_void_p] * 4,
+    ),
     "natten_amd_attention_forward": (
         ctypes.c_int,
         [ctypes.c_void_p] * 5 + [ctypes.c_int] * 8 + [ctypes.c_float] + [ctypes.c_void_p] * 4,
@@ -180,6 +184,38 @@ def fna_forward(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
             DTYPE_CODES[q.dtype], na_dim, q.shape[0], q.shape[1], k.shape[1], q.shape[2], k.shape[2], q.shape[3],
             _i32(q_shape), _i32(kv_shape), _i32(qkv_shape), _i32(kernel_size), _i32(stride), _i32(dilation),
+            _i32([1 if c else 0 for c in is_causal]), _i32(q_tile_shape), _i32(kv_tile_shape),
+            float(scale), *scales, _stream(q),
+        )
+    _check(rc)
+    return out, lse
+
+
+def fused_layout_supported(qkv_shape, dilation, kv_tile_shape) -> bool:
+    """Whether fna_forward_fused accepts this problem: no KV tile may reach past the input."""
+    return all(X % (d * t) == 0 for X, d, t in zip(qkv_shape, dilation, kv_tile_shape))
+
+
+def fna_forward_fused(
+    q: Tensor, k: Tensor, v: Tensor,
+    kernel_size, stride, dilation, is_causal, scale: float, q_tile_shape, kv_tile_shape,
+    q_scale: Optional[Tensor] = None, k_scale: Optional[Tensor] = None, v_scale: Optional[Tensor] = None,
+) -> Tuple[Tensor, Tensor]:
+    """Original-layout q [B, *X, H, D], k/v [B, *X, Hkv, D] -> (out like q, lse float32 [B, *X, H])."""
+    L = lib()
+    _require_gpu(q, k, v)
+    if q.dtype not in (torch.float16, torch.bfloat16):
+        raise NotImplementedError(f"natten_amd fna_forward_fused does not support {q.dtype}.")
+    na_dim = len(kernel_size)
+    qkv_shape = [int(x) for x in q.shape[1 : 1 + na_dim]]
+    scales = _scale_ptrs(q.flatten(1, na_dim), k.flatten(1, na_dim), q_scale, k_scale, v_scale)
+    out = torch.empty_like(q)
+    lse = torch.empty(q.shape[:-1], dtype=torch.float32, device=q.device)
+    with torch.cuda.device(q.device):
+        rc = L.natten_amd_fna_forward_fused(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
+            DTYPE_CODES[q.dtype], na_dim, q.shape[0], q.shape[-2], k.shape[-2], q.shape[-1],
+            _i32(qkv_shape), _i32(kernel_size), _i32(stride), _i32(dilation),
             _i32([1 if c else 0 for c in is_causal]), _i32(q_tile_shape), _i32(kv_tile_shape),
             float(scale), *scales, _stream(q),
         )

@@ -51,6 +51,14 @@ struct FnaParams {
   const float* q_scale;  // [heads_q]
   const float* k_scale;  // [heads_kv]
   const float* v_scale;  // [heads_kv]
+  // Operand layout.  fused == 0: q, k, v, o, lse are token-permuted sequences
+  // [batch * groups, seqlen, heads, D] (tile rows contiguous).  fused == 1: they are the
+  // original tensors [batch, X0, X1, X2, heads, D]; the kernel gathers the rows of a tile itself
+  // (every dilation group's extent must be a multiple of the KV tile in each dimension, so
+  // that no KV tile reaches past the input).
+  int fused;
+  int tok_stride[3];  // tokens per unit step of an original coordinate: X1*X2, X2, 1
+  int tokens;         // X0 * X1 * X2
 };
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
@@ -253,6 +261,8 @@ fna_fwd_kernel(const FnaParams p) {
   // the far end so that the Q tiles with the longest KV loops start first.
   int extent[3], q_first[3], box_tile0[3], box_n[3];
   int qtile_idx;  // position of the tile in the permuted sequence (dimension 0 fastest)
+  int tok_step[3];  // fused layout: tokens per unit step of a coordinate inside a dilation group
+  int group_tok = 0;  // fused layout: token of the dilation group's first element
   {
     int gl = bg % p.num_groups;
     int tc[3];
@@ -268,6 +278,8 @@ fna_fwd_kernel(const FnaParams p) {
       const int gi = gl % p.dil[a];
       gl /= p.dil[a];
       extent[a] = na_group_extent(p.qkv_shape[a], p.dil[a], gi);
+      tok_step[a] = p.dil[a] * p.tok_stride[a];
+      group_tok += gi * p.tok_stride[a];
       q_first[a] = tc[a] * p.q_tile[a];
       const int qf = q_first[a], ql = qf + p.q_tile[a] - 1;
       const bool c = p.causal[a] != 0;
@@ -335,9 +347,20 @@ fna_fwd_kernel(const FnaParams p) {
 
   const int64_t q_row_stride = int64_t(p.heads_q) * D;
   const int64_t kv_row_stride = int64_t(p.heads_kv) * D;
-  const T* qbase = reinterpret_cast<const T*>(p.q) + int64_t(bg) * p.seqlen_q * q_row_stride + int64_t(head) * D;
-  const T* kbase = reinterpret_cast<const T*>(p.k) + int64_t(bg) * p.seqlen_kv * kv_row_stride + int64_t(head_kv) * D;
-  const T* vbase = reinterpret_cast<const T*>(p.v) + int64_t(bg) * p.seqlen_kv * kv_row_stride + int64_t(head_kv) * D;
+  // first row of this (batch, dilation group): rows are then addressed by permuted row index
+  // (permuted layout) or by token offset inside the group (fused layout)
+  const int64_t q_row_base = p.fused ? int64_t(bg / p.num_groups) * p.tokens + group_tok : int64_t(bg) * p.seqlen_q;
+  const int64_t kv_row_base = p.fused ? int64_t(bg / p.num_groups) * p.tokens + group_tok : int64_t(bg) * p.seqlen_kv;
+  const T* qbase = reinterpret_cast<const T*>(p.q) + q_row_base * q_row_stride + int64_t(head) * D;
+  const T* kbase = reinterpret_cast<const T*>(p.k) + kv_row_base * kv_row_stride + int64_t(head_kv) * D;
+  const T* vbase = reinterpret_cast<const T*>(p.v) + kv_row_base * kv_row_stride + int64_t(head_kv) * D;
+  // row (permuted) or token offset (fused) of position `r` (dimension 0 fastest) of a KV tile
+  auto kv_tile_pos = [&](int r) {
+    if (!p.fused) return r;
+    const int t0 = r % p.kv_tile[0];
+    r /= p.kv_tile[0];
+    return t0 * tok_step[0] + (r % p.kv_tile[1]) * tok_step[1] + (r / p.kv_tile[1]) * tok_step[2];
+  };
 
   // ---- async tile loads -------------------------------------------------------------------------
   // Copy i of wave w fills LDS chunks (w*PER + i)*64 .. +63 of the tile (chunk P: row P / CPR,
@@ -348,7 +371,12 @@ fna_fwd_kernel(const FnaParams p) {
   // the per-lane offset again), and copy i + 4 lies a whole number of swizzle periods (16 rows
   // or more) below copy i, so it reuses that copy's per-lane offset on a shifted base.
   constexpr int NOFF = PER < 4 ? PER : 4;
+  constexpr int kImmBias = 3 * 1024;  // largest immediate offset of a copy
   constexpr int ROWS_PER_4 = 256 / CPR;  // rows between copy i and copy i + 4
+  // Copy i + 4 (only waves with eight copies have one) sets one more bit of the tile position;
+  // tile extents are powers of two, so that bit moves one coordinate by a fixed amount and the
+  // row (permuted) or token (fused) distance to copy i is the same for every lane.
+  const int64_t bytes_per_4 = int64_t(kv_tile_pos(ROWS_PER_4 % KVT)) * (kv_row_stride * 2);
   int ld_row[NOFF];
   uint32_t ld_koff[NOFF], ld_voff[NOFF];
 #pragma unroll
@@ -357,12 +385,14 @@ fna_fwd_kernel(const FnaParams p) {
     ld_row[i] = P / CPR;
     const int slot = P % CPR;
     // XOR swizzles are involutions: slot -> source chunk uses the same function
-    ld_koff[i] = uint32_t(ld_row[i]) * uint32_t(kv_row_stride * 2) + uint32_t(L::k_slot(ld_row[i], slot) * 16);
-    ld_voff[i] = uint32_t(ld_row[i]) * uint32_t(kv_row_stride * 2) + uint32_t(L::v_slot(ld_row[i], slot) * 16);
+    const uint32_t pos = uint32_t(kv_tile_pos(ld_row[i]));
+    ld_koff[i] = pos * uint32_t(kv_row_stride * 2) + uint32_t(L::k_slot(ld_row[i], slot) * 16);
+    ld_voff[i] = pos * uint32_t(kv_row_stride * 2) + uint32_t(L::v_slot(ld_row[i], slot) * 16);
     if constexpr (!RAGGED) {
-      // never negative: copy i starts at least 64 * i / CPR rows of at least 16 * CPR bytes into the tile
-      ld_koff[i] -= uint32_t(i * 1024);
-      ld_voff[i] -= uint32_t(i * 1024);
+      // the instruction adds its immediate i * 1024 to the global address as well: take it off
+      // here, on top of a bias that keeps the offset non-negative and is taken off the tile base
+      ld_koff[i] += uint32_t(kImmBias - i * 1024);
+      ld_voff[i] += uint32_t(kImmBias - i * 1024);
     }
   }
   // One operand tile in flight: uniform source base, LDS destination of this wave's share.
@@ -375,7 +405,7 @@ fna_fwd_kernel(const FnaParams p) {
   auto make_copy = [&](const T* base, char* dst, int kv_row0) {
     TileCopy c;
     kv_row0 = __builtin_amdgcn_readfirstlane(kv_row0);  // uniform by construction; keeps the base in scalar registers
-    c.src = reinterpret_cast<const char*>(base) + int64_t(kv_row0) * kv_row_stride * 2;
+    c.src = reinterpret_cast<const char*>(base) + int64_t(kv_row0) * kv_row_stride * 2 - (RAGGED ? 0 : kImmBias);
     c.lds0 = lds_address(dst) + uint32_t(wave * PER * 1024);
     c.row0 = kv_row0;
     c.inside = kv_row0 + KVT <= p.seqlen_kv;
@@ -387,7 +417,7 @@ fna_fwd_kernel(const FnaParams p) {
     if constexpr (I < PER) {
       if (CHUNKS % (NT * PER) == 0 || (wave * PER + I) * 64 < CHUNKS) {
         constexpr int IMM = (I % 4) * 1024;
-        const char* src = c.src + int64_t(I / 4) * ROWS_PER_4 * (kv_row_stride * 2);
+        const char* src = c.src + int64_t(I / 4) * bytes_per_4;
         uint32_t voff = off[I % 4];
         if constexpr (RAGGED) {
           if (!c.inside) {
@@ -420,7 +450,7 @@ fna_fwd_kernel(const FnaParams p) {
   // KV tile stream: dimension 2 fastest, dimension 0 slowest.  The load stream runs up to two
   // tiles ahead of the softmax, so tile descriptors are produced in order and handed down.
   struct TileInfo {
-    int row0;       // first row of the tile in the permuted KV sequence
+    int row0;       // first row of the tile in the permuted KV sequence / token offset of its origin (fused)
     int origin[3];  // coordinate of its first token
     bool full;      // every key of the tile is attended by every query of this wave
     bool skip;      // no key of the tile is attended by any query of this wave
@@ -437,7 +467,8 @@ fna_fwd_kernel(const FnaParams p) {
       t.full = t.full && (t.origin[a] >= wave_full_lo[a]) && (end <= wave_full_hi[a]);
       t.skip = t.skip || (end <= wave_lo[a]) || (t.origin[a] >= wave_hi[a]);
     }
-    t.row0 = ((box_tile0[0] + itc[0]) + p.kv_tiled[0] * ((box_tile0[1] + itc[1]) + p.kv_tiled[1] * (box_tile0[2] + itc[2]))) * KVT;
+    t.row0 = p.fused ? t.origin[0] * tok_step[0] + t.origin[1] * tok_step[1] + t.origin[2] * tok_step[2]
+                     : ((box_tile0[0] + itc[0]) + p.kv_tiled[0] * ((box_tile0[1] + itc[1]) + p.kv_tiled[1] * (box_tile0[2] + itc[2]))) * KVT;
     if (++itc[2] == box_n[2]) {
       itc[2] = 0;
       if (++itc[1] == box_n[1]) {
@@ -456,7 +487,7 @@ fna_fwd_kernel(const FnaParams p) {
 
   // ---- per-lane setup: this lane's query rows, their windows, Q fragments ---------------------
   int wst[MQ][3], wen[MQ][3];
-  int tile_row[MQ];  // this lane's row inside the permuted Q tile, per row block
+  int q_row[MQ];     // this lane's row of the permuted sequence / token offset in the group (fused), or -1
   vec8 qf[MQ][KSTEPS];
 #pragma unroll
   for (int mb = 0; mb < MQ; ++mb) {
@@ -466,15 +497,27 @@ fna_fwd_kernel(const FnaParams p) {
     r /= p.q_tile[2];
     off[1] = r % p.q_tile[1];
     off[0] = r / p.q_tile[1];
-    tile_row[mb] = off[0] + p.q_tile[0] * (off[1] + p.q_tile[1] * off[2]);
-    const int row = qtile_idx * QT + tile_row[mb];
+    int row = qtile_idx * QT + off[0] + p.q_tile[0] * (off[1] + p.q_tile[1] * off[2]);
+    bool valid = row < p.seqlen_q;
+    int row_c = na_min(row, p.seqlen_q - 1);
+    if (p.fused) {
+      // queries past the end of the dilation group are padding: computed on a clamped copy, never stored
+      row = 0;
+      row_c = 0;
+      valid = true;
+    }
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
       const int c = q_first[a] + off[a];
       wst[mb][a] = na_window_start(c, p.ksize[a], p.stride[a], extent[a], p.causal[a] != 0);
       wen[mb][a] = na_window_end(c, wst[mb][a], p.ksize[a], extent[a], p.causal[a] != 0);
+      if (p.fused) {
+        valid = valid && (c < extent[a]);
+        row += c * tok_step[a];
+        row_c += na_min(c, extent[a] - 1) * tok_step[a];
+      }
     }
-    const int row_c = na_min(row, p.seqlen_q - 1);
+    q_row[mb] = valid ? row : -1;
     const T* qrow = qbase + int64_t(row_c) * q_row_stride + g * 8;
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) qf[mb][ks] = *reinterpret_cast<const vec8*>(qrow + ks * 16);
@@ -810,13 +853,13 @@ fna_fwd_kernel(const FnaParams p) {
   wait_vmcnt<0>();  // the last iterations' copies into the unused stage must land before the LDS is released
 
   // ---- epilogue: O = acc / rowsum, LSE = ln(rowsum) + scale * rowmax -------------------------
-  T* obase = reinterpret_cast<T*>(p.o) + int64_t(bg) * p.seqlen_q * q_row_stride + int64_t(head) * D;
+  T* obase = reinterpret_cast<T*>(p.o) + q_row_base * q_row_stride + int64_t(head) * D;
 #pragma unroll
   for (int mb = 0; mb < MQ; ++mb) {
     const float l = l_run[mb] + __shfl_xor(l_run[mb], 32);
     const float inv = (l > 0.f) ? out_scale / l : 0.f;
-    const int row = qtile_idx * QT + tile_row[mb];
-    if (row < p.seqlen_q) {
+    const int row = q_row[mb];
+    if (row >= 0) {
       T* orow = obase + int64_t(row) * q_row_stride;
 #pragma unroll
       for (int db = 0; db < DB; ++db)
@@ -830,7 +873,7 @@ fna_fwd_kernel(const FnaParams p) {
         }
       if (g == 0) {
         const float lse = (l > 0.f) ? (m_run[mb] * sm_scale + __logf(l)) : -INFINITY;
-        p.lse[(int64_t(bg) * p.seqlen_q + row) * p.heads_q + head] = lse;
+        p.lse[(q_row_base + row) * p.heads_q + head] = lse;
       }
     }
   }

@@ -125,6 +125,47 @@ int check_common(const char* what, const void* q, const void* k, const void* v, 
   return 0;
 }
 
+// Shared by the permuted and the fused entry points: checks the neighborhood parameters and fills
+// everything but the operand layout.  q_shape / kv_shape: padded per-group token layouts.
+int fill_fna_params(const char* what, FnaParams& p, int na_dim, const int* q_shape, const int* kv_shape,
+                    const int32_t* qkv_shape, const int32_t* kernel_size, const int32_t* stride,
+                    const int32_t* dilation, const int32_t* is_causal, const int32_t* q_tile_shape,
+                    const int32_t* kv_tile_shape) {
+  memset(&p, 0, sizeof(p));
+  p.num_groups = 1;
+  for (int a = 0; a < 3; ++a) {
+    const bool used = a < na_dim;
+    p.qkv_shape[a] = used ? qkv_shape[a] : 1;
+    p.ksize[a] = used ? kernel_size[a] : 1;
+    p.stride[a] = used ? stride[a] : 1;
+    p.dil[a] = used ? dilation[a] : 1;
+    p.causal[a] = used ? (is_causal[a] != 0) : 0;
+    p.q_tile[a] = used ? q_tile_shape[a] : 1;
+    p.kv_tile[a] = used ? kv_tile_shape[a] : 1;
+    const int qs = used ? q_shape[a] : 1, ks = used ? kv_shape[a] : 1;
+    if (p.qkv_shape[a] < 1 || p.dil[a] < 1 || p.stride[a] < 1 || p.q_tile[a] < 1 || p.kv_tile[a] < 1 ||
+        (used && p.ksize[a] < 2))
+      return fail("%s: invalid parameter along dimension %d", what, a);
+    if (p.ksize[a] * p.dil[a] > p.qkv_shape[a])
+      return fail("%s: kernel_size * dilation exceeds the input along dimension %d (%d * %d > %d)", what, a,
+                  p.ksize[a], p.dil[a], p.qkv_shape[a]);
+    if (p.stride[a] > p.ksize[a])
+      return fail("%s: stride exceeds kernel_size along dimension %d (%d > %d)", what, a, p.stride[a], p.ksize[a]);
+    if (qs % p.q_tile[a] != 0 || ks % p.kv_tile[a] != 0)
+      return fail("%s: padded layouts must be multiples of the tile shapes (dimension %d)", what, a);
+    const int need = na_ceil_div(p.qkv_shape[a], p.dil[a]);
+    if (qs < need || ks < need)
+      return fail("%s: q_shape / kv_shape smaller than the dilation group extent along dimension %d", what, a);
+    if (p.kv_tile[a] > 512) return fail("%s: KV tile extent above 512 along dimension %d", what, a);
+    p.q_tiled[a] = qs / p.q_tile[a];
+    p.kv_tiled[a] = ks / p.kv_tile[a];
+    p.num_groups *= p.dil[a];
+  }
+  p.tok_stride[2] = 1;
+  p.tok_stride[1] = p.qkv_shape[2];
+  p.tok_stride[0] = p.qkv_shape[2] * p.qkv_shape[1];
+  return 0;
+}
 }  // namespace
 
 extern "C" {
@@ -157,39 +198,14 @@ int natten_amd_fna_forward(const void* q, const void* k, const void* v, void* ou
   if (!q_shape || !kv_shape || !qkv_shape || !kernel_size || !stride || !dilation || !is_causal || !q_tile_shape ||
       !kv_tile_shape)
     return fail("fna_forward: null shape argument");
-
   FnaParams p;
-  memset(&p, 0, sizeof(p));
+  if (int rc = fill_fna_params("fna_forward", p, na_dim, q_shape, kv_shape, qkv_shape, kernel_size, stride, dilation,
+                               is_causal, q_tile_shape, kv_tile_shape))
+    return rc;
   int qs[3] = {1, 1, 1}, ks[3] = {1, 1, 1};
-  p.num_groups = 1;
-  for (int a = 0; a < 3; ++a) {
-    const bool used = a < na_dim;
-    p.qkv_shape[a] = used ? qkv_shape[a] : 1;
-    p.ksize[a] = used ? kernel_size[a] : 1;
-    p.stride[a] = used ? stride[a] : 1;
-    p.dil[a] = used ? dilation[a] : 1;
-    p.causal[a] = used ? (is_causal[a] != 0) : 0;
-    p.q_tile[a] = used ? q_tile_shape[a] : 1;
-    p.kv_tile[a] = used ? kv_tile_shape[a] : 1;
-    qs[a] = used ? q_shape[a] : 1;
-    ks[a] = used ? kv_shape[a] : 1;
-    if (p.qkv_shape[a] < 1 || p.dil[a] < 1 || p.stride[a] < 1 || p.q_tile[a] < 1 || p.kv_tile[a] < 1 ||
-        (used && p.ksize[a] < 2))
-      return fail("fna_forward: invalid parameter along dimension %d", a);
-    if (p.ksize[a] * p.dil[a] > p.qkv_shape[a])
-      return fail("fna_forward: kernel_size * dilation exceeds the input along dimension %d (%d * %d > %d)", a,
-                  p.ksize[a], p.dil[a], p.qkv_shape[a]);
-    if (p.stride[a] > p.ksize[a])
-      return fail("fna_forward: stride exceeds kernel_size along dimension %d (%d > %d)", a, p.stride[a], p.ksize[a]);
-    if (qs[a] % p.q_tile[a] != 0 || ks[a] % p.kv_tile[a] != 0)
-      return fail("fna_forward: padded layouts must be multiples of the tile shapes (dimension %d)", a);
-    const int need = na_ceil_div(p.qkv_shape[a], p.dil[a]);
-    if (qs[a] < need || ks[a] < need)
-      return fail("fna_forward: q_shape / kv_shape smaller than the dilation group extent along dimension %d", a);
-    if (p.kv_tile[a] > 512) return fail("fna_forward: KV tile extent above 512 along dimension %d", a);
-    p.q_tiled[a] = qs[a] / p.q_tile[a];
-    p.kv_tiled[a] = ks[a] / p.kv_tile[a];
-    p.num_groups *= p.dil[a];
+  for (int a = 0; a < na_dim; ++a) {
+    qs[a] = q_shape[a];
+    ks[a] = kv_shape[a];
   }
   if (prod3(qs) != seqlen_q || prod3(ks) != seqlen_kv)
     return fail("fna_forward: seqlen_q / seqlen_kv do not match q_shape / kv_shape (%d vs %d, %d vs %d)", prod3(qs),
@@ -210,6 +226,65 @@ int natten_amd_fna_forward(const void* q, const void* k, const void* v, void* ou
   p.q_scale = q_scale;
   p.k_scale = k_scale;
   p.v_scale = v_scale;
+  set_wg_layout(p, 1);
+  return dispatch_dtype(p, dtype, head_dim, prod3(p.q_tile), prod3(p.kv_tile), static_cast<hipStream_t>(stream));
+}
+
+int natten_amd_fna_forward_fused(const void* q, const void* k, const void* v, void* out, float* lse, int dtype,
+                                 int na_dim, int batch, int heads_q, int heads_kv, int head_dim,
+                                 const int32_t* qkv_shape, const int32_t* kernel_size, const int32_t* stride,
+                                 const int32_t* dilation, const int32_t* is_causal, const int32_t* q_tile_shape,
+                                 const int32_t* kv_tile_shape, float scale, const float* q_scale,
+                                 const float* k_scale, const float* v_scale, void* stream) {
+  g_error[0] = 0;
+  if (na_dim < 1 || na_dim > 3) return fail("fna_forward_fused: na_dim must be 1, 2 or 3, got %d", na_dim);
+  if (!qkv_shape || !kernel_size || !stride || !dilation || !is_causal || !q_tile_shape || !kv_tile_shape)
+    return fail("fna_forward_fused: null shape argument");
+  int qs[3] = {1, 1, 1}, ks[3] = {1, 1, 1};
+  long long tokens = 1;
+  for (int a = 0; a < na_dim; ++a) {
+    if (qkv_shape[a] < 1 || dilation[a] < 1 || q_tile_shape[a] < 1 || kv_tile_shape[a] < 1)
+      return fail("fna_forward_fused: invalid parameter along dimension %d", a);
+    // every dilation group must have the same extent, a multiple of the KV tile: no KV tile
+    // may reach past the input, because the kernel gathers whole tiles without bounds checks
+    if (qkv_shape[a] % dilation[a] != 0 || (qkv_shape[a] / dilation[a]) % kv_tile_shape[a] != 0)
+      return fail("fna_forward_fused: the input extent %d along dimension %d is not a multiple of dilation * KV tile "
+                  "(%d * %d); use the token-permuted entry point",
+                  qkv_shape[a], a, dilation[a], kv_tile_shape[a]);
+    const int ext = qkv_shape[a] / dilation[a];
+    qs[a] = na_ceil_div(ext, q_tile_shape[a]) * q_tile_shape[a];
+    ks[a] = ext;
+    tokens *= qkv_shape[a];
+  }
+  if (tokens > 0x7fffffffLL) return fail("fna_forward_fused: more than 2^31 tokens per batch");
+  if (int rc = check_common("fna_forward_fused", q, k, v, out, lse, batch, prod3(qs), prod3(ks), heads_q, heads_kv,
+                            head_dim))
+    return rc;
+  FnaParams p;
+  if (int rc = fill_fna_params("fna_forward_fused", p, na_dim, qs, ks, qkv_shape, kernel_size, stride, dilation,
+                               is_causal, q_tile_shape, kv_tile_shape))
+    return rc;
+  // per-lane byte offsets inside a KV tile are 32-bit
+  long long span = 0;
+  for (int a = 0; a < 3; ++a) span += (long long)(p.kv_tile[a] - 1) * p.dil[a] * p.tok_stride[a];
+  if ((span + 1) * heads_kv * head_dim * 2 + 8192 >= 0x7fffffffLL)
+    return fail("fna_forward_fused: a KV tile spans more than 2^31 bytes of the input; use the token-permuted entry point");
+  p.q = q;
+  p.k = k;
+  p.v = v;
+  p.o = out;
+  p.lse = lse;
+  p.batch = batch * p.num_groups;
+  p.heads_q = heads_q;
+  p.heads_kv = heads_kv;
+  p.seqlen_q = prod3(qs);
+  p.seqlen_kv = prod3(ks);
+  p.scale = scale;
+  p.q_scale = q_scale;
+  p.k_scale = k_scale;
+  p.v_scale = v_scale;
+  p.fused = 1;
+  p.tokens = int(tokens);
   set_wg_layout(p, 1);
   return dispatch_dtype(p, dtype, head_dim, prod3(p.q_tile), prod3(p.kv_tile), static_cast<hipStream_t>(stream));
 }

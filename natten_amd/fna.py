@@ -94,8 +94,13 @@ def amd_fna_generic(
     k_scale=None,
     v_scale=None,
     out_dtype: Optional[torch.dtype] = None,
+    fused: Optional[bool] = None,
 ) -> Union[Tensor, Tuple[Tensor, Tensor]]:
-    """8-bit float operands (e4m3fn / e5m2) are widened to bf16 (exactly) by the token permute and
+    """`fused` selects the one-launch path that gathers tiles from the original tensors (None:
+    whenever the problem allows it); otherwise tokens are permuted, multiplied and unpermuted
+    by separate kernels, as the reference does.  Both give bit-identical results.
+
+    8-bit float operands (e4m3fn / e5m2) are widened to bf16 (exactly) by the token permute and
     multiplied in bf16; `q_scale`, `k_scale`, `v_scale` (number or per-head tensor) are their
     dequantisation scales.  `out_dtype` defaults to the dtype of `query`, as in the reference."""
     na_tensor_checks(query, key, value, must_match_head_dims=True)
@@ -115,6 +120,28 @@ def amd_fna_generic(
 
     in_dtype = query.dtype
     widen = is_fp8(in_dtype)
+    fusable = (not widen) and _lib.fused_layout_supported(query.shape[1 : 1 + na_dim], dilation, kv_tile_shape)
+    if fused and not fusable:
+        raise ValueError(
+            "natten_amd: the fused path needs 16-bit operands and an input extent that is a multiple of "
+            f"dilation * KV tile in every dimension; got {tuple(query.shape[1:1 + na_dim])}, {dilation=}, "
+            f"{kv_tile_shape=}, {in_dtype}."
+        )
+    if fusable and fused is not False:
+        output, lse = _lib.fna_forward_fused(
+            query.contiguous(), key.contiguous(), value.contiguous(), kernel_size, stride, dilation, is_causal,
+            scale, q_tile_shape, kv_tile_shape,
+            q_scale=resolve_scale(q_scale, query.shape[-2], query.device, "q_scale"),
+            k_scale=resolve_scale(k_scale, key.shape[-2], query.device, "k_scale"),
+            v_scale=resolve_scale(v_scale, key.shape[-2], query.device, "v_scale"),
+        )
+        if d_pad != head_dim:
+            output = output[..., :head_dim].contiguous()
+        out_dtype = out_dtype or in_dtype
+        if output.dtype != out_dtype:
+            output = output.to(out_dtype)
+        return (output, lse) if return_lse else output
+
     q_scale = resolve_scale(q_scale, query.shape[-2], query.device, "q_scale")
     k_scale = resolve_scale(k_scale, key.shape[-2], query.device, "k_scale")
     v_scale = resolve_scale(v_scale, key.shape[-2], query.device, "v_scale")

@@ -8,6 +8,7 @@ import pytest
 import torch
 
 import natten_amd
+from natten_amd.fna import amd_fna_generic
 from tests import problems
 from tests.gpu_utils import assert_close, make_qkv, oracle_full, to_np, tuplify
 
@@ -29,6 +30,14 @@ def run_case(B, H, Hkv, D, shape, k, s, d, causal, dtype, q_tile=None, kv_tile=N
     tag = f"{shape} k={k} s={s} d={d} c={causal} {dtype} tiles={q_tile},{kv_tile}"
     assert_close("out " + tag, to_np(out), ref_o)
     assert_close("lse " + tag, to_np(lse), ref_l)
+    if any(kk_ != x for kk_, x in zip(k, shape)) or any(causal):
+        # not the dense-attention shortcut: whichever path the call above took (one launch on
+        # the original tensors, or permute + kernel + unpermute), the other one must agree bit for bit
+        with torch.no_grad():
+            out2, lse2 = amd_fna_generic(q, kk, v, k, s, d, causal, q_tile_shape=q_tile, kv_tile_shape=kv_tile,
+                                         return_lse=True, fused=False)
+        assert torch.equal(out, out2), "fused and permuted paths differ in the output: " + tag
+        assert torch.equal(lse, lse2), "fused and permuted paths differ in the LSE: " + tag
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])

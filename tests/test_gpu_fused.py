@@ -1,0 +1,77 @@
+"""GPU parity of the one-launch path that gathers tiles from the original tensors
+(natten_amd_fna_forward_fused) against the permute + kernel + unpermute path and the oracle."""
+
+import pytest
+import torch
+
+import natten_amd
+from natten_amd import _lib
+from natten_amd.fna import amd_fna_generic
+from tests.gpu_utils import assert_close, make_qkv, oracle_full, to_np
+
+pytestmark = pytest.mark.gpu
+
+CASES = [
+    # shape, kernel, stride, dilation, causal, q_tile, kv_tile, heads, heads_kv, D
+    ((256,), (9,), (1,), (1,), (True,), (128,), (64,), 2, 1, 64),
+    ((384,), (31,), (4,), (2,), (False,), (128,), (64,), 3, 3, 32),
+    ((32, 48), (7, 9), (1, 2), (1, 1), (False, True), (8, 16), (8, 8), 4, 2, 64),
+    ((32, 32), (5, 5), (1, 1), (2, 2), (False, False), (16, 8), (4, 16), 2, 2, 128),
+    # Q tile that does not divide the group extent (padding queries), KV tile that does
+    ((24, 40), (6, 8), (2, 3), (1, 1), (True, False), (16, 16), (8, 8), 2, 2, 64),
+    ((6, 16, 24), (4, 8, 8), (1, 8, 4), (1, 1, 1), (True, False, False), (2, 8, 8), (1, 8, 8), 2, 1, 64),
+    ((8, 16, 16), (3, 5, 4), (1, 2, 1), (2, 1, 2), (False, False, True), (4, 8, 8), (2, 4, 8), 2, 2, 128),
+    ((4, 32, 32), (2, 9, 11), (1, 1, 1), (1, 2, 1), (False, False, False), (1, 8, 8), (1, 8, 8), 1, 1, 32),
+]
+
+
+@pytest.mark.parametrize("case", CASES)
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_fused_equals_permuted_and_oracle(case, dtype):
+    shape, k, s, d, causal, qt, kt, H, Hkv, D = case
+    q, kk, v = make_qkv(2, shape, H, Hkv, D, dtype, seed=7)
+    assert _lib.fused_layout_supported(shape, d, kt)
+    with torch.no_grad():
+        out_f, lse_f = amd_fna_generic(q, kk, v, k, s, d, causal, q_tile_shape=qt, kv_tile_shape=kt, return_lse=True,
+                                       fused=True)
+        out_p, lse_p = amd_fna_generic(q, kk, v, k, s, d, causal, q_tile_shape=qt, kv_tile_shape=kt, return_lse=True,
+                                       fused=False)
+    assert torch.equal(out_f, out_p)
+    assert torch.equal(lse_f, lse_p)
+    ref_o, ref_l = oracle_full(q, kk, v, k, s, d, causal)
+    assert_close("out", to_np(out_f), ref_o)
+    assert_close("lse", to_np(lse_f), ref_l)
+
+
+def test_fused_rejects_inputs_that_kv_tiles_overrun():
+    q, kk, v = make_qkv(1, (20, 24), 2, 2, 64, torch.bfloat16, seed=1)
+    args = ((5, 7), (1, 1), (1, 1), (False, False))
+    assert not _lib.fused_layout_supported((20, 24), (1, 1), (8, 8))
+    with pytest.raises(ValueError):
+        amd_fna_generic(q, kk, v, *args, q_tile_shape=(16, 8), kv_tile_shape=(8, 8), fused=True)
+    with pytest.raises(RuntimeError):
+        _lib.fna_forward_fused(q, kk, v, *args, 0.125, (16, 8), (8, 8))
+    # the default picks the permuted path and still matches the oracle
+    with torch.no_grad():
+        out, lse = natten_amd.na2d(q, kk, v, *args, q_tile_shape=(16, 8), kv_tile_shape=(8, 8), return_lse=True)
+    ref_o, ref_l = oracle_full(q, kk, v, *args)
+    assert_close("out", to_np(out), ref_o)
+    assert_close("lse", to_np(lse), ref_l)
+
+
+def test_fused_with_dequantisation_scales():
+    q, kk, v = make_qkv(1, (16, 16), 4, 2, 64, torch.bfloat16, seed=3)
+    sq = torch.tensor([0.5, 1.0, 2.0, 0.25], device="cuda")
+    sk = torch.tensor([1.5, 0.75], device="cuda")
+    sv = torch.tensor([2.0, 0.5], device="cuda")
+    args = ((5, 5), (1, 1), (1, 1), (False, False))
+    with torch.no_grad():
+        out_f, lse_f = amd_fna_generic(q, kk, v, *args, return_lse=True, q_scale=sq, k_scale=sk, v_scale=sv, fused=True)
+        out_p, lse_p = amd_fna_generic(q, kk, v, *args, return_lse=True, q_scale=sq, k_scale=sk, v_scale=sv, fused=False)
+    assert torch.equal(out_f, out_p) and torch.equal(lse_f, lse_p)
+    qd = q.float() * sq.view(1, 1, 1, -1, 1)
+    kd = kk.float() * sk.view(1, 1, 1, -1, 1)
+    vd = v.float() * sv.view(1, 1, 1, -1, 1)
+    ref_o, ref_l = oracle_full(qd, kd, vd, *args)
+    assert_close("out", to_np(out_f), ref_o, atol=2e-2, rtol=1e-2)
+    assert_close("lse", to_np(lse_f), ref_l)
