@@ -35,7 +35,7 @@ WORKLOADS = {
 # and calibrated on the permute kernel (a copy of known size); see profiles/fna_fwd_c4_na3d_bf16.md.
 # Keyed by (workload, q_tile_shape, kv_tile_shape); other combinations report null.
 MEASURED_TRAFFIC_BYTES = {
-    ("c4", (2, 8, 8), (1, 8, 8)): 2.84e10,
+    ("c4", (2, 8, 8), (1, 8, 8)): 2.82e10,
 }
 
 WORKLOAD_NAMES = {
