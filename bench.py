@@ -22,7 +22,9 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
-PEAK_TFLOPS = {"bf16": 2500.0, "fp16": 2500.0}  # MI355X dense MFMA peak
+# MI355X dense MFMA peak of the instruction the path multiplies with (e4m3 operands are widened
+# to bf16 exactly and multiplied by the bf16 instruction)
+PEAK_TFLOPS = {"bf16": 2500.0, "fp16": 2500.0, "e4m3": 2500.0}
 
 WORKLOADS = {
     # name: (B, H, layout, D, kernel, stride, dilation, causal, dtype, std)
@@ -30,6 +32,8 @@ WORKLOADS = {
     "c3": (1, 16, (128, 128), 128, (32, 32), (16, 16), (1, 1), (False, False), "fp16", 0.5),
     "c2": (2, 8, (64, 64), 64, (13, 13), (1, 1), (1, 1), (False, False), "bf16", 1.0),
     "c2d": (2, 8, (64, 64), 64, (13, 13), (1, 1), (2, 2), (False, False), "bf16", 1.0),
+    # e4m3 operands with per-head absmax scales, bf16 output; multiplied in bf16 after exact widening
+    "c5": (1, 16, (16, 64, 64), 128, (8, 16, 16), (4, 8, 8), (1, 2, 2), (False, False, False), "e4m3", 1.0),
 }
 # HBM-side traffic of one fused-kernel launch, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # and calibrated on the permute kernel (a copy of known size); see profiles/fna_fwd_c4_na3d_bf16.md.
@@ -43,6 +47,7 @@ WORKLOAD_NAMES = {
     "c3": "na2d fp16 B=1 H=16 128x128 D=128 k=(32,32) s=(16,16)",
     "c2": "na2d bf16 B=2 H=8 64x64 D=64 k=(13,13)",
     "c2d": "na2d bf16 B=2 H=8 64x64 D=64 k=(13,13) d=(2,2)",
+    "c5": "na3d e4m3 (per-head scales, bf16 out) B=1 H=16 16x64x64 D=128 k=(8,16,16) s=(4,8,8) d=(1,2,2)",
 }
 
 
@@ -139,16 +144,34 @@ def main():
     _lib.lib()  # no fallback: fail here when the HIP library is missing
     dev = torch.device("cuda:0")
     B, H, layout, D, kernel, stride, dilation, causal, dt_name, std = WORKLOADS[args.workload]
-    dtype = {"bf16": torch.bfloat16, "fp16": torch.float16}[dt_name]
+    quantised = dt_name == "e4m3"
+    dtype = {"bf16": torch.bfloat16, "fp16": torch.float16, "e4m3": torch.bfloat16}[dt_name]
     n = len(layout)
     gen = torch.Generator().manual_seed(0)
-    q, k, v = ((torch.randn((B, *layout, H, D), generator=gen) * std).to(dtype).to(dev) for _ in range(3))
+    q, k, v = ((torch.randn((B, *layout, H, D), generator=gen) * std).to(dev) for _ in range(3))
+    scales = {}
+    q8 = k8 = v8 = None
+    if quantised:
+        # per-head absmax scaling into the e4m3 range (max finite value 448)
+        def quantise(x):
+            sc = x.abs().amax(dim=tuple(range(x.dim() - 2)) + (x.dim() - 1,)).float() / 448.0
+            return (x / sc.view(-1, 1)).to(torch.float8_e4m3fn), sc
+
+        (q8, sq), (k8, sk), (v8, sv) = quantise(q), quantise(k), quantise(v)
+        scales = {"q_scale": sq, "k_scale": sk, "v_scale": sv, "out_dtype": torch.bfloat16}
+        # the dequantised values are what the result is checked against
+        q, k, v = (x8.float() * sc.view(-1, 1) for x8, sc in ((q8, sq), (k8, sk), (v8, sv)))
+    else:
+        q, k, v = (x.to(dtype) for x in (q, k, v))
     na = {1: natten_amd.na1d, 2: natten_amd.na2d, 3: natten_amd.na3d}[n]
     q_tile = tuple(int(x) for x in args.q_tile.split(",")) if args.q_tile else None
     kv_tile = tuple(int(x) for x in args.kv_tile.split(",")) if args.kv_tile else None
     q_tile, kv_tile = check_fna_forward_config(q, kernel, stride, dilation, causal, q_tile, kv_tile)
 
     def step():
+        if quantised:
+            return na(q8, k8, v8, kernel, stride, dilation, causal, q_tile_shape=q_tile, kv_tile_shape=kv_tile,
+                      return_lse=True, **scales)
         return na(q, k, v, kernel, stride, dilation, causal, q_tile_shape=q_tile, kv_tile_shape=kv_tile,
                   return_lse=True)
 
@@ -169,16 +192,26 @@ def main():
     from natten_amd.token_permute import token_permute_operation, token_unpermute_operation
 
     with torch.no_grad():
-        qp, qkv_shape, q_shape = token_permute_operation(q, q_tile, dilation)
-        kp, _, kv_shape = token_permute_operation(k, kv_tile, dilation)
-        vp, _, _ = token_permute_operation(v, kv_tile, dilation)
+        if quantised:
+            # the step's own route: widening permutes, then the bf16 kernel with the scales
+            qp, qkv_shape, q_shape = token_permute_operation(q8, q_tile, dilation, widen=True)
+            kp, _, kv_shape = token_permute_operation(k8, kv_tile, dilation, widen=True)
+            vp, _, _ = token_permute_operation(v8, kv_tile, dilation, widen=True)
+            kscales = {key: scales[key] for key in ("q_scale", "k_scale", "v_scale")}
+            tp_in = q8
+        else:
+            qp, qkv_shape, q_shape = token_permute_operation(q, q_tile, dilation)
+            kp, _, kv_shape = token_permute_operation(k, kv_tile, dilation)
+            vp, _, _ = token_permute_operation(v, kv_tile, dilation)
+            kscales = {}
+            tp_in = q
         scale = D**-0.5
 
-        fused = _lib.fused_layout_supported(layout, dilation, kv_tile)
+        fused = (not quantised) and _lib.fused_layout_supported(layout, dilation, kv_tile)
 
         def kern_permuted():
             return _lib.fna_forward(qp, kp, vp, kernel, stride, dilation, causal, scale, q_shape, kv_shape,
-                                    qkv_shape, q_tile, kv_tile)
+                                    qkv_shape, q_tile, kv_tile, **kscales)
 
         def kern():
             # the launch the step above makes
@@ -202,9 +235,9 @@ def main():
         kernel_ms = timed(kern, args.steps)
         kernel_permuted_ms = timed(kern_permuted, args.steps)
         op, lp = kern_permuted()
-        perm_ms = timed(lambda: token_permute_operation(q, q_tile, dilation), args.steps)
+        perm_ms = timed(lambda: token_permute_operation(tp_in, q_tile, dilation, widen=quantised), args.steps)
         unperm_ms = timed(lambda: token_unpermute_operation(op, qkv_shape, q_tile, dilation), args.steps)
-    q_bytes = q.numel() * q.element_size()
+    q_bytes = qp.numel() * qp.element_size() if quantised else q.numel() * q.element_size()
     achieved = flops / (kernel_ms * 1e-3) / 1e12
     peak = PEAK_TFLOPS[dt_name]
     dense_flops = 4.0 * B * H * D * float(q.numel() // (B * H * D)) ** 2
@@ -220,7 +253,7 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": dt_name,
+        "dtype": "bf16" if quantised else dt_name,
         "data": "synthetic",
         "config": {
             "workload": WORKLOAD_NAMES[args.workload],
@@ -236,7 +269,7 @@ def main():
         "token_permute": {
             "permute_q_ms": perm_ms,
             "unpermute_o_ms": unperm_ms,
-            "permute_GBps": 2 * q_bytes / (perm_ms * 1e-3) / 1e9,
+            "permute_GBps": (1.5 if quantised else 2) * q_bytes / (perm_ms * 1e-3) / 1e9,
             "unpermute_GBps": 2 * q_bytes / (unperm_ms * 1e-3) / 1e9,
         },
         "roofline": {
@@ -247,7 +280,8 @@ def main():
             "unit": "TFLOP/s",
             "frac": achieved / peak,
             "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, tuple(q_tile), tuple(kv_tile))),
-            "algorithmic_bytes": 4 * q_bytes + lse.numel() * 4,
+            "algorithmic_bytes": (4 * q.numel() * (1 if quantised else q.element_size())
+                                  + (q.numel() if quantised else 0) + lse.numel() * 4),
         },
     }
     if not args.no_mfma_probe:

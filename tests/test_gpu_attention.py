@@ -151,3 +151,14 @@ def test_attention_errors():
         natten_amd.attention(q, q, q, cumulative_seqlen_Q=torch.zeros(2, dtype=torch.int32))
     with pytest.raises(NotImplementedError):
         natten_amd.attention(q.float(), q.float(), q.float())
+
+
+def test_mfma_probe_reports_plausible_rates():
+    # diagnostic entry point: constant operands run at a higher clock than random ones, and
+    # neither exceeds the data-sheet peak
+    from natten_amd import _lib
+
+    rnd, rnd_ghz = _lib.mfma_probe(random_operands=True, iters=2000)
+    const, const_ghz = _lib.mfma_probe(random_operands=False, iters=2000)
+    assert 100.0 < rnd < 2600.0 and 100.0 < const < 2600.0
+    assert 0.3 < rnd_ghz < 2.6 and 0.3 < const_ghz < 2.6
