@@ -146,3 +146,21 @@ def test_c_oracle_window_equals_numpy():
             st = int(O.window_start(i, k, s, L, c))
             en = int(O.window_end(i, st, k, L, c))
             assert c_oracle.window(i, k, s, L, c) == (st, en)
+
+
+def test_hand_worked_window_tables():
+    # tables derived by hand from the definition (tests/golden/README.md), not by any code
+    import json
+    import os
+
+    path = os.path.join(os.path.dirname(__file__), "golden", "window_tables.json")
+    for c in json.load(open(path))["cases"]:
+        L, k, s, causal = c["L"], c["kernel"], c["stride"], c["causal"]
+        start = [int(O.window_start(i, k, s, L, causal)) for i in range(L)]
+        end = [int(O.window_end(i, start[i], k, L, causal)) for i in range(L)]
+        assert start == c["start"], (c, start)
+        assert end == c["end"], (c, end)
+        # the C oracle and the dense mask agree with the same tables
+        mask = O.na_mask_dense((L,), (k,), (s,), (1,), (causal,))
+        for i in range(L):
+            assert mask[i].nonzero()[0].tolist() == list(range(c["start"][i], c["end"][i]))
