@@ -22,9 +22,8 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
-# MI355X dense MFMA peak of the instruction the path multiplies with (e4m3 operands are widened
-# to bf16 exactly and multiplied by the bf16 instruction)
-PEAK_TFLOPS = {"bf16": 2500.0, "fp16": 2500.0, "e4m3": 2500.0}
+# MI355X dense MFMA peak of the instruction the path multiplies with
+PEAK_TFLOPS = {"bf16": 2500.0, "fp16": 2500.0, "e4m3": 5000.0}
 
 WORKLOADS = {
     # name: (B, H, layout, D, kernel, stride, dilation, causal, dtype, std)
@@ -32,7 +31,7 @@ WORKLOADS = {
     "c3": (1, 16, (128, 128), 128, (32, 32), (16, 16), (1, 1), (False, False), "fp16", 0.5),
     "c2": (2, 8, (64, 64), 64, (13, 13), (1, 1), (1, 1), (False, False), "bf16", 1.0),
     "c2d": (2, 8, (64, 64), 64, (13, 13), (1, 1), (2, 2), (False, False), "bf16", 1.0),
-    # e4m3 operands with per-head absmax scales, bf16 output; multiplied in bf16 after exact widening
+    # e4m3 operands with per-head absmax scales, bf16 output; multiplied by the 8-bit matrix instruction
     "c5": (1, 16, (16, 64, 64), 128, (8, 16, 16), (4, 8, 8), (1, 2, 2), (False, False, False), "e4m3", 1.0),
 }
 # HBM-side traffic of one fused-kernel launch, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
@@ -70,7 +69,7 @@ def count_attended(layout, k, s, d, c):
     return total
 
 
-def cpu_baseline(q, k, v, kernel, stride, dilation, causal, out_gpu, lse_gpu, seconds_target=15.0):
+def cpu_baseline(q, k, v, kernel, stride, dilation, causal, out_gpu, lse_gpu, seconds_target=15.0, tol=1e-2):
     """C oracle on a bounded sample of this workload's queries, all heads, host cores."""
     import numpy as np
 
@@ -101,7 +100,7 @@ def cpu_baseline(q, k, v, kernel, stride, dilation, causal, out_gpu, lse_gpu, se
     got_l = lse_gpu.reshape(B, N, H)[torch_idx(bat), torch_idx(tok)].float().cpu().numpy()
     err_o = float(np.abs(got_o - ref_o).max())
     err_l = float(np.abs(got_l - ref_l).max())
-    ok = bool(((np.abs(got_o - ref_o) <= 1e-2 + 1e-2 * np.abs(ref_o)).all())
+    ok = bool(((np.abs(got_o - ref_o) <= tol + tol * np.abs(ref_o)).all())
               and ((np.abs(got_l - ref_l) <= 1e-2 + 1e-2 * np.abs(ref_l)).all()))
     return {
         "value": flops / dt / 1e12,
@@ -109,7 +108,7 @@ def cpu_baseline(q, k, v, kernel, stride, dilation, causal, out_gpu, lse_gpu, se
         "cores": threads,
         "kind": "port",
         "sample": f"C oracle (float64), {nq} random queries x {H} heads of this workload, {dt:.1f} s wall",
-        "parity_on_sample": {"ok": ok, "max_abs_err_out": err_o, "max_abs_err_lse": err_l, "atol_rtol": 1e-2},
+        "parity_on_sample": {"ok": ok, "max_abs_err_out": err_o, "max_abs_err_lse": err_l, "atol_rtol": tol},
     }
 
 
@@ -193,10 +192,9 @@ def main():
 
     with torch.no_grad():
         if quantised:
-            # the step's own route: widening permutes, then the bf16 kernel with the scales
-            qp, qkv_shape, q_shape = token_permute_operation(q8, q_tile, dilation, widen=True)
-            kp, _, kv_shape = token_permute_operation(k8, kv_tile, dilation, widen=True)
-            vp, _, _ = token_permute_operation(v8, kv_tile, dilation, widen=True)
+            qp, qkv_shape, q_shape = token_permute_operation(q8, q_tile, dilation)
+            kp, _, kv_shape = token_permute_operation(k8, kv_tile, dilation)
+            vp, _, _ = token_permute_operation(v8, kv_tile, dilation)
             kscales = {key: scales[key] for key in ("q_scale", "k_scale", "v_scale")}
             tp_in = q8
         else:
@@ -207,7 +205,7 @@ def main():
             tp_in = q
         scale = D**-0.5
 
-        fused = (not quantised) and _lib.fused_layout_supported(layout, dilation, kv_tile)
+        fused = _lib.fused_layout_supported(layout, dilation, kv_tile)
 
         def kern_permuted():
             return _lib.fna_forward(qp, kp, vp, kernel, stride, dilation, causal, scale, q_shape, kv_shape,
@@ -215,6 +213,9 @@ def main():
 
         def kern():
             # the launch the step above makes
+            if fused and quantised:
+                return _lib.fna_forward_fused(q8, k8, v8, kernel, stride, dilation, causal, scale, q_tile, kv_tile,
+                                              **kscales)
             if fused:
                 return _lib.fna_forward_fused(q, k, v, kernel, stride, dilation, causal, scale, q_tile, kv_tile)
             return kern_permuted()
@@ -235,9 +236,9 @@ def main():
         kernel_ms = timed(kern, args.steps)
         kernel_permuted_ms = timed(kern_permuted, args.steps)
         op, lp = kern_permuted()
-        perm_ms = timed(lambda: token_permute_operation(tp_in, q_tile, dilation, widen=quantised), args.steps)
+        perm_ms = timed(lambda: token_permute_operation(tp_in, q_tile, dilation), args.steps)
         unperm_ms = timed(lambda: token_unpermute_operation(op, qkv_shape, q_tile, dilation), args.steps)
-    q_bytes = qp.numel() * qp.element_size() if quantised else q.numel() * q.element_size()
+    q_bytes = qp.numel() * qp.element_size()
     achieved = flops / (kernel_ms * 1e-3) / 1e12
     peak = PEAK_TFLOPS[dt_name]
     dense_flops = 4.0 * B * H * D * float(q.numel() // (B * H * D)) ** 2
@@ -253,7 +254,7 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "bf16" if quantised else dt_name,
+        "dtype": dt_name,
         "data": "synthetic",
         "config": {
             "workload": WORKLOAD_NAMES[args.workload],
@@ -269,11 +270,11 @@ def main():
         "token_permute": {
             "permute_q_ms": perm_ms,
             "unpermute_o_ms": unperm_ms,
-            "permute_GBps": (1.5 if quantised else 2) * q_bytes / (perm_ms * 1e-3) / 1e9,
-            "unpermute_GBps": 2 * q_bytes / (unperm_ms * 1e-3) / 1e9,
+            "permute_GBps": 2 * q_bytes / (perm_ms * 1e-3) / 1e9,
+            "unpermute_GBps": 2 * op.numel() * op.element_size() / (unperm_ms * 1e-3) / 1e9,
         },
         "roofline": {
-            "kernel": "fna_fwd_kernel",
+            "kernel": "fna_fwd_fp8_kernel" if quantised else "fna_fwd_kernel",
             "bound": "mfma",
             "achieved": achieved,
             "peak": peak,
@@ -295,7 +296,10 @@ def main():
             "constant_operands": {"TFLOP/s": const_tflops, "shader_clock_GHz": const_ghz},
         }
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(q, k, v, kernel, stride, dilation, causal, out, lse)
+        # 16-bit operands: atol = rtol = 1e-2; 8-bit matrix path (P rounded to e4m3, relative error
+        # up to 2^-4 per probability): atol = rtol = 2^-4
+        result["cpu_baseline"] = cpu_baseline(q, k, v, kernel, stride, dilation, causal, out, lse,
+                                              tol=2.0**-4 if quantised else 1e-2)
     print(json.dumps(result), flush=True)
 
 

@@ -34,9 +34,9 @@ extern "C" {
 /* Element types of Q/K/V (`dtype` arguments). */
 #define NATTEN_AMD_F16 0
 #define NATTEN_AMD_BF16 1
-#define NATTEN_AMD_F8E4M3 2 /* OCP e4m3fn: source type of natten_amd_token_permute_widen only */
+#define NATTEN_AMD_F8E4M3 2 /* OCP e4m3fn operands, bf16 output */
 #define NATTEN_AMD_F32 3    /* merge payloads only */
-#define NATTEN_AMD_F8E5M2 4 /* OCP e5m2: source type of natten_amd_token_permute_widen only */
+#define NATTEN_AMD_F8E5M2 4 /* OCP e5m2 operands, bf16 output */
 
 /* ABI version; bumped whenever a signature changes. */
 int natten_amd_abi_version(void);
@@ -49,7 +49,7 @@ const char* natten_amd_last_error(void);
  *
  *   q   [batch, seqlen_q,  heads_q,  head_dim]   contiguous
  *   k,v [batch, seqlen_kv, heads_kv, head_dim]   contiguous, heads_q % heads_kv == 0
- *   out [batch, seqlen_q,  heads_q,  head_dim]   dtype of q
+ *   out [batch, seqlen_q,  heads_q,  head_dim]   dtype of q (bf16 for 8-bit float operands)
  *   lse [batch, seqlen_q,  heads_q]              float32, natural log of the sum of exp(scale*q.k)
  *
  * `batch` already includes the dilation groups (batch index = b * prod(dilation) + group,
@@ -57,15 +57,18 @@ const char* natten_amd_last_error(void);
  * layouts the permuted sequences were built from (seqlen = product), qkv_shape the original
  * token layout.  All shape-like arrays hold `na_dim` entries.  Tiles are multi-dimensional;
  * their element counts must be a supported (Q tile, KV tile) pair, see
- * natten_amd_fna_supported_tiles().  head_dim must be 32, 64 or 128.  dtype is F16 or BF16.
+ * natten_amd_fna_supported_tiles().  head_dim must be 32, 64 or 128 (64 or 128 for 8-bit floats).
  *
  * q_scale [heads_q], k_scale [heads_kv], v_scale [heads_kv] are optional device arrays of
  * per-head dequantisation scales (NULL = 1): logits are scale * q_scale[h] * k_scale[hkv] * q.k,
  * the output is multiplied by v_scale[hkv], and lse is the log-sum-exp of those logits.
- * Quantised 8-bit float operands (the reference passes e4m3 / e5m2 tensors to this same entry
- * point, csrc/src/blackwell_fna_forward.cu:81-222) are served in two steps: widen them to bf16
- * while permuting with natten_amd_token_permute_widen (exact), then call this function with
- * dtype BF16 and the scales.  Passing an 8-bit dtype code here is an error.
+ *
+ * 8-bit float operands (dtype F8E4M3 / F8E5M2; the reference passes such tensors to this same
+ * entry point, csrc/src/blackwell_fna_forward.cu:81-222) are multiplied by the 8-bit matrix
+ * instruction with the probabilities rounded to e4m3, as the reference rounds them to the operand
+ * type; tiles must be 128 x 64 tokens.  A more accurate, slower route for the same operands:
+ * widen them to bf16 while permuting (natten_amd_token_permute_widen, exact) and call this
+ * function with dtype BF16 and the scales.
  */
 int natten_amd_fna_forward(const void* q, const void* k, const void* v, void* out, float* lse,
                            int dtype, int na_dim, int batch, int seqlen_q, int seqlen_kv,

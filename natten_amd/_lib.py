@@ -173,11 +173,12 @@ def fna_forward(
     q_scale [H], k_scale / v_scale [Hkv]: optional float32 per-head dequantisation scales."""
     L = lib()
     _require_gpu(q, k, v)
-    if q.dtype not in (torch.float16, torch.bfloat16):
+    if q.dtype not in (torch.float16, torch.bfloat16) + FP8_DTYPES:
         raise NotImplementedError(f"natten_amd fna_forward does not support {q.dtype}.")
     na_dim = len(kernel_size)
     scales = _scale_ptrs(q, k, q_scale, k_scale, v_scale)
-    out = torch.empty_like(q)
+    # 8-bit float operands are multiplied by the 8-bit matrix instruction; the result is bf16
+    out = torch.empty(q.shape, dtype=torch.bfloat16 if q.dtype in FP8_DTYPES else q.dtype, device=q.device)
     lse = torch.empty(q.shape[:-1], dtype=torch.float32, device=q.device)
     with torch.cuda.device(q.device):
         rc = L.natten_amd_fna_forward(
@@ -204,12 +205,12 @@ def fna_forward_fused(
     """Original-layout q [B, *X, H, D], k/v [B, *X, Hkv, D] -> (out like q, lse float32 [B, *X, H])."""
     L = lib()
     _require_gpu(q, k, v)
-    if q.dtype not in (torch.float16, torch.bfloat16):
+    if q.dtype not in (torch.float16, torch.bfloat16) + FP8_DTYPES:
         raise NotImplementedError(f"natten_amd fna_forward_fused does not support {q.dtype}.")
     na_dim = len(kernel_size)
     qkv_shape = [int(x) for x in q.shape[1 : 1 + na_dim]]
     scales = _scale_ptrs(q.flatten(1, na_dim), k.flatten(1, na_dim), q_scale, k_scale, v_scale)
-    out = torch.empty_like(q)
+    out = torch.empty(q.shape, dtype=torch.bfloat16 if q.dtype in FP8_DTYPES else q.dtype, device=q.device)
     lse = torch.empty(q.shape[:-1], dtype=torch.float32, device=q.device)
     with torch.cuda.device(q.device):
         rc = L.natten_amd_fna_forward_fused(

@@ -12,6 +12,7 @@
 #include <type_traits>
 
 #include "fna_fwd.hpp"
+#include "fna_fwd_fp8.hpp"
 #include "merge.hpp"
 #include "mfma_probe.hpp"
 #include "na_math.hpp"
@@ -76,6 +77,16 @@ int launch_fna(const FnaParams& p, hipStream_t stream) {
   return check_launch("fna_forward");
 }
 
+template <bool E5M2, int D>
+int launch_fna_fp8(const FnaParams& p, hipStream_t stream) {
+  constexpr int QT = 128;
+  if ((p.seqlen_q + QT - 1) / QT != p.num_q_tiles) return fail("fna_forward: internal tile count mismatch");
+  const long long wgs = (long long)((p.total_groups + kNumXcd - 1) / kNumXcd) * kNumXcd * p.wg_group;
+  if (wgs > 0x7fffffffLL) return fail("fna_forward: problem needs more than 2^31 workgroups");
+  hipLaunchKernelGGL((fna_fwd_fp8_kernel<E5M2, D, 4>), dim3((unsigned)wgs), dim3(256), 0, stream, p);
+  return check_launch("fna_forward");
+}
+
 template <typename T, int D>
 int dispatch_tiles(const FnaParams& p, int qt, int kvt, hipStream_t stream) {
   if (p.seqlen_kv % kvt != 0) {
@@ -104,9 +115,19 @@ int dispatch_dtype(const FnaParams& p, int dtype, int head_dim, int qt, int kvt,
     case NATTEN_AMD_F16: return dispatch_head_dim<_Float16>(p, head_dim, qt, kvt, stream);
     case NATTEN_AMD_BF16: return dispatch_head_dim<__bf16>(p, head_dim, qt, kvt, stream);
   }
-  if (dtype == NATTEN_AMD_F8E4M3 || dtype == NATTEN_AMD_F8E5M2)
-    return fail("8-bit float operands are widened by natten_amd_token_permute_widen; pass the bf16 result and "
-                "the dequantisation scales here");
+  if (dtype == NATTEN_AMD_F8E4M3 || dtype == NATTEN_AMD_F8E5M2) {
+    // 8-bit float operands, bf16 output: one kernel configuration
+    if (qt != 128 || kvt != 64)
+      return fail("fna_forward: 8-bit float operands need a Q tile of 128 and a KV tile of 64 tokens, got %d and %d", qt,
+                  kvt);
+    if (p.seqlen_kv % kvt != 0)
+      return fail("fna_forward: seqlen_kv (%d) must be a multiple of the KV tile (%d tokens)", p.seqlen_kv, kvt);
+    if (head_dim != 64 && head_dim != 128)
+      return fail("fna_forward: 8-bit float operands need head_dim 64 or 128, got %d", head_dim);
+    const bool e5m2 = dtype == NATTEN_AMD_F8E5M2;
+    if (head_dim == 128) return e5m2 ? launch_fna_fp8<true, 128>(p, stream) : launch_fna_fp8<false, 128>(p, stream);
+    return e5m2 ? launch_fna_fp8<true, 64>(p, stream) : launch_fna_fp8<false, 64>(p, stream);
+  }
   return fail("fna_forward: unsupported dtype code %d", dtype);
 }
 
@@ -175,6 +196,12 @@ int natten_amd_abi_version(void) { return 2; }
 const char* natten_amd_last_error(void) { return g_error; }
 
 int natten_amd_fna_supported_tiles(int dtype, int head_dim, int32_t* q_sizes, int32_t* kv_sizes, int capacity) {
+  if (dtype == NATTEN_AMD_F8E4M3 || dtype == NATTEN_AMD_F8E5M2) {
+    if (head_dim != 64 && head_dim != 128) return 0;
+    if (capacity > 0 && q_sizes) q_sizes[0] = 128;
+    if (capacity > 0 && kv_sizes) kv_sizes[0] = 64;
+    return 1;
+  }
   if (dtype != NATTEN_AMD_F16 && dtype != NATTEN_AMD_BF16) return 0;
   if (head_dim != 32 && head_dim != 64 && head_dim != 128) return 0;
   for (int i = 0; i < kNumTileConfigs && i < capacity; ++i) {
@@ -267,7 +294,7 @@ int natten_amd_fna_forward_fused(const void* q, const void* k, const void* v, vo
   // per-lane byte offsets inside a KV tile are 32-bit
   long long span = 0;
   for (int a = 0; a < 3; ++a) span += (long long)(p.kv_tile[a] - 1) * p.dil[a] * p.tok_stride[a];
-  if ((span + 1) * heads_kv * head_dim * 2 + 8192 >= 0x7fffffffLL)
+  if ((span + 1) * heads_kv * head_dim * 2 + 8192 >= 0x7fffffffLL)  // (16-bit rows; 8-bit ones are shorter)
     return fail("fna_forward_fused: a KV tile spans more than 2^31 bytes of the input; use the token-permuted entry point");
   p.q = q;
   p.k = k;

@@ -78,6 +78,13 @@ def can_run_amd_fna(query: Tensor, key: Tensor, value: Tensor, raise_error: bool
 _pad_head_dim = pad_head_dim
 
 
+def _prod(t) -> int:
+    out = 1
+    for x in t:
+        out *= int(x)
+    return out
+
+
 def amd_fna_generic(
     query: Tensor,
     key: Tensor,
@@ -95,14 +102,17 @@ def amd_fna_generic(
     v_scale=None,
     out_dtype: Optional[torch.dtype] = None,
     fused: Optional[bool] = None,
+    fp8_matmul: Optional[bool] = None,
 ) -> Union[Tensor, Tuple[Tensor, Tensor]]:
     """`fused` selects the one-launch path that gathers tiles from the original tensors (None:
     whenever the problem allows it); otherwise tokens are permuted, multiplied and unpermuted
     by separate kernels, as the reference does.  Both give bit-identical results.
 
-    8-bit float operands (e4m3fn / e5m2) are widened to bf16 (exactly) by the token permute and
-    multiplied in bf16; `q_scale`, `k_scale`, `v_scale` (number or per-head tensor) are their
-    dequantisation scales.  `out_dtype` defaults to the dtype of `query`, as in the reference."""
+    8-bit float operands (e4m3fn / e5m2): `q_scale`, `k_scale`, `v_scale` (number or per-head
+    tensor) are their dequantisation scales; `out_dtype` defaults to the dtype of `query`, as in
+    the reference.  `fp8_matmul` (None: whenever head dim and tiles allow) multiplies them with
+    the 8-bit matrix instruction, P rounded to e4m3 as the reference does; False widens them to
+    bf16 (exactly) in the token permute and multiplies in bf16, which is slower and more accurate."""
     na_tensor_checks(query, key, value, must_match_head_dims=True)
     can_run_amd_fna(query, key, value, raise_error=True)
     na_dim = query.dim() - 3
@@ -119,11 +129,21 @@ def amd_fna_generic(
         query, key, value = (_pad_head_dim(t, d_pad) for t in (query, key, value))
 
     in_dtype = query.dtype
-    widen = is_fp8(in_dtype)
+    fp8_ok = (
+        is_fp8(in_dtype) and d_pad in (64, 128)
+        and _prod(q_tile_shape) == 128 and _prod(kv_tile_shape) == 64
+    )
+    if fp8_matmul and not fp8_ok:
+        raise ValueError(
+            "natten_amd: the 8-bit matrix path needs e4m3 / e5m2 operands, head_dim of 64 or 128 (after padding) and "
+            f"tiles of 128 x 64 tokens; got {in_dtype}, head_dim {head_dim}, {q_tile_shape=}, {kv_tile_shape=}."
+        )
+    use_fp8 = fp8_ok and fp8_matmul is not False
+    widen = is_fp8(in_dtype) and not use_fp8
     fusable = (not widen) and _lib.fused_layout_supported(query.shape[1 : 1 + na_dim], dilation, kv_tile_shape)
     if fused and not fusable:
         raise ValueError(
-            "natten_amd: the fused path needs 16-bit operands and an input extent that is a multiple of "
+            "natten_amd: the fused path needs operands that are not widened and an input extent that is a multiple of "
             f"dilation * KV tile in every dimension; got {tuple(query.shape[1:1 + na_dim])}, {dilation=}, "
             f"{kv_tile_shape=}, {in_dtype}."
         )

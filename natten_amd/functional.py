@@ -107,6 +107,7 @@ def neighborhood_attention_generic(
     k_scale=None,
     v_scale=None,
     out_dtype: Optional[torch.dtype] = None,
+    fp8_matmul: Optional[bool] = None,
 ) -> Union[Tensor, Tuple[Tensor, Tensor]]:
     na_tensor_checks(query, key, value)
     additional_kv_tensor_checks(query, key, value, additional_keys, additional_values)
@@ -147,7 +148,7 @@ def neighborhood_attention_generic(
         query, key, value, kernel_size=kernel_size, stride=stride, dilation=dilation, is_causal=is_causal,
         scale=scale, q_tile_shape=q_tile_shape, kv_tile_shape=kv_tile_shape, return_lse=True,
         q_scale=q_scale, k_scale=k_scale, v_scale=v_scale,
-        out_dtype=work_dtype if has_additional_attention else final_dtype,
+        out_dtype=work_dtype if has_additional_attention else final_dtype, fp8_matmul=fp8_matmul,
     )
 
     if has_additional_attention:
@@ -193,6 +194,7 @@ def _make_na(na_dim: int, name: str):
         k_scale=None,
         v_scale=None,
         out_dtype: Optional[torch.dtype] = None,
+        fp8_matmul: Optional[bool] = None,
     ) -> Union[Tensor, Tuple[Tensor, Tensor]]:
         if query.dim() != na_dim + 3:
             raise ValueError(
@@ -207,7 +209,7 @@ def _make_na(na_dim: int, name: str):
             backward_kv_tile_shape=backward_kv_tile_shape, backward_kv_splits=backward_kv_splits,
             backward_use_pt_reduction=backward_use_pt_reduction, run_persistent_kernel=run_persistent_kernel,
             kernel_schedule=kernel_schedule, torch_compile=torch_compile, return_lse=return_lse,
-            q_scale=q_scale, k_scale=k_scale, v_scale=v_scale, out_dtype=out_dtype,
+            q_scale=q_scale, k_scale=k_scale, v_scale=v_scale, out_dtype=out_dtype, fp8_matmul=fp8_matmul,
         )
 
     op.__name__ = name
@@ -219,8 +221,9 @@ def _make_na(na_dim: int, name: str):
         "kernel_size * dilation <= input size); is_causal: bool or tuple.  additional_keys / additional_values "
         "`[batch, seqlen, heads_kv, head_dim]` add context every query attends to.  Returns the output and, with "
         "`return_lse=True`, the float32 logsumexp `[batch, *tokens, heads]`.  For e4m3 / e5m2 operands `q_scale`, "
-        "`k_scale`, `v_scale` (number or per-head tensor) are the dequantisation scales and `out_dtype` the result "
-        "type (default: the operands' type)."
+        "`k_scale`, `v_scale` (number or per-head tensor) are the dequantisation scales, `out_dtype` the result "
+        "type (default: the operands' type) and `fp8_matmul=False` trades the 8-bit matrix instruction for "
+        "bf16 products on exactly widened operands (slower, more accurate)."
     )
     return op
 

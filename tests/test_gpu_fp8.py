@@ -1,10 +1,16 @@
 """GPU parity for quantised 8-bit float operands (e4m3fn / e5m2 with per-head scales).
 
-The widening token permute must be bit-exact (every 8-bit float value is a bf16 value); the
-attention results are compared with the float64 oracle evaluated on the DEQUANTISED inputs.
-Tolerance: atol = rtol = 1e-2, the same as for bf16 operands, because the operands enter the
-bf16 matrix instructions exactly and only P and the output are rounded to bf16.  (The reference
-rounds P to 8 bits and tests with atol 0.5 for e4m3, tests/test_blackwell_fna.py:107.)"""
+The attention results are compared with the float64 oracle evaluated on the DEQUANTISED inputs.
+Two routes, two stated tolerances:
+  * 8-bit matrix instruction (default when head dim and tiles allow), P rounded to e4m3 as the
+    reference does.  Each probability then carries a relative error of up to 2^-4 (half a unit
+    of its 3-bit mantissa), so |out - ref| <= 2^-4 * max|V| holds for every element whatever the
+    window (checked as the absolute tolerance), and over a whole tensor the errors average out:
+    rms(out - ref) <= 3e-2 * rms(ref) (checked; observed 1.9e-2 to 2.5e-2).  LSE is computed
+    from unrounded probabilities: atol = rtol = 1e-2 as for 16-bit operands (observed 2e-5).
+    The reference tests the same arithmetic with atol 0.5 (tests/test_blackwell_fna.py:107).
+  * fp8_matmul=False: operands widened exactly to bf16 by the token permute (bit-exact, every
+    8-bit float value is a bf16 value) and multiplied in bf16: atol = rtol = 1e-2, as for bf16."""
 
 import numpy as np
 import pytest
@@ -20,6 +26,19 @@ pytestmark = pytest.mark.gpu
 
 E4M3_MAX = 448.0
 E5M2_MAX = 57344.0
+
+
+def check_out(name, fp8_matmul, got, ref, v_dequantised):
+    """Output tolerance of the two routes (see the module docstring)."""
+    if fp8_matmul is False:
+        assert_close(name, got, ref)
+        return
+    bound = 2.0**-4 * float(v_dequantised.abs().max())
+    assert_close(name, got, ref, atol=bound, rtol=0.0)
+    got, ref = np.asarray(got, dtype=np.float64), np.asarray(ref, dtype=np.float64)
+    rms_err, rms_ref = np.sqrt(((got - ref) ** 2).mean()), np.sqrt((ref**2).mean())
+    assert rms_err <= 3e-2 * rms_ref, f"{name}: rms error {rms_err:.4e} above 3e-2 of rms(ref) {rms_ref:.4e}"
+
 
 
 def quantise_per_head(x, dtype):
@@ -65,7 +84,7 @@ def test_widen_permute_matches_oracle(shape, tile, dil):
     assert np.array_equal(to_np(raw), ref)
 
 
-def _sampled(qd, kd, vd, out, lse, kernel, stride, dilation, causal, n_samples, seed):
+def _sampled(qd, kd, vd, out, lse, kernel, stride, dilation, causal, n_samples, seed, fp8_matmul=False):
     B = qd.shape[0]
     n = qd.dim() - 3
     N = int(np.prod(qd.shape[1 : 1 + n]))
@@ -77,11 +96,12 @@ def _sampled(qd, kd, vd, out, lse, kernel, stride, dilation, causal, n_samples, 
     ref_o, ref_l, _ = c_oracle.na_rows(to_np(qd), to_np(kd), to_np(vd), kernel, stride, dilation, causal, None, bat,
                                        tok, threads=8)
     ti, bi = torch.as_tensor(tok), torch.as_tensor(bat)
-    assert_close("sampled out", to_np(out.reshape(B, N, H, D)[bi, ti]), ref_o)
+    check_out("sampled out", fp8_matmul, to_np(out.reshape(B, N, H, D)[bi, ti]), ref_o, vd)
     assert_close("sampled lse", to_np(lse.reshape(B, N, H)[bi, ti]), ref_l)
 
 
-def test_config5_e4m3_full_size_sampled():
+@pytest.mark.parametrize("fp8_matmul", [True, False])
+def test_config5_e4m3_full_size_sampled(fp8_matmul):
     # na3d e4m3, B=1, heads 16, 16x64x64, D=128, kernel (8,16,16), stride (4,8,8), dilation (1,2,2)
     gen = torch.Generator().manual_seed(0)
     shape, H, D = (16, 64, 64), 16, 128
@@ -90,21 +110,22 @@ def test_config5_e4m3_full_size_sampled():
     args = ((8, 16, 16), (4, 8, 8), (1, 2, 2))
     with torch.no_grad():
         out, lse = natten_amd.na3d(q8, k8, v8, *args, return_lse=True, q_scale=sq, k_scale=sk, v_scale=sv,
-                                   out_dtype=torch.bfloat16)
+                                   out_dtype=torch.bfloat16, fp8_matmul=fp8_matmul)
     assert out.dtype == torch.bfloat16 and lse.dtype == torch.float32
     qd, kd, vd = dequantise(q8, sq), dequantise(k8, sk), dequantise(v8, sv)
-    _sampled(qd, kd, vd, out, lse, *args, (False, False, False), n_samples=96, seed=5)
+    _sampled(qd, kd, vd, out, lse, *args, (False, False, False), n_samples=96, seed=5, fp8_matmul=fp8_matmul)
     assert torch.isfinite(out).all() and torch.isfinite(lse).all()
     # doubling v_scale doubles the output bit-exactly and leaves LSE alone
     with torch.no_grad():
         out2, lse2 = natten_amd.na3d(q8, k8, v8, *args, return_lse=True, q_scale=sq, k_scale=sk, v_scale=sv * 2,
-                                     out_dtype=torch.bfloat16)
+                                     out_dtype=torch.bfloat16, fp8_matmul=fp8_matmul)
     assert torch.equal(out2, out * 2) and torch.equal(lse2, lse)
 
 
+@pytest.mark.parametrize("fp8_matmul", [True, False])
 @pytest.mark.parametrize("dtype", [torch.float8_e4m3fn, torch.float8_e5m2])
 @pytest.mark.parametrize("causal", [False, True])
-def test_small_fp8_problems_match_oracle(dtype, causal):
+def test_small_fp8_problems_match_oracle(dtype, causal, fp8_matmul):
     gen = torch.Generator().manual_seed(11)
     B, shape, H, Hkv, D = 2, (14, 20), 4, 2, 48
     q = torch.randn((B, *shape, H, D), generator=gen).cuda()
@@ -114,10 +135,10 @@ def test_small_fp8_problems_match_oracle(dtype, causal):
     kernel, stride, dil, cz = (5, 6), (2, 3), (2, 1), (causal, False)
     with torch.no_grad():
         out, lse = natten_amd.na2d(q8, k8, v8, kernel, stride, dil, cz, return_lse=True, q_scale=sq, k_scale=sk,
-                                   v_scale=sv, out_dtype=torch.bfloat16)
+                                   v_scale=sv, out_dtype=torch.bfloat16, fp8_matmul=fp8_matmul)
     qd, kd, vd = dequantise(q8, sq), dequantise(k8, sk), dequantise(v8, sv)
     ref_o, ref_l = c_oracle.na_forward(to_np(qd), to_np(kd), to_np(vd), kernel, stride, dil, cz, None)
-    assert_close("out", to_np(out), ref_o)
+    check_out("out", fp8_matmul, to_np(out), ref_o, vd)
     assert_close("lse", to_np(lse), ref_l)
 
 
@@ -151,10 +172,45 @@ def test_fp8_dense_attention_and_additional_kv():
     ref_o, ref_l = O.attention_forward(to_np(qd), to_np(kd), to_np(vd))
     assert_close("dense out", to_np(out), ref_o)
     assert_close("dense lse", to_np(lse), ref_l)
-    with torch.no_grad():
-        out, lse = natten_amd.na1d(q8, k8, v8, 7, additional_keys=ak8, additional_values=av8, return_lse=True,
-                                   q_scale=sq, k_scale=sk, v_scale=sv, out_dtype=torch.bfloat16)
     ref_o, ref_l = O.na_forward(to_np(qd), to_np(kd), to_np(vd), (7,), additional_keys=to_np(akd),
                                 additional_values=to_np(avd))
-    assert_close("na + additional out", to_np(out), ref_o)
-    assert_close("na + additional lse", to_np(lse), ref_l)
+    for fp8_matmul in (False, None):
+        with torch.no_grad():
+            out, lse = natten_amd.na1d(q8, k8, v8, 7, additional_keys=ak8, additional_values=av8, return_lse=True,
+                                       q_scale=sq, k_scale=sk, v_scale=sv, out_dtype=torch.bfloat16,
+                                       fp8_matmul=fp8_matmul)
+        check_out("na + additional out", fp8_matmul, to_np(out), ref_o, torch.cat([vd, avd], dim=1))
+        assert_close("na + additional lse", to_np(lse), ref_l)
+
+
+@pytest.mark.parametrize("dtype", [torch.float8_e4m3fn, torch.float8_e5m2])
+@pytest.mark.parametrize("D", [64, 128])
+def test_fp8_matmul_fused_equals_permuted(dtype, D):
+    # the 8-bit kernel on the original tensors and on token-permuted bytes: bit-identical
+    from natten_amd.fna import amd_fna_generic
+
+    gen = torch.Generator().manual_seed(9)
+    shape, H, Hkv = (4, 16, 32), 4, 2
+    q = torch.randn((2, *shape, H, D), generator=gen).cuda()
+    k = torch.randn((2, *shape, Hkv, D), generator=gen).cuda()
+    v = torch.randn((2, *shape, Hkv, D), generator=gen).cuda()
+    (q8, sq), (k8, sk), (v8, sv) = (quantise_per_head(t, dtype) for t in (q, k, v))
+    args = ((3, 7, 9), (1, 2, 3), (1, 2, 1), (True, False, False))
+    kw = dict(q_tile_shape=(2, 8, 8), kv_tile_shape=(2, 4, 8), return_lse=True, q_scale=sq, k_scale=sk, v_scale=sv,
+              out_dtype=torch.bfloat16, fp8_matmul=True)
+    with torch.no_grad():
+        out_f, lse_f = amd_fna_generic(q8, k8, v8, *args, fused=True, **kw)
+        out_p, lse_p = amd_fna_generic(q8, k8, v8, *args, fused=False, **kw)
+    assert torch.equal(out_f, out_p) and torch.equal(lse_f, lse_p)
+    qd, kd, vd = dequantise(q8, sq), dequantise(k8, sk), dequantise(v8, sv)
+    ref_o, ref_l = c_oracle.na_forward(to_np(qd), to_np(kd), to_np(vd), *args, None)
+    check_out("out", True, to_np(out_f), ref_o, vd)
+    assert_close("lse", to_np(lse_f), ref_l)
+
+
+def test_fp8_matmul_rejects_unsupported_shapes():
+    from natten_amd.fna import amd_fna_generic
+
+    q, k, v = (torch.zeros((1, 64, 2, 32), dtype=torch.float8_e4m3fn, device="cuda") for _ in range(3))
+    with pytest.raises(ValueError):
+        amd_fna_generic(q, k, v, (9,), fp8_matmul=True)  # head_dim 32 has no 8-bit instance
