@@ -104,6 +104,7 @@ def _try_load():
         _load_error = f"natten_amd: failed to load {LIB_PATH}: {e}"
 
 
+@torch.compiler.assume_constant_result
 def has_lib() -> bool:
     _try_load()
     return _lib is not None

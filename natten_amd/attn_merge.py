@@ -10,7 +10,7 @@ from typing import List, Tuple
 
 from torch import Tensor
 
-from . import _lib
+from . import _lib, torch_ops
 
 
 def merge_attentions(
@@ -50,7 +50,7 @@ def merge_attentions(
     out = work(outputs[0])
     lse = lse_tensors[0].float().contiguous()
     for o, l in zip(outputs[1:], lse_tensors[1:]):
-        out, lse = _lib.merge_two(out, lse, work(o.to(outputs[0].dtype)), l.float().contiguous())
+        out, lse = torch_ops.merge_two(out, lse, work(o.to(outputs[0].dtype)), l.float().contiguous())
     return out.to(out_dtype), lse
 
 

@@ -9,7 +9,7 @@ from typing import Optional, Tuple, Union
 import torch
 from torch import Tensor
 
-from . import _lib
+from . import _lib, torch_ops
 from .checks import fmha_tensor_checks
 from .fna import SUPPORTED_DTYPES, is_fp8, pad_head_dim, resolve_scale
 from .tile_config import padded_head_dim
@@ -43,8 +43,8 @@ def amd_fmha(
     q, k, v = (pad_head_dim(t.contiguous(), d_pad).contiguous() for t in (query, key, value))
     if is_fp8(query.dtype):
         # a one-token tile with no dilation is the identity permutation: a plain widening copy
-        q, k, v = (_lib.token_permute(t, (1,), (1,), True, widen=True) for t in (q, k, v))
-    out, lse = _lib.attention_forward(
+        q, k, v = (torch_ops.token_permute(t, (1,), (1,), True, widen=True) for t in (q, k, v))
+    out, lse = torch_ops.attention_forward(
         q, k, v, bool(is_causal), scale,
         q_scale=resolve_scale(q_scale, q.shape[-2], q.device, "q_scale"),
         k_scale=resolve_scale(k_scale, k.shape[-2], q.device, "k_scale"),

@@ -11,7 +11,7 @@ from typing import Optional, Tuple, Union
 import torch
 from torch import Tensor
 
-from . import _lib
+from . import _lib, torch_ops
 from .checks import check_all_args, check_args_against_input, na_tensor_checks
 from .tile_config import check_fna_forward_config, padded_head_dim
 from .token_permute import token_permute_operation, token_unpermute_operation
@@ -148,7 +148,7 @@ def amd_fna_generic(
             f"{kv_tile_shape=}, {in_dtype}."
         )
     if fusable and fused is not False:
-        output, lse = _lib.fna_forward_fused(
+        output, lse = torch_ops.fna_forward_fused(
             query.contiguous(), key.contiguous(), value.contiguous(), kernel_size, stride, dilation, is_causal,
             scale, q_tile_shape, kv_tile_shape,
             q_scale=resolve_scale(q_scale, query.shape[-2], query.device, "q_scale"),
@@ -170,7 +170,7 @@ def amd_fna_generic(
     k_perm, _, kv_shape = token_permute_operation(key, kv_tile_shape, dilation, flip_tiled_dims=True, widen=widen)
     v_perm, _, _ = token_permute_operation(value, kv_tile_shape, dilation, flip_tiled_dims=True, widen=widen)
 
-    out_perm, lse_perm = _lib.fna_forward(
+    out_perm, lse_perm = torch_ops.fna_forward(
         q_perm, k_perm, v_perm, kernel_size, stride, dilation, is_causal, scale,
         q_shape, kv_shape, qkv_shape, q_tile_shape, kv_tile_shape,
         q_scale=q_scale, k_scale=k_scale, v_scale=v_scale,

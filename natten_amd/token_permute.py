@@ -12,7 +12,7 @@ from typing import Optional, Tuple
 
 from torch import Tensor
 
-from . import _lib
+from . import _lib, torch_ops
 
 DimensionType = Tuple[int, ...]
 
@@ -49,7 +49,7 @@ def token_permute_operation(
     tensor = tensor.contiguous()
     token_layout = tuple(int(x) for x in tensor.shape[1 : 1 + na_dim])
     post = tuple(_ceil_div(_ceil_div(x, t), d) * t for x, t, d in zip(token_layout, tile_shape, dilation_))
-    out = _lib.token_permute(tensor, tile_shape, dilation_, flip_tiled_dims, widen=widen)
+    out = torch_ops.token_permute(tensor, tile_shape, dilation_, flip_tiled_dims, widen=widen)
     return out, token_layout, post
 
 
@@ -74,6 +74,6 @@ def token_unpermute_operation(
             f"{groups} ({dilation_=}), got batch={tensor.shape[0]}."
         )
     tensor = tensor.contiguous()
-    return _lib.token_unpermute(
+    return torch_ops.token_unpermute(
         tensor, tuple(int(x) for x in token_layout_shape), tuple(int(t) for t in tile_shape), dilation_, flip_tiled_dims
     )

@@ -1,0 +1,52 @@
+"""The public operations under a tracing compiler (torch.compile): the drivers route the native
+calls through torch custom operators whose fake implementations give shapes and dtypes, so
+the whole call traces into one graph (reference: src/natten/_libnatten/torch_wrappers.py:716-751).
+
+The CPU tests trace with fake device tensors (no GPU is touched); the GPU test runs the
+compiled function and compares it with the eager call bit for bit."""
+
+import pytest
+import torch
+from torch._subclasses.fake_tensor import FakeTensorMode
+
+import natten_amd
+
+CASES = {
+    "na2d one launch": (lambda q, k, v: natten_amd.na2d(q, k, v, (5, 5), (1, 1), (1, 1), return_lse=True),
+                        [(1, 16, 16, 2, 64)] * 3),
+    "na2d permuted": (lambda q, k, v: natten_amd.na2d(q, k, v, (5, 7), (1, 1), (1, 1), return_lse=True),
+                      [(1, 20, 24, 2, 64)] * 3),
+    "na1d additional kv": (lambda q, k, v, ak, av: natten_amd.na1d(q, k, v, 7, additional_keys=ak, additional_values=av,
+                                                                   return_lse=True),
+                           [(1, 70, 2, 64)] * 3 + [(1, 13, 2, 64)] * 2),
+    "attention": (lambda q, k, v: natten_amd.attention(q, k, v, is_causal=True, return_lse=True), [(2, 100, 4, 32)] * 3),
+    "na3d padded head dim": (lambda q, k, v: natten_amd.na3d(q, k, v, (2, 5, 5), return_lse=True),
+                             [(1, 4, 8, 8, 2, 40)] * 3),
+    "na2d whole-input window": (lambda q, k, v: natten_amd.na2d(q, k, v, (8, 8), return_lse=True), [(1, 8, 8, 2, 64)] * 3),
+}
+
+
+@pytest.mark.parametrize("name", sorted(CASES))
+def test_traces_into_one_graph_with_fake_tensors(name):
+    fn, shapes = CASES[name]
+    torch._dynamo.reset()
+    with FakeTensorMode():
+        args = [torch.empty(s, device="cuda", dtype=torch.bfloat16) for s in shapes]
+        compiled = torch.compile(fn, backend="eager", fullgraph=True)
+        with torch.no_grad():
+            out, lse = compiled(*args)
+    assert tuple(out.shape) == tuple(shapes[0]) and out.dtype == torch.bfloat16
+    assert tuple(lse.shape) == tuple(shapes[0][:-1]) and lse.dtype == torch.float32
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ["na2d one launch", "na2d permuted", "na1d additional kv"])
+def test_compiled_equals_eager(name):
+    fn, shapes = CASES[name]
+    torch._dynamo.reset()
+    gen = torch.Generator().manual_seed(0)
+    args = [torch.randn(s, generator=gen).to(torch.bfloat16).cuda() for s in shapes]
+    with torch.no_grad():
+        ref_out, ref_lse = fn(*args)
+        out, lse = torch.compile(fn, backend="aot_eager", fullgraph=True)(*args)
+    assert torch.equal(out, ref_out) and torch.equal(lse, ref_lse)
