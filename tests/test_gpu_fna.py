@@ -42,7 +42,7 @@ def run_case(B, H, Hkv, D, shape, k, s, d, causal, dtype, q_tile=None, kv_tile=N
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_config1_shape_na1d(dtype):
-    # BASELINE config 1's problem (B=1, heads=2, L=256, D=32, k=7) on the GPU path
+    # the first benchmark configuration's problem (B=1, heads=2, L=256, D=32, k=7) on the GPU path
     run_case(1, 2, 2, 32, (256,), 7, 1, 1, False, dtype)
 
 
