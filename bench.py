@@ -35,7 +35,7 @@ WORKLOADS = {
     "c5": (1, 16, (16, 64, 64), 128, (8, 16, 16), (4, 8, 8), (1, 2, 2), (False, False, False), "e4m3", 1.0),
 }
 # HBM-side traffic of one fused-kernel launch, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# and calibrated on the permute kernel (a copy of known size); see profiles/fna_fwd_c4_na3d_bf16.md.
+# and calibrated on the permute kernel (a copy of known size); the summary of that run is kept with the profiles.
 # Keyed by (workload, q_tile_shape, kv_tile_shape); other combinations report null.
 MEASURED_TRAFFIC_BYTES = {
     ("c4", (2, 8, 8), (1, 8, 8)): 2.82e10,

@@ -162,3 +162,22 @@ def test_mfma_probe_reports_plausible_rates():
     const, const_ghz = _lib.mfma_probe(random_operands=False, iters=2000)
     assert 100.0 < rnd < 2600.0 and 100.0 < const < 2600.0
     assert 0.3 < rnd_ghz < 2.6 and 0.3 < const_ghz < 2.6
+
+
+def test_neighborhood_attention_layer_matches_its_parts():
+    # the layer = qkv projection, na2d, output projection (reference src/natten/modules.py:83-123)
+    import natten_amd
+
+    torch.manual_seed(0)
+    layer = natten_amd.NeighborhoodAttention2D(embed_dim=128, num_heads=4, kernel_size=(5, 7), stride=(1, 2),
+                                               is_causal=(False, True)).cuda().to(torch.bfloat16)
+    x = torch.randn(2, 16, 24, 128, device="cuda", dtype=torch.bfloat16)
+    with torch.no_grad():
+        y = layer(x)
+        qkv = layer.qkv(x).reshape(2, 16, 24, 3, 4, 32)
+        ref = layer.proj(natten_amd.na2d(qkv[:, :, :, 0], qkv[:, :, :, 1], qkv[:, :, :, 2], (5, 7), (1, 2), 1,
+                                         (False, True)).reshape(2, 16, 24, 128))
+    assert y.shape == x.shape and torch.equal(y, ref)
+    with pytest.raises(ValueError):
+        layer(x[0])
+    assert set(layer.state_dict()) == {"qkv.weight", "qkv.bias", "proj.weight", "proj.bias"}
