@@ -18,7 +18,9 @@
  *   natten_amd_token_unpermute  <- token_unpermute_{1,2,3}d csrc/include/natten/token_permute.h:54-74
  *   natten_amd_attention_forward<- blackwell_fmha_forward   csrc/include/natten/blackwell_fmha.h
  *                                  (dense attention used for additional keys/values and for
- *                                  kernel_size == input size; no variable-length batches)
+ *                                  kernel_size == input size)
+ *   natten_amd_attention_forward_varlen <- the same function with cumulative_seqlen_Q / _KV,
+ *                                  max_seqlen_Q / _KV (csrc/include/natten/blackwell_fmha.h:34-50)
  *   natten_amd_merge_attentions <- the elementwise merge of src/natten/attn_merge.py:48-105
  *                                  (the reference runs it as framework ops; here it is one kernel)
  */
@@ -118,6 +120,26 @@ int natten_amd_attention_forward(const void* q, const void* k, const void* v, vo
                                  int heads_q, int heads_kv, int head_dim, int is_causal,
                                  float scale, const float* q_scale, const float* k_scale,
                                  const float* v_scale, void* stream);
+
+/*
+ * Dense attention forward on sequence-packed operands (variable-length batches).
+ *   q / out [total_seqlen_q, heads_q, head_dim], k / v [total_seqlen_kv, heads_kv, head_dim],
+ *   lse [total_seqlen_q, heads_q] float32.  Sequence b (0 <= b < num_seqs) owns query rows
+ *   cumulative_seqlen_q[b] .. cumulative_seqlen_q[b+1]-1 and key rows likewise; the two int32
+ *   arrays of num_seqs + 1 entries live in device memory.  max_seqlen_* bound the sequence
+ *   lengths (the launch is sized from them; rows of a longer sequence would not be computed).
+ *   The causal mask is top-left aligned per sequence.  A sequence without keys gets
+ *   out = 0 and lse = -inf.  Rows that belong to no sequence are not written.
+ *   16-bit float operands only.
+ */
+int natten_amd_attention_forward_varlen(const void* q, const void* k, const void* v, void* out,
+                                        float* lse, int dtype, int num_seqs, int total_seqlen_q,
+                                        int total_seqlen_kv, int max_seqlen_q, int max_seqlen_kv,
+                                        int heads_q, int heads_kv, int head_dim,
+                                        const int32_t* cumulative_seqlen_q,
+                                        const int32_t* cumulative_seqlen_kv, int is_causal,
+                                        float scale, const float* q_scale, const float* k_scale,
+                                        const float* v_scale, void* stream);
 
 /*
  * Token permute: src [batch, *token_layout, heads, head_dim] -> dst

@@ -19,7 +19,7 @@ from torch import Tensor
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libnatten_amd.so")
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 DTYPE_CODES = {
     torch.float16: 0,
@@ -55,6 +55,11 @@ _SIGNATURES = {
     "natten_amd_attention_forward": (
         ctypes.c_int,
         [ctypes.c_void_p] * 5 + [ctypes.c_int] * 8 + [ctypes.c_float] + [ctypes.c_void_p] * 4,
+    ),
+    "natten_amd_attention_forward_varlen": (
+        ctypes.c_int,
+        [ctypes.c_void_p] * 5 + [ctypes.c_int] * 9 + [ctypes.c_void_p] * 2 + [ctypes.c_int, ctypes.c_float]
+        + [ctypes.c_void_p] * 4,
     ),
     "natten_amd_token_permute_widen": (
         ctypes.c_int,
@@ -242,6 +247,39 @@ def attention_forward(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(), DTYPE_CODES[q.dtype],
             q.shape[0], q.shape[1], k.shape[1], q.shape[2], k.shape[2], q.shape[3], 1 if is_causal else 0,
             float(scale), *scales, _stream(q),
+        )
+    _check(rc)
+    return out, lse
+
+
+def attention_forward_varlen(
+    q: Tensor, k: Tensor, v: Tensor, cumulative_seqlen_q: Tensor, cumulative_seqlen_kv: Tensor,
+    max_seqlen_q: int, max_seqlen_kv: int, is_causal: bool, scale: float,
+    q_scale: Optional[Tensor] = None, k_scale: Optional[Tensor] = None, v_scale: Optional[Tensor] = None,
+) -> Tuple[Tensor, Tensor]:
+    """Sequence-packed dense attention: q [1, total_q, H, D], k/v [1, total_kv, Hkv, D], int32
+    device arrays of cumulative lengths (leading 0) -> (out, lse float32 [1, total_q, H]).  Rows
+    that belong to no sequence come back as zeros."""
+    L = lib()
+    _require_gpu(q, k, v, cumulative_seqlen_q, cumulative_seqlen_kv)
+    if q.dtype not in (torch.float16, torch.bfloat16):
+        raise NotImplementedError(f"natten_amd attention_forward_varlen does not support {q.dtype}.")
+    if q.shape[0] != 1 or k.shape[0] != 1:
+        raise ValueError("variable-length attention takes the sequence-packed layout (batch = 1).")
+    for c in (cumulative_seqlen_q, cumulative_seqlen_kv):
+        if c.dtype != torch.int32 or c.dim() != 1 or not c.is_contiguous():
+            raise ValueError("cumulative sequence lengths must be contiguous 1-D int32 tensors.")
+    if cumulative_seqlen_q.shape[0] != cumulative_seqlen_kv.shape[0] or cumulative_seqlen_q.shape[0] < 2:
+        raise ValueError("cumulative sequence lengths must match in size and hold at least 2 entries.")
+    scales = _scale_ptrs(q, k, q_scale, k_scale, v_scale)
+    out = torch.zeros_like(q)
+    lse = torch.zeros(q.shape[:-1], dtype=torch.float32, device=q.device)
+    with torch.cuda.device(q.device):
+        rc = L.natten_amd_attention_forward_varlen(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(), DTYPE_CODES[q.dtype],
+            cumulative_seqlen_q.shape[0] - 1, q.shape[1], k.shape[1], int(max_seqlen_q), int(max_seqlen_kv),
+            q.shape[2], k.shape[2], q.shape[3], cumulative_seqlen_q.data_ptr(), cumulative_seqlen_kv.data_ptr(),
+            1 if is_causal else 0, float(scale), *scales, _stream(q),
         )
     _check(rc)
     return out, lse

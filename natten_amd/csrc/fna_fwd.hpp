@@ -59,6 +59,11 @@ struct FnaParams {
   int fused;
   int tok_stride[3];  // tokens per unit step of an original coordinate: X1*X2, X2, 1
   int tokens;         // X0 * X1 * X2
+  // Sequence-packed dense attention (RAGGED instances only; null otherwise): `batch` sequences
+  // lie back to back in one row range, sequence b owns query rows cu_q[b] .. cu_q[b+1]-1 and
+  // key rows cu_kv[b] .. cu_kv[b+1]-1; q_tiled[0] then counts the Q tiles of the longest one.
+  const int32_t* cu_q;   // [batch + 1]
+  const int32_t* cu_kv;  // [batch + 1]
 };
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
@@ -256,6 +261,42 @@ fna_fwd_kernel(const FnaParams p) {
   }
   const int head_kv = head / (p.heads_q / p.heads_kv);
 
+  // sequence lengths, window and row range of this batch entry: launch constants, except for
+  // sequence-packed dense attention, where every batch entry is a sequence of its own
+  int seqlen_q = p.seqlen_q, seqlen_kv = p.seqlen_kv;
+  int ksz[3] = {p.ksize[0], p.ksize[1], p.ksize[2]};
+  int shp[3] = {p.qkv_shape[0], p.qkv_shape[1], p.qkv_shape[2]};
+  int64_t q_seq_row0 = int64_t(bg) * p.seqlen_q, kv_seq_row0 = int64_t(bg) * p.seqlen_kv;
+  if constexpr (RAGGED) {
+    if (p.cu_q != nullptr) {
+      const int q0 = p.cu_q[bg], kv0 = p.cu_kv[bg];
+      seqlen_q = p.cu_q[bg + 1] - q0;
+      seqlen_kv = p.cu_kv[bg + 1] - kv0;
+      q_seq_row0 = q0;
+      kv_seq_row0 = kv0;
+      ksz[0] = seqlen_kv;
+      shp[0] = seqlen_kv;
+      // Q tiles are counted for the longest sequence: the ones past the end of this one have nothing to do
+      int t0 = qtile_rm;
+      if (p.causal[0]) t0 = p.q_tiled[0] - 1 - t0;
+      if (t0 * QT >= seqlen_q) return;
+      if (seqlen_kv <= 0) {
+        // no keys: the softmax runs over an empty set, O = 0 and LSE = -inf
+        T* o = reinterpret_cast<T*>(p.o) + (q_seq_row0 * p.heads_q + head) * D;
+        for (int i = tid; i < QT * (D / 8); i += NT) {
+          const int row = t0 * QT + i / (D / 8);
+          if (row < seqlen_q) {
+            typedef T tx8 __attribute__((ext_vector_type(8)));
+            *reinterpret_cast<tx8*>(o + int64_t(row) * p.heads_q * D + (i % (D / 8)) * 8) = tx8{};
+          }
+        }
+        for (int i = tid; i < QT; i += NT)
+          if (t0 * QT + i < seqlen_q) p.lse[(q_seq_row0 + t0 * QT + i) * p.heads_q + head] = -INFINITY;
+        return;
+      }
+    }
+  }
+
   // ---- workgroup-uniform setup: dilation group, Q tile origin, KV tile box -------------------
   // qtile_rm enumerates Q tiles with dimension 0 slowest; causal dimension 0 is walked from
   // the far end so that the Q tiles with the longest KV loops start first.
@@ -277,15 +318,15 @@ fna_fwd_kernel(const FnaParams p) {
     for (int a = 0; a < 3; ++a) {
       const int gi = gl % p.dil[a];
       gl /= p.dil[a];
-      extent[a] = na_group_extent(p.qkv_shape[a], p.dil[a], gi);
+      extent[a] = na_group_extent(shp[a], p.dil[a], gi);
       tok_step[a] = p.dil[a] * p.tok_stride[a];
       group_tok += gi * p.tok_stride[a];
       q_first[a] = tc[a] * p.q_tile[a];
       const int qf = q_first[a], ql = qf + p.q_tile[a] - 1;
       const bool c = p.causal[a] != 0;
-      const int st_f = na_window_start(qf, p.ksize[a], p.stride[a], extent[a], c);
-      const int st_l = na_window_start(ql, p.ksize[a], p.stride[a], extent[a], c);
-      const int en_l = na_window_end(ql, st_l, p.ksize[a], extent[a], c);
+      const int st_f = na_window_start(qf, ksz[a], p.stride[a], extent[a], c);
+      const int st_l = na_window_start(ql, ksz[a], p.stride[a], extent[a], c);
+      const int en_l = na_window_end(ql, st_l, ksz[a], extent[a], c);
       box_tile0[a] = st_f / p.kv_tile[a];
       box_n[a] = na_ceil_div(en_l, p.kv_tile[a]) - box_tile0[a];
     }
@@ -324,10 +365,10 @@ fna_fwd_kernel(const FnaParams p) {
       // rows past the end of an unpadded sequence (dense attention) are clamped like the loads
       const int qmin = q_first[a] + f[a], qmax = q_first[a] + na_min(l[a], p.q_tile[a] - 1);
       const bool c = p.causal[a] != 0;
-      const int st_min = na_window_start(qmin, p.ksize[a], p.stride[a], extent[a], c);
-      const int en_min = na_window_end(qmin, st_min, p.ksize[a], extent[a], c);
-      const int st_max = na_window_start(qmax, p.ksize[a], p.stride[a], extent[a], c);
-      const int en_max = na_window_end(qmax, st_max, p.ksize[a], extent[a], c);
+      const int st_min = na_window_start(qmin, ksz[a], p.stride[a], extent[a], c);
+      const int en_min = na_window_end(qmin, st_min, ksz[a], extent[a], c);
+      const int st_max = na_window_start(qmax, ksz[a], p.stride[a], extent[a], c);
+      const int en_max = na_window_end(qmax, st_max, ksz[a], extent[a], c);
       wave_lo[a] = st_min;
       wave_hi[a] = en_max;
       wave_full_lo[a] = st_max;
@@ -349,8 +390,8 @@ fna_fwd_kernel(const FnaParams p) {
   const int64_t kv_row_stride = int64_t(p.heads_kv) * D;
   // first row of this (batch, dilation group): rows are then addressed by permuted row index
   // (permuted layout) or by token offset inside the group (fused layout)
-  const int64_t q_row_base = p.fused ? int64_t(bg / p.num_groups) * p.tokens + group_tok : int64_t(bg) * p.seqlen_q;
-  const int64_t kv_row_base = p.fused ? int64_t(bg / p.num_groups) * p.tokens + group_tok : int64_t(bg) * p.seqlen_kv;
+  const int64_t q_row_base = p.fused ? int64_t(bg / p.num_groups) * p.tokens + group_tok : q_seq_row0;
+  const int64_t kv_row_base = p.fused ? int64_t(bg / p.num_groups) * p.tokens + group_tok : kv_seq_row0;
   const T* qbase = reinterpret_cast<const T*>(p.q) + q_row_base * q_row_stride + int64_t(head) * D;
   const T* kbase = reinterpret_cast<const T*>(p.k) + kv_row_base * kv_row_stride + int64_t(head_kv) * D;
   const T* vbase = reinterpret_cast<const T*>(p.v) + kv_row_base * kv_row_stride + int64_t(head_kv) * D;
@@ -408,7 +449,7 @@ fna_fwd_kernel(const FnaParams p) {
     c.src = reinterpret_cast<const char*>(base) + int64_t(kv_row0) * kv_row_stride * 2 - (RAGGED ? 0 : kImmBias);
     c.lds0 = lds_address(dst) + uint32_t(wave * PER * 1024);
     c.row0 = kv_row0;
-    c.inside = kv_row0 + KVT <= p.seqlen_kv;
+    c.inside = kv_row0 + KVT <= seqlen_kv;
     return c;
   };
   // issues copy I (0 <= I < PER) of a tile
@@ -423,7 +464,7 @@ fna_fwd_kernel(const FnaParams p) {
           if (!c.inside) {
             // last, partial tile of an unpadded sequence: rows past the end are masked; read the
             // last valid row instead so that no out-of-bounds address is formed
-            const int over = na_max(c.row0 + ld_row[I % 4] + (I / 4) * ROWS_PER_4 - (p.seqlen_kv - 1), 0);
+            const int over = na_max(c.row0 + ld_row[I % 4] + (I / 4) * ROWS_PER_4 - (seqlen_kv - 1), 0);
             voff -= uint32_t(over) * uint32_t(kv_row_stride * 2);
           }
           // the clamped per-lane offset may be smaller than the immediate: take the immediate
@@ -498,8 +539,8 @@ fna_fwd_kernel(const FnaParams p) {
     off[1] = r % p.q_tile[1];
     off[0] = r / p.q_tile[1];
     int row = qtile_idx * QT + off[0] + p.q_tile[0] * (off[1] + p.q_tile[1] * off[2]);
-    bool valid = row < p.seqlen_q;
-    int row_c = na_min(row, p.seqlen_q - 1);
+    bool valid = row < seqlen_q;
+    int row_c = na_min(row, seqlen_q - 1);
     if (p.fused) {
       // queries past the end of the dilation group are padding: computed on a clamped copy, never stored
       row = 0;
@@ -509,8 +550,8 @@ fna_fwd_kernel(const FnaParams p) {
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
       const int c = q_first[a] + off[a];
-      wst[mb][a] = na_window_start(c, p.ksize[a], p.stride[a], extent[a], p.causal[a] != 0);
-      wen[mb][a] = na_window_end(c, wst[mb][a], p.ksize[a], extent[a], p.causal[a] != 0);
+      wst[mb][a] = na_window_start(c, ksz[a], p.stride[a], extent[a], p.causal[a] != 0);
+      wen[mb][a] = na_window_end(c, wst[mb][a], ksz[a], extent[a], p.causal[a] != 0);
       if (p.fused) {
         valid = valid && (c < extent[a]);
         row += c * tok_step[a];

@@ -89,8 +89,8 @@ int launch_fna_fp8(const FnaParams& p, hipStream_t stream) {
 
 template <typename T, int D>
 int dispatch_tiles(const FnaParams& p, int qt, int kvt, hipStream_t stream) {
-  if (p.seqlen_kv % kvt != 0) {
-    // key sequences that end inside a tile: dense attention on unpadded sequences only
+  if (p.seqlen_kv % kvt != 0 || p.cu_q != nullptr) {
+    // key sequences that end inside a tile: dense attention on unpadded or packed sequences only
     if (qt == 128 && kvt == 64) return launch_fna<T, D, 4, 1, true, 64>(p, stream);
     return fail("fna_forward: seqlen_kv (%d) must be a multiple of the KV tile (%d tokens)", p.seqlen_kv, kvt);
   }
@@ -191,7 +191,7 @@ int fill_fna_params(const char* what, FnaParams& p, int na_dim, const int* q_sha
 
 extern "C" {
 
-int natten_amd_abi_version(void) { return 2; }
+int natten_amd_abi_version(void) { return 3; }
 
 const char* natten_amd_last_error(void) { return g_error; }
 
@@ -359,6 +359,59 @@ int natten_amd_attention_forward(const void* q, const void* k, const void* v, vo
   p.q_scale = q_scale;
   p.k_scale = k_scale;
   p.v_scale = v_scale;
+  set_wg_layout(p, 1);
+  return dispatch_dtype(p, dtype, head_dim, QT, KVT, static_cast<hipStream_t>(stream));
+}
+
+int natten_amd_attention_forward_varlen(const void* q, const void* k, const void* v, void* out, float* lse, int dtype,
+                                        int num_seqs, int total_seqlen_q, int total_seqlen_kv, int max_seqlen_q,
+                                        int max_seqlen_kv, int heads_q, int heads_kv, int head_dim,
+                                        const int32_t* cumulative_seqlen_q, const int32_t* cumulative_seqlen_kv,
+                                        int is_causal, float scale, const float* q_scale, const float* k_scale,
+                                        const float* v_scale, void* stream) {
+  g_error[0] = 0;
+  const char* what = "attention_forward_varlen";
+  if (int rc = check_common(what, q, k, v, out, lse, num_seqs, total_seqlen_q, total_seqlen_kv, heads_q, heads_kv,
+                            head_dim))
+    return rc;
+  if (!cumulative_seqlen_q || !cumulative_seqlen_kv) return fail("%s: null cumulative sequence length array", what);
+  if (max_seqlen_q < 1 || max_seqlen_kv < 1 || max_seqlen_q > total_seqlen_q || max_seqlen_kv > total_seqlen_kv)
+    return fail("%s: maximum sequence lengths (%d, %d) must lie in 1 .. total (%d, %d)", what, max_seqlen_q,
+                max_seqlen_kv, total_seqlen_q, total_seqlen_kv);
+  if (dtype != NATTEN_AMD_F16 && dtype != NATTEN_AMD_BF16)
+    return fail("%s: only 16-bit float operands are supported, got dtype code %d", what, dtype);
+  constexpr int QT = 128, KVT = 64;
+  FnaParams p;
+  memset(&p, 0, sizeof(p));
+  for (int a = 0; a < 3; ++a) {
+    p.qkv_shape[a] = p.ksize[a] = p.stride[a] = p.dil[a] = p.q_tile[a] = p.kv_tile[a] = p.q_tiled[a] = p.kv_tiled[a] = 1;
+  }
+  // one batch entry per sequence; the kernel reads every sequence's own lengths (window =
+  // its whole key sequence) from the cumulative arrays, the launch is sized for the longest
+  p.ksize[0] = max_seqlen_kv;
+  p.qkv_shape[0] = max_seqlen_kv;
+  p.causal[0] = is_causal != 0;
+  p.q_tile[0] = QT;
+  p.kv_tile[0] = KVT;
+  p.q_tiled[0] = na_ceil_div(max_seqlen_q, QT);
+  p.kv_tiled[0] = na_ceil_div(max_seqlen_kv, KVT);
+  p.num_groups = 1;
+  p.q = q;
+  p.k = k;
+  p.v = v;
+  p.o = out;
+  p.lse = lse;
+  p.batch = num_seqs;
+  p.heads_q = heads_q;
+  p.heads_kv = heads_kv;
+  p.seqlen_q = max_seqlen_q;
+  p.seqlen_kv = max_seqlen_kv;
+  p.scale = scale;
+  p.q_scale = q_scale;
+  p.k_scale = k_scale;
+  p.v_scale = v_scale;
+  p.cu_q = cumulative_seqlen_q;
+  p.cu_kv = cumulative_seqlen_kv;
   set_wg_layout(p, 1);
   return dispatch_dtype(p, dtype, head_dim, QT, KVT, static_cast<hipStream_t>(stream));
 }

@@ -19,11 +19,13 @@ from .checks import (
     additional_kv_tensor_checks,
     check_all_args,
     check_args_against_input,
+    fmha_tensor_checks,
     is_self_attention,
     na_tensor_checks,
 )
 from .fmha import amd_fmha
 from .fna import amd_fna_generic, is_fp8
+from .utils.varlen import varlen_tensor_checks
 
 _BACKEND_FNA = "amd-fna"
 _BACKEND_FMHA = "amd-fmha"
@@ -62,20 +64,27 @@ def attention(
 ) -> Union[Tensor, Tuple[Tensor, Tensor]]:
     """Dot product attention on `[batch, seqlen, heads, head_dim]` tensors (heads last).
 
-    `is_causal` is top-left aligned.  Returns the output, and the float32 logsumexp
+    `is_causal` is top-left aligned.  Variable-length batches use the sequence-packed layout
+    (batch = 1, sequences back to back): pass either `seqlens_Q` / `seqlens_KV` (int32 device
+    tensors; costs a synchronisation) or `cumulative_seqlen_{Q,KV}` and `max_seqlen_{Q,KV}` from
+    `natten_amd.utils.varlen.generate_varlen_parameters`
+    (reference: src/natten/functional.py:74-348).  Returns the output, and the float32 logsumexp
     `[batch, seqlen, heads]` when `return_lse=True`.  For e4m3 / e5m2 operands `q_scale`, `k_scale`,
     `v_scale` (number or per-head tensor) are the dequantisation scales and `out_dtype` the
     result type (default: the operands' type, as in the reference).
     """
-    if any(x is not None for x in (seqlens_Q, seqlens_KV, cumulative_seqlen_Q, cumulative_seqlen_KV)) or any(
-        x not in (None, 0) for x in (max_seqlen_Q, max_seqlen_KV)
-    ):
-        raise NotImplementedError("natten_amd does not implement variable-length attention.")
+    fmha_tensor_checks(query, key, value, must_match_head_dims=True)
+    cumulative_seqlen_Q, cumulative_seqlen_KV, max_seqlen_Q, max_seqlen_KV = varlen_tensor_checks(
+        query, key, value, seqlens_Q=seqlens_Q, seqlens_KV=seqlens_KV, cumulative_seqlen_Q=cumulative_seqlen_Q,
+        cumulative_seqlen_KV=cumulative_seqlen_KV, max_seqlen_Q=max_seqlen_Q, max_seqlen_KV=max_seqlen_KV,
+    )
     if backend not in (None, _BACKEND_FMHA):
         raise NotImplementedError(f"Unrecognized attention backend {backend}; natten_amd provides '{_BACKEND_FMHA}'.")
     return amd_fmha(
         query, key, value, is_causal=is_causal, scale=scale, return_lse=return_lse,
         q_scale=q_scale, k_scale=k_scale, v_scale=v_scale, out_dtype=out_dtype,
+        cumulative_seqlen_Q=cumulative_seqlen_Q, cumulative_seqlen_KV=cumulative_seqlen_KV,
+        max_seqlen_Q=max_seqlen_Q, max_seqlen_KV=max_seqlen_KV,
     )
 
 

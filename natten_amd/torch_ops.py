@@ -68,6 +68,23 @@ def _(q, k, v, is_causal, scale, q_scale, k_scale, v_scale):
     return torch.empty_like(q), q.new_empty(q.shape[:-1], dtype=torch.float32)
 
 
+@torch.library.custom_op("natten_amd::attention_forward_varlen", mutates_args=(), device_types="cuda")
+def _attention_forward_varlen_op(
+    q: Tensor, k: Tensor, v: Tensor, cumulative_seqlen_q: Tensor, cumulative_seqlen_kv: Tensor,
+    max_seqlen_q: int, max_seqlen_kv: int, is_causal: bool, scale: float, q_scale: Optional[Tensor],
+    k_scale: Optional[Tensor], v_scale: Optional[Tensor],
+) -> Tuple[Tensor, Tensor]:
+    return _lib.attention_forward_varlen(q, k, v, cumulative_seqlen_q, cumulative_seqlen_kv, max_seqlen_q,
+                                         max_seqlen_kv, is_causal, scale, q_scale=q_scale, k_scale=k_scale,
+                                         v_scale=v_scale)
+
+
+@_attention_forward_varlen_op.register_fake
+def _(q, k, v, cumulative_seqlen_q, cumulative_seqlen_kv, max_seqlen_q, max_seqlen_kv, is_causal, scale, q_scale,
+      k_scale, v_scale):
+    return torch.empty_like(q), q.new_empty(q.shape[:-1], dtype=torch.float32)
+
+
 def _permuted_shape(x: Tensor, tile_shape: List[int], dilation: List[int]) -> List[int]:
     na_dim = x.dim() - 3
     groups, seqlen = 1, 1
@@ -146,6 +163,17 @@ def attention_forward(q, k, v, is_causal, scale, q_scale=None, k_scale=None, v_s
     if _tracing():
         return _attention_forward_op(q, k, v, bool(is_causal), float(scale), q_scale, k_scale, v_scale)
     return _lib.attention_forward(q, k, v, is_causal, scale, q_scale=q_scale, k_scale=k_scale, v_scale=v_scale)
+
+
+def attention_forward_varlen(q, k, v, cumulative_seqlen_q, cumulative_seqlen_kv, max_seqlen_q, max_seqlen_kv,
+                             is_causal, scale, q_scale=None, k_scale=None, v_scale=None):
+    if _tracing():
+        return _attention_forward_varlen_op(q, k, v, cumulative_seqlen_q, cumulative_seqlen_kv, int(max_seqlen_q),
+                                            int(max_seqlen_kv), bool(is_causal), float(scale), q_scale, k_scale,
+                                            v_scale)
+    return _lib.attention_forward_varlen(q, k, v, cumulative_seqlen_q, cumulative_seqlen_kv, max_seqlen_q,
+                                         max_seqlen_kv, is_causal, scale, q_scale=q_scale, k_scale=k_scale,
+                                         v_scale=v_scale)
 
 
 def token_permute(x, tile_shape, dilation, flip_tiled_dims, widen=False):

@@ -147,7 +147,7 @@ def test_attention_errors():
         natten_amd.attention(q, q[:, :, :1], q)
     with pytest.raises(ValueError):
         natten_amd.attention(q, q[:, :8], q)
-    with pytest.raises(NotImplementedError):
+    with pytest.raises(ValueError):  # cumulative lengths without their partner and the maxima
         natten_amd.attention(q, q, q, cumulative_seqlen_Q=torch.zeros(2, dtype=torch.int32))
     with pytest.raises(NotImplementedError):
         natten_amd.attention(q.float(), q.float(), q.float())
