@@ -98,3 +98,44 @@ def na_forward(q, k, v, kernel_size, stride, dilation, is_causal, scale=None, th
     qt = np.tile(np.arange(N), B)
     o, l, _ = na_rows(q, k, v, kernel_size, stride, dilation, is_causal, scale, qb, qt, threads)
     return o.reshape(*q.shape[:-1], q.shape[-1]), l.reshape(q.shape[:-1])
+
+
+def na_backward(q, k, v, d_out, kernel_size, stride, dilation, is_causal, scale=None, threads: int = 8):
+    """Gradients (dq, dk, dv), float64, of sum(out * d_out) for neighborhood attention on heads-last
+    float32 tensors [B, *X, H, D]; the work is split over (batch, KV head) pairs."""
+    q = np.ascontiguousarray(q, dtype=np.float32)
+    k = np.ascontiguousarray(k, dtype=np.float32)
+    v = np.ascontiguousarray(v, dtype=np.float32)
+    d_out = np.ascontiguousarray(d_out, dtype=np.float32)
+    assert d_out.shape == q.shape and k.shape == v.shape
+    n = q.ndim - 3
+    X = _pad3(q.shape[1 : 1 + n], n, 1)
+    B, H, D = q.shape[0], q.shape[-2], q.shape[-1]
+    Hkv = k.shape[-2]
+    ks = _pad3(kernel_size, n, 1)
+    st = _pad3(stride, n, 1)
+    dl = _pad3(dilation, n, 1)
+    ca = _pad3([int(bool(c)) for c in is_causal], n, 0)
+    scale = float(scale) if scale is not None else float(D) ** -0.5
+    dq = np.zeros(q.shape, dtype=np.float64)
+    dk = np.zeros(k.shape, dtype=np.float64)
+    dv = np.zeros(v.shape, dtype=np.float64)
+    I3 = ctypes.c_int * 3
+    L = lib()
+    L.na_oracle_backward.restype = ctypes.c_int64
+
+    def run(job):
+        b, hk = job
+        return L.na_oracle_backward(
+            q.ctypes.data_as(ctypes.c_void_p), k.ctypes.data_as(ctypes.c_void_p),
+            v.ctypes.data_as(ctypes.c_void_p), d_out.ctypes.data_as(ctypes.c_void_p), ctypes.c_int(b), I3(*X),
+            ctypes.c_int(H), ctypes.c_int(Hkv), ctypes.c_int(D), I3(*ks), I3(*st), I3(*dl), I3(*ca),
+            ctypes.c_double(scale), ctypes.c_int(hk), ctypes.c_int(hk + 1),
+            dq.ctypes.data_as(ctypes.c_void_p), dk.ctypes.data_as(ctypes.c_void_p),
+            dv.ctypes.data_as(ctypes.c_void_p))
+
+    jobs = [(b, hk) for b in range(B) for hk in range(Hkv)]
+    with ThreadPoolExecutor(max(1, min(threads, len(jobs)))) as ex:
+        visited = list(ex.map(run, jobs))
+    assert all(x >= 0 for x in visited)
+    return dq, dk, dv

@@ -1,5 +1,5 @@
 /*
- * CPU oracle (plain C) for neighborhood attention forward, evaluated query by query.
+ * CPU oracle (plain C) for neighborhood attention forward and backward, evaluated query by query.
  *
  * TEST INFRASTRUCTURE ONLY: this file is the checker for the HIP path (tests, smoke, the bench's
  * CPU-baseline leg).  Nothing shipped links or calls it.
@@ -114,6 +114,99 @@ int64_t na_oracle_rows(const float* q, const float* k, const float* v, int B, co
     }
   }
   free(logits);
+  free(keyidx);
+  return visited;
+}
+
+/*
+ * Backward: gradients of sum(out * d_out) with respect to q, k, v, for the q heads of the KV
+ * heads hk_lo .. hk_hi-1 of batch entry b (callers split the work over disjoint ranges, so
+ * no two calls write the same gradient rows).  Restates the naive backward kernels of
+ *   csrc/include/natten/cuda/reference/fna_reference_backward.hpp:60-150 (dQ), :165-265 (dK),
+ *   :282-380 (dV):   P = exp(scale * q.k - LSE),  dS = P * scale * (dO.v - dO.o),
+ *   dQ = sum_j dS k_j,  dK_j = sum_i dS q_i,  dV_j = sum_i P dO_i
+ * one query at a time over its window.  LSE is recomputed here and dO.o is evaluated as
+ * sum_j P_j (dO.v_j), the same number, so the forward output is not an input.  The gradient of
+ * the returned LSE is not propagated, as in the reference.
+ * d_out [B, X0, X1, X2, H, D] float32; dq like q, dk / dv like k (float64, zero-initialised by
+ * the caller).
+ */
+int64_t na_oracle_backward(const float* q, const float* k, const float* v, const float* d_out, int b,
+                           const int* X /*3*/, int H, int Hkv, int D, const int* ksz, const int* stride,
+                           const int* dil, const int* causal, double scale, int hk_lo, int hk_hi,
+                           double* dq, double* dk, double* dv) {
+  const int64_t N = (int64_t)X[0] * X[1] * X[2];
+  const int rep = H / Hkv;
+  int64_t visited = 0;
+  int maxw = 1;
+  for (int a = 0; a < 3; ++a) maxw *= (X[a] < 1 ? 1 : X[a]);
+  double* prob = (double*)malloc(sizeof(double) * (size_t)maxw);
+  double* dprob = (double*)malloc(sizeof(double) * (size_t)maxw);
+  int64_t* keyidx = (int64_t*)malloc(sizeof(int64_t) * (size_t)maxw);
+  if (!prob || !dprob || !keyidx) return -1;
+  for (int64_t t = 0; t < N; ++t) {
+    int c[3] = {(int)(t / ((int64_t)X[1] * X[2])), (int)((t / X[2]) % X[1]), (int)(t % X[2])};
+    int st[3], en[3], g[3];
+    for (int a = 0; a < 3; ++a) {
+      g[a] = c[a] % dil[a];
+      int L = fix_extent(X[a], dil[a], g[a]);
+      int i = c[a] / dil[a];
+      st[a] = win_start(i, ksz[a], stride[a], L, causal[a]);
+      en[a] = win_end(i, st[a], ksz[a], L, causal[a]);
+    }
+    int w = 0;
+    for (int j0 = st[0]; j0 < en[0]; ++j0)
+      for (int j1 = st[1]; j1 < en[1]; ++j1)
+        for (int j2 = st[2]; j2 < en[2]; ++j2) {
+          int64_t x0 = (int64_t)j0 * dil[0] + g[0], x1 = (int64_t)j1 * dil[1] + g[1],
+                  x2 = (int64_t)j2 * dil[2] + g[2];
+          keyidx[w++] = (x0 * X[1] + x1) * X[2] + x2;
+        }
+    for (int h = hk_lo * rep; h < hk_hi * rep; ++h) {
+      const int hk = h / rep;
+      const int64_t qoff = (((int64_t)b * N + t) * H + h) * D;
+      const float* qrow = q + qoff;
+      const float* dorow = d_out + qoff;
+      double m = -INFINITY;
+      for (int j = 0; j < w; ++j) {
+        const float* krow = k + (((int64_t)b * N + keyidx[j]) * Hkv + hk) * D;
+        double acc = 0.0;
+        for (int e = 0; e < D; ++e) acc += (double)qrow[e] * (double)krow[e];
+        prob[j] = acc * scale;
+        if (prob[j] > m) m = prob[j];
+      }
+      double sum = 0.0;
+      for (int j = 0; j < w; ++j) {
+        prob[j] = exp(prob[j] - m);
+        sum += prob[j];
+      }
+      double delta = 0.0;
+      for (int j = 0; j < w; ++j) {
+        prob[j] /= sum;
+        const float* vrow = v + (((int64_t)b * N + keyidx[j]) * Hkv + hk) * D;
+        double acc = 0.0;
+        for (int e = 0; e < D; ++e) acc += (double)dorow[e] * (double)vrow[e];
+        dprob[j] = acc;
+        delta += prob[j] * acc;
+      }
+      double* dqrow = dq + qoff;
+      for (int j = 0; j < w; ++j) {
+        const int64_t koff = (((int64_t)b * N + keyidx[j]) * Hkv + hk) * D;
+        const double ds = prob[j] * (dprob[j] - delta) * scale;
+        const float* krow = k + koff;
+        double* dkrow = dk + koff;
+        double* dvrow = dv + koff;
+        for (int e = 0; e < D; ++e) {
+          dqrow[e] += ds * (double)krow[e];
+          dkrow[e] += ds * (double)qrow[e];
+          dvrow[e] += prob[j] * (double)dorow[e];
+        }
+      }
+      visited += w;
+    }
+  }
+  free(prob);
+  free(dprob);
   free(keyidx);
   return visited;
 }

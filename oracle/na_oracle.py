@@ -240,6 +240,64 @@ def na_forward(
     return o.reshape(B, *shape, H, vf.shape[-1]), lse.reshape(B, *shape, H)
 
 
+def masked_attention_backward(q, k, v, d_out, mask: Optional[np.ndarray], scale: float):
+    """Gradients of sum(out * d_out) for `masked_attention`, float64, as dense matrix algebra:
+    P = softmax(scale q k^T + mask), dV = P^T dO, dP = dO V^T, dS = P * (dP - rowsum(P * dP)),
+    dQ = scale dS K, dK = scale dS^T Q  (fna_reference_backward.hpp:116-131, :231-246 evaluate
+    the same terms one pair at a time).  The gradient of the LSE output is not propagated."""
+    q = np.asarray(q, dtype=np.float64)
+    k = np.asarray(k, dtype=np.float64)
+    v = np.asarray(v, dtype=np.float64)
+    d_out = np.asarray(d_out, dtype=np.float64)
+    B, Nq, H, D = q.shape
+    Hkv = k.shape[2]
+    rep = H // Hkv
+    dq = np.zeros_like(q)
+    dk = np.zeros_like(k)
+    dv = np.zeros_like(v)
+    for b in range(B):
+        for h in range(H):
+            hk = h // rep
+            s = (q[b, :, h, :] @ k[b, :, hk, :].T) * scale
+            if mask is not None:
+                s = np.where(mask, s, -np.inf)
+            p = np.exp(s - s.max(axis=-1, keepdims=True))
+            p /= p.sum(axis=-1, keepdims=True)
+            dp = d_out[b, :, h, :] @ v[b, :, hk, :].T
+            ds = p * (dp - (p * dp).sum(axis=-1, keepdims=True)) * scale
+            dq[b, :, h, :] = ds @ k[b, :, hk, :]
+            dk[b, :, hk, :] += ds.T @ q[b, :, h, :]
+            dv[b, :, hk, :] += p.T @ d_out[b, :, h, :]
+    return dq, dk, dv
+
+
+def na_backward(q, k, v, d_out, kernel_size, stride=1, dilation=1, is_causal=False, scale: Optional[float] = None):
+    """Neighborhood attention backward on heads-last tensors [B, *X, H, D] -> (dQ, dK, dV)."""
+    q = np.asarray(q)
+    shape = q.shape[1:-2]
+    B, H, D = q.shape[0], q.shape[-2], q.shape[-1]
+    N = int(np.prod(shape))
+    scale = float(scale) if scale is not None else float(D) ** -0.5
+    mask = na_mask_dense(shape, kernel_size, stride, dilation, is_causal)
+    k = np.asarray(k)
+    v = np.asarray(v)
+    dq, dk, dv = masked_attention_backward(
+        q.reshape(B, N, H, D), k.reshape(B, N, k.shape[-2], D), v.reshape(B, N, v.shape[-2], v.shape[-1]),
+        np.asarray(d_out).reshape(B, N, H, v.shape[-1]), mask, scale)
+    return dq.reshape(q.shape), dk.reshape(k.shape), dv.reshape(v.shape)
+
+
+def attention_backward(q, k, v, d_out, is_causal=False, scale: Optional[float] = None):
+    """Dense attention backward [B, S, H, D] with optional top-left causal mask -> (dQ, dK, dV)."""
+    q = np.asarray(q)
+    k = np.asarray(k)
+    scale = float(scale) if scale is not None else float(q.shape[-1]) ** -0.5
+    mask = None
+    if is_causal:
+        mask = np.arange(q.shape[1])[:, None] >= np.arange(k.shape[1])[None, :]
+    return masked_attention_backward(q, k, v, d_out, mask, scale)
+
+
 def attention_forward(q, k, v, is_causal=False, scale: Optional[float] = None):
     """Dense attention [B, S, H, D] with optional top-left causal mask -> (O, LSE)."""
     q = np.asarray(q)
