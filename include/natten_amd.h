@@ -21,6 +21,11 @@
  *                                  kernel_size == input size)
  *   natten_amd_attention_forward_varlen <- the same function with cumulative_seqlen_Q / _KV,
  *                                  max_seqlen_Q / _KV (csrc/include/natten/blackwell_fmha.h:34-50)
+ *   natten_amd_fna_backward     <- blackwell_na{1,2,3}d_backward
+ *                                  csrc/include/natten/blackwell_fna.h:92-160
+ *   natten_amd_attention_backward <- blackwell_fmha_backward csrc/include/natten/blackwell_fmha.h:52-73
+ *                                  (fixed-length batches)
+ *   natten_amd_compute_delta    <- compute_delta            csrc/include/natten/compute_delta.h:33-36
  *   natten_amd_merge_attentions <- the elementwise merge of src/natten/attn_merge.py:48-105
  *                                  (the reference runs it as framework ops; here it is one kernel)
  */
@@ -140,6 +145,58 @@ int natten_amd_attention_forward_varlen(const void* q, const void* k, const void
                                         const int32_t* cumulative_seqlen_kv, int is_causal,
                                         float scale, const float* q_scale, const float* k_scale,
                                         const float* v_scale, void* stream);
+
+/*
+ * Host-only helper (no GPU work): the interval of query coordinates 0 .. num_queries-1 whose
+ * window meets the key coordinates key_first .. key_last of one dimension of `extent` keys:
+ * what the dK/dV kernel iterates over per KV tile (the role of get_trip_count in
+ * csrc/include/natten/cuda/fna_blackwell/collective/fna_fusion_bwd.hpp:256-318).  An empty
+ * interval comes back as *first_query > *last_query.
+ */
+int natten_amd_query_range(int key_first, int key_last, int kernel_size, int stride, int extent,
+                           int num_queries, int is_causal, int32_t* first_query,
+                           int32_t* last_query);
+
+/*
+ * delta[i] = sum_d out[i, d] * d_out[i, d] for `items` rows of head_dim contiguous elements
+ * (any layout whose last dimension is head_dim: items = batch * tokens * heads).  float32 result.
+ */
+int natten_amd_compute_delta(const void* out, const void* d_out, float* delta, int dtype,
+                             int64_t items, int head_dim, void* stream);
+
+/*
+ * Fused neighborhood attention backward on token-permuted operands.
+ *   q, d_out, dq [batch, seqlen_q, heads_q, head_dim]; k, v, dk, dv [batch, seqlen_kv, heads_kv,
+ *   head_dim]; lse, delta [batch, seqlen_q, heads_q] float32 (lse from the forward pass, natural
+ *   log; delta from natten_amd_compute_delta), all permuted like the forward operands
+ *   (dimension 0 fastest inside a tile, dilation groups folded into batch).
+ *   Both tile shapes must hold 128 tokens and their last extent above 1 must be even; q_shape /
+ *   kv_shape are the padded per-group layouts (multiples of the tiles), seqlen = their product.
+ * dq, dk, dv are written completely (padding rows get zeros); nothing is accumulated through
+ * memory, results are deterministic.  The gradient of the LSE output is not propagated (as in
+ * the reference).  16-bit float operands, head_dim 32 / 64 / 128.
+ */
+int natten_amd_fna_backward(const void* q, const void* k, const void* v, const void* d_out,
+                            const float* lse, const float* delta, void* dq, void* dk, void* dv,
+                            int dtype, int na_dim, int batch, int seqlen_q, int seqlen_kv,
+                            int heads_q, int heads_kv, int head_dim, const int32_t* q_shape,
+                            const int32_t* kv_shape, const int32_t* qkv_shape,
+                            const int32_t* kernel_size, const int32_t* stride,
+                            const int32_t* dilation, const int32_t* is_causal,
+                            const int32_t* q_tile_shape, const int32_t* kv_tile_shape, float scale,
+                            void* stream);
+
+/*
+ * Dense attention backward (optional top-left causal mask).  Operands as above with
+ * sequences zero-padded to padded_seqlen_q / padded_seqlen_kv rows (multiples of 128);
+ * seqlen_q / seqlen_kv are the true lengths.
+ */
+int natten_amd_attention_backward(const void* q, const void* k, const void* v, const void* d_out,
+                                  const float* lse, const float* delta, void* dq, void* dk,
+                                  void* dv, int dtype, int batch, int seqlen_q, int seqlen_kv,
+                                  int padded_seqlen_q, int padded_seqlen_kv, int heads_q,
+                                  int heads_kv, int head_dim, int is_causal, float scale,
+                                  void* stream);
 
 /*
  * Token permute: src [batch, *token_layout, heads, head_dim] -> dst

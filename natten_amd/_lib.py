@@ -19,7 +19,7 @@ from torch import Tensor
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libnatten_amd.so")
 
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 DTYPE_CODES = {
     torch.float16: 0,
@@ -60,6 +60,19 @@ _SIGNATURES = {
         ctypes.c_int,
         [ctypes.c_void_p] * 5 + [ctypes.c_int] * 9 + [ctypes.c_void_p] * 2 + [ctypes.c_int, ctypes.c_float]
         + [ctypes.c_void_p] * 4,
+    ),
+    "natten_amd_query_range": (ctypes.c_int, [ctypes.c_int] * 7 + [ctypes.c_void_p] * 2),
+    "natten_amd_compute_delta": (
+        ctypes.c_int,
+        [ctypes.c_void_p] * 3 + [ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_void_p],
+    ),
+    "natten_amd_fna_backward": (
+        ctypes.c_int,
+        [ctypes.c_void_p] * 9 + [ctypes.c_int] * 8 + [ctypes.c_void_p] * 9 + [ctypes.c_float, ctypes.c_void_p],
+    ),
+    "natten_amd_attention_backward": (
+        ctypes.c_int,
+        [ctypes.c_void_p] * 9 + [ctypes.c_int] * 10 + [ctypes.c_float, ctypes.c_void_p],
     ),
     "natten_amd_token_permute_widen": (
         ctypes.c_int,
@@ -283,6 +296,76 @@ def attention_forward_varlen(
         )
     _check(rc)
     return out, lse
+
+
+def query_range(key_first: int, key_last: int, kernel_size: int, stride: int, extent: int, num_queries: int,
+                is_causal: bool) -> Tuple[int, int]:
+    """(first, last) query coordinate whose window meets keys key_first .. key_last (host arithmetic only)."""
+    first, last = ctypes.c_int32(), ctypes.c_int32()
+    _check(lib().natten_amd_query_range(int(key_first), int(key_last), int(kernel_size), int(stride), int(extent),
+                                        int(num_queries), 1 if is_causal else 0, ctypes.byref(first),
+                                        ctypes.byref(last)))
+    return first.value, last.value
+
+
+def compute_delta(out: Tensor, d_out: Tensor) -> Tensor:
+    """rowsum(out * d_out) over the last dimension, float32, shape out.shape[:-1]."""
+    L = lib()
+    _require_gpu(out, d_out)
+    if out.dtype not in (torch.float16, torch.bfloat16) or d_out.dtype != out.dtype or d_out.shape != out.shape:
+        raise ValueError("compute_delta needs two fp16 / bf16 tensors of the same shape and dtype.")
+    delta = torch.empty(out.shape[:-1], dtype=torch.float32, device=out.device)
+    with torch.cuda.device(out.device):
+        rc = L.natten_amd_compute_delta(out.data_ptr(), d_out.data_ptr(), delta.data_ptr(), DTYPE_CODES[out.dtype],
+                                        delta.numel(), out.shape[-1], _stream(out))
+    _check(rc)
+    return delta
+
+
+def fna_backward(
+    q: Tensor, k: Tensor, v: Tensor, d_out: Tensor, lse: Tensor, delta: Tensor, kernel_size, stride, dilation,
+    is_causal, scale: float, q_shape, kv_shape, qkv_shape, q_tile_shape, kv_tile_shape,
+) -> Tuple[Tensor, Tensor, Tensor]:
+    """Backward on token-permuted operands (128-token tiles on both sides) -> (dq, dk, dv)."""
+    L = lib()
+    _require_gpu(q, k, v, d_out, lse, delta)
+    if q.dtype not in (torch.float16, torch.bfloat16):
+        raise NotImplementedError(f"natten_amd fna_backward does not support {q.dtype}.")
+    if lse.dtype != torch.float32 or delta.dtype != torch.float32:
+        raise ValueError("lse and delta must be float32.")
+    na_dim = len(kernel_size)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    with torch.cuda.device(q.device):
+        rc = L.natten_amd_fna_backward(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), d_out.data_ptr(), lse.data_ptr(), delta.data_ptr(),
+            dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), DTYPE_CODES[q.dtype], na_dim, q.shape[0], q.shape[1],
+            k.shape[1], q.shape[2], k.shape[2], q.shape[3], _i32(q_shape), _i32(kv_shape), _i32(qkv_shape),
+            _i32(kernel_size), _i32(stride), _i32(dilation), _i32([1 if c else 0 for c in is_causal]),
+            _i32(q_tile_shape), _i32(kv_tile_shape), float(scale), _stream(q),
+        )
+    _check(rc)
+    return dq, dk, dv
+
+
+def attention_backward(
+    q: Tensor, k: Tensor, v: Tensor, d_out: Tensor, lse: Tensor, delta: Tensor, seqlen_q: int, seqlen_kv: int,
+    is_causal: bool, scale: float,
+) -> Tuple[Tensor, Tensor, Tensor]:
+    """Dense attention backward on operands zero-padded to multiples of 128 rows -> (dq, dk, dv), padded alike."""
+    L = lib()
+    _require_gpu(q, k, v, d_out, lse, delta)
+    if q.dtype not in (torch.float16, torch.bfloat16):
+        raise NotImplementedError(f"natten_amd attention_backward does not support {q.dtype}.")
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    with torch.cuda.device(q.device):
+        rc = L.natten_amd_attention_backward(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), d_out.data_ptr(), lse.data_ptr(), delta.data_ptr(),
+            dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), DTYPE_CODES[q.dtype], q.shape[0], int(seqlen_q),
+            int(seqlen_kv), q.shape[1], k.shape[1], q.shape[2], k.shape[2], q.shape[3], 1 if is_causal else 0,
+            float(scale), _stream(q),
+        )
+    _check(rc)
+    return dq, dk, dv
 
 
 def _ceil_div(a: int, b: int) -> int:

@@ -38,4 +38,30 @@ NA_HD int na_window_end(int i, int start, int k, int L, bool causal) {
 // Number of tokens of dilation group g along a dimension of extent X.
 NA_HD int na_group_extent(int X, int d, int g) { return X / d + 1 - ((g + (d - X % d)) / d); }
 
+// The queries that attend key coordinates j0 .. j1 of a dimension form an interval, because
+// window start and end are non-decreasing in the query coordinate: its first element is the
+// first query whose window ends past j0, its last the last query whose window starts at or
+// before j1 (queries 0 .. Lq-1, keys of extent L).  Both by bisection.  An empty interval comes
+// back as first > last.
+NA_HD int na_first_query_attending(int j0, int k, int s, int L, int Lq, bool causal) {
+  int lo = 0, hi = Lq;  // answer in [lo, hi]; hi == Lq: none
+  while (lo < hi) {
+    const int mid = (lo + hi) / 2;
+    const int st = na_window_start(mid, k, s, L, causal);
+    if (na_window_end(mid, st, k, L, causal) > j0) hi = mid;
+    else lo = mid + 1;
+  }
+  return lo;
+}
+
+NA_HD int na_last_query_attending(int j1, int k, int s, int L, int Lq, bool causal) {
+  int lo = -1, hi = Lq - 1;  // answer in [lo, hi]; lo == -1: none
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) / 2;
+    if (na_window_start(mid, k, s, L, causal) <= j1) lo = mid;
+    else hi = mid - 1;
+  }
+  return lo;
+}
+
 }  // namespace natten_amd

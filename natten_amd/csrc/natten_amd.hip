@@ -11,6 +11,7 @@
 
 #include <type_traits>
 
+#include "fna_bwd.hpp"
 #include "fna_fwd.hpp"
 #include "fna_fwd_fp8.hpp"
 #include "merge.hpp"
@@ -191,7 +192,7 @@ int fill_fna_params(const char* what, FnaParams& p, int na_dim, const int* q_sha
 
 extern "C" {
 
-int natten_amd_abi_version(void) { return 3; }
+int natten_amd_abi_version(void) { return 4; }
 
 const char* natten_amd_last_error(void) { return g_error; }
 
@@ -414,6 +415,210 @@ int natten_amd_attention_forward_varlen(const void* q, const void* k, const void
   p.cu_kv = cumulative_seqlen_kv;
   set_wg_layout(p, 1);
   return dispatch_dtype(p, dtype, head_dim, QT, KVT, static_cast<hipStream_t>(stream));
+}
+
+// ---- backward ---------------------------------------------------------------------------------
+
+extern "C++" {
+template <typename T, int D>
+static int launch_bwd(const FnaBwdParams& p, hipStream_t stream) {
+  const long long wg_q = (long long)p.batch * p.heads_q * prod3(p.q_tiled);
+  const long long wg_kv = (long long)p.batch * p.heads_kv * prod3(p.kv_tiled);
+  if (wg_q > 0x7fffffffLL || wg_kv > 0x7fffffffLL) return fail("fna_backward: problem needs more than 2^31 workgroups");
+  hipLaunchKernelGGL((fna_bwd_kernel<T, D, false>), dim3((unsigned)wg_q), dim3(256), 0, stream, p);
+  if (int rc = check_launch("fna_backward (dQ)")) return rc;
+  hipLaunchKernelGGL((fna_bwd_kernel<T, D, true>), dim3((unsigned)wg_kv), dim3(256), 0, stream, p);
+  return check_launch("fna_backward (dK, dV)");
+}
+
+template <typename T>
+static int dispatch_bwd_head_dim(const FnaBwdParams& p, int head_dim, hipStream_t stream) {
+  switch (head_dim) {
+    case 32: return launch_bwd<T, 32>(p, stream);
+    case 64: return launch_bwd<T, 64>(p, stream);
+    case 128: return launch_bwd<T, 128>(p, stream);
+  }
+  return fail("fna_backward: head_dim must be 32, 64 or 128, got %d", head_dim);
+}
+
+static int dispatch_bwd(const FnaBwdParams& p, int dtype, int head_dim, hipStream_t stream) {
+  switch (dtype) {
+    case NATTEN_AMD_F16: return dispatch_bwd_head_dim<_Float16>(p, head_dim, stream);
+    case NATTEN_AMD_BF16: return dispatch_bwd_head_dim<__bf16>(p, head_dim, stream);
+  }
+  return fail("fna_backward: only 16-bit float operands are supported, got dtype code %d", dtype);
+}
+}  // extern "C++"
+
+// last dimension of extent > 1 (0 for a one-token tile)
+static int split_dim_of(const int* tile) {
+  int s = 0;
+  for (int a = 0; a < 3; ++a)
+    if (tile[a] > 1) s = a;
+  return s;
+}
+
+static int check_bwd_pointers(const char* what, const void* q, const void* k, const void* v, const void* d_out,
+                              const float* lse, const float* delta, void* dq, void* dk, void* dv) {
+  if (!q || !k || !v || !d_out || !lse || !delta || !dq || !dk || !dv) return fail("%s: null pointer argument", what);
+  const uintptr_t all = reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v) |
+                        reinterpret_cast<uintptr_t>(d_out) | reinterpret_cast<uintptr_t>(dq) |
+                        reinterpret_cast<uintptr_t>(dk) | reinterpret_cast<uintptr_t>(dv);
+  if (all & 15) return fail("%s: q, k, v, d_out, dq, dk and dv must be 16-byte aligned", what);
+  return 0;
+}
+
+int natten_amd_fna_backward(const void* q, const void* k, const void* v, const void* d_out, const float* lse,
+                            const float* delta, void* dq, void* dk, void* dv, int dtype, int na_dim, int batch,
+                            int seqlen_q, int seqlen_kv, int heads_q, int heads_kv, int head_dim,
+                            const int32_t* q_shape, const int32_t* kv_shape, const int32_t* qkv_shape,
+                            const int32_t* kernel_size, const int32_t* stride, const int32_t* dilation,
+                            const int32_t* is_causal, const int32_t* q_tile_shape, const int32_t* kv_tile_shape,
+                            float scale, void* stream) {
+  g_error[0] = 0;
+  const char* what = "fna_backward";
+  if (int rc = check_bwd_pointers(what, q, k, v, d_out, lse, delta, dq, dk, dv)) return rc;
+  if (int rc = check_common(what, q, k, v, dq, lse, batch, seqlen_q, seqlen_kv, heads_q, heads_kv, head_dim)) return rc;
+  if (na_dim < 1 || na_dim > 3) return fail("%s: na_dim must be 1, 2 or 3, got %d", what, na_dim);
+  if (!q_shape || !kv_shape || !qkv_shape || !kernel_size || !stride || !dilation || !is_causal || !q_tile_shape ||
+      !kv_tile_shape)
+    return fail("%s: null shape argument", what);
+  FnaParams f;
+  if (int rc = fill_fna_params(what, f, na_dim, q_shape, kv_shape, qkv_shape, kernel_size, stride, dilation, is_causal,
+                               q_tile_shape, kv_tile_shape))
+    return rc;
+  if (prod3(f.q_tile) != 128 || prod3(f.kv_tile) != 128)
+    return fail("%s: Q and KV tiles must hold 128 tokens each, got %d and %d", what, prod3(f.q_tile), prod3(f.kv_tile));
+  FnaBwdParams p;
+  memset(&p, 0, sizeof(p));
+  p.q_split = split_dim_of(f.q_tile);
+  p.kv_split = split_dim_of(f.kv_tile);
+  if (f.q_tile[p.q_split] % 2 != 0 || f.kv_tile[p.kv_split] % 2 != 0)
+    return fail("%s: the last tile extent above 1 must be even", what);
+  int groups = 1;
+  for (int a = 0; a < 3; ++a) {
+    p.qkv_shape[a] = f.qkv_shape[a];
+    p.ksize[a] = f.ksize[a];
+    p.stride[a] = f.stride[a];
+    p.dil[a] = f.dil[a];
+    p.causal[a] = f.causal[a];
+    p.q_tile[a] = f.q_tile[a];
+    p.kv_tile[a] = f.kv_tile[a];
+    p.q_tiled[a] = f.q_tiled[a];
+    p.kv_tiled[a] = f.kv_tiled[a];
+    groups *= f.dil[a];
+  }
+  if (batch % groups != 0) return fail("%s: batch (%d) must be a multiple of prod(dilation) (%d)", what, batch, groups);
+  if (seqlen_q != prod3(p.q_tiled) * 128 || seqlen_kv != prod3(p.kv_tiled) * 128)
+    return fail("%s: sequence lengths (%d, %d) do not match the padded layouts (%d, %d)", what, seqlen_q, seqlen_kv,
+                prod3(p.q_tiled) * 128, prod3(p.kv_tiled) * 128);
+  p.q = q;
+  p.k = k;
+  p.v = v;
+  p.d_out = d_out;
+  p.lse = lse;
+  p.delta = delta;
+  p.dq = dq;
+  p.dk = dk;
+  p.dv = dv;
+  p.batch = batch;
+  p.heads_q = heads_q;
+  p.heads_kv = heads_kv;
+  p.seqlen_q = seqlen_q;
+  p.seqlen_kv = seqlen_kv;
+  p.num_groups = groups;
+  p.q_extent0 = 0;
+  p.scale = scale;
+  return dispatch_bwd(p, dtype, head_dim, static_cast<hipStream_t>(stream));
+}
+
+int natten_amd_attention_backward(const void* q, const void* k, const void* v, const void* d_out, const float* lse,
+                                  const float* delta, void* dq, void* dk, void* dv, int dtype, int batch,
+                                  int seqlen_q, int seqlen_kv, int padded_seqlen_q, int padded_seqlen_kv, int heads_q,
+                                  int heads_kv, int head_dim, int is_causal, float scale, void* stream) {
+  g_error[0] = 0;
+  const char* what = "attention_backward";
+  if (int rc = check_bwd_pointers(what, q, k, v, d_out, lse, delta, dq, dk, dv)) return rc;
+  if (int rc = check_common(what, q, k, v, dq, lse, batch, seqlen_q, seqlen_kv, heads_q, heads_kv, head_dim)) return rc;
+  if (padded_seqlen_q % 128 != 0 || padded_seqlen_kv % 128 != 0 || padded_seqlen_q < seqlen_q ||
+      padded_seqlen_kv < seqlen_kv)
+    return fail("%s: padded sequence lengths (%d, %d) must be multiples of 128 that cover (%d, %d)", what,
+                padded_seqlen_q, padded_seqlen_kv, seqlen_q, seqlen_kv);
+  // the 1-D neighborhood problem whose window is the whole key sequence, with its own query count
+  FnaBwdParams p;
+  memset(&p, 0, sizeof(p));
+  for (int a = 0; a < 3; ++a) {
+    p.qkv_shape[a] = p.ksize[a] = p.stride[a] = p.dil[a] = p.q_tile[a] = p.kv_tile[a] = p.q_tiled[a] = p.kv_tiled[a] = 1;
+  }
+  p.qkv_shape[0] = seqlen_kv;
+  p.ksize[0] = seqlen_kv;
+  p.causal[0] = is_causal != 0;
+  p.q_tile[0] = p.kv_tile[0] = 128;
+  p.q_tiled[0] = padded_seqlen_q / 128;
+  p.kv_tiled[0] = padded_seqlen_kv / 128;
+  p.q_extent0 = seqlen_q;
+  p.q = q;
+  p.k = k;
+  p.v = v;
+  p.d_out = d_out;
+  p.lse = lse;
+  p.delta = delta;
+  p.dq = dq;
+  p.dk = dk;
+  p.dv = dv;
+  p.batch = batch;
+  p.heads_q = heads_q;
+  p.heads_kv = heads_kv;
+  p.seqlen_q = padded_seqlen_q;
+  p.seqlen_kv = padded_seqlen_kv;
+  p.num_groups = 1;
+  p.scale = scale;
+  return dispatch_bwd(p, dtype, head_dim, static_cast<hipStream_t>(stream));
+}
+
+int natten_amd_query_range(int key_first, int key_last, int kernel_size, int stride, int extent, int num_queries,
+                           int is_causal, int32_t* first_query, int32_t* last_query) {
+  g_error[0] = 0;
+  if (!first_query || !last_query) return fail("query_range: null pointer argument");
+  if (kernel_size < 1 || stride < 1 || extent < 1 || num_queries < 1 || kernel_size > extent || stride > kernel_size ||
+      key_first < 0 || key_last < key_first || key_last >= extent)
+    return fail("query_range: invalid argument");
+  *first_query = na_first_query_attending(key_first, kernel_size, stride, extent, num_queries, is_causal != 0);
+  *last_query = na_last_query_attending(key_last, kernel_size, stride, extent, num_queries, is_causal != 0);
+  return 0;
+}
+
+int natten_amd_compute_delta(const void* out, const void* d_out, float* delta, int dtype, int64_t items, int head_dim,
+                             void* stream) {
+  g_error[0] = 0;
+  if (!out || !d_out || !delta) return fail("compute_delta: null pointer argument");
+  if (items < 0) return fail("compute_delta: negative item count");
+  if ((reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(d_out)) & 15)
+    return fail("compute_delta: out and d_out must be 16-byte aligned");
+  if (items == 0) return 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+#define NA_DELTA_LAUNCH(TYPE, DD)                                                                              \
+  do {                                                                                                         \
+    const int64_t blocks = (items * ((DD) / 8) + 255) / 256;                                                   \
+    if (blocks > 0x7fffffffLL) return fail("compute_delta: too many rows");                                    \
+    hipLaunchKernelGGL((delta_kernel<TYPE, DD>), dim3((unsigned)blocks), dim3(256), 0, s,                      \
+                       static_cast<const TYPE*>(out), static_cast<const TYPE*>(d_out), delta, items);          \
+  } while (0)
+#define NA_DELTA_DTYPE(DD)                                              \
+  do {                                                                  \
+    if (dtype == NATTEN_AMD_F16) NA_DELTA_LAUNCH(_Float16, DD);         \
+    else if (dtype == NATTEN_AMD_BF16) NA_DELTA_LAUNCH(__bf16, DD);     \
+    else return fail("compute_delta: unsupported dtype code %d", dtype); \
+  } while (0)
+  switch (head_dim) {
+    case 32: NA_DELTA_DTYPE(32); break;
+    case 64: NA_DELTA_DTYPE(64); break;
+    case 128: NA_DELTA_DTYPE(128); break;
+    default: return fail("compute_delta: head_dim must be 32, 64 or 128, got %d", head_dim);
+  }
+#undef NA_DELTA_DTYPE
+#undef NA_DELTA_LAUNCH
+  return check_launch("compute_delta");
 }
 
 // widen: 0 = copy the payload, NATTEN_AMD_F8E4M3 / NATTEN_AMD_F8E5M2 = 8-bit float source, bf16 destination

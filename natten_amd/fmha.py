@@ -42,10 +42,20 @@ def amd_fmha(
         raise NotImplementedError(f"natten_amd attention supports head_dim <= 128, multiple of 8; got {head_dim}.")
     if is_fp8(query.dtype) and head_dim % 16 != 0:
         raise NotImplementedError(f"natten_amd attention needs head_dim % 16 == 0 for 8-bit floats; got {head_dim}.")
-    if torch.is_grad_enabled() and (query.requires_grad or key.requires_grad or value.requires_grad):
-        raise NotImplementedError("natten_amd implements the forward pass only; call it under torch.no_grad().")
     scale = scale or head_dim**-0.5
     d_pad = padded_head_dim(head_dim)
+    if torch.is_grad_enabled() and (query.requires_grad or key.requires_grad or value.requires_grad):
+        if is_fp8(query.dtype) or cumulative_seqlen_Q is not None:
+            raise NotImplementedError(
+                "natten_amd attention has a backward pass for fp16 / bf16 fixed-length batches only."
+            )
+        q, k, v = (pad_head_dim(t, d_pad) for t in (query, key, value))
+        out, lse = AmdFmhaFunction.apply(q, k, v, bool(is_causal), float(scale))
+        if d_pad != head_dim:
+            out = out[..., :head_dim]
+        if out_dtype is not None and out.dtype != out_dtype:
+            out = out.to(out_dtype)
+        return (out, lse) if return_lse else out
     q, k, v = (pad_head_dim(t.contiguous(), d_pad).contiguous() for t in (query, key, value))
     if is_fp8(query.dtype):
         # a one-token tile with no dilation is the identity permutation: a plain widening copy
@@ -75,3 +85,41 @@ def amd_fmha(
     if return_lse:
         return out, lse
     return out
+
+
+def _pad_rows(x: Tensor, rows: int) -> Tensor:
+    """Zero-pads dimension 1 to `rows`."""
+    if x.shape[1] == rows:
+        return x.contiguous()
+    pad = [0, 0] * (x.dim() - 2) + [0, rows - x.shape[1]]
+    return torch.nn.functional.pad(x, pad).contiguous()
+
+
+class AmdFmhaFunction(torch.autograd.Function):
+    """Dense attention with a backward pass (fp16 / bf16, fixed-length batches): the backward
+    kernels of neighborhood attention on the 1-D problem whose window is the whole key sequence,
+    sequences zero-padded to multiples of 128 rows.  Counterpart of the reference's
+    src/natten/backends/blackwell_fmha.py:52-170; the gradient of LSE is not propagated."""
+
+    @staticmethod
+    def forward(ctx, query, key, value, is_causal, scale):
+        with torch.no_grad():
+            out, lse = _lib.attention_forward(query.contiguous(), key.contiguous(), value.contiguous(), is_causal, scale)
+        ctx.save_for_backward(query, key, value, out, lse)
+        ctx.args = (is_causal, scale)
+        ctx.mark_non_differentiable(lse)
+        return out, lse
+
+    @staticmethod
+    def backward(ctx, d_out, d_lse):
+        query, key, value, out, lse = ctx.saved_tensors
+        is_causal, scale = ctx.args
+        d_out = d_out.contiguous()
+        delta = _lib.compute_delta(out.contiguous(), d_out)
+        sq, skv = query.shape[1], key.shape[1]
+        pq, pkv = -(-sq // 128) * 128, -(-skv // 128) * 128
+        dq, dk, dv = _lib.attention_backward(
+            _pad_rows(query, pq), _pad_rows(key, pkv), _pad_rows(value, pkv), _pad_rows(d_out, pq),
+            _pad_rows(lse, pq), _pad_rows(delta, pq), sq, skv, is_causal, scale,
+        )
+        return dq[:, :sq], dk[:, :skv], dv[:, :skv], None, None

@@ -1,7 +1,9 @@
-"""Driver of the MI355X fused neighborhood attention forward:
-token permute -> fused kernel -> token unpermute (output and LSE).
+"""Driver of the MI355X fused neighborhood attention:
+forward = token permute -> fused kernel -> token unpermute (output and LSE), or one launch on
+the original tensors; backward = delta, token permutes, the dQ and dK/dV kernels, unpermutes.
 
-Forward half of the reference's src/natten/backends/blackwell_fna.py:90-165 and :332-407.
+Counterpart of the reference's src/natten/backends/blackwell_fna.py:72-318 (autograd function)
+and :332-407 (driver).
 """
 
 from __future__ import annotations
@@ -13,7 +15,7 @@ from torch import Tensor
 
 from . import _lib, torch_ops
 from .checks import check_all_args, check_args_against_input, na_tensor_checks
-from .tile_config import check_fna_forward_config, padded_head_dim
+from .tile_config import check_fna_backward_config, check_fna_forward_config, padded_head_dim
 from .token_permute import token_permute_operation, token_unpermute_operation
 
 SUPPORTED_DTYPES = (torch.float16, torch.bfloat16, torch.float8_e4m3fn, torch.float8_e5m2)
@@ -69,9 +71,8 @@ def can_run_amd_fna(query: Tensor, key: Tensor, value: Tensor, raise_error: bool
         return no(f"natten_amd FNA supports head_dim <= 128 that is a multiple of 8, got {query.shape[-1]}.")
     if is_fp8(query.dtype) and query.shape[-1] % 16 != 0:
         return no(f"natten_amd FNA needs head dims that are multiples of 16 for 8-bit floats, got {query.shape[-1]}.")
-    if query.requires_grad or key.requires_grad or value.requires_grad:
-        if torch.is_grad_enabled():
-            return no("natten_amd implements the forward pass only; call it under torch.no_grad().")
+    if is_fp8(query.dtype) and torch.is_grad_enabled() and (query.requires_grad or key.requires_grad or value.requires_grad):
+        return no("natten_amd has no backward pass for 8-bit float operands.")
     return True
 
 
@@ -103,6 +104,8 @@ def amd_fna_generic(
     out_dtype: Optional[torch.dtype] = None,
     fused: Optional[bool] = None,
     fp8_matmul: Optional[bool] = None,
+    backward_q_tile_shape=None,
+    backward_kv_tile_shape=None,
 ) -> Union[Tensor, Tuple[Tensor, Tensor]]:
     """`fused` selects the one-launch path that gathers tiles from the original tensors (None:
     whenever the problem allows it); otherwise tokens are permuted, multiplied and unpermuted
@@ -127,6 +130,20 @@ def amd_fna_generic(
     if d_pad != head_dim:
         # zero columns change neither q.k nor the first head_dim output columns
         query, key, value = (_pad_head_dim(t, d_pad) for t in (query, key, value))
+
+    if torch.is_grad_enabled() and (query.requires_grad or key.requires_grad or value.requires_grad):
+        bwd_q_tile, bwd_kv_tile = check_fna_backward_config(
+            query, kernel_size, stride, dilation, is_causal, backward_q_tile_shape, backward_kv_tile_shape
+        )
+        output, lse = AmdFnaFunction.apply(
+            query, key, value, kernel_size, stride, dilation, is_causal, scale, q_tile_shape, kv_tile_shape,
+            bwd_q_tile, bwd_kv_tile, fused,
+        )
+        if d_pad != head_dim:
+            output = output[..., :head_dim]
+        if out_dtype is not None and output.dtype != out_dtype:
+            output = output.to(out_dtype)
+        return (output, lse) if return_lse else output
 
     in_dtype = query.dtype
     fp8_ok = (
@@ -188,3 +205,51 @@ def amd_fna_generic(
     if return_lse:
         return output, lse
     return output
+
+
+class AmdFnaFunction(torch.autograd.Function):
+    """Neighborhood attention with a backward pass (fp16 / bf16, head dims the kernels take).
+
+    Mirrors the reference's autograd function (src/natten/backends/blackwell_fna.py:72-318):
+    the forward saves q, k, v, out and LSE; the backward computes delta = rowsum(dO * O), permutes
+    q, dO, LSE, delta with the backward Q tile and k, v with the backward KV tile, runs the dQ and
+    the dK/dV kernels, and unpermutes the three gradients.  The gradient of the LSE output is
+    not propagated, as in the reference."""
+
+    @staticmethod
+    def forward(ctx, query, key, value, kernel_size, stride, dilation, is_causal, scale, q_tile_shape, kv_tile_shape,
+                bwd_q_tile_shape, bwd_kv_tile_shape, fused):
+        with torch.no_grad():
+            output, lse = amd_fna_generic(
+                query, key, value, kernel_size, stride, dilation, is_causal, scale, q_tile_shape, kv_tile_shape,
+                return_lse=True, fused=fused,
+            )
+        ctx.save_for_backward(query, key, value, output, lse)
+        ctx.na_args = (kernel_size, stride, dilation, is_causal, scale, bwd_q_tile_shape, bwd_kv_tile_shape)
+        ctx.mark_non_differentiable(lse)
+        return output, lse
+
+    @staticmethod
+    def backward(ctx, d_output, d_lse):
+        query, key, value, output, lse = ctx.saved_tensors
+        kernel_size, stride, dilation, is_causal, scale, q_tile, kv_tile = ctx.na_args
+        d_output = d_output.contiguous()
+        delta = _lib.compute_delta(output.contiguous(), d_output)
+
+        def perm(x, tile):
+            return token_permute_operation(x.contiguous(), tile, dilation, flip_tiled_dims=True)
+
+        q_perm, qkv_shape, q_shape = perm(query, q_tile)
+        do_perm, _, _ = perm(d_output, q_tile)
+        lse_perm, _, _ = perm(lse.unsqueeze(-1), q_tile)
+        delta_perm, _, _ = perm(delta.unsqueeze(-1), q_tile)
+        k_perm, _, kv_shape = perm(key, kv_tile)
+        v_perm, _, _ = perm(value, kv_tile)
+        dq_perm, dk_perm, dv_perm = _lib.fna_backward(
+            q_perm, k_perm, v_perm, do_perm, lse_perm.squeeze(-1).contiguous(), delta_perm.squeeze(-1).contiguous(),
+            kernel_size, stride, dilation, is_causal, scale, q_shape, kv_shape, qkv_shape, q_tile, kv_tile,
+        )
+        dq = token_unpermute_operation(dq_perm, qkv_shape, q_tile, dilation, flip_tiled_dims=True)
+        dk = token_unpermute_operation(dk_perm, qkv_shape, kv_tile, dilation, flip_tiled_dims=True)
+        dv = token_unpermute_operation(dv_perm, qkv_shape, kv_tile, dilation, flip_tiled_dims=True)
+        return (dq, dk, dv) + (None,) * 10

@@ -127,6 +127,13 @@ def neighborhood_attention_generic(
         raise NotImplementedError(f"Unrecognized backend {backend}; natten_amd provides '{_BACKEND_FNA}'.")
 
     has_additional_attention = additional_keys is not None and additional_values is not None
+    if has_additional_attention and torch.is_grad_enabled() and any(
+        t.requires_grad for t in (query, key, value, additional_keys, additional_values)
+    ):
+        raise NotImplementedError(
+            "natten_amd has no backward pass through the merge with additional keys / values; "
+            "call it under torch.no_grad()."
+        )
     attn_kwargs = dict(attention_kwargs or {})
     attn_kwargs.pop("torch_compile", None)
 
@@ -158,6 +165,7 @@ def neighborhood_attention_generic(
         scale=scale, q_tile_shape=q_tile_shape, kv_tile_shape=kv_tile_shape, return_lse=True,
         q_scale=q_scale, k_scale=k_scale, v_scale=v_scale,
         out_dtype=work_dtype if has_additional_attention else final_dtype, fp8_matmul=fp8_matmul,
+        backward_q_tile_shape=backward_q_tile_shape, backward_kv_tile_shape=backward_kv_tile_shape,
     )
 
     if has_additional_attention:

@@ -122,6 +122,44 @@ def check_fna_forward_config(
     return q_tile_shape, kv_tile_shape
 
 
+BACKWARD_TILE_SIZE = 128  # tokens per Q tile and per KV tile of the backward kernels
+
+
+def check_fna_backward_config(
+    input_tensor: torch.Tensor, kernel_size: DimensionType, stride: DimensionType, dilation: DimensionType,
+    is_causal: Tuple[bool, ...], q_tile_shape: Optional[DimensionType] = None,
+    kv_tile_shape: Optional[DimensionType] = None,
+) -> Tuple[DimensionType, DimensionType]:
+    """Validate user tile shapes of the backward pass or choose defaults (the role of the reference's
+    check_cutlass_blackwell_fna_backward_config, src/natten/backends/configs/checks.py).  Both tiles
+    hold 128 tokens; the last extent above 1 must be even (the other role streams half tiles)."""
+    na_dim = input_tensor.dim() - 3
+    layout = tuple(int(x) for x in input_tensor.shape[1 : 1 + na_dim])
+    if (q_tile_shape is None) != (kv_tile_shape is None):
+        raise ValueError("`backward_q_tile_shape` and `backward_kv_tile_shape` must be given together or not at all.")
+    if q_tile_shape is None:
+        return choose_tile_shapes(layout, tuple(kernel_size), tuple(stride), tuple(dilation), tuple(is_causal),
+                                  BACKWARD_TILE_SIZE, BACKWARD_TILE_SIZE)
+    from .checks import check_tile_shape
+
+    q_tile_shape = check_tile_shape(q_tile_shape, na_dim, "backward_q_tile_shape")
+    kv_tile_shape = check_tile_shape(kv_tile_shape, na_dim, "backward_kv_tile_shape")
+    for name, t in (("backward_q_tile_shape", q_tile_shape), ("backward_kv_tile_shape", kv_tile_shape)):
+        last = [x for x in t if x > 1]
+        if math.prod(t) != BACKWARD_TILE_SIZE or not last or last[-1] % 2 != 0:
+            raise ValueError(
+                f"Unsupported {name}={t}: backward tiles hold {BACKWARD_TILE_SIZE} tokens and their last extent "
+                "above 1 must be even."
+            )
+    return q_tile_shape, kv_tile_shape
+
+
+def get_all_backward_tile_shapes(na_dim: int) -> List[Tuple[DimensionType, DimensionType]]:
+    """Every legal (backward_q_tile_shape, backward_kv_tile_shape) of power-of-two extents."""
+    shapes = _factorisations(BACKWARD_TILE_SIZE, na_dim)
+    return [(qt, kt) for qt in shapes for kt in shapes]
+
+
 def get_all_tile_shapes(na_dim: int) -> List[Tuple[DimensionType, DimensionType]]:
     """Every legal (q_tile_shape, kv_tile_shape) for an na_dim-dimensional problem."""
     out = []

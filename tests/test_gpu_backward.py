@@ -1,0 +1,171 @@
+"""GPU parity of the backward pass: gradients from the public API (autograd function over the
+C ABI: delta, token permutes, dQ and dK/dV kernels) against the CPU oracle's float64 gradients on
+the same (already rounded) inputs, with q, k, v, dO ~ N(0, 1).
+
+Tolerance: fp16 atol = rtol = 1e-2; bf16 atol = rtol = 2e-2.  The kernels round P and
+dS = P (dP - delta) to the operand type before the second matrix product, as the reference's
+kernels do; |dP| ~ sqrt(head_dim), so one bf16 rounding of dS (2^-9 relative) is worth up to
+~1e-2 in a gradient whose window holds few keys.  The reference's own bar is atol 1e-2, rtol 0
+on gradients twenty times smaller (dO ~ 0.05 N(0, 1): tests/test_blackwell_fna.py:104-109,
+tests/utils.py:117-120), i.e. ten times looser than this one."""
+
+import numpy as np
+import pytest
+import torch
+
+import natten_amd
+from natten_amd.tile_config import get_all_backward_tile_shapes
+from oracle import c_oracle
+from oracle import na_oracle as O
+from tests.gpu_utils import assert_close, make_qkv, to_np, tuplify
+
+pytestmark = pytest.mark.gpu
+
+NA = {1: natten_amd.na1d, 2: natten_amd.na2d, 3: natten_amd.na3d}
+TOL = {torch.float16: 1e-2, torch.bfloat16: 2e-2}
+
+
+def run_backward(B, H, Hkv, D, shape, k, s, d, causal, dtype, bq=None, bkv=None, seed=0):
+    n = len(shape)
+    k, s, d, causal = (tuplify(x, n) for x in (k, s, d, causal))
+    q, kk, v = make_qkv(B, shape, H, Hkv, D, dtype, seed=seed)
+    gen = torch.Generator().manual_seed(seed + 1000)
+    d_out = torch.randn(q.shape, generator=gen).to(dtype).cuda()
+    q.requires_grad_(True)
+    kk.requires_grad_(True)
+    v.requires_grad_(True)
+    out = NA[n](q, kk, v, k, s, d, causal, backward_q_tile_shape=bq, backward_kv_tile_shape=bkv)
+    out.backward(d_out)
+    torch.cuda.synchronize()
+    ref = c_oracle.na_backward(to_np(q), to_np(kk), to_np(v), to_np(d_out), k, s, d, causal)
+    tag = f"{shape} k={k} s={s} d={d} c={causal} H={H}/{Hkv} D={D} {dtype} tiles={bq},{bkv}"
+    for name, got, r in zip(("dq", "dk", "dv"), (q.grad, kk.grad, v.grad), ref):
+        assert got is not None and got.dtype == dtype and got.shape == r.shape, name
+        assert_close(f"{name} {tag}", to_np(got), r, atol=TOL[dtype], rtol=TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_backward_1d(dtype):
+    run_backward(1, 2, 2, 32, (256,), 7, 1, 1, False, dtype)
+    run_backward(2, 4, 2, 64, (300,), 33, 4, 2, True, dtype, seed=1)
+    run_backward(1, 2, 1, 128, (77,), 9, 3, 1, False, dtype, seed=2)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_backward_2d(dtype):
+    run_backward(2, 2, 2, 64, (20, 24), (5, 7), (2, 1), (1, 2), (False, True), dtype, seed=3)
+    run_backward(1, 4, 1, 128, (32, 32), (13, 13), (1, 1), (1, 1), (False, False), dtype, seed=4)
+    run_backward(1, 2, 2, 48, (17, 19), (4, 6), (2, 3), (2, 1), (True, True), dtype, seed=5)  # head_dim padded to 64
+
+
+def test_backward_3d():
+    run_backward(1, 2, 1, 64, (9, 16, 24), (4, 8, 8), (1, 8, 4), 1, (True, False, False), torch.bfloat16, seed=6)
+    run_backward(1, 2, 2, 32, (6, 10, 9), (3, 4, 5), (1, 2, 2), (2, 1, 1), (False, True, False), torch.float16, seed=7)
+    run_backward(2, 1, 1, 128, (8, 8, 8), (3, 3, 3), 1, 1, False, torch.bfloat16, seed=8)
+
+
+def test_backward_every_tile_shape_2d():
+    for i, (bq, bkv) in enumerate(get_all_backward_tile_shapes(2)):
+        if i % 3 == 0:  # a third of the 64 pairs: every Q shape and every KV shape occurs
+            run_backward(1, 2, 1, 32, (40, 36), (9, 6), (2, 1), (1, 2), (True, False), torch.bfloat16, bq, bkv, seed=i)
+
+
+def test_backward_tile_shapes_3d():
+    for bq, bkv in [((2, 8, 8), (2, 8, 8)), ((1, 8, 16), (4, 4, 8)), ((8, 4, 4), (1, 2, 64)), ((128, 1, 1), (1, 128, 1))]:
+        run_backward(1, 2, 2, 64, (10, 12, 20), (4, 5, 6), (1, 2, 3), 1, (True, False, False), torch.float16, bq, bkv, seed=9)
+
+
+def test_backward_random_sweep():
+    rng = np.random.default_rng(77)
+    done = 0
+    while done < 16:
+        n = int(rng.integers(1, 4))
+        shape = tuple(int(rng.integers(4, {1: 300, 2: 36, 3: 12}[n])) for _ in range(n))
+        d = tuple(int(rng.integers(1, max(2, x // 4 + 1))) for x in shape)
+        if any(x // dd < 2 for x, dd in zip(shape, d)):
+            continue
+        k = tuple(int(rng.integers(2, x // dd + 1)) for x, dd in zip(shape, d))
+        if all(kk * dd == x for kk, dd, x in zip(k, d, shape)) and n > 1:
+            continue
+        s = tuple(int(rng.integers(1, kk + 1)) for kk in k)
+        causal = tuple(bool(rng.integers(0, 2)) for _ in range(n))
+        Hkv = int(rng.choice([1, 2]))
+        H = Hkv * int(rng.choice([1, 2]))
+        D = int(rng.choice([32, 64, 128]))
+        run_backward(1, H, Hkv, D, shape, k, s, d, causal, [torch.bfloat16, torch.float16][done % 2], seed=done)
+        done += 1
+
+
+ATTN_CASES = [
+    # B, Sq, Skv, H, Hkv, D, causal
+    (2, 128, 128, 2, 2, 64, False),
+    (1, 125, 300, 2, 1, 128, False),
+    (1, 300, 125, 4, 2, 32, True),   # top-left causal, more queries than keys
+    (1, 77, 77, 3, 3, 64, True),
+    (1, 5, 1, 2, 2, 64, False),
+    (1, 130, 9, 4, 2, 48, False),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_attention_backward(dtype):
+    for i, (B, Sq, Skv, H, Hkv, D, causal) in enumerate(ATTN_CASES):
+        gen = torch.Generator().manual_seed(i)
+        q = torch.randn((B, Sq, H, D), generator=gen).to(dtype).cuda().requires_grad_(True)
+        k = torch.randn((B, Skv, Hkv, D), generator=gen).to(dtype).cuda().requires_grad_(True)
+        v = torch.randn((B, Skv, Hkv, D), generator=gen).to(dtype).cuda().requires_grad_(True)
+        d_out = torch.randn((B, Sq, H, D), generator=gen).to(dtype).cuda()
+        out, lse = natten_amd.attention(q, k, v, is_causal=causal, return_lse=True)
+        out.backward(d_out)
+        ref = O.attention_backward(to_np(q), to_np(k), to_np(v), to_np(d_out), is_causal=causal)
+        tag = f"attention {(B, Sq, Skv, H, Hkv, D, causal)} {dtype}"
+        for name, got, r in zip(("dq", "dk", "dv"), (q.grad, k.grad, v.grad), ref):
+            assert_close(f"{name} {tag}", to_np(got), r, atol=TOL[dtype], rtol=TOL[dtype])
+
+
+def test_full_window_backward_takes_the_attention_path():
+    q, kk, v = make_qkv(1, (8, 12), 2, 2, 64, torch.float16, seed=3)
+    d_out = torch.randn(q.shape, generator=torch.Generator().manual_seed(5)).to(q.dtype).cuda()
+    for t in (q, kk, v):
+        t.requires_grad_(True)
+    natten_amd.na2d(q, kk, v, (8, 12)).backward(d_out)
+    ref = O.na_backward(to_np(q), to_np(kk), to_np(v), to_np(d_out), (8, 12))
+    for name, got, r in zip(("dq", "dk", "dv"), (q.grad, kk.grad, v.grad), ref):
+        assert_close(name, to_np(got), r)
+
+
+def test_compute_delta_matches_numpy():
+    from natten_amd import _lib
+
+    for D in (32, 64, 128):
+        gen = torch.Generator().manual_seed(D)
+        o = torch.randn((3, 37, 5, D), generator=gen).to(torch.bfloat16).cuda()
+        do = torch.randn((3, 37, 5, D), generator=gen).to(torch.bfloat16).cuda()
+        got = _lib.compute_delta(o, do)
+        ref = (to_np(o).astype(np.float64) * to_np(do)).sum(-1)
+        assert got.dtype == torch.float32 and got.shape == o.shape[:-1]
+        assert_close(f"delta D={D}", to_np(got), ref, atol=1e-4, rtol=1e-5)
+
+
+def test_backward_is_deterministic():
+    q, kk, v = make_qkv(1, (24, 24), 2, 1, 64, torch.bfloat16, seed=11)
+    d_out = torch.randn(q.shape, generator=torch.Generator().manual_seed(12)).to(q.dtype).cuda()
+    grads = []
+    for _ in range(2):
+        qq, k2, v2 = (t.clone().requires_grad_(True) for t in (q, kk, v))
+        natten_amd.na2d(qq, k2, v2, (7, 5), (2, 1), is_causal=(True, False)).backward(d_out)
+        grads.append((qq.grad, k2.grad, v2.grad))
+    for a, b in zip(*grads):
+        assert torch.equal(a, b)
+
+
+def test_backward_argument_errors():
+    q, kk, v = make_qkv(1, (16, 16), 2, 2, 32, torch.bfloat16, seed=0)
+    q.requires_grad_(True)
+    with pytest.raises(ValueError):
+        natten_amd.na2d(q, kk, v, 3, backward_q_tile_shape=(8, 8), backward_kv_tile_shape=(8, 16))
+    with pytest.raises(ValueError):
+        natten_amd.na2d(q, kk, v, 3, backward_q_tile_shape=(8, 16))
+    ak = torch.zeros(1, 5, 2, 32, dtype=torch.bfloat16).cuda()
+    with pytest.raises(NotImplementedError):
+        natten_amd.na2d(q, kk, v, 3, additional_keys=ak, additional_values=ak)

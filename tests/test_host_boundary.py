@@ -5,6 +5,7 @@ import ctypes
 import os
 import re
 
+import numpy as np
 import pytest
 import torch
 
@@ -110,3 +111,26 @@ def test_cpu_tensors_are_rejected_not_emulated():
         natten_amd.attention(q.flatten(1, 2), q.flatten(1, 2), q.flatten(1, 2))
     with pytest.raises(RuntimeError):
         natten_amd.token_permute_operation(q, (4, 4))
+
+
+def test_query_range_matches_brute_force():
+    """The interval of queries whose window meets a run of keys (what the dK/dV kernel iterates
+    over): the library's bisection against an exhaustive scan with the oracle's window functions."""
+    from natten_amd import _lib
+    from oracle import na_oracle as O
+
+    rng = np.random.default_rng(5)
+    cases = [(L, k, s, c) for L in (1, 2, 7, 16, 33) for k in range(1, L + 1) for s in range(1, k + 1) for c in (False, True)
+             if not (k == 1 and L > 1)]
+    for L, k, s, c in cases:
+        win = [(int(O.window_start(q, k, s, L, c)),) for q in range(L)]
+        win = [(st, int(O.window_end(q, st, k, L, c))) for q, (st,) in enumerate(win)]
+        for _ in range(6):
+            j0 = int(rng.integers(0, L))
+            j1 = int(rng.integers(j0, min(L, j0 + 9)))
+            hits = [q for q, (st, en) in enumerate(win) if en > j0 and st <= j1]
+            first, last = _lib.query_range(j0, j1, k, s, L, L, c)
+            if hits:
+                assert (first, last) == (hits[0], hits[-1]), (L, k, s, c, j0, j1)
+            else:
+                assert first > last, (L, k, s, c, j0, j1)
