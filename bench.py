@@ -118,6 +118,110 @@ def torch_idx(a):
     return torch.as_tensor(a, dtype=torch.long)
 
 
+def bench_backward(args, q, k, v, kernel, stride, dilation, causal, dt_name):
+    """Secondary measurement: one step = forward + backward through the public API; the backward
+    kernels (dQ role + dK/dV role of fna_bwd_kernel) are timed on their own with HIP events.
+    Work is counted as 2.5 x the forward's algorithmic FLOP (five matrix products against two)."""
+    import torch
+
+    import natten_amd
+    from natten_amd import _lib
+    from natten_amd.tile_config import check_fna_backward_config
+    from natten_amd.token_permute import token_permute_operation
+
+    n = q.dim() - 3
+    B, H, D = q.shape[0], q.shape[-2], q.shape[-1]
+    layout = tuple(q.shape[1 : 1 + n])
+    na = {1: natten_amd.na1d, 2: natten_amd.na2d, 3: natten_amd.na3d}[n]
+    q_tile = tuple(int(x) for x in args.q_tile.split(",")) if args.q_tile else None
+    kv_tile = tuple(int(x) for x in args.kv_tile.split(",")) if args.kv_tile else None
+    q_tile, kv_tile = check_fna_backward_config(q, kernel, stride, dilation, causal, q_tile, kv_tile)
+    gen = torch.Generator().manual_seed(1)
+    d_out = torch.randn(q.shape, generator=gen).to(q.dtype).to(q.device)
+    q, k, v = (t.clone().requires_grad_(True) for t in (q, k, v))
+
+    def step():
+        q.grad = k.grad = v.grad = None
+        out = na(q, k, v, kernel, stride, dilation, causal, backward_q_tile_shape=q_tile,
+                 backward_kv_tile_shape=kv_tile)
+        out.backward(d_out)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    with torch.no_grad():
+        out, lse = na(q, k, v, kernel, stride, dilation, causal, return_lse=True)
+        delta = _lib.compute_delta(out, d_out)
+
+        def perm(x, t):
+            return token_permute_operation(x.contiguous(), t, dilation, flip_tiled_dims=True)
+
+        qp, qkv_shape, q_shape = perm(q, q_tile)
+        dop = perm(d_out, q_tile)[0]
+        lp = perm(lse.unsqueeze(-1), q_tile)[0].squeeze(-1).contiguous()
+        dp = perm(delta.unsqueeze(-1), q_tile)[0].squeeze(-1).contiguous()
+        kp, _, kv_shape = perm(k, kv_tile)
+        vp = perm(v, kv_tile)[0]
+
+        def kern():
+            return _lib.fna_backward(qp, kp, vp, dop, lp, dp, kernel, stride, dilation, causal, D**-0.5, q_shape,
+                                     kv_shape, qkv_shape, q_tile, kv_tile)
+
+        for _ in range(2):
+            kern()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(args.steps):
+            kern()
+        e1.record()
+        torch.cuda.synchronize()
+        kernel_ms = e0.elapsed_time(e1) / args.steps
+    fwd_flops = 4.0 * B * H * D * count_attended(layout, kernel, stride, dilation, causal)
+    achieved = 2.5 * fwd_flops / (kernel_ms * 1e-3) / 1e12
+    peak = PEAK_TFLOPS[dt_name]
+    print(json.dumps({
+        "metric": "FNA fwd+bwd ms per step and effective TFLOP/s of the backward kernels, 1 GPU",
+        "value": 3.5 * fwd_flops / (ms_per_step * 1e-3) / 1e12,
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": dt_name,
+        "data": "synthetic",
+        "config": {
+            "workload": WORKLOAD_NAMES[args.workload] + ", forward + backward",
+            "backward_q_tile_shape": list(q_tile),
+            "backward_kv_tile_shape": list(kv_tile),
+            "path": "forward (one launch when the layout allows) + delta + token permutes + dQ and dK/dV kernels + unpermutes",
+        },
+        "na_flop_per_step": 3.5 * fwd_flops,
+        "backward_kernels_ms": kernel_ms,
+        "roofline": {
+            "kernel": "fna_bwd_kernel (dQ role + dK/dV role)",
+            "bound": "mfma",
+            "achieved": achieved,
+            "peak": peak,
+            "unit": "TFLOP/s",
+            "frac": achieved / peak,
+            "traffic": None,
+            "algorithmic_flop": 2.5 * fwd_flops,
+        },
+        "cpu_baseline": None,
+    }), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -126,6 +230,8 @@ def main():
     ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS))
     ap.add_argument("--q-tile", type=str, default=None, help="comma separated, e.g. 2,8,8")
     ap.add_argument("--kv-tile", type=str, default=None)
+    ap.add_argument("--backward", action="store_true",
+                    help="measure the backward pass (forward + backward step, backward kernels) instead of the forward metric")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-mfma-probe", action="store_true")
     args = ap.parse_args()
@@ -166,6 +272,13 @@ def main():
     q_tile = tuple(int(x) for x in args.q_tile.split(",")) if args.q_tile else None
     kv_tile = tuple(int(x) for x in args.kv_tile.split(",")) if args.kv_tile else None
     q_tile, kv_tile = check_fna_forward_config(q, kernel, stride, dilation, causal, q_tile, kv_tile)
+
+    if args.backward:
+        if quantised:
+            print("bench.py: there is no backward pass for 8-bit float operands.", file=sys.stderr)
+            sys.exit(2)
+        bench_backward(args, q, k, v, kernel, stride, dilation, causal, dt_name)
+        return
 
     def step():
         if quantised:

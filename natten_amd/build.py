@@ -18,6 +18,9 @@ HIPCC_FLAGS = [
     "-fPIC",
     # keep the compiler from forming packed-fp32 VALU instructions
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # matrix instructions accumulate in ordinary vector registers: kernels that run one wave per
+    # SIMD otherwise shuttle their accumulators to and from the accumulation registers every iteration
+    "-mllvm", "-amdgpu-mfma-vgpr-form=1",
 ]
 
 

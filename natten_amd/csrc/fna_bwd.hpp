@@ -1,18 +1,20 @@
 // Fused neighborhood attention backward for gfx950 (MI355X).
 //
-// One kernel template, two roles.  A workgroup owns a "stationary" tile of 128 rows (one row
-// per lane and 32-row block, four waves) and streams 64-row tiles of the other side through
-// LDS:
-//   dQ role  : stationary = queries (operands Q, dO; result dQ), streamed = keys (K, V)
-//   dKV role : stationary = keys    (operands K, V; results dK, dV), streamed = queries (Q, dO)
+// One kernel template, several roles.  A workgroup owns a "stationary" tile of 128 rows (one
+// row per lane and 32-row block, four waves) and streams 64-row tiles of the other side
+// through LDS:
+//   dQ role     : stationary = queries (operands Q, dO; result dQ), streamed = keys (K, V)
+//   dK, dV, dKV : stationary = keys    (operands K, V; results dK and / or dV), streamed = queries (Q, dO)
 // Per streamed tile, with Y1/Y2 the streamed and X1/X2 the stationary operands:
 //   S^T  = Y1 X1^T,  dP^T = Y2 X2^T                     (32x32x16 MFMA, the lane owns a stationary row)
 //   P    = exp2(c S - log2e LSE) on unmasked pairs, 0 elsewhere;  dS = P (dP - delta)
 //   acc1^T += Y1^T dS^T   (dQ = scale * sum_k dS k  /  dK = scale * sum_q dS q)
-//   acc2^T += Y2^T P^T    (dKV role only: dV = sum_q P dO)
-// LSE and delta = rowsum(dO * O) belong to the query: per-lane scalars in the dQ role, a small
-// per-tile LDS table in the dKV role.  Nothing is accumulated through memory, so both results
-// are deterministic.
+//   acc2^T += Y2^T P^T    (dV = sum_q P dO)
+// The dK and dV roles exist next to the combined one because at head dim 128 the combined
+// accumulators, stationary fragments and both products no longer fit the 256 vector registers
+// a matrix instruction can address directly.  LSE and delta = rowsum(dO * O) belong to the
+// query: per-lane scalars in the dQ role, a small per-tile LDS table in the others.  Nothing
+// is accumulated through memory, so the results are deterministic.
 //
 // What it restates (not the code): SHI-Labs/NATTEN
 //   csrc/include/natten/cuda/reference/fna_reference_backward.hpp:60-150, :165-265, :282-380
@@ -50,9 +52,14 @@ struct FnaBwdParams {
   float scale;
 };
 
-template <typename T, int D, bool KV_STATIONARY>
+enum BwdRole : int { kBwdDQ = 0, kBwdDK = 1, kBwdDV = 2, kBwdDKV = 3 };
+
+template <typename T, int D, int ROLE>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
 fna_bwd_kernel(const FnaBwdParams p) {
+  constexpr bool KV_STATIONARY = ROLE != kBwdDQ;
+  constexpr bool HAS_DS = ROLE != kBwdDV;                    // dP, dS and acc1 (dQ or dK)
+  constexpr bool HAS_PV = ROLE == kBwdDV || ROLE == kBwdDKV;  // acc2 (dV)
   constexpr int NT = 256;
   constexpr int AT = 128;  // stationary rows
   constexpr int BT = 64;   // streamed rows per tile
@@ -66,18 +73,30 @@ fna_bwd_kernel(const FnaBwdParams p) {
   constexpr int CHUNKS = BT * CPR;
   constexpr int PER = CHUNKS / NT;
   static_assert(CHUNKS % NT == 0 && PER >= 1, "a streamed tile must be a whole number of workgroup-wide copies");
+  static_assert(NSB == 2, "the slot schedule is written for two 32-row sub-blocks");
   using M = Mma<T>;
   using vec8 = typename M::vec8;
+  using vec2 = typename M::vec2;
 
-  // two stages of: Y1 in the layout of b128 row reads, Y1 in the layout of transpose reads, Y2 likewise
-  __shared__ __attribute__((aligned(1024))) char sY1k[2 * TILE_BYTES];
-  __shared__ __attribute__((aligned(1024))) char sY1t[2 * TILE_BYTES];
-  __shared__ __attribute__((aligned(1024))) char sY2k[2 * TILE_BYTES];
-  __shared__ __attribute__((aligned(1024))) char sY2t[KV_STATIONARY ? 2 * TILE_BYTES : 1024];
-  __shared__ __attribute__((aligned(16))) uint32_t sTabA[2 * BT];
-  __shared__ __attribute__((aligned(16))) uint32_t sTabB[2 * BT];
-  __shared__ __attribute__((aligned(16))) float sLse[2 * BT];
-  __shared__ __attribute__((aligned(16))) float sDelta[2 * BT];
+  // Tile copies per stage: Y1 in the layout of b128 row reads (for S), Y1 in the layout of
+  // transpose reads (for acc1), Y2 in row layout (for dP), Y2 in transpose layout (for acc2).
+#ifndef NA_BWD_DV_STAGES
+#define NA_BWD_DV_STAGES 2
+#endif
+  constexpr int NS = (ROLE == kBwdDKV && D == 128) ? 2 : (ROLE == kBwdDV ? NA_BWD_DV_STAGES : 3);  // stages: tiles are copied NS - 1 ahead
+  constexpr int SZ_1K = NS * TILE_BYTES;
+  constexpr int SZ_1T = HAS_DS ? NS * TILE_BYTES : 1024;
+  constexpr int SZ_2K = HAS_DS ? NS * TILE_BYTES : 1024;
+  constexpr int SZ_2T = HAS_PV ? NS * TILE_BYTES : 1024;
+  __shared__ __attribute__((aligned(1024))) char sY1k[SZ_1K];
+  __shared__ __attribute__((aligned(1024))) char sY1t[SZ_1T];
+  __shared__ __attribute__((aligned(1024))) char sY2k[SZ_2K];
+  __shared__ __attribute__((aligned(1024))) char sY2t[SZ_2T];
+  __shared__ __attribute__((aligned(16))) uint32_t sTabA[NS * BT];
+  __shared__ __attribute__((aligned(16))) uint32_t sTabB[NS * BT];
+  __shared__ __attribute__((aligned(16))) float sLse[NS * BT];
+  __shared__ __attribute__((aligned(16))) float sDelta[NS * BT];
+  __shared__ __attribute__((aligned(16))) float sSpare[BT];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -97,19 +116,32 @@ fna_bwd_kernel(const FnaBwdParams p) {
   const int split_dim = KV_STATIONARY ? p.q_split : p.kv_split;  // of the streamed side
 
   // ---- workgroup -> (batch * group, head, stationary tile) --------------------------------------
+  // Workgroup ids go round-robin to the 8 XCDs; each XCD takes one contiguous eighth of the
+  // (batch, head, tile) space, so that the workgroups resident on an XCD are neighbouring tiles
+  // of one head and find each other's streamed tiles in that XCD's L2.
   const int num_a = a_tiled[0] * a_tiled[1] * a_tiled[2];
-  const int at = int(blockIdx.x) % num_a;
-  const int head_a = (int(blockIdx.x) / num_a) % heads_a;
-  const int bg = int(blockIdx.x) / (num_a * heads_a);
+  const int total_wg = p.batch * heads_a * num_a;
+  const int chunk = (total_wg + kNumXcd - 1) / kNumXcd;
+  const int lin = (int(blockIdx.x) % kNumXcd) * chunk + int(blockIdx.x) / kNumXcd;
+  if (lin >= total_wg) return;
+  // Within a head the tiles are taken with dimension 0 slowest: the workgroups running side by
+  // side are then neighbours in the faster dimensions at the same dimension-0 position and
+  // walk the same streamed tiles at about the same time.
+  int tc[3];
+  {
+    const int rm = lin % num_a;
+    tc[2] = rm % a_tiled[2];
+    tc[1] = (rm / a_tiled[2]) % a_tiled[1];
+    tc[0] = rm / (a_tiled[2] * a_tiled[1]);
+  }
+  const int at = tc[0] + a_tiled[0] * (tc[1] + a_tiled[1] * tc[2]);  // position in the permuted sequence
+  const int head_a = (lin / num_a) % heads_a;
+  const int bg = lin / (num_a * heads_a);
 
-  int extent[3], q_extent[3], a_first[3], b_sub[3], box_tile0[3], box_n[3];
+  int extent[3], q_extent[3], a_first[3], b_sub[3], box_tile0[3], box_n[3], full_t0[3], full_t1[3];
   bool empty = false;
   {
     int gl = bg % p.num_groups;
-    int tc[3];
-    tc[0] = at % a_tiled[0];
-    tc[1] = (at / a_tiled[0]) % a_tiled[1];
-    tc[2] = at / (a_tiled[0] * a_tiled[1]);
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
       const int gi = gl % p.dil[a];
@@ -137,6 +169,29 @@ fna_bwd_kernel(const FnaBwdParams p) {
       hi = na_max(hi, lo);
       box_tile0[a] = lo / b_sub[a];
       box_n[a] = hi / b_sub[a] + 1 - box_tile0[a];
+      // Streamed tiles every row of which pairs with every row of the stationary tile (no mask
+      // needed) form an interval of tile coordinates per dimension, again by monotonicity:
+      // streamed coordinates flo .. fhi pair with all stationary ones.
+      int flo, fhi;
+      if constexpr (!KV_STATIONARY) {
+        const int qf = a_first[a], ql = qf + a_tile[a] - 1;  // rows past the extent use the last window
+        const int st_l = na_window_start(ql, p.ksize[a], p.stride[a], extent[a], c);
+        const int st_f = na_window_start(qf, p.ksize[a], p.stride[a], extent[a], c);
+        flo = st_l;
+        fhi = na_window_end(qf, st_f, p.ksize[a], extent[a], c) - 1;
+      } else {
+        const int j0 = a_first[a], j1 = j0 + a_tile[a] - 1;
+        if (j1 >= extent[a]) {
+          flo = 1;  // the tile holds padding keys: never whole
+          fhi = 0;
+        } else {
+          flo = na_first_query_attending(j1, p.ksize[a], p.stride[a], extent[a], q_extent[a], c);
+          fhi = na_last_query_attending(j0, p.ksize[a], p.stride[a], extent[a], q_extent[a], c);
+        }
+      }
+      full_t0[a] = na_max(na_ceil_div(na_max(flo, 0), b_sub[a]), box_tile0[a]);
+      full_t1[a] = na_min((fhi + 1) / b_sub[a], box_tile0[a] + box_n[a]);  // one past the last whole tile
+      if (fhi < 0 || full_t1[a] < full_t0[a]) full_t1[a] = full_t0[a];
     }
   }
 
@@ -164,6 +219,11 @@ fna_bwd_kernel(const FnaBwdParams p) {
         *reinterpret_cast<tx4*>(orow + db * 32 + 8 * j + 4 * g) = o4;
       }
   };
+  auto store_results = [&](const f32x16_t (&a1)[DB], const f32x16_t (&a2)[DB], float scale1) {
+    if constexpr (ROLE == kBwdDQ) store_rows(p.dq, a1, scale1);
+    if constexpr (ROLE == kBwdDK || ROLE == kBwdDKV) store_rows(p.dk, a1, scale1);
+    if constexpr (HAS_PV) store_rows(p.dv, a2, scale1 == 0.f ? 0.f : 1.f);
+  };
 
   f32x16_t acc1[DB], acc2[DB];
 #pragma unroll
@@ -173,28 +233,23 @@ fna_bwd_kernel(const FnaBwdParams p) {
 
   if (empty) {
     // padding rows, or rows nothing attends: their gradients are zero
-    if constexpr (KV_STATIONARY) {
-      store_rows(p.dk, acc1, 0.f);
-      store_rows(p.dv, acc2, 0.f);
-    } else {
-      store_rows(p.dq, acc1, 0.f);
-    }
+    store_results(acc1, acc2, 0.f);
     return;
   }
 
   // stationary operand fragments: row r_in, elements 16*ks + 8*g .. +7
   const T* x1 = reinterpret_cast<const T*>(KV_STATIONARY ? p.k : p.q) + a_row * a_stride + int64_t(head_a) * D + g * 8;
   const T* x2 = reinterpret_cast<const T*>(KV_STATIONARY ? p.v : p.d_out) + a_row * a_stride + int64_t(head_a) * D + g * 8;
-  vec8 x1f[KSTEPS], x2f[KSTEPS];
+  vec8 x1f[KSTEPS], x2f[HAS_DS ? KSTEPS : 1];
 #pragma unroll
   for (int ks = 0; ks < KSTEPS; ++ks) {
     x1f[ks] = *reinterpret_cast<const vec8*>(x1 + ks * 16);
-    x2f[ks] = *reinterpret_cast<const vec8*>(x2 + ks * 16);
+    if constexpr (HAS_DS) x2f[ks] = *reinterpret_cast<const vec8*>(x2 + ks * 16);
   }
 
   // mask state of the lane
   int wst[3] = {0, 0, 0}, wen[3] = {0, 0, 0};  // dQ role: window of the lane's query
-  uint32_t key_packed = 0;                     // dKV role: in-tile coordinates of the lane's key
+  uint32_t key_packed = 0;                     // other roles: in-tile coordinates of the lane's key
   float lse_l = 0.f, delta_l = 0.f;
   if constexpr (!KV_STATIONARY) {
 #pragma unroll
@@ -217,8 +272,6 @@ fna_bwd_kernel(const FnaBwdParams p) {
   }
 
   // ---- streamed tiles ---------------------------------------------------------------------------
-  const int total = box_n[0] * box_n[1] * box_n[2];
-  const int n_iter = KV_STATIONARY ? total * rep : total;
   const T* y1_all = reinterpret_cast<const T*>(KV_STATIONARY ? p.q : p.k);
   const T* y2_all = reinterpret_cast<const T*>(KV_STATIONARY ? p.d_out : p.v);
 
@@ -237,39 +290,65 @@ fna_bwd_kernel(const FnaBwdParams p) {
     int row0;       // its first row in the streamed side's permuted sequence
     int head_b;
   };
-  auto tile_of = [&](int it) {
+  // The streamed tiles in visiting order: dimension 2 fastest, dimension 0 slowest; the
+  // key-stationary roles walk the box once per query head of the key head's group.  The box is
+  // walked twice: first the tiles that need the element mask, then the whole ones (see full_t0).
+  const int total = box_n[0] * box_n[1] * box_n[2];
+  const int n_whole = (full_t1[0] - full_t0[0]) * (full_t1[1] - full_t0[1]) * (full_t1[2] - full_t0[2]);
+  int walk[3] = {0, 0, 0}, walk_head = 0;
+  auto is_whole = [&]() {
+    bool w = true;
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+      const int c = box_tile0[a] + walk[a];
+      w = w && (c >= full_t0[a]) && (c < full_t1[a]);
+    }
+    return w;
+  };
+  auto advance = [&]() {
+    if (++walk[2] == box_n[2]) {
+      walk[2] = 0;
+      if (++walk[1] == box_n[1]) {
+        walk[1] = 0;
+        if (++walk[0] == box_n[0]) {
+          walk[0] = 0;
+          ++walk_head;
+        }
+      }
+    }
+  };
+  // next tile of the wanted class; past the last one the walk runs into later heads, whose
+  // descriptors are never used
+  auto next_tile = [&](bool want_whole, int remaining) {
+    if (remaining > 0)
+      while (is_whole() != want_whole) advance();
     Tile t;
-    const int j = it % total;
-    int c[3];
-    c[2] = j % box_n[2];
-    c[1] = (j / box_n[2]) % box_n[1];
-    c[0] = j / (box_n[2] * box_n[1]);
     int cc[3], half = 0;
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
-      c[a] += box_tile0[a];
-      t.origin[a] = c[a] * b_sub[a];
+      const int c = box_tile0[a] + walk[a];
+      t.origin[a] = c * b_sub[a];
       const bool split = (a == split_dim);
-      half |= split ? (c[a] & 1) : 0;
-      cc[a] = split ? (c[a] >> 1) : c[a];
+      half |= split ? (c & 1) : 0;
+      cc[a] = split ? (c >> 1) : c;
     }
     t.row0 = (cc[0] + b_tiled[0] * (cc[1] + b_tiled[1] * cc[2])) * AT + half * BT;
-    t.head_b = KV_STATIONARY ? head_a * rep + it / total : head_a / rep;
+    t.head_b = KV_STATIONARY ? head_a * rep + walk_head : head_a / rep;
+    advance();
     return t;
   };
 
-  auto issue = [&](int it, int stage) {
-    const Tile t = tile_of(it);
-    const int64_t row = int64_t(bg) * seq_b + t.row0;
+  // in-tile coordinates of streamed position `lane` (the window tables below are built by wave 0)
+  int qo[3];
+  qo[0] = lane % b_sub[0];
+  qo[1] = (lane / b_sub[0]) % b_sub[1];
+  qo[2] = lane / (b_sub[0] * b_sub[1]);
+
+  const uint32_t stat_off = uint32_t(lane) * uint32_t(p.heads_q) * 4u;  // byte offset of streamed row `lane` in lse / delta
+  auto issue = [&](const Tile& t, int stage, bool masked) {
     if constexpr (KV_STATIONARY) {
-      // Per streamed query: its window relative to this workgroup's key tile, and its LSE / delta.
-      // Done ahead of the tile copies, so that waiting for these loads does not wait for the copies.
-      if (wave == 0) {
-        const int e = lane;
-        int qo[3];
-        qo[0] = e % b_sub[0];
-        qo[1] = (e / b_sub[0]) % b_sub[1];
-        qo[2] = e / (b_sub[0] * b_sub[1]);
+      if (wave == 0 && masked) {
+        // per streamed query: its window relative to this workgroup's key tile
         uint32_t addc = 0, subc = 0;
         bool valid = true;
 #pragma unroll
@@ -283,13 +362,18 @@ fna_bwd_kernel(const FnaBwdParams p) {
           addc |= uint32_t(512 - lo) << (10 * a);
           subc |= uint32_t(511 + hi) << (10 * a);
         }
-        sTabA[stage * BT + e] = valid ? addc : 0u;  // no guard bit survives a zero addend
-        sTabB[stage * BT + e] = valid ? subc : 0u;
-      } else if (wave == 1) {
-        sLse[stage * BT + lane] = p.lse[(row + lane) * p.heads_q + t.head_b] * kLog2e;
-      } else if (wave == 2) {
-        sDelta[stage * BT + lane] = p.delta[(row + lane) * p.heads_q + t.head_b];
+        sTabA[stage * BT + lane] = valid ? addc : 0u;  // no guard bit survives a zero addend
+        sTabB[stage * BT + lane] = valid ? subc : 0u;
       }
+    }
+    const int64_t row = int64_t(bg) * seq_b + t.row0;
+    if constexpr (KV_STATIONARY) {
+      // LSE / delta of the tile's 64 queries: one asynchronous 4-byte-per-lane copy each
+      // (wave 1, wave 2; wave 3 and, without delta, wave 2 make the same number of copies into a
+      // spare row so that every wave counts the same number of outstanding copies per tile)
+      const float* src = (wave == 2 && HAS_DS ? p.delta : p.lse) + row * p.heads_q + t.head_b;
+      float* dst = (wave == 1) ? &sLse[stage * BT] : (wave == 2 && HAS_DS) ? &sDelta[stage * BT] : &sSpare[0];
+      if (wave != 0) async_copy4_asm(src, stat_off, lds_address(dst));
     }
     const T* y1 = y1_all + row * b_stride + int64_t(t.head_b) * D;
     const T* y2 = y2_all + row * b_stride + int64_t(t.head_b) * D;
@@ -298,9 +382,9 @@ fna_bwd_kernel(const FnaBwdParams p) {
     for (int i = 0; i < PER; ++i) {
       const uint32_t d = dst + uint32_t(i * NT * 16);
       async_copy16_asm<0>(y1, off_k[i], lds_address(sY1k) + d);
-      async_copy16_asm<0>(y1, off_t[i], lds_address(sY1t) + d);
-      async_copy16_asm<0>(y2, off_k[i], lds_address(sY2k) + d);
-      if constexpr (KV_STATIONARY) async_copy16_asm<0>(y2, off_t[i], lds_address(sY2t) + d);
+      if constexpr (HAS_DS) async_copy16_asm<0>(y1, off_t[i], lds_address(sY1t) + d);
+      if constexpr (HAS_DS) async_copy16_asm<0>(y2, off_k[i], lds_address(sY2k) + d);
+      if constexpr (HAS_PV) async_copy16_asm<0>(y2, off_t[i], lds_address(sY2t) + d);
     }
   };
 
@@ -327,100 +411,197 @@ fna_bwd_kernel(const FnaBwdParams p) {
 
   const float c_log2 = p.scale * kLog2e;
 
-  issue(0, 0);
-  for (int it = 0; it < n_iter; ++it) {
-    const int stage = it & 1;
-    wait_vmcnt<0>();
-    __syncthreads();  // tile `it` and its tables are in LDS; everyone is done with the other stage
-    if (it + 1 < n_iter) issue(it + 1, stage ^ 1);
-
+  // One streamed tile.  The matrix instructions form one sequence of "slots" (first the
+  // products S and dP of the two 32-row sub-blocks, then the accumulations of the two
+  // sub-blocks); a slot is one operand fragment read ahead from LDS, one MFMA and its share of
+  // the vector work: the probabilities of sub-block 0 run under the products of sub-block 1,
+  // those of sub-block 1 under the accumulations of sub-block 0.  Slots are fenced so that the
+  // compiler keeps the interleaving.
+  constexpr int WP = HAS_DS ? 2 : 1;                       // products per k-step (S, dP)
+  constexpr int W = (HAS_DS ? 1 : 0) + (HAS_PV ? 1 : 0);   // accumulators fed per transposed fragment position
+  constexpr int NP = WP * KSTEPS;                          // product slots per sub-block
+  constexpr int N1 = 2 * NP;
+  constexpr int NC = 2 * DB * W;                           // accumulation slots per sub-block
+  constexpr int G = N1 + 2 * NC;
+#ifndef NA_BWD_PF
+#define NA_BWD_PF 3
+#endif
+  constexpr int PF = NA_BWD_PF;                            // fragments read ahead
+  auto tile_body = [&](auto masked_tag, int stage, uint32_t addc, uint32_t subc) __attribute__((always_inline)) {
+    constexpr bool MASKED = decltype(masked_tag)::value;
     const char* y1k = sY1k + stage * TILE_BYTES;
-    const char* y1t = sY1t + stage * TILE_BYTES;
-    const char* y2k = sY2k + stage * TILE_BYTES;
-    const char* y2t = sY2t + (KV_STATIONARY ? stage * TILE_BYTES : 0);
+    const char* y1t = sY1t + (HAS_DS ? stage * TILE_BYTES : 0);
+    const char* y2k = sY2k + (HAS_DS ? stage * TILE_BYTES : 0);
+    const char* y2t = sY2t + (HAS_PV ? stage * TILE_BYTES : 0);
+
+    auto frag = [&](auto x_tag) {
+      constexpr int x = decltype(x_tag)::value;
+      if constexpr (x < N1) {
+        constexpr int sb = x / NP, ks = (x % NP) / WP, which = x % WP;
+        return row_frag(which ? y2k : y1k, sb, ks);
+      } else {
+        constexpr int n = x - N1;
+        constexpr int sb = n / NC, idx = n % NC, h = idx / (DB * W), db = (idx / W) % DB;
+        constexpr bool to_acc1 = HAS_DS && (idx % W == 0);
+        return tr_frag(to_acc1 ? y1t : y2t, sb, h, db);
+      }
+    };
 
     f32x16_t S[NSB], dP[NSB];
-#pragma unroll
-    for (int sb = 0; sb < NSB; ++sb) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) S[sb][r] = dP[sb][r] = 0.f;
-#pragma unroll
-      for (int ks = 0; ks < KSTEPS; ++ks) {
-        S[sb] = M::run(row_frag(y1k, sb, ks), x1f[ks], S[sb]);
-        dP[sb] = M::run(row_frag(y2k, sb, ks), x2f[ks], dP[sb]);
-      }
-    }
-
-    // mask constants of the lane for this tile
-    uint32_t addc = 0, subc = 0;
-    if constexpr (!KV_STATIONARY) {
-      const Tile t = tile_of(it);
-#pragma unroll
-      for (int a = 0; a < 3; ++a) {
-        const int lo = na_min(na_max(wst[a] - t.origin[a], 0), b_sub[a]);
-        const int hi = na_min(na_max(wen[a] - t.origin[a], 0), b_sub[a]);
-        addc |= uint32_t(512 - lo) << (10 * a);
-        subc |= uint32_t(511 + hi) << (10 * a);
-      }
-    }
-
     vec8 pf[NSB][2], dsf[NSB][2];
-#pragma unroll
-    for (int sb = 0; sb < NSB; ++sb)
-#pragma unroll
-      for (int jj = 0; jj < 4; ++jj) {
-        const int e0 = sb * 32 + 8 * jj + 4 * g;  // the lane's registers 4*jj .. 4*jj+3 are streamed rows e0 .. e0+3
-        u32x4_t ta, tb;
-        float ls[4], dl[4];
+    // tables of the streamed rows, four rows (8*jj + 4*g + i of a sub-block) at a time; the
+    // group after the one in use is read ahead
+    u32x4_t ta[2], tb[2];
+    f32x4_t ls4[2], dl4[2];
+    auto load_group = [&](auto gi_tag) {
+      constexpr int gi = decltype(gi_tag)::value;  // sub-block * 4 + jj
+      if constexpr (gi < 2 * 4) {
+        const int e0 = (gi / 4) * 32 + 8 * (gi % 4) + 4 * g;
         if constexpr (KV_STATIONARY) {
-          ta = *reinterpret_cast<const u32x4_t*>(&sTabA[stage * BT + e0]);
-          tb = *reinterpret_cast<const u32x4_t*>(&sTabB[stage * BT + e0]);
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            ls[i] = sLse[stage * BT + e0 + i];
-            dl[i] = sDelta[stage * BT + e0 + i];
+          if constexpr (MASKED) {
+            ta[gi & 1] = *reinterpret_cast<const u32x4_t*>(&sTabA[stage * BT + e0]);
+            tb[gi & 1] = *reinterpret_cast<const u32x4_t*>(&sTabB[stage * BT + e0]);
           }
-        } else {
-          ta = *reinterpret_cast<const u32x4_t*>(&sTabA[e0]);
-          tb = ta;
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            ls[i] = lse_l;
-            dl[i] = delta_l;
-          }
-        }
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int r = 4 * jj + i;
-          uint32_t ok;
-          if constexpr (KV_STATIONARY) ok = (key_packed + ta[i]) & (tb[i] - key_packed) & kGuardBits;
-          else ok = (ta[i] + addc) & (subc - ta[i]) & kGuardBits;
-          const float x = fast_exp2(S[sb][r] * c_log2 - ls[i]);
-          const float pv = (ok == kGuardBits) ? x : 0.f;
-          const float ds = pv * (dP[sb][r] - dl[i]);
-          pf[sb][r / 8][r % 8] = static_cast<T>(pv);
-          dsf[sb][r / 8][r % 8] = static_cast<T>(ds);
+          ls4[gi & 1] = *reinterpret_cast<const f32x4_t*>(&sLse[stage * BT + e0]) * kLog2e;
+          if constexpr (HAS_DS) dl4[gi & 1] = *reinterpret_cast<const f32x4_t*>(&sDelta[stage * BT + e0]);
+        } else if constexpr (MASKED) {
+          ta[gi & 1] = *reinterpret_cast<const u32x4_t*>(&sTabA[e0]);
         }
       }
-
-#pragma unroll
-    for (int sb = 0; sb < NSB; ++sb)
-#pragma unroll
-      for (int h = 0; h < 2; ++h)
-#pragma unroll
-        for (int db = 0; db < DB; ++db) {
-          acc1[db] = M::run(tr_frag(y1t, sb, h, db), dsf[sb][h], acc1[db]);
-          if constexpr (KV_STATIONARY) acc2[db] = M::run(tr_frag(y2t, sb, h, db), pf[sb][h], acc2[db]);
+    };
+    float held_p = 0.f, held_ds = 0.f;
+    auto elem = [&](auto sb_tag, auto r_tag) {
+      constexpr int sb = decltype(sb_tag)::value, r = decltype(r_tag)::value;
+      constexpr int jj = (sb * 4 + r / 4) & 1, i = r % 4;
+      if constexpr (i == 0) load_group(std::integral_constant<int, sb * 4 + r / 4 + 1>{});
+      float x;
+      if constexpr (KV_STATIONARY) x = fast_exp2(S[sb][r] * c_log2 - ls4[jj][i]);
+      else x = fast_exp2(S[sb][r] * c_log2 - lse_l);
+      if constexpr (MASKED) {
+        uint32_t ok;
+        if constexpr (KV_STATIONARY) ok = (key_packed + ta[jj][i]) & (tb[jj][i] - key_packed) & kGuardBits;
+        else ok = (ta[jj][i] + addc) & (subc - ta[jj][i]) & kGuardBits;
+        x = (ok == kGuardBits) ? x : 0.f;
+      }
+      float ds = 0.f;
+      if constexpr (HAS_DS) {
+        if constexpr (KV_STATIONARY) ds = x * (dP[sb][r] - dl4[jj][i]);
+        else ds = x * (dP[sb][r] - delta_l);
+      }
+      if constexpr (r % 2 == 0) {
+        pin(x);
+        held_p = x;
+        if constexpr (HAS_DS) {
+          pin(ds);
+          held_ds = ds;
         }
-  }
-  wait_vmcnt<0>();
+      } else {
+        if constexpr (HAS_PV) {
+          vec2 p2 = {static_cast<T>(held_p), static_cast<T>(x)};
+          uint32_t pb = __builtin_bit_cast(uint32_t, p2);
+          pin(pb);
+          p2 = __builtin_bit_cast(vec2, pb);
+          pf[sb][r / 8][r % 8 - 1] = p2[0];
+          pf[sb][r / 8][r % 8] = p2[1];
+        }
+        if constexpr (HAS_DS) {
+          vec2 d2 = {static_cast<T>(held_ds), static_cast<T>(ds)};
+          uint32_t db_ = __builtin_bit_cast(uint32_t, d2);
+          pin(db_);
+          d2 = __builtin_bit_cast(vec2, db_);
+          dsf[sb][r / 8][r % 8 - 1] = d2[0];
+          dsf[sb][r / 8][r % 8] = d2[1];
+        }
+      }
+    };
 
-  if constexpr (KV_STATIONARY) {
-    store_rows(p.dk, acc1, p.scale);
-    store_rows(p.dv, acc2, 1.f);
-  } else {
-    store_rows(p.dq, acc1, p.scale);
-  }
+    vec8 fr[G];
+    for_range<0, PF>([&](auto x_tag) { fr[decltype(x_tag)::value] = frag(x_tag); });
+    load_group(std::integral_constant<int, 0>{});
+    for_range<0, G>([&](auto x_tag) __attribute__((always_inline)) {
+      constexpr int x = decltype(x_tag)::value;
+      if constexpr (x + PF < G) fr[x + PF] = frag(std::integral_constant<int, x + PF>{});
+      if constexpr (x < N1) {
+        constexpr int sb = x / NP, ks = (x % NP) / WP, which = x % WP;
+        f32x16_t zero;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) zero[r] = 0.f;
+        if constexpr (which == 0) S[sb] = M::run(fr[x], x1f[ks], ks == 0 ? zero : S[sb]);
+        else dP[sb] = M::run(fr[x], x2f[ks], ks == 0 ? zero : dP[sb]);
+        if constexpr (sb == 1) {
+          // probabilities of sub-block 0
+          constexpr int s = x - NP;
+          constexpr int e_lo = (16 * s) / NP, e_hi = (16 * (s + 1)) / NP;
+          for_range<e_lo, e_hi - e_lo>([&](auto r_tag) { elem(std::integral_constant<int, 0>{}, r_tag); });
+        }
+      } else {
+        constexpr int n = x - N1;
+        constexpr int sb = n / NC, idx = n % NC, h = idx / (DB * W), db = (idx / W) % DB;
+        constexpr bool to_acc1 = HAS_DS && (idx % W == 0);
+        if constexpr (to_acc1) acc1[db] = M::run(fr[x], dsf[sb][h], acc1[db]);
+        else acc2[db] = M::run(fr[x], pf[sb][h], acc2[db]);
+        if constexpr (sb == 0) {
+          // probabilities of sub-block 1
+          constexpr int e_lo = (16 * idx) / NC, e_hi = (16 * (idx + 1)) / NC;
+          for_range<e_lo, e_hi - e_lo>([&](auto r_tag) { elem(std::integral_constant<int, 1>{}, r_tag); });
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    });
+  };
+
+  // ---- pipeline: tile `it` is multiplied while tiles it+1 .. it+NS-1 are in flight ----------------
+  // Descriptor queue: d[0] = tile `it`, d[k] = tile it + k.
+  constexpr int CPT = PER * (1 + (HAS_DS ? 2 : 0) + (HAS_PV ? 1 : 0));  // tile copies per thread and tile
+  auto run_pass = [&](auto masked_tag, int n_iter) __attribute__((always_inline)) {
+    constexpr bool MASKED = decltype(masked_tag)::value;
+    if (n_iter <= 0) return;
+    walk[0] = walk[1] = walk[2] = 0;
+    walk_head = 0;
+    Tile d[NS];
+#pragma unroll
+    for (int k = 0; k < NS; ++k) d[k] = next_tile(!MASKED, n_iter - k);
+#pragma unroll
+    for (int k = 0; k < NS - 1; ++k)
+      if (k < n_iter) issue(d[k], k, MASKED);
+
+    for (int it = 0; it < n_iter; ++it) {
+      const int stage = it % NS;
+      // this thread's copies of tile `it` have landed once at most those of the later tiles in
+      // flight (one tile with three stages, none with two) are outstanding; wave 0 makes one
+      // copy less per tile in the key-stationary roles
+      if (NS == 3 && it + 1 < n_iter) {
+        if (KV_STATIONARY && wave != 0) wait_vmcnt<CPT + 1>();
+        else wait_vmcnt<CPT>();
+      } else {
+        wait_vmcnt<0>();
+      }
+      __syncthreads();  // tile `it` and its tables are in LDS; everyone is done with the stage of tile it - 1
+      if (it + NS - 1 < n_iter) issue(d[NS - 1], (it + NS - 1) % NS, MASKED);
+
+      uint32_t addc = 0, subc = 0;
+      if constexpr (MASKED && !KV_STATIONARY) {
+#pragma unroll
+        for (int a = 0; a < 3; ++a) {
+          const int lo = na_min(na_max(wst[a] - d[0].origin[a], 0), b_sub[a]);
+          const int hi = na_min(na_max(wen[a] - d[0].origin[a], 0), b_sub[a]);
+          addc |= uint32_t(512 - lo) << (10 * a);
+          subc |= uint32_t(511 + hi) << (10 * a);
+        }
+      }
+      tile_body(masked_tag, stage, addc, subc);
+#pragma unroll
+      for (int k = 0; k + 1 < NS; ++k) d[k] = d[k + 1];
+      d[NS - 1] = next_tile(!MASKED, n_iter - it - NS);
+    }
+    wait_vmcnt<0>();
+    __syncthreads();  // the stages are free for the next pass
+  };
+  const int heads_walked = KV_STATIONARY ? rep : 1;
+  run_pass(std::true_type{}, (total - n_whole) * heads_walked);
+  run_pass(std::false_type{}, n_whole * heads_walked);
+
+  store_results(acc1, acc2, p.scale);
 }
 
 // delta[item] = sum_d out[item, d] * d_out[item, d] over `items` rows of D contiguous elements

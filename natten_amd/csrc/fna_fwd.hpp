@@ -71,6 +71,7 @@ typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
 typedef short s16x4_t __attribute__((ext_vector_type(4)));
 typedef short s16x8_t __attribute__((ext_vector_type(8)));
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
@@ -140,6 +141,22 @@ static __device__ __forceinline__ void async_copy16_asm(const void* base, uint32
       "global_load_lds_dwordx4 %1, %2 offset:%3"
       :
       : "s"(lds_addr), "v"(voff), "s"(base), "n"(IMM)
+      : "memory", "m0");
+}
+
+// The 4-byte-per-lane form: lane i's dword from `base + voff` lands at LDS address `lds_addr + 4 * i`.
+static __device__ __forceinline__ void async_copy4_asm(const void* base, uint32_t voff, uint32_t lds_addr) {
+  const uint64_t b = reinterpret_cast<uint64_t>(base);
+  const uint64_t ub = (uint64_t(uint32_t(__builtin_amdgcn_readfirstlane(int(b >> 32)))) << 32) |
+                      uint32_t(__builtin_amdgcn_readfirstlane(int(uint32_t(b))));
+  base = reinterpret_cast<const void*>(ub);
+  lds_addr = uint32_t(__builtin_amdgcn_readfirstlane(int(lds_addr)));
+  asm volatile(
+      "s_mov_b32 m0, %0\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dword %1, %2"
+      :
+      : "s"(lds_addr), "v"(voff), "s"(base)
       : "memory", "m0");
 }
 

@@ -422,13 +422,24 @@ int natten_amd_attention_forward_varlen(const void* q, const void* k, const void
 extern "C++" {
 template <typename T, int D>
 static int launch_bwd(const FnaBwdParams& p, hipStream_t stream) {
-  const long long wg_q = (long long)p.batch * p.heads_q * prod3(p.q_tiled);
-  const long long wg_kv = (long long)p.batch * p.heads_kv * prod3(p.kv_tiled);
+  // grids are padded to a multiple of the 8 XCDs: each XCD takes a contiguous eighth of the tiles
+  auto grid = [](long long wgs) { return (wgs + kNumXcd - 1) / kNumXcd * kNumXcd; };
+  const long long wg_q = grid((long long)p.batch * p.heads_q * prod3(p.q_tiled));
+  const long long wg_kv = grid((long long)p.batch * p.heads_kv * prod3(p.kv_tiled));
   if (wg_q > 0x7fffffffLL || wg_kv > 0x7fffffffLL) return fail("fna_backward: problem needs more than 2^31 workgroups");
-  hipLaunchKernelGGL((fna_bwd_kernel<T, D, false>), dim3((unsigned)wg_q), dim3(256), 0, stream, p);
+  hipLaunchKernelGGL((fna_bwd_kernel<T, D, kBwdDQ>), dim3((unsigned)wg_q), dim3(256), 0, stream, p);
   if (int rc = check_launch("fna_backward (dQ)")) return rc;
-  hipLaunchKernelGGL((fna_bwd_kernel<T, D, true>), dim3((unsigned)wg_kv), dim3(256), 0, stream, p);
-  return check_launch("fna_backward (dK, dV)");
+  if constexpr (D == 128) {
+    // dK and dV separately: their accumulators, fragments and products together exceed the
+    // registers a matrix instruction addresses directly
+    hipLaunchKernelGGL((fna_bwd_kernel<T, D, kBwdDK>), dim3((unsigned)wg_kv), dim3(256), 0, stream, p);
+    if (int rc = check_launch("fna_backward (dK)")) return rc;
+    hipLaunchKernelGGL((fna_bwd_kernel<T, D, kBwdDV>), dim3((unsigned)wg_kv), dim3(256), 0, stream, p);
+    return check_launch("fna_backward (dV)");
+  } else {
+    hipLaunchKernelGGL((fna_bwd_kernel<T, D, kBwdDKV>), dim3((unsigned)wg_kv), dim3(256), 0, stream, p);
+    return check_launch("fna_backward (dK, dV)");
+  }
 }
 
 template <typename T>
