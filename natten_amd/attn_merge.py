@@ -1,13 +1,19 @@
 """merge_attentions: combine partial attentions over disjoint key sets of the same queries.
 
 Same API and validation as the reference's src/natten/attn_merge.py:193-292; the arithmetic
-(:83-95) runs as one HIP kernel per pair.  `torch_compile` and `use_autograd_fix` are accepted
-for signature compatibility and ignored (forward only, nothing to compile)."""
+(:83-95) runs as one HIP kernel per pair.  `torch_compile` is accepted for signature
+compatibility and ignored.  With tensors that require grad the merge is an autograd function
+that, like the reference's (:130-190), overwrites the partial outputs and LSEs saved by the
+originating attention operations with the merged ones and hands every one of them the merged
+output's gradient: each attention backward then computes the gradient of attention over the
+joint context.  This only works on the tensors those operations returned (or contiguous views of
+them), as in the reference."""
 
 from __future__ import annotations
 
 from typing import List, Tuple
 
+import torch
 from torch import Tensor
 
 from . import _lib, torch_ops
@@ -44,6 +50,14 @@ def merge_attentions(
                 f"LSE tensors must match outputs in shape except last dim ({shape=}), but got LSE {i} with "
                 f"shape={lse.shape}."
             )
+    if torch.is_grad_enabled() and any(t.requires_grad for t in outputs):
+        if not use_autograd_fix:
+            raise NotImplementedError("natten_amd merges differentiable partial attentions only with use_autograd_fix=True.")
+        return MergeAttentionsFunction.apply(*outputs, *lse_tensors)
+    return _merge(list(outputs), list(lse_tensors))
+
+
+def _merge(outputs: List[Tensor], lse_tensors: List[Tensor]) -> Tuple[Tensor, Tensor]:
     out_dtype = outputs[0].dtype
     # more than two partials: keep the running result in float32 between pairwise merges
     work = (lambda t: t.float().contiguous()) if len(outputs) > 2 else (lambda t: t.contiguous())
@@ -52,6 +66,29 @@ def merge_attentions(
     for o, l in zip(outputs[1:], lse_tensors[1:]):
         out, lse = torch_ops.merge_two(out, lse, work(o.to(outputs[0].dtype)), l.float().contiguous())
     return out.to(out_dtype), lse
+
+
+class MergeAttentionsFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, *args):
+        n = len(args) // 2
+        outputs, lses = args[:n], args[n:]
+        with torch.no_grad():
+            merged_out, merged_lse = _merge(list(outputs), list(lses))
+        ctx.n = n
+        ctx.save_for_backward(merged_out, merged_lse, *outputs, *lses)
+        return merged_out, merged_lse
+
+    @staticmethod
+    def backward(ctx, grad_out, grad_lse):
+        n = ctx.n
+        merged_out, merged_lse = ctx.saved_tensors[:2]
+        outputs = ctx.saved_tensors[2 : 2 + n]
+        lses = ctx.saved_tensors[2 + n :]
+        for output, lse in zip(outputs, lses):
+            output.data.copy_(merged_out.data.reshape(output.shape))
+            lse.data.copy_(merged_lse.data.reshape(lse.shape))
+        return (grad_out,) * n + (None,) * n
 
 
 __all__ = ["merge_attentions"]

@@ -49,10 +49,7 @@ def amd_fmha(
             raise NotImplementedError(
                 "natten_amd attention has a backward pass for fp16 / bf16 fixed-length batches only."
             )
-        q, k, v = (pad_head_dim(t, d_pad) for t in (query, key, value))
-        out, lse = AmdFmhaFunction.apply(q, k, v, bool(is_causal), float(scale))
-        if d_pad != head_dim:
-            out = out[..., :head_dim]
+        out, lse = AmdFmhaFunction.apply(query, key, value, bool(is_causal), float(scale))
         if out_dtype is not None and out.dtype != out_dtype:
             out = out.to(out_dtype)
         return (out, lse) if return_lse else out
@@ -99,12 +96,13 @@ class AmdFmhaFunction(torch.autograd.Function):
     """Dense attention with a backward pass (fp16 / bf16, fixed-length batches): the backward
     kernels of neighborhood attention on the 1-D problem whose window is the whole key sequence,
     sequences zero-padded to multiples of 128 rows.  Counterpart of the reference's
-    src/natten/backends/blackwell_fmha.py:52-170; the gradient of LSE is not propagated."""
+    src/natten/backends/blackwell_fmha.py:52-170; the gradient of LSE is not propagated.  The saved
+    output and LSE are the returned tensors themselves (see AmdFnaFunction)."""
 
     @staticmethod
     def forward(ctx, query, key, value, is_causal, scale):
         with torch.no_grad():
-            out, lse = _lib.attention_forward(query.contiguous(), key.contiguous(), value.contiguous(), is_causal, scale)
+            out, lse = amd_fmha(query, key, value, is_causal=is_causal, scale=scale, return_lse=True)
         ctx.save_for_backward(query, key, value, out, lse)
         ctx.args = (is_causal, scale)
         ctx.mark_non_differentiable(lse)
@@ -114,12 +112,16 @@ class AmdFmhaFunction(torch.autograd.Function):
     def backward(ctx, d_out, d_lse):
         query, key, value, out, lse = ctx.saved_tensors
         is_causal, scale = ctx.args
-        d_out = d_out.contiguous()
-        delta = _lib.compute_delta(out.contiguous(), d_out)
+        head_dim = query.shape[-1]
+        d_pad = padded_head_dim(head_dim)
+        query, key, value, out, d_out = (
+            pad_head_dim(t.contiguous(), d_pad).contiguous() for t in (query, key, value, out, d_out)
+        )
+        delta = _lib.compute_delta(out, d_out)
         sq, skv = query.shape[1], key.shape[1]
         pq, pkv = -(-sq // 128) * 128, -(-skv // 128) * 128
         dq, dk, dv = _lib.attention_backward(
             _pad_rows(query, pq), _pad_rows(key, pkv), _pad_rows(value, pkv), _pad_rows(d_out, pq),
             _pad_rows(lse, pq), _pad_rows(delta, pq), sq, skv, is_causal, scale,
         )
-        return dq[:, :sq], dk[:, :skv], dv[:, :skv], None, None
+        return dq[:, :sq, :, :head_dim], dk[:, :skv, :, :head_dim], dv[:, :skv, :, :head_dim], None, None

@@ -127,10 +127,6 @@ def amd_fna_generic(
     head_dim = query.shape[-1]
     scale = scale or head_dim**-0.5
     d_pad = padded_head_dim(head_dim)
-    if d_pad != head_dim:
-        # zero columns change neither q.k nor the first head_dim output columns
-        query, key, value = (_pad_head_dim(t, d_pad) for t in (query, key, value))
-
     if torch.is_grad_enabled() and (query.requires_grad or key.requires_grad or value.requires_grad):
         bwd_q_tile, bwd_kv_tile = check_fna_backward_config(
             query, kernel_size, stride, dilation, is_causal, backward_q_tile_shape, backward_kv_tile_shape
@@ -139,11 +135,12 @@ def amd_fna_generic(
             query, key, value, kernel_size, stride, dilation, is_causal, scale, q_tile_shape, kv_tile_shape,
             bwd_q_tile, bwd_kv_tile, fused,
         )
-        if d_pad != head_dim:
-            output = output[..., :head_dim]
         if out_dtype is not None and output.dtype != out_dtype:
             output = output.to(out_dtype)
         return (output, lse) if return_lse else output
+    if d_pad != head_dim:
+        # zero columns change neither q.k nor the first head_dim output columns
+        query, key, value = (_pad_head_dim(t, d_pad) for t in (query, key, value))
 
     in_dtype = query.dtype
     fp8_ok = (
@@ -214,7 +211,9 @@ class AmdFnaFunction(torch.autograd.Function):
     the forward saves q, k, v, out and LSE; the backward computes delta = rowsum(dO * O), permutes
     q, dO, LSE, delta with the backward Q tile and k, v with the backward KV tile, runs the dQ and
     the dK/dV kernels, and unpermutes the three gradients.  The gradient of the LSE output is
-    not propagated, as in the reference."""
+    not propagated, as in the reference.  The saved output and LSE are the returned tensors
+    themselves: `merge_attentions` overwrites them with the merged ones before this backward
+    runs, which makes it the backward of attention over the joint context."""
 
     @staticmethod
     def forward(ctx, query, key, value, kernel_size, stride, dilation, is_causal, scale, q_tile_shape, kv_tile_shape,
@@ -233,8 +232,13 @@ class AmdFnaFunction(torch.autograd.Function):
     def backward(ctx, d_output, d_lse):
         query, key, value, output, lse = ctx.saved_tensors
         kernel_size, stride, dilation, is_causal, scale, q_tile, kv_tile = ctx.na_args
-        d_output = d_output.contiguous()
-        delta = _lib.compute_delta(output.contiguous(), d_output)
+        head_dim = query.shape[-1]
+        d_pad = padded_head_dim(head_dim)
+        # zero columns add nothing to q.k, dO.v or rowsum(dO * O); their gradients are dropped
+        query, key, value, output, d_output = (
+            pad_head_dim(t.contiguous(), d_pad).contiguous() for t in (query, key, value, output, d_output)
+        )
+        delta = _lib.compute_delta(output, d_output)
 
         def perm(x, tile):
             return token_permute_operation(x.contiguous(), tile, dilation, flip_tiled_dims=True)
@@ -252,4 +256,6 @@ class AmdFnaFunction(torch.autograd.Function):
         dq = token_unpermute_operation(dq_perm, qkv_shape, q_tile, dilation, flip_tiled_dims=True)
         dk = token_unpermute_operation(dk_perm, qkv_shape, kv_tile, dilation, flip_tiled_dims=True)
         dv = token_unpermute_operation(dv_perm, qkv_shape, kv_tile, dilation, flip_tiled_dims=True)
+        if d_pad != head_dim:
+            dq, dk, dv = (t[..., :head_dim].contiguous() for t in (dq, dk, dv))
         return (dq, dk, dv) + (None,) * 10

