@@ -92,3 +92,104 @@ def test_permute_round_trip_full_size():
     idx = 1 + 15 * (1 + 6 * 2)
     tile = p[0, idx * 128 : (idx + 1) * 128].reshape(8, 8, 2, 24, 128)  # dimension 0 fastest
     assert torch.equal(tile.permute(2, 1, 0, 3, 4), blk)
+
+
+# ---- backward at full size ---------------------------------------------------------------------------
+
+
+def _window(shape, kernel, stride, causal, coord):
+    from oracle import na_oracle as O
+
+    st = [int(O.window_start(c, k, s, L, ca)) for c, k, s, L, ca in zip(coord, kernel, stride, shape, causal)]
+    en = [int(O.window_end(c, s0, k, L, ca)) for c, s0, k, L, ca in zip(coord, st, kernel, shape, causal)]
+    return st, en
+
+
+def _backward_sampled(fn, shape, H, D, kernel, stride, causal, dtype, std, n_q, n_k, seed, tol):
+    """Forward + backward at full size; sampled rows of dQ and of dK / dV against float64 arithmetic.
+
+    A dQ row needs only its query's window.  A dK / dV row sums over the queries that attend the key
+    (found with the host-side query range, then filtered with the window test); their
+    probabilities use the LSE and the delta = dO.O of the forward result, which the forward tests
+    above pin, so the check costs one dot product per (query, key) pair."""
+    from natten_amd import _lib
+
+    n = len(shape)
+    q, k, v = make_qkv(1, shape, H, H, D, dtype, seed=seed, std=std)
+    d_out = torch.randn(q.shape, generator=torch.Generator().manual_seed(seed + 1)).to(dtype).cuda()
+    for t in (q, k, v):
+        t.requires_grad_(True)
+    out, lse = fn(q, k, v, kernel, stride, 1, causal, return_lse=True)
+    out.backward(d_out)
+    torch.cuda.synchronize()
+    scale = float(D) ** -0.5
+    N = int(np.prod(shape))
+    flat = lambda t: t.detach().reshape(N, H, D)
+    qf, kf, vf, dof, of = flat(q), flat(k), flat(v), flat(d_out), flat(out)
+    lsef = lse.detach().reshape(N, H)
+    dq, dk, dv = flat(q.grad), flat(k.grad), flat(v.grad)
+    rng = np.random.default_rng(seed)
+    strides = np.array([int(np.prod(shape[a + 1 :])) for a in range(n)])
+
+    def box_tokens(st, en):
+        grids = np.meshgrid(*[np.arange(s0, e0) for s0, e0 in zip(st, en)], indexing="ij")
+        return sum(g.reshape(-1) * int(sd) for g, sd in zip(grids, strides))
+
+    for _ in range(n_q):
+        tok = int(rng.integers(0, N))
+        coord = [int(x) for x in np.unravel_index(tok, shape)]
+        st, en = _window(shape, kernel, stride, causal, coord)
+        keys = torch.as_tensor(box_tokens(st, en), device="cuda")
+        qi, doi = qf[tok].double(), dof[tok].double()          # [H, D]
+        kw, vw = kf[keys].double(), vf[keys].double()          # [W, H, D]
+        s = torch.einsum("hd,whd->hw", qi, kw) * scale
+        p = torch.softmax(s, dim=-1)
+        dp = torch.einsum("hd,whd->hw", doi, vw)
+        ds = p * (dp - (p * dp).sum(-1, keepdim=True)) * scale
+        ref = torch.einsum("hw,whd->hd", ds, kw)
+        assert_close(f"dq row {coord}", to_np(dq[tok]), ref.cpu().numpy(), atol=tol, rtol=tol)
+
+    for _ in range(n_k):
+        tok = int(rng.integers(0, N))
+        coord = [int(x) for x in np.unravel_index(tok, shape)]
+        rng_q = [_lib.query_range(c, c, kk, ss, L, L, ca) for c, kk, ss, L, ca in zip(coord, kernel, stride, shape, causal)]
+        cand = box_tokens([r[0] for r in rng_q], [r[1] + 1 for r in rng_q])
+        keep = []
+        for t in cand:
+            qc = [int(x) for x in np.unravel_index(int(t), shape)]
+            st, en = _window(shape, kernel, stride, causal, qc)
+            if all(s0 <= c < e0 for s0, e0, c in zip(st, en, coord)):
+                keep.append(int(t))
+        assert keep, "every key is attended by some query"
+        qs = torch.as_tensor(keep, device="cuda")
+        qa, doa, oa = qf[qs].double(), dof[qs].double(), of[qs].double()   # [Nq, H, D]
+        kj, vj = kf[tok].double(), vf[tok].double()                        # [H, D]
+        p = torch.exp(torch.einsum("nhd,hd->nh", qa, kj) * scale - lsef[qs].double())
+        dp = torch.einsum("nhd,hd->nh", doa, vj)
+        ds = p * (dp - (doa * oa).sum(-1)) * scale
+        assert_close(f"dk row {coord}", to_np(dk[tok]), torch.einsum("nh,nhd->hd", ds, qa).cpu().numpy(), atol=tol, rtol=tol)
+        assert_close(f"dv row {coord}", to_np(dv[tok]), torch.einsum("nh,nhd->hd", p, doa).cpu().numpy(), atol=tol, rtol=tol)
+
+    # size-independent property: the gradients are linear in dO.  In bf16 a factor of two is exact
+    # (it commutes with every rounding); in fp16 the rounded dS of long rows reaches the subnormal
+    # range, where it does not, so the comparison there is to a few units of the last place.
+    g1 = [t.grad.clone() for t in (q, k, v)]
+    for t in (q, k, v):
+        t.grad = None
+    fn(q, k, v, kernel, stride, 1, causal).backward(d_out * 2)
+    for name, a, b in zip(("dq", "dk", "dv"), g1, (q.grad, k.grad, v.grad)):
+        assert torch.isfinite(b).all()
+        if dtype == torch.bfloat16:
+            assert torch.equal(a * 2, b), f"doubling dO must double {name} bit-exactly"
+        else:
+            assert torch.allclose(b.float(), a.float() * 2, atol=1e-4, rtol=4e-3), f"doubling dO must double {name}"
+
+
+def test_config3_backward_full_size_sampled():
+    _backward_sampled(natten_amd.na2d, (128, 128), 16, 128, (32, 32), (16, 16), (False, False), torch.float16, 0.5,
+                      n_q=24, n_k=12, seed=5, tol=1e-2)
+
+
+def test_config4_backward_full_size_sampled():
+    _backward_sampled(natten_amd.na3d, (30, 48, 80), 24, 128, (18, 24, 24), (1, 8, 8), (True, False, False),
+                      torch.bfloat16, 1.0, n_q=12, n_k=4, seed=6, tol=2e-2)
