@@ -117,10 +117,10 @@ class AmdFmhaFunction(torch.autograd.Function):
         query, key, value, out, d_out = (
             pad_head_dim(t.contiguous(), d_pad).contiguous() for t in (query, key, value, out, d_out)
         )
-        delta = _lib.compute_delta(out, d_out)
+        delta = torch_ops.compute_delta(out, d_out)
         sq, skv = query.shape[1], key.shape[1]
         pq, pkv = -(-sq // 128) * 128, -(-skv // 128) * 128
-        dq, dk, dv = _lib.attention_backward(
+        dq, dk, dv = torch_ops.attention_backward(
             _pad_rows(query, pq), _pad_rows(key, pkv), _pad_rows(value, pkv), _pad_rows(d_out, pq),
             _pad_rows(lse, pq), _pad_rows(delta, pq), sq, skv, is_causal, scale,
         )

@@ -238,7 +238,7 @@ class AmdFnaFunction(torch.autograd.Function):
         query, key, value, output, d_output = (
             pad_head_dim(t.contiguous(), d_pad).contiguous() for t in (query, key, value, output, d_output)
         )
-        delta = _lib.compute_delta(output, d_output)
+        delta = torch_ops.compute_delta(output, d_output)
 
         def perm(x, tile):
             return token_permute_operation(x.contiguous(), tile, dilation, flip_tiled_dims=True)
@@ -249,7 +249,7 @@ class AmdFnaFunction(torch.autograd.Function):
         delta_perm, _, _ = perm(delta.unsqueeze(-1), q_tile)
         k_perm, _, kv_shape = perm(key, kv_tile)
         v_perm, _, _ = perm(value, kv_tile)
-        dq_perm, dk_perm, dv_perm = _lib.fna_backward(
+        dq_perm, dk_perm, dv_perm = torch_ops.fna_backward(
             q_perm, k_perm, v_perm, do_perm, lse_perm.squeeze(-1).contiguous(), delta_perm.squeeze(-1).contiguous(),
             kernel_size, stride, dilation, is_causal, scale, q_shape, kv_shape, qkv_shape, q_tile, kv_tile,
         )

@@ -85,6 +85,45 @@ def _(q, k, v, cumulative_seqlen_q, cumulative_seqlen_kv, max_seqlen_q, max_seql
     return torch.empty_like(q), q.new_empty(q.shape[:-1], dtype=torch.float32)
 
 
+@torch.library.custom_op("natten_amd::compute_delta", mutates_args=(), device_types="cuda")
+def _compute_delta_op(out: Tensor, d_out: Tensor) -> Tensor:
+    return _lib.compute_delta(out, d_out)
+
+
+@_compute_delta_op.register_fake
+def _(out, d_out):
+    return out.new_empty(out.shape[:-1], dtype=torch.float32)
+
+
+@torch.library.custom_op("natten_amd::fna_backward", mutates_args=(), device_types="cuda")
+def _fna_backward_op(
+    q: Tensor, k: Tensor, v: Tensor, d_out: Tensor, lse: Tensor, delta: Tensor, kernel_size: List[int],
+    stride: List[int], dilation: List[int], is_causal: List[bool], scale: float, q_shape: List[int],
+    kv_shape: List[int], qkv_shape: List[int], q_tile_shape: List[int], kv_tile_shape: List[int],
+) -> Tuple[Tensor, Tensor, Tensor]:
+    return _lib.fna_backward(q, k, v, d_out, lse, delta, kernel_size, stride, dilation, is_causal, scale, q_shape,
+                             kv_shape, qkv_shape, q_tile_shape, kv_tile_shape)
+
+
+@_fna_backward_op.register_fake
+def _(q, k, v, d_out, lse, delta, kernel_size, stride, dilation, is_causal, scale, q_shape, kv_shape, qkv_shape,
+      q_tile_shape, kv_tile_shape):
+    return torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+
+
+@torch.library.custom_op("natten_amd::attention_backward", mutates_args=(), device_types="cuda")
+def _attention_backward_op(
+    q: Tensor, k: Tensor, v: Tensor, d_out: Tensor, lse: Tensor, delta: Tensor, seqlen_q: int, seqlen_kv: int,
+    is_causal: bool, scale: float,
+) -> Tuple[Tensor, Tensor, Tensor]:
+    return _lib.attention_backward(q, k, v, d_out, lse, delta, seqlen_q, seqlen_kv, is_causal, scale)
+
+
+@_attention_backward_op.register_fake
+def _(q, k, v, d_out, lse, delta, seqlen_q, seqlen_kv, is_causal, scale):
+    return torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+
+
 def _permuted_shape(x: Tensor, tile_shape: List[int], dilation: List[int]) -> List[int]:
     na_dim = x.dim() - 3
     groups, seqlen = 1, 1
@@ -174,6 +213,29 @@ def attention_forward_varlen(q, k, v, cumulative_seqlen_q, cumulative_seqlen_kv,
     return _lib.attention_forward_varlen(q, k, v, cumulative_seqlen_q, cumulative_seqlen_kv, max_seqlen_q,
                                          max_seqlen_kv, is_causal, scale, q_scale=q_scale, k_scale=k_scale,
                                          v_scale=v_scale)
+
+
+def compute_delta(out, d_out):
+    if _tracing():
+        return _compute_delta_op(out, d_out)
+    return _lib.compute_delta(out, d_out)
+
+
+def fna_backward(q, k, v, d_out, lse, delta, kernel_size, stride, dilation, is_causal, scale, q_shape, kv_shape,
+                 qkv_shape, q_tile_shape, kv_tile_shape):
+    if _tracing():
+        return _fna_backward_op(q, k, v, d_out, lse, delta, _ints(kernel_size), _ints(stride), _ints(dilation),
+                                [bool(c) for c in is_causal], float(scale), _ints(q_shape), _ints(kv_shape),
+                                _ints(qkv_shape), _ints(q_tile_shape), _ints(kv_tile_shape))
+    return _lib.fna_backward(q, k, v, d_out, lse, delta, kernel_size, stride, dilation, is_causal, scale, q_shape,
+                             kv_shape, qkv_shape, q_tile_shape, kv_tile_shape)
+
+
+def attention_backward(q, k, v, d_out, lse, delta, seqlen_q, seqlen_kv, is_causal, scale):
+    if _tracing():
+        return _attention_backward_op(q, k, v, d_out, lse, delta, int(seqlen_q), int(seqlen_kv), bool(is_causal),
+                                      float(scale))
+    return _lib.attention_backward(q, k, v, d_out, lse, delta, seqlen_q, seqlen_kv, is_causal, scale)
 
 
 def token_permute(x, tile_shape, dilation, flip_tiled_dims, widen=False):

@@ -50,3 +50,42 @@ def test_compiled_equals_eager(name):
         ref_out, ref_lse = fn(*args)
         out, lse = torch.compile(fn, backend="aot_eager", fullgraph=True)(*args)
     assert torch.equal(out, ref_out) and torch.equal(lse, ref_lse)
+
+
+GRAD_CASES = {
+    "na2d": (lambda q, k, v: natten_amd.na2d(q, k, v, (5, 7), (2, 1), (1, 1), (False, True)), [(1, 20, 24, 2, 64)] * 3),
+    "na3d padded head dim": (lambda q, k, v: natten_amd.na3d(q, k, v, (2, 5, 5)), [(1, 4, 8, 8, 2, 40)] * 3),
+    "attention": (lambda q, k, v: natten_amd.attention(q, k, v, is_causal=True), [(2, 100, 4, 32)] * 3),
+}
+
+
+@pytest.mark.parametrize("name", sorted(GRAD_CASES))
+def test_forward_and_backward_trace_with_fake_tensors(name):
+    # Inputs that require grad: dynamo has to trace the autograd function's forward *and* backward
+    # (it turns both into graphs of custom operators) to compile the call at all.  The backward
+    # itself is not run here: the autograd engine wants a real device for "cuda" tensors; the
+    # GPU test below runs the compiled training step.
+    fn, shapes = GRAD_CASES[name]
+    torch._dynamo.reset()
+    with FakeTensorMode():
+        args = [torch.empty(s, device="cuda", dtype=torch.bfloat16, requires_grad=True) for s in shapes]
+        out = torch.compile(fn, backend="eager", fullgraph=True)(*args)
+        assert out.requires_grad and out.grad_fn is not None
+        assert tuple(out.shape) == tuple(shapes[0]) and out.dtype == torch.bfloat16
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", sorted(GRAD_CASES))
+def test_compiled_training_step_equals_eager(name):
+    fn, shapes = GRAD_CASES[name]
+    torch._dynamo.reset()
+    gen = torch.Generator().manual_seed(0)
+    base = [torch.randn(s, generator=gen).to(torch.bfloat16).cuda() for s in shapes]
+    d_out = torch.randn(shapes[0], generator=gen).to(torch.bfloat16).cuda()
+    grads = []
+    for f in (fn, torch.compile(fn, backend="aot_eager", fullgraph=True)):
+        args = [t.clone().requires_grad_(True) for t in base]
+        f(*args).backward(d_out)
+        grads.append([a.grad for a in args])
+    for a, b in zip(*grads):
+        assert torch.equal(a, b)
