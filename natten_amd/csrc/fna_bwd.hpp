@@ -78,20 +78,14 @@ fna_bwd_kernel(const FnaBwdParams p) {
   using vec8 = typename M::vec8;
   using vec2 = typename M::vec2;
 
-  // Tile copies per stage: Y1 in the layout of b128 row reads (for S), Y1 in the layout of
-  // transpose reads (for acc1), Y2 in row layout (for dP), Y2 in transpose layout (for acc2).
-#ifndef NA_BWD_DV_STAGES
-#define NA_BWD_DV_STAGES 2
-#endif
-  constexpr int NS = (ROLE == kBwdDKV && D == 128) ? 2 : (ROLE == kBwdDV ? NA_BWD_DV_STAGES : 3);  // stages: tiles are copied NS - 1 ahead
-  constexpr int SZ_1K = NS * TILE_BYTES;
-  constexpr int SZ_1T = HAS_DS ? NS * TILE_BYTES : 1024;
-  constexpr int SZ_2K = HAS_DS ? NS * TILE_BYTES : 1024;
-  constexpr int SZ_2T = HAS_PV ? NS * TILE_BYTES : 1024;
-  __shared__ __attribute__((aligned(1024))) char sY1k[SZ_1K];
-  __shared__ __attribute__((aligned(1024))) char sY1t[SZ_1T];
-  __shared__ __attribute__((aligned(1024))) char sY2k[SZ_2K];
-  __shared__ __attribute__((aligned(1024))) char sY2t[SZ_2T];
+  // One copy of Y1 and one of Y2 per stage, in the layout that serves row reads (S, dP) and
+  // transpose reads (the accumulations) alike.
+  // Stages: tiles are copied NS - 1 ahead.  The dV role at head dim 128 fits two workgroups on a
+  // CU with two stages (which beats one workgroup with three); the others are held to one
+  // workgroup by their registers.
+  constexpr int NS = (ROLE == kBwdDV && D == 128) ? 2 : 3;
+  __shared__ __attribute__((aligned(1024))) char sY1[NS * TILE_BYTES];
+  __shared__ __attribute__((aligned(1024))) char sY2[NS * TILE_BYTES];
   __shared__ __attribute__((aligned(16))) uint32_t sTabA[NS * BT];
   __shared__ __attribute__((aligned(16))) uint32_t sTabB[NS * BT];
   __shared__ __attribute__((aligned(16))) float sLse[NS * BT];
@@ -276,13 +270,12 @@ fna_bwd_kernel(const FnaBwdParams p) {
   const T* y2_all = reinterpret_cast<const T*>(KV_STATIONARY ? p.d_out : p.v);
 
   // copy i of a thread moves chunk P = i * NT + tid of the tile (row P / CPR, LDS slot P % CPR)
-  uint32_t off_k[PER], off_t[PER];
+  uint32_t off_u[PER];
 #pragma unroll
   for (int i = 0; i < PER; ++i) {
     const int P = i * NT + tid;
     const int row = P / CPR, slot = P % CPR;
-    off_k[i] = uint32_t(row) * uint32_t(b_stride * 2) + uint32_t(L::k_slot(row, slot) * 16);
-    off_t[i] = uint32_t(row) * uint32_t(b_stride * 2) + uint32_t(L::v_slot(row, slot) * 16);
+    off_u[i] = uint32_t(row) * uint32_t(b_stride * 2) + uint32_t(L::u_slot(row, slot) * 16);
   }
 
   struct Tile {
@@ -381,17 +374,15 @@ fna_bwd_kernel(const FnaBwdParams p) {
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
       const uint32_t d = dst + uint32_t(i * NT * 16);
-      async_copy16_asm<0>(y1, off_k[i], lds_address(sY1k) + d);
-      if constexpr (HAS_DS) async_copy16_asm<0>(y1, off_t[i], lds_address(sY1t) + d);
-      if constexpr (HAS_DS) async_copy16_asm<0>(y2, off_k[i], lds_address(sY2k) + d);
-      if constexpr (HAS_PV) async_copy16_asm<0>(y2, off_t[i], lds_address(sY2t) + d);
+      async_copy16_asm<0>(y1, off_u[i], lds_address(sY1) + d);
+      async_copy16_asm<0>(y2, off_u[i], lds_address(sY2) + d);
     }
   };
 
   // lane-constant LDS read offsets (same fragment layouts as the forward kernel)
   int k_off[KSTEPS];
 #pragma unroll
-  for (int ks = 0; ks < KSTEPS; ++ks) k_off[ks] = l32 * ROWB + L::k_slot(l32, ks * 2 + g) * 16;
+  for (int ks = 0; ks < KSTEPS; ++ks) k_off[ks] = l32 * ROWB + L::u_slot(l32, ks * 2 + g) * 16;
   const int l16 = lane & 15;
   const int v_e = l16 >> 2, v_j4 = l16 & 3;
   const int v_row = 4 * g + v_e;
@@ -404,8 +395,8 @@ fna_bwd_kernel(const FnaBwdParams p) {
   auto tr_frag = [&](const char* s, int sb, int h, int db) {
     const int r0 = sb * 32 + h * 16 + v_row;
     const int c = db * 4 + v_chunk;
-    const s16x4_t lo = lds_read_tr16(s + r0 * ROWB + v_sub + L::v_slot(r0, c) * 16);
-    const s16x4_t hi = lds_read_tr16(s + (r0 + 8) * ROWB + v_sub + L::v_slot(r0 + 8, c) * 16);
+    const s16x4_t lo = lds_read_tr16(s + r0 * ROWB + v_sub + L::u_slot(r0, c) * 16);
+    const s16x4_t hi = lds_read_tr16(s + (r0 + 8) * ROWB + v_sub + L::u_slot(r0 + 8, c) * 16);
     return __builtin_bit_cast(vec8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
   };
 
@@ -423,27 +414,22 @@ fna_bwd_kernel(const FnaBwdParams p) {
   constexpr int N1 = 2 * NP;
   constexpr int NC = 2 * DB * W;                           // accumulation slots per sub-block
   constexpr int G = N1 + 2 * NC;
-#ifndef NA_BWD_PF
-#define NA_BWD_PF 3
-#endif
-  constexpr int PF = NA_BWD_PF;                            // fragments read ahead
+  constexpr int PF = 3;                                    // fragments read ahead
   auto tile_body = [&](auto masked_tag, int stage, uint32_t addc, uint32_t subc) __attribute__((always_inline)) {
     constexpr bool MASKED = decltype(masked_tag)::value;
-    const char* y1k = sY1k + stage * TILE_BYTES;
-    const char* y1t = sY1t + (HAS_DS ? stage * TILE_BYTES : 0);
-    const char* y2k = sY2k + (HAS_DS ? stage * TILE_BYTES : 0);
-    const char* y2t = sY2t + (HAS_PV ? stage * TILE_BYTES : 0);
+    const char* y1 = sY1 + stage * TILE_BYTES;
+    const char* y2 = sY2 + stage * TILE_BYTES;
 
     auto frag = [&](auto x_tag) {
       constexpr int x = decltype(x_tag)::value;
       if constexpr (x < N1) {
         constexpr int sb = x / NP, ks = (x % NP) / WP, which = x % WP;
-        return row_frag(which ? y2k : y1k, sb, ks);
+        return row_frag(which ? y2 : y1, sb, ks);
       } else {
         constexpr int n = x - N1;
         constexpr int sb = n / NC, idx = n % NC, h = idx / (DB * W), db = (idx / W) % DB;
         constexpr bool to_acc1 = HAS_DS && (idx % W == 0);
-        return tr_frag(to_acc1 ? y1t : y2t, sb, h, db);
+        return tr_frag(to_acc1 ? y1 : y2, sb, h, db);
       }
     };
 
@@ -552,7 +538,7 @@ fna_bwd_kernel(const FnaBwdParams p) {
 
   // ---- pipeline: tile `it` is multiplied while tiles it+1 .. it+NS-1 are in flight ----------------
   // Descriptor queue: d[0] = tile `it`, d[k] = tile it + k.
-  constexpr int CPT = PER * (1 + (HAS_DS ? 2 : 0) + (HAS_PV ? 1 : 0));  // tile copies per thread and tile
+  constexpr int CPT = 2 * PER;  // tile copies per thread and tile
   auto run_pass = [&](auto masked_tag, int n_iter) __attribute__((always_inline)) {
     constexpr bool MASKED = decltype(masked_tag)::value;
     if (n_iter <= 0) return;

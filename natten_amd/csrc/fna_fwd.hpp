@@ -220,6 +220,13 @@ struct FnaSmem {
   static constexpr int BYTES = STAGES * 2 * TILE_BYTES + KVT * 4;  // static LDS of the kernel
   static __host__ __device__ constexpr int k_slot(int r, int c) { return c ^ ((r / RPL) % CPR); }
   static __host__ __device__ constexpr int v_slot(int r, int c) { return c ^ (2 * ((r / RPL) % (CPR / 2))); }
+  // One layout that serves both kinds of read (the backward kernels read the same tile both
+  // ways): the XOR pattern runs through the even values over the first half of a 16-row period
+  // (what the transpose reads need) and through the odd ones over the second half (so that the
+  // 16 rows of a b128 column read still hit 16 different slots).
+  static __host__ __device__ constexpr int u_slot(int r, int c) {
+    return c ^ ((2 * ((r / RPL) % (CPR / 2))) | (((r / RPL) / (CPR / 2)) & 1));
+  }
 };
 
 // MQ 32-row query blocks per wave.  MQ = 1 runs two waves per SIMD (256 registers each);
