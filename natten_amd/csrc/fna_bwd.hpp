@@ -285,49 +285,62 @@ fna_bwd_kernel(const FnaBwdParams p) {
   };
   // The streamed tiles in visiting order: dimension 2 fastest, dimension 0 slowest; the
   // key-stationary roles walk the box once per query head of the key head's group.  The box is
-  // walked twice: first the tiles that need the element mask, then the whole ones (see full_t0).
+  // walked twice: first the tiles that need the element mask (the box minus the inner box of
+  // whole tiles, see full_t0), then the whole ones (the inner box itself).
   const int total = box_n[0] * box_n[1] * box_n[2];
   const int n_whole = (full_t1[0] - full_t0[0]) * (full_t1[1] - full_t0[1]) * (full_t1[2] - full_t0[2]);
-  int walk[3] = {0, 0, 0}, walk_head = 0;
-  auto is_whole = [&]() {
-    bool w = true;
-#pragma unroll
-    for (int a = 0; a < 3; ++a) {
-      const int c = box_tile0[a] + walk[a];
-      w = w && (c >= full_t0[a]) && (c < full_t1[a]);
-    }
-    return w;
-  };
-  auto advance = [&]() {
-    if (++walk[2] == box_n[2]) {
-      walk[2] = 0;
-      if (++walk[1] == box_n[1]) {
-        walk[1] = 0;
-        if (++walk[0] == box_n[0]) {
-          walk[0] = 0;
+  const int head_b0 = KV_STATIONARY ? head_a * rep : head_a / rep;
+  int wc[3], walk_head = 0;  // position of the walk in absolute tile coordinates
+  // one step inside the box of the pass (WHOLE: the inner box, else the whole box)
+  auto step = [&](auto whole_tag) {
+    constexpr bool WHOLE = decltype(whole_tag)::value;
+    auto lo = [&](int a) { return WHOLE ? full_t0[a] : box_tile0[a]; };
+    auto hi = [&](int a) { return WHOLE ? full_t1[a] : box_tile0[a] + box_n[a]; };
+    if (++wc[2] == hi(2)) {
+      wc[2] = lo(2);
+      if (++wc[1] == hi(1)) {
+        wc[1] = lo(1);
+        if (++wc[0] == hi(0)) {
+          wc[0] = lo(0);
           ++walk_head;
         }
       }
     }
   };
-  // next tile of the wanted class; past the last one the walk runs into later heads, whose
-  // descriptors are never used
-  auto next_tile = [&](bool want_whole, int remaining) {
-    if (remaining > 0)
-      while (is_whole() != want_whole) advance();
+  // masked pass: a position at the start of a run of whole tiles jumps to the run's end
+  auto skip_whole = [&]() {
+    while (n_whole > 0 && wc[2] == full_t0[2] && wc[1] >= full_t0[1] && wc[1] < full_t1[1] && wc[0] >= full_t0[0] &&
+           wc[0] < full_t1[0]) {
+      wc[2] = full_t1[2] - 1;
+      step(std::false_type{});
+    }
+  };
+  auto start_walk = [&](auto whole_tag) {
+    constexpr bool WHOLE = decltype(whole_tag)::value;
+#pragma unroll
+    for (int a = 0; a < 3; ++a) wc[a] = WHOLE ? full_t0[a] : box_tile0[a];
+    walk_head = 0;
+    if constexpr (!WHOLE) skip_whole();
+  };
+  // descriptor of the current position, then on to the next one; `more` = tiles of this pass still
+  // to come after this one (past the last one the position is never used)
+  auto next_tile = [&](auto whole_tag, bool more) {
+    constexpr bool WHOLE = decltype(whole_tag)::value;
     Tile t;
     int cc[3], half = 0;
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
-      const int c = box_tile0[a] + walk[a];
-      t.origin[a] = c * b_sub[a];
+      t.origin[a] = wc[a] * b_sub[a];
       const bool split = (a == split_dim);
-      half |= split ? (c & 1) : 0;
-      cc[a] = split ? (c >> 1) : c;
+      half |= split ? (wc[a] & 1) : 0;
+      cc[a] = split ? (wc[a] >> 1) : wc[a];
     }
     t.row0 = (cc[0] + b_tiled[0] * (cc[1] + b_tiled[1] * cc[2])) * AT + half * BT;
-    t.head_b = KV_STATIONARY ? head_a * rep + walk_head : head_a / rep;
-    advance();
+    t.head_b = KV_STATIONARY ? head_b0 + walk_head : head_b0;
+    if (more) {
+      step(whole_tag);
+      if constexpr (!WHOLE) skip_whole();
+    }
     return t;
   };
 
@@ -337,6 +350,8 @@ fna_bwd_kernel(const FnaBwdParams p) {
   qo[1] = (lane / b_sub[0]) % b_sub[1];
   qo[2] = lane / (b_sub[0] * b_sub[1]);
 
+  const uint32_t lds_y1 = uint32_t(__builtin_amdgcn_readfirstlane(int(lds_address(sY1))));
+  const uint32_t lds_y2 = uint32_t(__builtin_amdgcn_readfirstlane(int(lds_address(sY2))));
   const uint32_t stat_off = uint32_t(lane) * uint32_t(p.heads_q) * 4u;  // byte offset of streamed row `lane` in lse / delta
   auto issue = [&](const Tile& t, int stage, bool masked) {
     if constexpr (KV_STATIONARY) {
@@ -368,14 +383,14 @@ fna_bwd_kernel(const FnaBwdParams p) {
       float* dst = (wave == 1) ? &sLse[stage * BT] : (wave == 2 && HAS_DS) ? &sDelta[stage * BT] : &sSpare[0];
       if (wave != 0) async_copy4_asm(src, stat_off, lds_address(dst));
     }
-    const T* y1 = y1_all + row * b_stride + int64_t(t.head_b) * D;
-    const T* y2 = y2_all + row * b_stride + int64_t(t.head_b) * D;
-    const uint32_t dst = uint32_t(stage * TILE_BYTES + wave * 1024);
+    const int64_t elem = row * b_stride + int64_t(t.head_b) * D;
+    const uint64_t y1 = uniform64(y1_all + elem), y2 = uniform64(y2_all + elem);
+    const uint32_t dst = uint32_t(__builtin_amdgcn_readfirstlane(stage * TILE_BYTES + wave * 1024));
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
       const uint32_t d = dst + uint32_t(i * NT * 16);
-      async_copy16_asm<0>(y1, off_u[i], lds_address(sY1) + d);
-      async_copy16_asm<0>(y2, off_u[i], lds_address(sY2) + d);
+      async_copy16_uniform(y1, off_u[i], lds_y1 + d);
+      async_copy16_uniform(y2, off_u[i], lds_y2 + d);
     }
   };
 
@@ -542,14 +557,27 @@ fna_bwd_kernel(const FnaBwdParams p) {
   auto run_pass = [&](auto masked_tag, int n_iter) __attribute__((always_inline)) {
     constexpr bool MASKED = decltype(masked_tag)::value;
     if (n_iter <= 0) return;
-    walk[0] = walk[1] = walk[2] = 0;
-    walk_head = 0;
-    Tile d[NS];
+    start_walk(std::integral_constant<bool, !MASKED>{});
+    // dQ role, masked pass: origins of the tiles in flight (the lane's mask constants need the
+    // origin of the tile being multiplied); og<k> = origin of tile it + k
+    constexpr bool NEED_ORIGIN = MASKED && !KV_STATIONARY;
+    int og0[3] = {0, 0, 0}, og1[3] = {0, 0, 0}, og2[3] = {0, 0, 0};
+    if (0 < n_iter && NS > 1) {
+      const Tile t = next_tile(std::integral_constant<bool, !MASKED>{}, 1 < n_iter);
+      issue(t, 0, MASKED);
+      if constexpr (NEED_ORIGIN) {
 #pragma unroll
-    for (int k = 0; k < NS; ++k) d[k] = next_tile(!MASKED, n_iter - k);
+        for (int a = 0; a < 3; ++a) og0[a] = t.origin[a];
+      }
+    }
+    if (1 < n_iter && NS > 2) {
+      const Tile t = next_tile(std::integral_constant<bool, !MASKED>{}, 2 < n_iter);
+      issue(t, 1, MASKED);
+      if constexpr (NEED_ORIGIN) {
 #pragma unroll
-    for (int k = 0; k < NS - 1; ++k)
-      if (k < n_iter) issue(d[k], k, MASKED);
+        for (int a = 0; a < 3; ++a) og1[a] = t.origin[a];
+      }
+    }
 
     for (int it = 0; it < n_iter; ++it) {
       const int stage = it % NS;
@@ -563,22 +591,33 @@ fna_bwd_kernel(const FnaBwdParams p) {
         wait_vmcnt<0>();
       }
       __syncthreads();  // tile `it` and its tables are in LDS; everyone is done with the stage of tile it - 1
-      if (it + NS - 1 < n_iter) issue(d[NS - 1], (it + NS - 1) % NS, MASKED);
+      if (it + NS - 1 < n_iter) {
+        const Tile t = next_tile(std::integral_constant<bool, !MASKED>{}, it + NS < n_iter);
+        issue(t, (it + NS - 1) % NS, MASKED);
+        if constexpr (NEED_ORIGIN) {
+#pragma unroll
+          for (int a = 0; a < 3; ++a) (NS == 3 ? og2[a] : og1[a]) = t.origin[a];
+        }
+      }
 
       uint32_t addc = 0, subc = 0;
-      if constexpr (MASKED && !KV_STATIONARY) {
+      if constexpr (NEED_ORIGIN) {
 #pragma unroll
         for (int a = 0; a < 3; ++a) {
-          const int lo = na_min(na_max(wst[a] - d[0].origin[a], 0), b_sub[a]);
-          const int hi = na_min(na_max(wen[a] - d[0].origin[a], 0), b_sub[a]);
+          const int lo = na_min(na_max(wst[a] - og0[a], 0), b_sub[a]);
+          const int hi = na_min(na_max(wen[a] - og0[a], 0), b_sub[a]);
           addc |= uint32_t(512 - lo) << (10 * a);
           subc |= uint32_t(511 + hi) << (10 * a);
         }
       }
       tile_body(masked_tag, stage, addc, subc);
+      if constexpr (NEED_ORIGIN) {
 #pragma unroll
-      for (int k = 0; k + 1 < NS; ++k) d[k] = d[k + 1];
-      d[NS - 1] = next_tile(!MASKED, n_iter - it - NS);
+        for (int a = 0; a < 3; ++a) {
+          og0[a] = og1[a];
+          og1[a] = og2[a];
+        }
+      }
     }
     wait_vmcnt<0>();
     __syncthreads();  // the stages are free for the next pass

@@ -160,6 +160,24 @@ static __device__ __forceinline__ void async_copy4_asm(const void* base, uint32_
       : "memory", "m0");
 }
 
+// The same copy for callers whose `base` and `lds_addr` already live in scalar registers
+// (made uniform once per tile with readfirstlane), which saves three moves per copy.
+static __device__ __forceinline__ void async_copy16_uniform(uint64_t base, uint32_t voff, uint32_t lds_addr) {
+  asm volatile(
+      "s_mov_b32 m0, %0\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dwordx4 %1, %2"
+      :
+      : "s"(lds_addr), "v"(voff), "s"(base)
+      : "memory", "m0");
+}
+
+static __device__ __forceinline__ uint64_t uniform64(const void* p) {
+  const uint64_t b = reinterpret_cast<uint64_t>(p);
+  return (uint64_t(uint32_t(__builtin_amdgcn_readfirstlane(int(b >> 32)))) << 32) |
+         uint32_t(__builtin_amdgcn_readfirstlane(int(uint32_t(b))));
+}
+
 static __device__ __forceinline__ uint32_t lds_address(const void* p) {
 #pragma clang diagnostic push
 #pragma clang diagnostic ignored "-Wold-style-cast"
