@@ -45,11 +45,15 @@ def amd_fmha(
     scale = scale or head_dim**-0.5
     d_pad = padded_head_dim(head_dim)
     if torch.is_grad_enabled() and (query.requires_grad or key.requires_grad or value.requires_grad):
-        if is_fp8(query.dtype) or cumulative_seqlen_Q is not None:
-            raise NotImplementedError(
-                "natten_amd attention has a backward pass for fp16 / bf16 fixed-length batches only."
+        if is_fp8(query.dtype):
+            raise NotImplementedError("natten_amd attention has no backward pass for 8-bit float operands.")
+        if cumulative_seqlen_Q is not None:
+            out, lse = AmdFmhaVarlenFunction.apply(
+                query, key, value, bool(is_causal), float(scale), cumulative_seqlen_Q, cumulative_seqlen_KV,
+                int(max_seqlen_Q), int(max_seqlen_KV),
             )
-        out, lse = AmdFmhaFunction.apply(query, key, value, bool(is_causal), float(scale))
+        else:
+            out, lse = AmdFmhaFunction.apply(query, key, value, bool(is_causal), float(scale))
         if out_dtype is not None and out.dtype != out_dtype:
             out = out.to(out_dtype)
         return (out, lse) if return_lse else out
@@ -125,3 +129,48 @@ class AmdFmhaFunction(torch.autograd.Function):
             _pad_rows(lse, pq), _pad_rows(delta, pq), sq, skv, is_causal, scale,
         )
         return dq[:, :sq, :, :head_dim], dk[:, :skv, :, :head_dim], dv[:, :skv, :, :head_dim], None, None
+
+
+class AmdFmhaVarlenFunction(torch.autograd.Function):
+    """Variable-length dense attention with a backward pass.  The forward is the sequence-packed
+    kernel; the backward runs the fixed-length backward kernels once per sequence (on zero-padded
+    copies of its rows), which costs one device-to-host copy of the cumulative lengths and one
+    set of launches per sequence.  Counterpart of the varlen arguments of
+    src/natten/backends/blackwell_fmha.py:52-170."""
+
+    @staticmethod
+    def forward(ctx, query, key, value, is_causal, scale, cu_q, cu_kv, max_q, max_kv):
+        with torch.no_grad():
+            out, lse = amd_fmha(query, key, value, is_causal=is_causal, scale=scale, return_lse=True,
+                                cumulative_seqlen_Q=cu_q, cumulative_seqlen_KV=cu_kv, max_seqlen_Q=max_q,
+                                max_seqlen_KV=max_kv)
+        ctx.save_for_backward(query, key, value, out, lse, cu_q, cu_kv)
+        ctx.args = (is_causal, scale)
+        ctx.mark_non_differentiable(lse)
+        return out, lse
+
+    @staticmethod
+    def backward(ctx, d_out, d_lse):
+        query, key, value, out, lse, cu_q, cu_kv = ctx.saved_tensors
+        is_causal, scale = ctx.args
+        head_dim = query.shape[-1]
+        d_pad = padded_head_dim(head_dim)
+        q, k, v, o, do = (pad_head_dim(t.contiguous(), d_pad).contiguous() for t in (query, key, value, out, d_out))
+        delta = torch_ops.compute_delta(o, do)
+        dq, dk, dv = torch.zeros_like(q), torch.zeros_like(k), torch.zeros_like(v)
+        bounds_q, bounds_kv = cu_q.tolist(), cu_kv.tolist()
+        for b in range(len(bounds_q) - 1):
+            q0, q1, k0, k1 = bounds_q[b], bounds_q[b + 1], bounds_kv[b], bounds_kv[b + 1]
+            sq, skv = q1 - q0, k1 - k0
+            if sq <= 0 or skv <= 0:
+                continue  # no queries, or no keys (output 0, nothing to differentiate)
+            pq, pkv = -(-sq // 128) * 128, -(-skv // 128) * 128
+            g = torch_ops.attention_backward(
+                _pad_rows(q[:, q0:q1], pq), _pad_rows(k[:, k0:k1], pkv), _pad_rows(v[:, k0:k1], pkv),
+                _pad_rows(do[:, q0:q1], pq), _pad_rows(lse[:, q0:q1], pq), _pad_rows(delta[:, q0:q1], pq),
+                sq, skv, is_causal, scale,
+            )
+            dq[:, q0:q1] = g[0][:, :sq]
+            dk[:, k0:k1] = g[1][:, :skv]
+            dv[:, k0:k1] = g[2][:, :skv]
+        return (dq[..., :head_dim], dk[..., :head_dim], dv[..., :head_dim]) + (None,) * 6
