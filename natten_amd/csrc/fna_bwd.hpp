@@ -55,7 +55,7 @@ struct FnaBwdParams {
 enum BwdRole : int { kBwdDQ = 0, kBwdDK = 1, kBwdDV = 2, kBwdDKV = 3 };
 
 template <typename T, int D, int ROLE>
-__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
 fna_bwd_kernel(const FnaBwdParams p) {
   constexpr bool KV_STATIONARY = ROLE != kBwdDQ;
   constexpr bool HAS_DS = ROLE != kBwdDV;                    // dP, dS and acc1 (dQ or dK)
@@ -80,10 +80,9 @@ fna_bwd_kernel(const FnaBwdParams p) {
 
   // One copy of Y1 and one of Y2 per stage, in the layout that serves row reads (S, dP) and
   // transpose reads (the accumulations) alike.
-  // Stages: tiles are copied NS - 1 ahead.  The dV role at head dim 128 fits two workgroups on a
-  // CU with two stages (which beats one workgroup with three); the others are held to one
-  // workgroup by their registers.
-  constexpr int NS = (ROLE == kBwdDV && D == 128) ? 2 : 3;
+  // Stages: tiles are copied NS - 1 ahead.  Two stages at head dim 128 keep a workgroup under
+  // half of the CU's LDS, so that two workgroups (two waves per SIMD) share a CU.
+  constexpr int NS = D == 128 ? 2 : 3;
   __shared__ __attribute__((aligned(1024))) char sY1[NS * TILE_BYTES];
   __shared__ __attribute__((aligned(1024))) char sY2[NS * TILE_BYTES];
   __shared__ __attribute__((aligned(16))) uint32_t sTabA[NS * BT];
@@ -417,76 +416,84 @@ fna_bwd_kernel(const FnaBwdParams p) {
 
   const float c_log2 = p.scale * kLog2e;
 
-  // One streamed tile.  The matrix instructions form one sequence of "slots" (first the
-  // products S and dP of the two 32-row sub-blocks, then the accumulations of the two
-  // sub-blocks); a slot is one operand fragment read ahead from LDS, one MFMA and its share of
-  // the vector work: the probabilities of sub-block 0 run under the products of sub-block 1,
-  // those of sub-block 1 under the accumulations of sub-block 0.  Slots are fenced so that the
-  // compiler keeps the interleaving.
+  // One streamed tile: its two 32-row sub-blocks one after the other, each as products (S, dP),
+  // probabilities, accumulations.  Only one sub-block's products are live at a time, which keeps
+  // the kernel within 256 registers: two workgroups share a CU, and the other wave of a SIMD
+  // fills the gaps of this one (a measured 1.2-1.3 x over interleaving the sub-blocks inside
+  // one wave per SIMD).  The matrix instructions form one sequence of fenced "slots", each with
+  // its operand fragment read from LDS a few slots ahead.
   constexpr int WP = HAS_DS ? 2 : 1;                       // products per k-step (S, dP)
   constexpr int W = (HAS_DS ? 1 : 0) + (HAS_PV ? 1 : 0);   // accumulators fed per transposed fragment position
   constexpr int NP = WP * KSTEPS;                          // product slots per sub-block
   constexpr int N1 = 2 * NP;
   constexpr int NC = 2 * DB * W;                           // accumulation slots per sub-block
   constexpr int G = N1 + 2 * NC;
-  constexpr int PF = 3;                                    // fragments read ahead
+  constexpr int PF = 2;                                    // fragments read ahead
   auto tile_body = [&](auto masked_tag, int stage, uint32_t addc, uint32_t subc) __attribute__((always_inline)) {
     constexpr bool MASKED = decltype(masked_tag)::value;
     const char* y1 = sY1 + stage * TILE_BYTES;
     const char* y2 = sY2 + stage * TILE_BYTES;
 
+    // slot x of the tile: a product slot (sub-block, index i < NP) or an accumulation slot (i < NC)
+    struct Slot {
+      bool prod;
+      int sb, i;
+    };
+    auto slot_of = [](int x) constexpr {
+      const int sb = x / (NP + NC), z = x % (NP + NC);
+      return Slot{z < NP, sb, z < NP ? z : z - NP};
+    };
     auto frag = [&](auto x_tag) {
-      constexpr int x = decltype(x_tag)::value;
-      if constexpr (x < N1) {
-        constexpr int sb = x / NP, ks = (x % NP) / WP, which = x % WP;
-        return row_frag(which ? y2 : y1, sb, ks);
+      constexpr Slot sl = slot_of(decltype(x_tag)::value);
+      if constexpr (sl.prod) {
+        constexpr int ks = sl.i / WP, which = sl.i % WP;
+        return row_frag(which ? y2 : y1, sl.sb, ks);
       } else {
-        constexpr int n = x - N1;
-        constexpr int sb = n / NC, idx = n % NC, h = idx / (DB * W), db = (idx / W) % DB;
-        constexpr bool to_acc1 = HAS_DS && (idx % W == 0);
-        return tr_frag(to_acc1 ? y1 : y2, sb, h, db);
+        constexpr int h = sl.i / (DB * W), db = (sl.i / W) % DB;
+        constexpr bool to_acc1 = HAS_DS && (sl.i % W == 0);
+        return tr_frag(to_acc1 ? y1 : y2, sl.sb, h, db);
       }
     };
 
     f32x16_t S[NSB], dP[NSB];
     vec8 pf[NSB][2], dsf[NSB][2];
-    // tables of the streamed rows, four rows (8*jj + 4*g + i of a sub-block) at a time; the
-    // group after the one in use is read ahead
-    u32x4_t ta[2], tb[2];
-    f32x4_t ls4[2], dl4[2];
+    // tables of the streamed rows, four rows (8*jj + 4*g + i of a sub-block) at a time, read
+    // when they are needed (the other wave covers the wait)
+    u32x4_t ta, tb;
+    f32x4_t ls4, dl4;
     auto load_group = [&](auto gi_tag) {
       constexpr int gi = decltype(gi_tag)::value;  // sub-block * 4 + jj
       if constexpr (gi < 2 * 4) {
         const int e0 = (gi / 4) * 32 + 8 * (gi % 4) + 4 * g;
         if constexpr (KV_STATIONARY) {
           if constexpr (MASKED) {
-            ta[gi & 1] = *reinterpret_cast<const u32x4_t*>(&sTabA[stage * BT + e0]);
-            tb[gi & 1] = *reinterpret_cast<const u32x4_t*>(&sTabB[stage * BT + e0]);
+            ta = *reinterpret_cast<const u32x4_t*>(&sTabA[stage * BT + e0]);
+            tb = *reinterpret_cast<const u32x4_t*>(&sTabB[stage * BT + e0]);
           }
-          ls4[gi & 1] = *reinterpret_cast<const f32x4_t*>(&sLse[stage * BT + e0]) * kLog2e;
-          if constexpr (HAS_DS) dl4[gi & 1] = *reinterpret_cast<const f32x4_t*>(&sDelta[stage * BT + e0]);
+          ls4 = *reinterpret_cast<const f32x4_t*>(&sLse[stage * BT + e0]) * kLog2e;
+          if constexpr (HAS_DS) dl4 = *reinterpret_cast<const f32x4_t*>(&sDelta[stage * BT + e0]);
         } else if constexpr (MASKED) {
-          ta[gi & 1] = *reinterpret_cast<const u32x4_t*>(&sTabA[e0]);
+          ta = *reinterpret_cast<const u32x4_t*>(&sTabA[e0]);
         }
       }
     };
     float held_p = 0.f, held_ds = 0.f;
     auto elem = [&](auto sb_tag, auto r_tag) {
       constexpr int sb = decltype(sb_tag)::value, r = decltype(r_tag)::value;
-      constexpr int jj = (sb * 4 + r / 4) & 1, i = r % 4;
-      if constexpr (i == 0) load_group(std::integral_constant<int, sb * 4 + r / 4 + 1>{});
+      constexpr int i = r % 4;
+      if constexpr (i == 0) load_group(std::integral_constant<int, sb * 4 + r / 4>{});
       float x;
-      if constexpr (KV_STATIONARY) x = fast_exp2(S[sb][r] * c_log2 - ls4[jj][i]);
+      if constexpr (KV_STATIONARY) x = fast_exp2(S[sb][r] * c_log2 - ls4[i]);
       else x = fast_exp2(S[sb][r] * c_log2 - lse_l);
       if constexpr (MASKED) {
         uint32_t ok;
-        if constexpr (KV_STATIONARY) ok = (key_packed + ta[jj][i]) & (tb[jj][i] - key_packed) & kGuardBits;
-        else ok = (ta[jj][i] + addc) & (subc - ta[jj][i]) & kGuardBits;
+        if constexpr (KV_STATIONARY) ok = (key_packed + ta[i]) & (tb[i] - key_packed) & kGuardBits;
+        else ok = (ta[i] + addc) & (subc - ta[i]) & kGuardBits;
         x = (ok == kGuardBits) ? x : 0.f;
       }
       float ds = 0.f;
       if constexpr (HAS_DS) {
-        if constexpr (KV_STATIONARY) ds = x * (dP[sb][r] - dl4[jj][i]);
+        if constexpr (KV_STATIONARY) ds = x * (dP[sb][r] - dl4[i]);
         else ds = x * (dP[sb][r] - delta_l);
       }
       if constexpr (r % 2 == 0) {
@@ -518,34 +525,25 @@ fna_bwd_kernel(const FnaBwdParams p) {
 
     vec8 fr[G];
     for_range<0, PF>([&](auto x_tag) { fr[decltype(x_tag)::value] = frag(x_tag); });
-    load_group(std::integral_constant<int, 0>{});
     for_range<0, G>([&](auto x_tag) __attribute__((always_inline)) {
       constexpr int x = decltype(x_tag)::value;
+      constexpr Slot sl = slot_of(x);
+      constexpr int sb = sl.sb;
       if constexpr (x + PF < G) fr[x + PF] = frag(std::integral_constant<int, x + PF>{});
-      if constexpr (x < N1) {
-        constexpr int sb = x / NP, ks = (x % NP) / WP, which = x % WP;
+      if constexpr (sl.prod) {
+        constexpr int ks = sl.i / WP, which = sl.i % WP;
         f32x16_t zero;
 #pragma unroll
         for (int r = 0; r < 16; ++r) zero[r] = 0.f;
         if constexpr (which == 0) S[sb] = M::run(fr[x], x1f[ks], ks == 0 ? zero : S[sb]);
         else dP[sb] = M::run(fr[x], x2f[ks], ks == 0 ? zero : dP[sb]);
-        if constexpr (sb == 1) {
-          // probabilities of sub-block 0
-          constexpr int s = x - NP;
-          constexpr int e_lo = (16 * s) / NP, e_hi = (16 * (s + 1)) / NP;
-          for_range<e_lo, e_hi - e_lo>([&](auto r_tag) { elem(std::integral_constant<int, 0>{}, r_tag); });
-        }
+        // all probabilities of the sub-block once its products are complete
+        if constexpr (sl.i == NP - 1) for_range<0, 16>([&](auto r_tag) { elem(std::integral_constant<int, sb>{}, r_tag); });
       } else {
-        constexpr int n = x - N1;
-        constexpr int sb = n / NC, idx = n % NC, h = idx / (DB * W), db = (idx / W) % DB;
-        constexpr bool to_acc1 = HAS_DS && (idx % W == 0);
+        constexpr int h = sl.i / (DB * W), db = (sl.i / W) % DB;
+        constexpr bool to_acc1 = HAS_DS && (sl.i % W == 0);
         if constexpr (to_acc1) acc1[db] = M::run(fr[x], dsf[sb][h], acc1[db]);
         else acc2[db] = M::run(fr[x], pf[sb][h], acc2[db]);
-        if constexpr (sb == 0) {
-          // probabilities of sub-block 1
-          constexpr int e_lo = (16 * idx) / NC, e_hi = (16 * (idx + 1)) / NC;
-          for_range<e_lo, e_hi - e_lo>([&](auto r_tag) { elem(std::integral_constant<int, 1>{}, r_tag); });
-        }
       }
       __builtin_amdgcn_sched_barrier(0);
     });
