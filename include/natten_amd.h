@@ -167,9 +167,10 @@ int natten_amd_compute_delta(const void* out, const void* d_out, float* delta, i
 /*
  * Fused neighborhood attention backward on token-permuted operands.
  *   q, d_out, dq [batch, seqlen_q, heads_q, head_dim]; k, v, dk, dv [batch, seqlen_kv, heads_kv,
- *   head_dim]; lse, delta [batch, seqlen_q, heads_q] float32 (lse from the forward pass, natural
- *   log; delta from natten_amd_compute_delta), all permuted like the forward operands
- *   (dimension 0 fastest inside a tile, dilation groups folded into batch).
+ *   head_dim], permuted like the forward operands (dimension 0 fastest inside a tile, dilation
+ *   groups folded into batch); lse, delta float32, permuted the same way and then stored
+ *   head-major, [batch, heads_q, seqlen_q] (the kernels read 64 consecutive rows of one head at
+ *   a time); lse from the forward pass (natural log), delta from natten_amd_compute_delta.
  *   Both tile shapes must hold 128 tokens and their last extent above 1 must be even; q_shape /
  *   kv_shape are the padded per-group layouts (multiples of the tiles), seqlen = their product.
  * dq, dk, dv are written completely (padding rows get zeros); nothing is accumulated through
@@ -187,9 +188,9 @@ int natten_amd_fna_backward(const void* q, const void* k, const void* v, const v
                             void* stream);
 
 /*
- * Dense attention backward (optional top-left causal mask).  Operands as above with
- * sequences zero-padded to padded_seqlen_q / padded_seqlen_kv rows (multiples of 128);
- * seqlen_q / seqlen_kv are the true lengths.
+ * Dense attention backward (optional top-left causal mask).  Operands as above (lse and delta
+ * head-major) with sequences zero-padded to padded_seqlen_q / padded_seqlen_kv rows (multiples
+ * of 128); seqlen_q / seqlen_kv are the true lengths.
  */
 int natten_amd_attention_backward(const void* q, const void* k, const void* v, const void* d_out,
                                   const float* lse, const float* delta, void* dq, void* dk,

@@ -326,8 +326,10 @@ def fna_backward(
     q: Tensor, k: Tensor, v: Tensor, d_out: Tensor, lse: Tensor, delta: Tensor, kernel_size, stride, dilation,
     is_causal, scale: float, q_shape, kv_shape, qkv_shape, q_tile_shape, kv_tile_shape,
 ) -> Tuple[Tensor, Tensor, Tensor]:
-    """Backward on token-permuted operands (128-token tiles on both sides) -> (dq, dk, dv)."""
+    """Backward on token-permuted operands (128-token tiles on both sides) -> (dq, dk, dv).
+    lse, delta: [batch, seqlen_q, heads_q] as the permute gives them; the kernels take them head-major."""
     L = lib()
+    lse, delta = lse.transpose(1, 2).contiguous(), delta.transpose(1, 2).contiguous()
     _require_gpu(q, k, v, d_out, lse, delta)
     if q.dtype not in (torch.float16, torch.bfloat16):
         raise NotImplementedError(f"natten_amd fna_backward does not support {q.dtype}.")
@@ -351,8 +353,10 @@ def attention_backward(
     q: Tensor, k: Tensor, v: Tensor, d_out: Tensor, lse: Tensor, delta: Tensor, seqlen_q: int, seqlen_kv: int,
     is_causal: bool, scale: float,
 ) -> Tuple[Tensor, Tensor, Tensor]:
-    """Dense attention backward on operands zero-padded to multiples of 128 rows -> (dq, dk, dv), padded alike."""
+    """Dense attention backward on operands zero-padded to multiples of 128 rows -> (dq, dk, dv), padded alike.
+    lse, delta: [batch, padded seqlen_q, heads_q]; the kernels take them head-major."""
     L = lib()
+    lse, delta = lse.transpose(1, 2).contiguous(), delta.transpose(1, 2).contiguous()
     _require_gpu(q, k, v, d_out, lse, delta)
     if q.dtype not in (torch.float16, torch.bfloat16):
         raise NotImplementedError(f"natten_amd attention_backward does not support {q.dtype}.")

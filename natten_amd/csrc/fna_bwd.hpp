@@ -34,8 +34,8 @@ struct FnaBwdParams {
   const void* k;      // [batch, seqlen_kv, heads_kv, D]
   const void* v;
   const void* d_out;  // like q
-  const float* lse;   // [batch, seqlen_q, heads_q], natural log
-  const float* delta; // [batch, seqlen_q, heads_q], rowsum(d_out * out)
+  const float* lse;   // [batch, heads_q, seqlen_q] (head-major: a tile's values are contiguous), natural log
+  const float* delta; // [batch, heads_q, seqlen_q], rowsum(d_out * out)
   void* dq;
   void* dk;
   void* dv;
@@ -251,8 +251,9 @@ fna_bwd_kernel(const FnaBwdParams p) {
       wst[a] = na_window_start(c, p.ksize[a], p.stride[a], extent[a], p.causal[a] != 0);
       wen[a] = na_window_end(c, wst[a], p.ksize[a], extent[a], p.causal[a] != 0);
     }
-    lse_l = p.lse[a_row * p.heads_q + head_a] * kLog2e;
-    delta_l = p.delta[a_row * p.heads_q + head_a];
+    const int64_t stat_idx = (int64_t(bg) * p.heads_q + head_a) * seq_a + int64_t(at) * AT + r_in;
+    lse_l = p.lse[stat_idx] * kLog2e;
+    delta_l = p.delta[stat_idx];
     // in-tile coordinates of every streamed position, packed in 10-bit fields
     for (int i = tid; i < BT; i += NT) {
       const int t0 = i % b_sub[0];
@@ -351,7 +352,7 @@ fna_bwd_kernel(const FnaBwdParams p) {
 
   const uint32_t lds_y1 = uint32_t(__builtin_amdgcn_readfirstlane(int(lds_address(sY1))));
   const uint32_t lds_y2 = uint32_t(__builtin_amdgcn_readfirstlane(int(lds_address(sY2))));
-  const uint32_t stat_off = uint32_t(lane) * uint32_t(p.heads_q) * 4u;  // byte offset of streamed row `lane` in lse / delta
+  const uint32_t stat_off = uint32_t(lane) * 4u;  // byte offset of streamed row `lane` in lse / delta (head-major)
   auto issue = [&](const Tile& t, int stage, bool masked) {
     if constexpr (KV_STATIONARY) {
       if (wave == 0 && masked) {
@@ -378,7 +379,7 @@ fna_bwd_kernel(const FnaBwdParams p) {
       // LSE / delta of the tile's 64 queries: one asynchronous 4-byte-per-lane copy each
       // (wave 1, wave 2; wave 3 and, without delta, wave 2 make the same number of copies into a
       // spare row so that every wave counts the same number of outstanding copies per tile)
-      const float* src = (wave == 2 && HAS_DS ? p.delta : p.lse) + row * p.heads_q + t.head_b;
+      const float* src = (wave == 2 && HAS_DS ? p.delta : p.lse) + (int64_t(bg) * p.heads_q + t.head_b) * seq_b + t.row0;
       float* dst = (wave == 1) ? &sLse[stage * BT] : (wave == 2 && HAS_DS) ? &sDelta[stage * BT] : &sSpare[0];
       if (wave != 0) async_copy4_asm(src, stat_off, lds_address(dst));
     }
