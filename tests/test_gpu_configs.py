@@ -193,3 +193,16 @@ def test_config3_backward_full_size_sampled():
 def test_config4_backward_full_size_sampled():
     _backward_sampled(natten_amd.na3d, (30, 48, 80), 24, 128, (18, 24, 24), (1, 8, 8), (True, False, False),
                       torch.bfloat16, 1.0, n_q=12, n_k=4, seed=6, tol=2e-2)
+
+
+@pytest.mark.parametrize("dil", [(1, 1), (2, 2)])
+def test_config2_backward_full(dil):
+    # the second configuration is small enough for the C oracle to differentiate it completely
+    q, k, v = make_qkv(2, (64, 64), 8, 8, 64, torch.bfloat16, seed=0)
+    d_out = torch.randn(q.shape, generator=torch.Generator().manual_seed(3)).to(torch.bfloat16).cuda()
+    for t in (q, k, v):
+        t.requires_grad_(True)
+    natten_amd.na2d(q, k, v, (13, 13), (1, 1), dil).backward(d_out)
+    refs = c_oracle.na_backward(to_np(q), to_np(k), to_np(v), to_np(d_out), (13, 13), (1, 1), dil, (False, False))
+    for name, got, ref in zip(("dq", "dk", "dv"), (q.grad, k.grad, v.grad), refs):
+        assert_close(f"{name} dilation {dil}", to_np(got), ref, atol=2e-2, rtol=2e-2)
