@@ -126,6 +126,9 @@ fna_bwd_kernel(const FnaBwdParams p) {
     tc[2] = rm % a_tiled[2];
     tc[1] = (rm / a_tiled[2]) % a_tiled[1];
     tc[0] = rm / (a_tiled[2] * a_tiled[1]);
+    // a causal dimension 0: the query tiles with the longest key ranges are the last ones;
+    // they start first (key tiles are already in that order)
+    if (!KV_STATIONARY && p.causal[0]) tc[0] = a_tiled[0] - 1 - tc[0];
   }
   const int at = tc[0] + a_tiled[0] * (tc[1] + a_tiled[1] * tc[2]);  // position in the permuted sequence
   const int head_a = (lin / num_a) % heads_a;
