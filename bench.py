@@ -169,21 +169,35 @@ def bench_backward(args, q, k, v, kernel, stride, dilation, causal, dt_name):
         kp, _, kv_shape = perm(k, kv_tile)
         vp = perm(v, kv_tile)[0]
 
-        def kern():
+        fused = _lib.backward_fused_layout_supported(layout, dilation, q_tile, kv_tile)
+        qd, kd, vd = q.detach(), k.detach(), v.detach()
+
+        def kern_permuted():
             return _lib.fna_backward(qp, kp, vp, dop, lp, dp, kernel, stride, dilation, causal, D**-0.5, q_shape,
                                      kv_shape, qkv_shape, q_tile, kv_tile)
 
-        for _ in range(2):
-            kern()
-        e0 = torch.cuda.Event(enable_timing=True)
-        e1 = torch.cuda.Event(enable_timing=True)
-        torch.cuda.synchronize()
-        e0.record()
-        for _ in range(args.steps):
-            kern()
-        e1.record()
-        torch.cuda.synchronize()
-        kernel_ms = e0.elapsed_time(e1) / args.steps
+        def kern():
+            # the launches the step above makes
+            if fused:
+                return _lib.fna_backward_fused(qd, kd, vd, d_out, lse, delta, kernel, stride, dilation, causal,
+                                               D**-0.5, q_tile, kv_tile)
+            return kern_permuted()
+
+        def timed(fn):
+            for _ in range(2):
+                fn()
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            e0.record()
+            for _ in range(args.steps):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) / args.steps
+
+        kernel_ms = timed(kern)
+        kernel_permuted_ms = timed(kern_permuted)
     fwd_flops = 4.0 * B * H * D * count_attended(layout, kernel, stride, dilation, causal)
     achieved = 2.5 * fwd_flops / (kernel_ms * 1e-3) / 1e12
     peak = PEAK_TFLOPS[dt_name]
@@ -204,10 +218,12 @@ def bench_backward(args, q, k, v, kernel, stride, dilation, causal, dt_name):
             "workload": WORKLOAD_NAMES[args.workload] + ", forward + backward",
             "backward_q_tile_shape": list(q_tile),
             "backward_kv_tile_shape": list(kv_tile),
-            "path": "forward (one launch when the layout allows) + delta + token permutes + dQ and dK/dV kernels + unpermutes",
+            "path": ("forward (one launch) + delta + dQ, dK, dV kernels on the original tensors" if fused else
+                     "forward + delta + token permutes + dQ and dK/dV kernels + unpermutes"),
         },
         "na_flop_per_step": 3.5 * fwd_flops,
         "backward_kernels_ms": kernel_ms,
+        "backward_kernels_on_permuted_operands_ms": kernel_permuted_ms,
         "roofline": {
             "kernel": "fna_bwd_kernel (dQ role + dK/dV role)",
             "bound": "mfma",

@@ -23,6 +23,8 @@
  *                                  max_seqlen_Q / _KV (csrc/include/natten/blackwell_fmha.h:34-50)
  *   natten_amd_fna_backward     <- blackwell_na{1,2,3}d_backward
  *                                  csrc/include/natten/blackwell_fna.h:92-160
+ *   natten_amd_fna_backward_fused <- the reference driver's permutes + backward + unpermutes,
+ *                                  src/natten/backends/blackwell_fna.py:205-297, without the copies
  *   natten_amd_attention_backward <- blackwell_fmha_backward csrc/include/natten/blackwell_fmha.h:52-73
  *                                  (fixed-length batches)
  *   natten_amd_compute_delta    <- compute_delta            csrc/include/natten/compute_delta.h:33-36
@@ -186,6 +188,24 @@ int natten_amd_fna_backward(const void* q, const void* k, const void* v, const v
                             const int32_t* dilation, const int32_t* is_causal,
                             const int32_t* q_tile_shape, const int32_t* kv_tile_shape, float scale,
                             void* stream);
+
+/*
+ * The same backward on the original tensors: q, d_out, dq [batch, *qkv_shape, heads_q, head_dim],
+ * k, v, dk, dv [batch, *qkv_shape, heads_kv, head_dim], lse and delta head-major
+ * [batch, heads_q, prod(qkv_shape)].  The kernels gather and scatter the rows of their tiles
+ * themselves, which replaces the six token permutes and three unpermutes of the reference's
+ * backward driver (src/natten/backends/blackwell_fna.py:205-297); results are bit-identical to
+ * them.  Every extent must be a multiple of dilation x tile for both tile shapes (an error
+ * otherwise: use natten_amd_fna_backward on permuted operands).
+ */
+int natten_amd_fna_backward_fused(const void* q, const void* k, const void* v, const void* d_out,
+                                  const float* lse, const float* delta, void* dq, void* dk,
+                                  void* dv, int dtype, int na_dim, int batch, int heads_q,
+                                  int heads_kv, int head_dim, const int32_t* qkv_shape,
+                                  const int32_t* kernel_size, const int32_t* stride,
+                                  const int32_t* dilation, const int32_t* is_causal,
+                                  const int32_t* q_tile_shape, const int32_t* kv_tile_shape,
+                                  float scale, void* stream);
 
 /*
  * Dense attention backward (optional top-left causal mask).  Operands as above (lse and delta

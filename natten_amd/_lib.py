@@ -19,7 +19,7 @@ from torch import Tensor
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libnatten_amd.so")
 
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 DTYPE_CODES = {
     torch.float16: 0,
@@ -69,6 +69,10 @@ _SIGNATURES = {
     "natten_amd_fna_backward": (
         ctypes.c_int,
         [ctypes.c_void_p] * 9 + [ctypes.c_int] * 8 + [ctypes.c_void_p] * 9 + [ctypes.c_float, ctypes.c_void_p],
+    ),
+    "natten_amd_fna_backward_fused": (
+        ctypes.c_int,
+        [ctypes.c_void_p] * 9 + [ctypes.c_int] * 6 + [ctypes.c_void_p] * 7 + [ctypes.c_float, ctypes.c_void_p],
     ),
     "natten_amd_attention_backward": (
         ctypes.c_int,
@@ -344,6 +348,41 @@ def fna_backward(
             k.shape[1], q.shape[2], k.shape[2], q.shape[3], _i32(q_shape), _i32(kv_shape), _i32(qkv_shape),
             _i32(kernel_size), _i32(stride), _i32(dilation), _i32([1 if c else 0 for c in is_causal]),
             _i32(q_tile_shape), _i32(kv_tile_shape), float(scale), _stream(q),
+        )
+    _check(rc)
+    return dq, dk, dv
+
+
+def backward_fused_layout_supported(token_layout, dilation, q_tile_shape, kv_tile_shape) -> bool:
+    """Whether the backward kernels can work on the original tensors: no padding on either side."""
+    return all(
+        X % (d * tq) == 0 and X % (d * tk) == 0
+        for X, d, tq, tk in zip(token_layout, dilation, q_tile_shape, kv_tile_shape)
+    )
+
+
+def fna_backward_fused(
+    q: Tensor, k: Tensor, v: Tensor, d_out: Tensor, lse: Tensor, delta: Tensor, kernel_size, stride, dilation,
+    is_causal, scale: float, q_tile_shape, kv_tile_shape,
+) -> Tuple[Tensor, Tensor, Tensor]:
+    """Backward on the original tensors [B, *X, H, D] (lse, delta [B, *X, H]) -> (dq, dk, dv)."""
+    L = lib()
+    na_dim = len(kernel_size)
+    B, H = q.shape[0], q.shape[-2]
+    lse = lse.reshape(B, -1, H).transpose(1, 2).contiguous()
+    delta = delta.reshape(B, -1, H).transpose(1, 2).contiguous()
+    _require_gpu(q, k, v, d_out, lse, delta)
+    if q.dtype not in (torch.float16, torch.bfloat16):
+        raise NotImplementedError(f"natten_amd fna_backward_fused does not support {q.dtype}.")
+    if lse.dtype != torch.float32 or delta.dtype != torch.float32:
+        raise ValueError("lse and delta must be float32.")
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    with torch.cuda.device(q.device):
+        rc = L.natten_amd_fna_backward_fused(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), d_out.data_ptr(), lse.data_ptr(), delta.data_ptr(),
+            dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), DTYPE_CODES[q.dtype], na_dim, B, H, k.shape[-2], q.shape[-1],
+            _i32(q.shape[1 : 1 + na_dim]), _i32(kernel_size), _i32(stride), _i32(dilation),
+            _i32([1 if c else 0 for c in is_causal]), _i32(q_tile_shape), _i32(kv_tile_shape), float(scale), _stream(q),
         )
     _check(rc)
     return dq, dk, dv

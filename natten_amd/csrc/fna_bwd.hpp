@@ -50,6 +50,13 @@ struct FnaBwdParams {
   int q_split, kv_split;        // the dimension along which a 128-token tile of either side halves
                                 // (its last dimension of extent > 1, so that the halves are contiguous)
   float scale;
+  // Operand layout.  fused == 0: token-permuted sequences as described above.  fused == 1: the
+  // original tensors [batch, X0, X1, X2, heads, D] (lse / delta [batch, heads, X0 * X1 * X2]);
+  // the kernel gathers and scatters the rows of a tile itself.  Every extent must then be a
+  // multiple of dilation x tile for both tile shapes (no padding rows exist).
+  int fused;
+  int tok_stride[3];  // tokens per unit step of an original coordinate: X1*X2, X2, 1
+  int tokens;         // X0 * X1 * X2
 };
 
 enum BwdRole : int { kBwdDQ = 0, kBwdDK = 1, kBwdDV = 2, kBwdDKV = 3 };
@@ -135,6 +142,8 @@ fna_bwd_kernel(const FnaBwdParams p) {
   const int bg = lin / (num_a * heads_a);
 
   int extent[3], q_extent[3], a_first[3], b_sub[3], box_tile0[3], box_n[3], full_t0[3], full_t1[3];
+  int tok_step[3];    // original layout: tokens per unit step of a coordinate inside a dilation group
+  int group_tok = 0;  // original layout: token of the dilation group's first element
   bool empty = false;
   {
     int gl = bg % p.num_groups;
@@ -142,6 +151,8 @@ fna_bwd_kernel(const FnaBwdParams p) {
     for (int a = 0; a < 3; ++a) {
       const int gi = gl % p.dil[a];
       gl /= p.dil[a];
+      tok_step[a] = p.dil[a] * p.tok_stride[a];
+      group_tok += gi * p.tok_stride[a];
       extent[a] = na_group_extent(p.qkv_shape[a], p.dil[a], gi);
       q_extent[a] = (a == 0 && p.q_extent0 > 0) ? p.q_extent0 : extent[a];
       a_first[a] = tc[a] * a_tile[a];
@@ -197,7 +208,12 @@ fna_bwd_kernel(const FnaBwdParams p) {
   a_off[0] = r_in % a_tile[0];
   a_off[1] = (r_in / a_tile[0]) % a_tile[1];
   a_off[2] = r_in / (a_tile[0] * a_tile[1]);
-  const int64_t a_row = (int64_t(bg) * seq_a + int64_t(at) * AT + r_in);
+  // Row of the tensors / index into lse and delta: position in the permuted sequence, or the
+  // token of the lane's coordinate in the original layout.
+  const int a_tok = group_tok + (a_first[0] + a_off[0]) * tok_step[0] + (a_first[1] + a_off[1]) * tok_step[1] +
+                    (a_first[2] + a_off[2]) * tok_step[2];
+  const int64_t batch_row0 = p.fused ? int64_t(bg / p.num_groups) * p.tokens : 0;  // first row of the batch entry (original layout)
+  const int64_t a_row = p.fused ? batch_row0 + a_tok : (int64_t(bg) * seq_a + int64_t(at) * AT + r_in);
   const int64_t a_stride = int64_t(heads_a) * D;
   const int64_t b_stride = int64_t(heads_b) * D;
   const float kLog2e = 1.4426950408889634f;
@@ -254,7 +270,8 @@ fna_bwd_kernel(const FnaBwdParams p) {
       wst[a] = na_window_start(c, p.ksize[a], p.stride[a], extent[a], p.causal[a] != 0);
       wen[a] = na_window_end(c, wst[a], p.ksize[a], extent[a], p.causal[a] != 0);
     }
-    const int64_t stat_idx = (int64_t(bg) * p.heads_q + head_a) * seq_a + int64_t(at) * AT + r_in;
+    const int64_t stat_idx = p.fused ? (int64_t(bg / p.num_groups) * p.heads_q + head_a) * p.tokens + a_tok
+                                     : (int64_t(bg) * p.heads_q + head_a) * seq_a + int64_t(at) * AT + r_in;
     lse_l = p.lse[stat_idx] * kLog2e;
     delta_l = p.delta[stat_idx];
     // in-tile coordinates of every streamed position, packed in 10-bit fields
@@ -272,13 +289,20 @@ fna_bwd_kernel(const FnaBwdParams p) {
   const T* y1_all = reinterpret_cast<const T*>(KV_STATIONARY ? p.q : p.k);
   const T* y2_all = reinterpret_cast<const T*>(KV_STATIONARY ? p.d_out : p.v);
 
+  // row (permuted) or token offset (original layout) of position r (dimension 0 fastest) of a streamed tile
+  auto sub_pos = [&](int r) {
+    if (!p.fused) return r;
+    const int t0 = r % b_sub[0];
+    r /= b_sub[0];
+    return t0 * tok_step[0] + (r % b_sub[1]) * tok_step[1] + (r / b_sub[1]) * tok_step[2];
+  };
   // copy i of a thread moves chunk P = i * NT + tid of the tile (row P / CPR, LDS slot P % CPR)
   uint32_t off_u[PER];
 #pragma unroll
   for (int i = 0; i < PER; ++i) {
     const int P = i * NT + tid;
     const int row = P / CPR, slot = P % CPR;
-    off_u[i] = uint32_t(row) * uint32_t(b_stride * 2) + uint32_t(L::u_slot(row, slot) * 16);
+    off_u[i] = uint32_t(sub_pos(row)) * uint32_t(b_stride * 2) + uint32_t(L::u_slot(row, slot) * 16);
   }
 
   struct Tile {
@@ -338,7 +362,8 @@ fna_bwd_kernel(const FnaBwdParams p) {
       half |= split ? (wc[a] & 1) : 0;
       cc[a] = split ? (wc[a] >> 1) : wc[a];
     }
-    t.row0 = (cc[0] + b_tiled[0] * (cc[1] + b_tiled[1] * cc[2])) * AT + half * BT;
+    t.row0 = p.fused ? group_tok + t.origin[0] * tok_step[0] + t.origin[1] * tok_step[1] + t.origin[2] * tok_step[2]
+                     : (cc[0] + b_tiled[0] * (cc[1] + b_tiled[1] * cc[2])) * AT + half * BT;
     t.head_b = KV_STATIONARY ? head_b0 + walk_head : head_b0;
     if (more) {
       step(whole_tag);
@@ -355,7 +380,7 @@ fna_bwd_kernel(const FnaBwdParams p) {
 
   const uint32_t lds_y1 = uint32_t(__builtin_amdgcn_readfirstlane(int(lds_address(sY1))));
   const uint32_t lds_y2 = uint32_t(__builtin_amdgcn_readfirstlane(int(lds_address(sY2))));
-  const uint32_t stat_off = uint32_t(lane) * 4u;  // byte offset of streamed row `lane` in lse / delta (head-major)
+  const uint32_t stat_off = uint32_t(sub_pos(lane)) * 4u;  // byte offset of streamed row `lane` in lse / delta (head-major)
   auto issue = [&](const Tile& t, int stage, bool masked) {
     if constexpr (KV_STATIONARY) {
       if (wave == 0 && masked) {
@@ -377,12 +402,14 @@ fna_bwd_kernel(const FnaBwdParams p) {
         sTabB[stage * BT + lane] = valid ? subc : 0u;
       }
     }
-    const int64_t row = int64_t(bg) * seq_b + t.row0;
+    const int64_t row = p.fused ? batch_row0 + t.row0 : int64_t(bg) * seq_b + t.row0;
     if constexpr (KV_STATIONARY) {
       // LSE / delta of the tile's 64 queries: one asynchronous 4-byte-per-lane copy each
       // (wave 1, wave 2; wave 3 and, without delta, wave 2 make the same number of copies into a
       // spare row so that every wave counts the same number of outstanding copies per tile)
-      const float* src = (wave == 2 && HAS_DS ? p.delta : p.lse) + (int64_t(bg) * p.heads_q + t.head_b) * seq_b + t.row0;
+      const int64_t stat_row0 = p.fused ? (int64_t(bg / p.num_groups) * p.heads_q + t.head_b) * p.tokens + t.row0
+                                        : (int64_t(bg) * p.heads_q + t.head_b) * seq_b + t.row0;
+      const float* src = (wave == 2 && HAS_DS ? p.delta : p.lse) + stat_row0;
       float* dst = (wave == 1) ? &sLse[stage * BT] : (wave == 2 && HAS_DS) ? &sDelta[stage * BT] : &sSpare[0];
       if (wave != 0) async_copy4_asm(src, stat_off, lds_address(dst));
     }

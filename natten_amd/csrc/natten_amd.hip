@@ -192,7 +192,7 @@ int fill_fna_params(const char* what, FnaParams& p, int na_dim, const int* q_sha
 
 extern "C" {
 
-int natten_amd_abi_version(void) { return 4; }
+int natten_amd_abi_version(void) { return 5; }
 
 const char* natten_amd_last_error(void) { return g_error; }
 
@@ -540,6 +540,81 @@ int natten_amd_fna_backward(const void* q, const void* k, const void* v, const v
   p.num_groups = groups;
   p.q_extent0 = 0;
   p.scale = scale;
+  return dispatch_bwd(p, dtype, head_dim, static_cast<hipStream_t>(stream));
+}
+
+int natten_amd_fna_backward_fused(const void* q, const void* k, const void* v, const void* d_out, const float* lse,
+                                  const float* delta, void* dq, void* dk, void* dv, int dtype, int na_dim, int batch,
+                                  int heads_q, int heads_kv, int head_dim, const int32_t* qkv_shape,
+                                  const int32_t* kernel_size, const int32_t* stride, const int32_t* dilation,
+                                  const int32_t* is_causal, const int32_t* q_tile_shape, const int32_t* kv_tile_shape,
+                                  float scale, void* stream) {
+  g_error[0] = 0;
+  const char* what = "fna_backward_fused";
+  if (int rc = check_bwd_pointers(what, q, k, v, d_out, lse, delta, dq, dk, dv)) return rc;
+  if (na_dim < 1 || na_dim > 3) return fail("%s: na_dim must be 1, 2 or 3, got %d", what, na_dim);
+  if (!qkv_shape || !kernel_size || !stride || !dilation || !is_causal || !q_tile_shape || !kv_tile_shape)
+    return fail("%s: null shape argument", what);
+  // per-group layouts: without padding, which needs every extent to be a multiple of dilation x tile
+  int group_shape[3] = {1, 1, 1};
+  long long tokens = 1;
+  for (int a = 0; a < na_dim; ++a) {
+    if (qkv_shape[a] < 1 || dilation[a] < 1 || q_tile_shape[a] < 1 || kv_tile_shape[a] < 1)
+      return fail("%s: invalid parameter along dimension %d", what, a);
+    if (qkv_shape[a] % (dilation[a] * q_tile_shape[a]) != 0 || qkv_shape[a] % (dilation[a] * kv_tile_shape[a]) != 0)
+      return fail("%s: extent %d along dimension %d is not a multiple of dilation x tile (%d x %d, %d x %d); use the "
+                  "token-permuted entry point",
+                  what, qkv_shape[a], a, dilation[a], q_tile_shape[a], dilation[a], kv_tile_shape[a]);
+    group_shape[a] = qkv_shape[a] / dilation[a];
+    tokens *= qkv_shape[a];
+  }
+  if (tokens > 0x7fffffffLL) return fail("%s: more than 2^31 tokens", what);
+  FnaParams f;
+  if (int rc = fill_fna_params(what, f, na_dim, group_shape, group_shape, qkv_shape, kernel_size, stride, dilation,
+                               is_causal, q_tile_shape, kv_tile_shape))
+    return rc;
+  if (int rc = check_common(what, q, k, v, dq, lse, batch, int(tokens), int(tokens), heads_q, heads_kv, head_dim)) return rc;
+  if (prod3(f.q_tile) != 128 || prod3(f.kv_tile) != 128)
+    return fail("%s: Q and KV tiles must hold 128 tokens each, got %d and %d", what, prod3(f.q_tile), prod3(f.kv_tile));
+  FnaBwdParams p;
+  memset(&p, 0, sizeof(p));
+  p.q_split = split_dim_of(f.q_tile);
+  p.kv_split = split_dim_of(f.kv_tile);
+  if (f.q_tile[p.q_split] % 2 != 0 || f.kv_tile[p.kv_split] % 2 != 0)
+    return fail("%s: the last tile extent above 1 must be even", what);
+  int groups = 1;
+  for (int a = 0; a < 3; ++a) {
+    p.qkv_shape[a] = f.qkv_shape[a];
+    p.ksize[a] = f.ksize[a];
+    p.stride[a] = f.stride[a];
+    p.dil[a] = f.dil[a];
+    p.causal[a] = f.causal[a];
+    p.q_tile[a] = f.q_tile[a];
+    p.kv_tile[a] = f.kv_tile[a];
+    p.q_tiled[a] = f.q_tiled[a];
+    p.kv_tiled[a] = f.kv_tiled[a];
+    p.tok_stride[a] = f.tok_stride[a];
+    groups *= f.dil[a];
+  }
+  p.q = q;
+  p.k = k;
+  p.v = v;
+  p.d_out = d_out;
+  p.lse = lse;
+  p.delta = delta;
+  p.dq = dq;
+  p.dk = dk;
+  p.dv = dv;
+  p.batch = batch * groups;
+  p.heads_q = heads_q;
+  p.heads_kv = heads_kv;
+  p.seqlen_q = prod3(p.q_tiled) * 128;
+  p.seqlen_kv = prod3(p.kv_tiled) * 128;
+  p.num_groups = groups;
+  p.q_extent0 = 0;
+  p.scale = scale;
+  p.fused = 1;
+  p.tokens = int(tokens);
   return dispatch_bwd(p, dtype, head_dim, static_cast<hipStream_t>(stream));
 }
 

@@ -225,6 +225,7 @@ class AmdFnaFunction(torch.autograd.Function):
             )
         ctx.save_for_backward(query, key, value, output, lse)
         ctx.na_args = (kernel_size, stride, dilation, is_causal, scale, bwd_q_tile_shape, bwd_kv_tile_shape)
+        ctx.fused = fused
         ctx.mark_non_differentiable(lse)
         return output, lse
 
@@ -239,6 +240,17 @@ class AmdFnaFunction(torch.autograd.Function):
             pad_head_dim(t.contiguous(), d_pad).contiguous() for t in (query, key, value, output, d_output)
         )
         delta = torch_ops.compute_delta(output, d_output)
+        na_dim = len(kernel_size)
+        fusable = _lib.backward_fused_layout_supported(query.shape[1 : 1 + na_dim], dilation, q_tile, kv_tile)
+        if fusable and ctx.fused is not False:
+            # the kernels gather and scatter their tiles themselves: no permuted copies
+            dq, dk, dv = torch_ops.fna_backward_fused(
+                query, key, value, d_output, lse.contiguous(), delta, kernel_size, stride, dilation, is_causal, scale,
+                q_tile, kv_tile,
+            )
+            if d_pad != head_dim:
+                dq, dk, dv = (t[..., :head_dim].contiguous() for t in (dq, dk, dv))
+            return (dq, dk, dv) + (None,) * 10
 
         def perm(x, tile):
             return token_permute_operation(x.contiguous(), tile, dilation, flip_tiled_dims=True)

@@ -111,6 +111,21 @@ def _(q, k, v, d_out, lse, delta, kernel_size, stride, dilation, is_causal, scal
     return torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
 
 
+@torch.library.custom_op("natten_amd::fna_backward_fused", mutates_args=(), device_types="cuda")
+def _fna_backward_fused_op(
+    q: Tensor, k: Tensor, v: Tensor, d_out: Tensor, lse: Tensor, delta: Tensor, kernel_size: List[int],
+    stride: List[int], dilation: List[int], is_causal: List[bool], scale: float, q_tile_shape: List[int],
+    kv_tile_shape: List[int],
+) -> Tuple[Tensor, Tensor, Tensor]:
+    return _lib.fna_backward_fused(q, k, v, d_out, lse, delta, kernel_size, stride, dilation, is_causal, scale,
+                                   q_tile_shape, kv_tile_shape)
+
+
+@_fna_backward_fused_op.register_fake
+def _(q, k, v, d_out, lse, delta, kernel_size, stride, dilation, is_causal, scale, q_tile_shape, kv_tile_shape):
+    return torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+
+
 @torch.library.custom_op("natten_amd::attention_backward", mutates_args=(), device_types="cuda")
 def _attention_backward_op(
     q: Tensor, k: Tensor, v: Tensor, d_out: Tensor, lse: Tensor, delta: Tensor, seqlen_q: int, seqlen_kv: int,
@@ -229,6 +244,16 @@ def fna_backward(q, k, v, d_out, lse, delta, kernel_size, stride, dilation, is_c
                                 _ints(qkv_shape), _ints(q_tile_shape), _ints(kv_tile_shape))
     return _lib.fna_backward(q, k, v, d_out, lse, delta, kernel_size, stride, dilation, is_causal, scale, q_shape,
                              kv_shape, qkv_shape, q_tile_shape, kv_tile_shape)
+
+
+def fna_backward_fused(q, k, v, d_out, lse, delta, kernel_size, stride, dilation, is_causal, scale, q_tile_shape,
+                       kv_tile_shape):
+    if _tracing():
+        return _fna_backward_fused_op(q, k, v, d_out, lse, delta, _ints(kernel_size), _ints(stride), _ints(dilation),
+                                      [bool(c) for c in is_causal], float(scale), _ints(q_tile_shape),
+                                      _ints(kv_tile_shape))
+    return _lib.fna_backward_fused(q, k, v, d_out, lse, delta, kernel_size, stride, dilation, is_causal, scale,
+                                   q_tile_shape, kv_tile_shape)
 
 
 def attention_backward(q, k, v, d_out, lse, delta, seqlen_q, seqlen_kv, is_causal, scale):

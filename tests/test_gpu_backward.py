@@ -42,6 +42,16 @@ def run_backward(B, H, Hkv, D, shape, k, s, d, causal, dtype, bq=None, bkv=None,
     for name, got, r in zip(("dq", "dk", "dv"), (q.grad, kk.grad, v.grad), ref):
         assert got is not None and got.dtype == dtype and got.shape == r.shape, name
         assert_close(f"{name} {tag}", to_np(got), r, atol=TOL[dtype], rtol=TOL[dtype])
+    if not all(kk_ == x for kk_, x in zip(k, shape)) or any(causal):
+        # whichever layout the backward above worked on (the original tensors when no extent needs
+        # padding, token-permuted copies otherwise), the permuted route must agree bit for bit
+        from natten_amd.fna import amd_fna_generic
+
+        q2, k2, v2 = (t.detach().clone().requires_grad_(True) for t in (q, kk, v))
+        amd_fna_generic(q2, k2, v2, k, s, d, causal, backward_q_tile_shape=bq, backward_kv_tile_shape=bkv,
+                        fused=False).backward(d_out)
+        for name, a, b in zip(("dq", "dk", "dv"), (q.grad, kk.grad, v.grad), (q2.grad, k2.grad, v2.grad)):
+            assert torch.equal(a, b), f"original-layout and permuted backward differ in {name}: {tag}"
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
@@ -60,6 +70,11 @@ def test_backward_2d(dtype):
 
 def test_backward_3d():
     run_backward(1, 2, 1, 64, (9, 16, 24), (4, 8, 8), (1, 8, 4), 1, (True, False, False), torch.bfloat16, seed=6)
+    # extents that are multiples of dilation x tile: the backward works on the original tensors
+    run_backward(2, 4, 2, 128, (8, 16, 16), (3, 8, 8), (1, 4, 8), (2, 1, 1), (True, False, False), torch.bfloat16,
+                 (2, 8, 8), (4, 4, 8), seed=60)
+    run_backward(1, 2, 2, 64, (4, 32, 16), (2, 9, 5), (1, 3, 1), (1, 2, 1), (False, False, True), torch.float16,
+                 (2, 16, 4), (1, 8, 16), seed=61)
     run_backward(1, 2, 2, 32, (6, 10, 9), (3, 4, 5), (1, 2, 2), (2, 1, 1), (False, True, False), torch.float16, seed=7)
     run_backward(2, 1, 1, 128, (8, 8, 8), (3, 3, 3), 1, 1, False, torch.bfloat16, seed=8)
 
