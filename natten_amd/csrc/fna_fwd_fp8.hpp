@@ -499,7 +499,9 @@ fna_fwd_fp8_kernel(const FnaParams p) {
       });
       __builtin_amdgcn_sched_barrier(0);
     };
+    __builtin_amdgcn_s_setprio(1);  // as in the 16-bit kernel: the QK slots run at raised wave priority
     for_range<0, N_QK>(g1_slot);
+    __builtin_amdgcn_s_setprio(0);
 
     i32x8_t pf;
 #pragma unroll
