@@ -26,6 +26,8 @@
  *   natten_amd_fna_backward_fused <- the reference driver's permutes + backward + unpermutes,
  *                                  src/natten/backends/blackwell_fna.py:205-297, without the copies
  *   natten_amd_attention_backward <- blackwell_fmha_backward csrc/include/natten/blackwell_fmha.h:52-73
+ *   natten_amd_attention_backward_varlen <- the same function with cumulative_seqlen_Q / _KV,
+ *                                  max_seqlen_Q / _KV (csrc/include/natten/blackwell_fmha.h:52-73)
  *                                  (fixed-length batches)
  *   natten_amd_compute_delta    <- compute_delta            csrc/include/natten/compute_delta.h:33-36
  *   natten_amd_merge_attentions <- the elementwise merge of src/natten/attn_merge.py:48-105
@@ -218,6 +220,29 @@ int natten_amd_attention_backward(const void* q, const void* k, const void* v, c
                                   int padded_seqlen_q, int padded_seqlen_kv, int heads_q,
                                   int heads_kv, int head_dim, int is_causal, float scale,
                                   void* stream);
+
+/*
+ * Dense attention backward of a sequence-packed batch, one set of launches for all sequences.
+ * The operands hold the `num_seqs` sequences back to back, each zero-padded to a multiple of
+ * 128 rows: q, d_out, dq [1, rows_q, heads_q, head_dim], k, v, dk, dv [1, rows_kv, heads_kv,
+ * head_dim], lse and delta head-major [1, heads_q, rows_q]; rows_q and rows_kv are multiples
+ * of 128.  All four cumulative arrays are device int32 [num_seqs + 1]: sequence b has
+ * cu_seqlens_q[b+1] - cu_seqlens_q[b] queries, which are rows padded_cu_seqlens_q[b] ... of the
+ * operands (padded_cu_seqlens_* count padded lengths: multiples of 128, each covering the
+ * sequence); keys likewise.  max_seqlen_q / max_seqlen_kv bound the sequence lengths (they size
+ * the grid; rows of longer sequences would be left out).  Rows of dq, dk, dv outside every
+ * sequence's padded range are not written.  A sequence whose offsets do not fit the row counts
+ * is skipped by the kernels (the host cannot see the device arrays).  No host synchronisation.
+ */
+int natten_amd_attention_backward_varlen(const void* q, const void* k, const void* v,
+                                         const void* d_out, const float* lse, const float* delta,
+                                         void* dq, void* dk, void* dv, int dtype, int num_seqs,
+                                         int rows_q, int rows_kv, const int32_t* cu_seqlens_q,
+                                         const int32_t* cu_seqlens_kv,
+                                         const int32_t* padded_cu_seqlens_q,
+                                         const int32_t* padded_cu_seqlens_kv, int max_seqlen_q,
+                                         int max_seqlen_kv, int heads_q, int heads_kv,
+                                         int head_dim, int is_causal, float scale, void* stream);
 
 /*
  * Token permute: src [batch, *token_layout, heads, head_dim] -> dst

@@ -19,7 +19,7 @@ from torch import Tensor
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libnatten_amd.so")
 
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 DTYPE_CODES = {
     torch.float16: 0,
@@ -77,6 +77,11 @@ _SIGNATURES = {
     "natten_amd_attention_backward": (
         ctypes.c_int,
         [ctypes.c_void_p] * 9 + [ctypes.c_int] * 10 + [ctypes.c_float, ctypes.c_void_p],
+    ),
+    "natten_amd_attention_backward_varlen": (
+        ctypes.c_int,
+        [ctypes.c_void_p] * 9 + [ctypes.c_int] * 4 + [ctypes.c_void_p] * 4 + [ctypes.c_int] * 6
+        + [ctypes.c_float, ctypes.c_void_p],
     ),
     "natten_amd_token_permute_widen": (
         ctypes.c_int,
@@ -406,6 +411,37 @@ def attention_backward(
             dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), DTYPE_CODES[q.dtype], q.shape[0], int(seqlen_q),
             int(seqlen_kv), q.shape[1], k.shape[1], q.shape[2], k.shape[2], q.shape[3], 1 if is_causal else 0,
             float(scale), _stream(q),
+        )
+    _check(rc)
+    return dq, dk, dv
+
+
+def attention_backward_varlen(
+    q: Tensor, k: Tensor, v: Tensor, d_out: Tensor, lse: Tensor, delta: Tensor, cu_q: Tensor, cu_kv: Tensor,
+    padded_cu_q: Tensor, padded_cu_kv: Tensor, max_seqlen_q: int, max_seqlen_kv: int, is_causal: bool, scale: float,
+) -> Tuple[Tensor, Tensor, Tensor]:
+    """Dense attention backward of a sequence-packed batch whose sequences are each zero-padded to
+    a multiple of 128 rows -> (dq, dk, dv) in the same padded packing.  q, d_out [1, rows_q, H, D];
+    k, v [1, rows_kv, Hkv, D]; lse, delta [1, rows_q, H] (the kernels take them head-major); the
+    four cumulative arrays are device int32 [sequences + 1].  Rows outside every sequence's padded
+    range are left unwritten."""
+    L = lib()
+    lse, delta = lse.transpose(1, 2).contiguous(), delta.transpose(1, 2).contiguous()
+    _require_gpu(q, k, v, d_out, lse, delta, cu_q, cu_kv, padded_cu_q, padded_cu_kv)
+    if q.dtype not in (torch.float16, torch.bfloat16):
+        raise NotImplementedError(f"natten_amd attention_backward_varlen does not support {q.dtype}.")
+    cums = (cu_q, cu_kv, padded_cu_q, padded_cu_kv)
+    if any(c.dtype != torch.int32 or c.dim() != 1 or c.numel() != cu_q.numel() or not c.is_contiguous() for c in cums):
+        raise ValueError("cumulative sequence lengths must be contiguous int32 vectors of one length.")
+    if cu_q.numel() < 2 or q.shape[0] != 1 or k.shape[0] != 1:
+        raise ValueError("sequence-packed operands have batch 1 and at least one sequence.")
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    with torch.cuda.device(q.device):
+        rc = L.natten_amd_attention_backward_varlen(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), d_out.data_ptr(), lse.data_ptr(), delta.data_ptr(),
+            dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), DTYPE_CODES[q.dtype], cu_q.numel() - 1, q.shape[1], k.shape[1],
+            cu_q.data_ptr(), cu_kv.data_ptr(), padded_cu_q.data_ptr(), padded_cu_kv.data_ptr(), int(max_seqlen_q),
+            int(max_seqlen_kv), q.shape[2], k.shape[2], q.shape[3], 1 if is_causal else 0, float(scale), _stream(q),
         )
     _check(rc)
     return dq, dk, dv

@@ -57,11 +57,20 @@ struct FnaBwdParams {
   int fused;
   int tok_stride[3];  // tokens per unit step of an original coordinate: X1*X2, X2, 1
   int tokens;         // X0 * X1 * X2
+  // Sequence-packed dense attention (VARLEN instances only; null otherwise).  `batch` sequences
+  // lie back to back in one row range (the tensors have batch 1; seqlen_q / seqlen_kv count all
+  // their rows), each padded to a multiple of 128 rows: sequence b owns query rows
+  // pcu_q[b] .. pcu_q[b+1]-1 of which the first cu_q[b+1] - cu_q[b] are real, keys likewise;
+  // q_tiled[0] / kv_tiled[0] count the tiles of the longest sequence.
+  const int32_t* cu_q;    // [batch + 1] cumulative real lengths
+  const int32_t* cu_kv;
+  const int32_t* pcu_q;   // [batch + 1] cumulative padded lengths (row offsets into the tensors)
+  const int32_t* pcu_kv;
 };
 
 enum BwdRole : int { kBwdDQ = 0, kBwdDK = 1, kBwdDV = 2, kBwdDKV = 3 };
 
-template <typename T, int D, int ROLE>
+template <typename T, int D, int ROLE, bool VARLEN = false>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
 fna_bwd_kernel(const FnaBwdParams p) {
   constexpr bool KV_STATIONARY = ROLE != kBwdDQ;
@@ -141,10 +150,34 @@ fna_bwd_kernel(const FnaBwdParams p) {
   const int head_a = (lin / num_a) % heads_a;
   const int bg = lin / (num_a * heads_a);
 
+  // first rows of this batch entry's sequences, its lse / delta values of head 0, and the
+  // parameters a packed sequence overrides
+  int64_t seq_row_a = int64_t(bg) * seq_a, seq_row_b = int64_t(bg) * seq_b;
+  int64_t stat_row_q = int64_t(bg) * p.heads_q * p.seqlen_q;
+  int64_t stat_head_stride = p.seqlen_q;
+  int ksz[3] = {p.ksize[0], p.ksize[1], p.ksize[2]};
+  int keys0 = p.qkv_shape[0], queries0 = p.q_extent0;
+  bool empty = false;
+  if constexpr (VARLEN) {
+    const int q0 = p.cu_q[bg], kv0 = p.cu_kv[bg], pq0 = p.pcu_q[bg], pkv0 = p.pcu_kv[bg];
+    const int len_q = p.cu_q[bg + 1] - q0, len_kv = p.cu_kv[bg + 1] - kv0;
+    const int pad_q = p.pcu_q[bg + 1] - pq0, pad_kv = p.pcu_kv[bg + 1] - pkv0;
+    // offsets the tensors cannot hold are not followed
+    if (len_q < 0 || len_kv < 0 || pq0 < 0 || pkv0 < 0 || pad_q < len_q || pad_kv < len_kv ||
+        ((pq0 | pkv0 | pad_q | pad_kv) & 127) != 0 || pq0 + pad_q > p.seqlen_q || pkv0 + pad_kv > p.seqlen_kv)
+      return;
+    if (tc[0] * AT >= (KV_STATIONARY ? pad_kv : pad_q)) return;  // the longest sequence has more tiles than this one
+    seq_row_a = KV_STATIONARY ? pkv0 : pq0;
+    seq_row_b = KV_STATIONARY ? pq0 : pkv0;
+    stat_row_q = pq0;
+    keys0 = ksz[0] = na_max(len_kv, 1);
+    queries0 = na_max(len_q, 1);
+    empty = len_q == 0 || len_kv == 0;  // nothing attends, or attends to nothing: zero gradients
+  }
+
   int extent[3], q_extent[3], a_first[3], b_sub[3], box_tile0[3], box_n[3], full_t0[3], full_t1[3];
   int tok_step[3];    // original layout: tokens per unit step of a coordinate inside a dilation group
   int group_tok = 0;  // original layout: token of the dilation group's first element
-  bool empty = false;
   {
     int gl = bg % p.num_groups;
 #pragma unroll
@@ -153,8 +186,8 @@ fna_bwd_kernel(const FnaBwdParams p) {
       gl /= p.dil[a];
       tok_step[a] = p.dil[a] * p.tok_stride[a];
       group_tok += gi * p.tok_stride[a];
-      extent[a] = na_group_extent(p.qkv_shape[a], p.dil[a], gi);
-      q_extent[a] = (a == 0 && p.q_extent0 > 0) ? p.q_extent0 : extent[a];
+      extent[a] = na_group_extent(a == 0 ? keys0 : p.qkv_shape[a], p.dil[a], gi);
+      q_extent[a] = (a == 0 && queries0 > 0) ? queries0 : extent[a];
       a_first[a] = tc[a] * a_tile[a];
       b_sub[a] = (a == split_dim) ? b_tile[a] / 2 : b_tile[a];
       const bool c = p.causal[a] != 0;
@@ -162,14 +195,14 @@ fna_bwd_kernel(const FnaBwdParams p) {
       if constexpr (!KV_STATIONARY) {
         const int qf = a_first[a], ql = na_min(qf + a_tile[a], q_extent[a]) - 1;
         if (qf >= q_extent[a]) empty = true;
-        lo = na_window_start(qf, p.ksize[a], p.stride[a], extent[a], c);
-        const int st_l = na_window_start(na_max(ql, 0), p.ksize[a], p.stride[a], extent[a], c);
-        hi = na_window_end(na_max(ql, 0), st_l, p.ksize[a], extent[a], c) - 1;
+        lo = na_window_start(qf, ksz[a], p.stride[a], extent[a], c);
+        const int st_l = na_window_start(na_max(ql, 0), ksz[a], p.stride[a], extent[a], c);
+        hi = na_window_end(na_max(ql, 0), st_l, ksz[a], extent[a], c) - 1;
       } else {
         const int j0 = a_first[a], j1 = na_min(j0 + a_tile[a], extent[a]) - 1;
         if (j0 >= extent[a]) empty = true;
-        lo = na_first_query_attending(j0, p.ksize[a], p.stride[a], extent[a], q_extent[a], c);
-        hi = na_last_query_attending(na_max(j1, 0), p.ksize[a], p.stride[a], extent[a], q_extent[a], c);
+        lo = na_first_query_attending(j0, ksz[a], p.stride[a], extent[a], q_extent[a], c);
+        hi = na_last_query_attending(na_max(j1, 0), ksz[a], p.stride[a], extent[a], q_extent[a], c);
         if (lo > hi) empty = true;
       }
       lo = na_max(lo, 0);
@@ -182,18 +215,18 @@ fna_bwd_kernel(const FnaBwdParams p) {
       int flo, fhi;
       if constexpr (!KV_STATIONARY) {
         const int qf = a_first[a], ql = qf + a_tile[a] - 1;  // rows past the extent use the last window
-        const int st_l = na_window_start(ql, p.ksize[a], p.stride[a], extent[a], c);
-        const int st_f = na_window_start(qf, p.ksize[a], p.stride[a], extent[a], c);
+        const int st_l = na_window_start(ql, ksz[a], p.stride[a], extent[a], c);
+        const int st_f = na_window_start(qf, ksz[a], p.stride[a], extent[a], c);
         flo = st_l;
-        fhi = na_window_end(qf, st_f, p.ksize[a], extent[a], c) - 1;
+        fhi = na_window_end(qf, st_f, ksz[a], extent[a], c) - 1;
       } else {
         const int j0 = a_first[a], j1 = j0 + a_tile[a] - 1;
         if (j1 >= extent[a]) {
           flo = 1;  // the tile holds padding keys: never whole
           fhi = 0;
         } else {
-          flo = na_first_query_attending(j1, p.ksize[a], p.stride[a], extent[a], q_extent[a], c);
-          fhi = na_last_query_attending(j0, p.ksize[a], p.stride[a], extent[a], q_extent[a], c);
+          flo = na_first_query_attending(j1, ksz[a], p.stride[a], extent[a], q_extent[a], c);
+          fhi = na_last_query_attending(j0, ksz[a], p.stride[a], extent[a], q_extent[a], c);
         }
       }
       full_t0[a] = na_max(na_ceil_div(na_max(flo, 0), b_sub[a]), box_tile0[a]);
@@ -213,7 +246,7 @@ fna_bwd_kernel(const FnaBwdParams p) {
   const int a_tok = group_tok + (a_first[0] + a_off[0]) * tok_step[0] + (a_first[1] + a_off[1]) * tok_step[1] +
                     (a_first[2] + a_off[2]) * tok_step[2];
   const int64_t batch_row0 = p.fused ? int64_t(bg / p.num_groups) * p.tokens : 0;  // first row of the batch entry (original layout)
-  const int64_t a_row = p.fused ? batch_row0 + a_tok : (int64_t(bg) * seq_a + int64_t(at) * AT + r_in);
+  const int64_t a_row = p.fused ? batch_row0 + a_tok : (seq_row_a + int64_t(at) * AT + r_in);
   const int64_t a_stride = int64_t(heads_a) * D;
   const int64_t b_stride = int64_t(heads_b) * D;
   const float kLog2e = 1.4426950408889634f;
@@ -267,11 +300,11 @@ fna_bwd_kernel(const FnaBwdParams p) {
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
       const int c = a_first[a] + a_off[a];
-      wst[a] = na_window_start(c, p.ksize[a], p.stride[a], extent[a], p.causal[a] != 0);
-      wen[a] = na_window_end(c, wst[a], p.ksize[a], extent[a], p.causal[a] != 0);
+      wst[a] = na_window_start(c, ksz[a], p.stride[a], extent[a], p.causal[a] != 0);
+      wen[a] = na_window_end(c, wst[a], ksz[a], extent[a], p.causal[a] != 0);
     }
     const int64_t stat_idx = p.fused ? (int64_t(bg / p.num_groups) * p.heads_q + head_a) * p.tokens + a_tok
-                                     : (int64_t(bg) * p.heads_q + head_a) * seq_a + int64_t(at) * AT + r_in;
+                                     : stat_row_q + head_a * stat_head_stride + int64_t(at) * AT + r_in;
     lse_l = p.lse[stat_idx] * kLog2e;
     delta_l = p.delta[stat_idx];
     // in-tile coordinates of every streamed position, packed in 10-bit fields
@@ -391,8 +424,8 @@ fna_bwd_kernel(const FnaBwdParams p) {
         for (int a = 0; a < 3; ++a) {
           const int qc = t.origin[a] + qo[a];
           valid = valid && (qc < q_extent[a]);
-          const int st = na_window_start(qc, p.ksize[a], p.stride[a], extent[a], p.causal[a] != 0);
-          const int en = na_window_end(qc, st, p.ksize[a], extent[a], p.causal[a] != 0);
+          const int st = na_window_start(qc, ksz[a], p.stride[a], extent[a], p.causal[a] != 0);
+          const int en = na_window_end(qc, st, ksz[a], extent[a], p.causal[a] != 0);
           const int lo = na_min(na_max(st - a_first[a], 0), a_tile[a]);
           const int hi = na_min(na_max(en - a_first[a], 0), a_tile[a]);
           addc |= uint32_t(512 - lo) << (10 * a);
@@ -402,13 +435,13 @@ fna_bwd_kernel(const FnaBwdParams p) {
         sTabB[stage * BT + lane] = valid ? subc : 0u;
       }
     }
-    const int64_t row = p.fused ? batch_row0 + t.row0 : int64_t(bg) * seq_b + t.row0;
+    const int64_t row = p.fused ? batch_row0 + t.row0 : seq_row_b + t.row0;
     if constexpr (KV_STATIONARY) {
       // LSE / delta of the tile's 64 queries: one asynchronous 4-byte-per-lane copy each
       // (wave 1, wave 2; wave 3 and, without delta, wave 2 make the same number of copies into a
       // spare row so that every wave counts the same number of outstanding copies per tile)
       const int64_t stat_row0 = p.fused ? (int64_t(bg / p.num_groups) * p.heads_q + t.head_b) * p.tokens + t.row0
-                                        : (int64_t(bg) * p.heads_q + t.head_b) * seq_b + t.row0;
+                                        : stat_row_q + t.head_b * stat_head_stride + t.row0;
       const float* src = (wave == 2 && HAS_DS ? p.delta : p.lse) + stat_row0;
       float* dst = (wave == 1) ? &sLse[stage * BT] : (wave == 2 && HAS_DS) ? &sDelta[stage * BT] : &sSpare[0];
       if (wave != 0) async_copy4_asm(src, stat_off, lds_address(dst));

@@ -192,7 +192,7 @@ int fill_fna_params(const char* what, FnaParams& p, int na_dim, const int* q_sha
 
 extern "C" {
 
-int natten_amd_abi_version(void) { return 5; }
+int natten_amd_abi_version(void) { return 6; }
 
 const char* natten_amd_last_error(void) { return g_error; }
 
@@ -420,34 +420,35 @@ int natten_amd_attention_forward_varlen(const void* q, const void* k, const void
 // ---- backward ---------------------------------------------------------------------------------
 
 extern "C++" {
-template <typename T, int D>
+template <typename T, int D, bool VARLEN>
 static int launch_bwd(const FnaBwdParams& p, hipStream_t stream) {
   // grids are padded to a multiple of the 8 XCDs: each XCD takes a contiguous eighth of the tiles
   auto grid = [](long long wgs) { return (wgs + kNumXcd - 1) / kNumXcd * kNumXcd; };
   const long long wg_q = grid((long long)p.batch * p.heads_q * prod3(p.q_tiled));
   const long long wg_kv = grid((long long)p.batch * p.heads_kv * prod3(p.kv_tiled));
   if (wg_q > 0x7fffffffLL || wg_kv > 0x7fffffffLL) return fail("fna_backward: problem needs more than 2^31 workgroups");
-  hipLaunchKernelGGL((fna_bwd_kernel<T, D, kBwdDQ>), dim3((unsigned)wg_q), dim3(256), 0, stream, p);
+  hipLaunchKernelGGL((fna_bwd_kernel<T, D, kBwdDQ, VARLEN>), dim3((unsigned)wg_q), dim3(256), 0, stream, p);
   if (int rc = check_launch("fna_backward (dQ)")) return rc;
   if constexpr (D == 128) {
     // dK and dV separately: their accumulators, fragments and products together exceed the
     // registers a matrix instruction addresses directly
-    hipLaunchKernelGGL((fna_bwd_kernel<T, D, kBwdDK>), dim3((unsigned)wg_kv), dim3(256), 0, stream, p);
+    hipLaunchKernelGGL((fna_bwd_kernel<T, D, kBwdDK, VARLEN>), dim3((unsigned)wg_kv), dim3(256), 0, stream, p);
     if (int rc = check_launch("fna_backward (dK)")) return rc;
-    hipLaunchKernelGGL((fna_bwd_kernel<T, D, kBwdDV>), dim3((unsigned)wg_kv), dim3(256), 0, stream, p);
+    hipLaunchKernelGGL((fna_bwd_kernel<T, D, kBwdDV, VARLEN>), dim3((unsigned)wg_kv), dim3(256), 0, stream, p);
     return check_launch("fna_backward (dV)");
   } else {
-    hipLaunchKernelGGL((fna_bwd_kernel<T, D, kBwdDKV>), dim3((unsigned)wg_kv), dim3(256), 0, stream, p);
+    hipLaunchKernelGGL((fna_bwd_kernel<T, D, kBwdDKV, VARLEN>), dim3((unsigned)wg_kv), dim3(256), 0, stream, p);
     return check_launch("fna_backward (dK, dV)");
   }
 }
 
 template <typename T>
 static int dispatch_bwd_head_dim(const FnaBwdParams& p, int head_dim, hipStream_t stream) {
+  const bool varlen = p.cu_q != nullptr;  // sequence-packed dense attention
   switch (head_dim) {
-    case 32: return launch_bwd<T, 32>(p, stream);
-    case 64: return launch_bwd<T, 64>(p, stream);
-    case 128: return launch_bwd<T, 128>(p, stream);
+    case 32: return varlen ? launch_bwd<T, 32, true>(p, stream) : launch_bwd<T, 32, false>(p, stream);
+    case 64: return varlen ? launch_bwd<T, 64, true>(p, stream) : launch_bwd<T, 64, false>(p, stream);
+    case 128: return varlen ? launch_bwd<T, 128, true>(p, stream) : launch_bwd<T, 128, false>(p, stream);
   }
   return fail("fna_backward: head_dim must be 32, 64 or 128, got %d", head_dim);
 }
@@ -659,6 +660,59 @@ int natten_amd_attention_backward(const void* q, const void* k, const void* v, c
   p.seqlen_kv = padded_seqlen_kv;
   p.num_groups = 1;
   p.scale = scale;
+  return dispatch_bwd(p, dtype, head_dim, static_cast<hipStream_t>(stream));
+}
+
+int natten_amd_attention_backward_varlen(const void* q, const void* k, const void* v, const void* d_out,
+                                         const float* lse, const float* delta, void* dq, void* dk, void* dv, int dtype,
+                                         int num_seqs, int rows_q, int rows_kv, const int32_t* cu_seqlens_q,
+                                         const int32_t* cu_seqlens_kv, const int32_t* padded_cu_seqlens_q,
+                                         const int32_t* padded_cu_seqlens_kv, int max_seqlen_q, int max_seqlen_kv,
+                                         int heads_q, int heads_kv, int head_dim, int is_causal, float scale,
+                                         void* stream) {
+  g_error[0] = 0;
+  const char* what = "attention_backward_varlen";
+  if (int rc = check_bwd_pointers(what, q, k, v, d_out, lse, delta, dq, dk, dv)) return rc;
+  if (int rc = check_common(what, q, k, v, dq, lse, num_seqs, rows_q, rows_kv, heads_q, heads_kv, head_dim)) return rc;
+  if (!cu_seqlens_q || !cu_seqlens_kv || !padded_cu_seqlens_q || !padded_cu_seqlens_kv)
+    return fail("%s: null cumulative length argument", what);
+  if (rows_q % 128 != 0 || rows_kv % 128 != 0)
+    return fail("%s: the padded row counts (%d, %d) must be multiples of 128", what, rows_q, rows_kv);
+  if (max_seqlen_q < 1 || max_seqlen_kv < 1 || max_seqlen_q > rows_q || max_seqlen_kv > rows_kv)
+    return fail("%s: max_seqlen_q / max_seqlen_kv (%d, %d) must lie in 1 .. the row counts (%d, %d)", what,
+                max_seqlen_q, max_seqlen_kv, rows_q, rows_kv);
+  // per sequence: the 1-D neighborhood problem whose window is the whole key sequence
+  FnaBwdParams p;
+  memset(&p, 0, sizeof(p));
+  for (int a = 0; a < 3; ++a) {
+    p.qkv_shape[a] = p.ksize[a] = p.stride[a] = p.dil[a] = p.q_tile[a] = p.kv_tile[a] = p.q_tiled[a] = p.kv_tiled[a] = 1;
+  }
+  p.qkv_shape[0] = p.ksize[0] = max_seqlen_kv;  // replaced per sequence inside the kernel
+  p.q_extent0 = max_seqlen_q;
+  p.causal[0] = is_causal != 0;
+  p.q_tile[0] = p.kv_tile[0] = 128;
+  p.q_tiled[0] = (max_seqlen_q + 127) / 128;
+  p.kv_tiled[0] = (max_seqlen_kv + 127) / 128;
+  p.q = q;
+  p.k = k;
+  p.v = v;
+  p.d_out = d_out;
+  p.lse = lse;
+  p.delta = delta;
+  p.dq = dq;
+  p.dk = dk;
+  p.dv = dv;
+  p.batch = num_seqs;
+  p.heads_q = heads_q;
+  p.heads_kv = heads_kv;
+  p.seqlen_q = rows_q;
+  p.seqlen_kv = rows_kv;
+  p.num_groups = 1;
+  p.scale = scale;
+  p.cu_q = cu_seqlens_q;
+  p.cu_kv = cu_seqlens_kv;
+  p.pcu_q = padded_cu_seqlens_q;
+  p.pcu_kv = padded_cu_seqlens_kv;
   return dispatch_bwd(p, dtype, head_dim, static_cast<hipStream_t>(stream));
 }
 

@@ -131,12 +131,35 @@ class AmdFmhaFunction(torch.autograd.Function):
         return dq[:, :sq, :, :head_dim], dk[:, :skv, :, :head_dim], dv[:, :skv, :, :head_dim], None, None
 
 
+def _padded_packing(cu: Tensor, rows: int) -> Tuple[Tensor, Tensor, int]:
+    """A packing of the same sequences with every sequence padded to a multiple of 128 rows, from
+    device arithmetic only (no copy to the host): (padded cumulative lengths [sequences + 1] int32,
+    padded row of every packed row [rows] int64, row count of the padded packing).  The row count
+    is an upper bound the host can know: rows + 127 per sequence, rounded up to 128."""
+    num_seqs = cu.numel() - 1
+    cu = cu.to(torch.int32)
+    padded_len = (cu[1:] - cu[:-1] + 127) // 128 * 128
+    padded_cu = torch.cat([cu.new_zeros(1), torch.cumsum(padded_len, 0).to(torch.int32)])
+    row = torch.arange(rows, device=cu.device, dtype=torch.int32)
+    # the sequence of a packed row (empty sequences own no row; rows past the last sequence, which a
+    # consistent caller does not have, count to the last one and stay inside the bound)
+    seq = torch.searchsorted(cu[1:].contiguous(), row, right=True).clamp_(max=num_seqs - 1)
+    dest = (padded_cu[seq] + (row - cu[seq])).long()
+    return padded_cu, dest, -(-(rows + 127 * num_seqs) // 128) * 128
+
+
+def _to_padded_packing(x: Tensor, dest: Tensor, padded_rows: int) -> Tensor:
+    out = x.new_zeros((x.shape[0], padded_rows) + tuple(x.shape[2:]))
+    return out.index_copy_(1, dest, x)
+
+
 class AmdFmhaVarlenFunction(torch.autograd.Function):
     """Variable-length dense attention with a backward pass.  The forward is the sequence-packed
-    kernel; the backward runs the fixed-length backward kernels once per sequence (on zero-padded
-    copies of its rows), which costs one device-to-host copy of the cumulative lengths and one
-    set of launches per sequence.  Counterpart of the varlen arguments of
-    src/natten/backends/blackwell_fmha.py:52-170."""
+    kernel.  The backward kernels work on 128-row tiles that must not straddle two sequences, so
+    the backward first copies the operands into a packing whose sequences are padded to multiples
+    of 128 rows (index arithmetic on the device, no copy of the lengths to the host), runs one
+    set of launches for all sequences, and gathers the gradient rows back.  Counterpart of the
+    varlen arguments of src/natten/backends/blackwell_fmha.py:52-170."""
 
     @staticmethod
     def forward(ctx, query, key, value, is_causal, scale, cu_q, cu_kv, max_q, max_kv):
@@ -146,6 +169,7 @@ class AmdFmhaVarlenFunction(torch.autograd.Function):
                                 max_seqlen_KV=max_kv)
         ctx.save_for_backward(query, key, value, out, lse, cu_q, cu_kv)
         ctx.args = (is_causal, scale)
+        ctx.max_seqlens = (int(max_q), int(max_kv))
         ctx.mark_non_differentiable(lse)
         return out, lse
 
@@ -156,21 +180,19 @@ class AmdFmhaVarlenFunction(torch.autograd.Function):
         head_dim = query.shape[-1]
         d_pad = padded_head_dim(head_dim)
         q, k, v, o, do = (pad_head_dim(t.contiguous(), d_pad).contiguous() for t in (query, key, value, out, d_out))
+        max_q, max_kv = ctx.max_seqlens
+        if max_q == 0 or max_kv == 0 or q.shape[1] == 0 or k.shape[1] == 0:
+            # no sequence has both queries and keys: the output does not depend on the operands
+            return (torch.zeros_like(query), torch.zeros_like(key), torch.zeros_like(value)) + (None,) * 6
         delta = torch_ops.compute_delta(o, do)
-        dq, dk, dv = torch.zeros_like(q), torch.zeros_like(k), torch.zeros_like(v)
-        bounds_q, bounds_kv = cu_q.tolist(), cu_kv.tolist()
-        for b in range(len(bounds_q) - 1):
-            q0, q1, k0, k1 = bounds_q[b], bounds_q[b + 1], bounds_kv[b], bounds_kv[b + 1]
-            sq, skv = q1 - q0, k1 - k0
-            if sq <= 0 or skv <= 0:
-                continue  # no queries, or no keys (output 0, nothing to differentiate)
-            pq, pkv = -(-sq // 128) * 128, -(-skv // 128) * 128
-            g = torch_ops.attention_backward(
-                _pad_rows(q[:, q0:q1], pq), _pad_rows(k[:, k0:k1], pkv), _pad_rows(v[:, k0:k1], pkv),
-                _pad_rows(do[:, q0:q1], pq), _pad_rows(lse[:, q0:q1], pq), _pad_rows(delta[:, q0:q1], pq),
-                sq, skv, is_causal, scale,
-            )
-            dq[:, q0:q1] = g[0][:, :sq]
-            dk[:, k0:k1] = g[1][:, :skv]
-            dv[:, k0:k1] = g[2][:, :skv]
+        pcu_q, dest_q, rows_q = _padded_packing(cu_q, q.shape[1])
+        pcu_kv, dest_kv, rows_kv = _padded_packing(cu_kv, k.shape[1])
+        dq, dk, dv = torch_ops.attention_backward_varlen(
+            _to_padded_packing(q, dest_q, rows_q), _to_padded_packing(k, dest_kv, rows_kv),
+            _to_padded_packing(v, dest_kv, rows_kv), _to_padded_packing(do, dest_q, rows_q),
+            _to_padded_packing(lse, dest_q, rows_q), _to_padded_packing(delta, dest_q, rows_q),
+            cu_q.to(torch.int32).contiguous(), cu_kv.to(torch.int32).contiguous(), pcu_q, pcu_kv, max_q, max_kv,
+            is_causal, scale,
+        )
+        dq, dk, dv = dq.index_select(1, dest_q), dk.index_select(1, dest_kv), dv.index_select(1, dest_kv)
         return (dq[..., :head_dim], dk[..., :head_dim], dv[..., :head_dim]) + (None,) * 6

@@ -139,6 +139,20 @@ def _(q, k, v, d_out, lse, delta, seqlen_q, seqlen_kv, is_causal, scale):
     return torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
 
 
+@torch.library.custom_op("natten_amd::attention_backward_varlen", mutates_args=(), device_types="cuda")
+def _attention_backward_varlen_op(
+    q: Tensor, k: Tensor, v: Tensor, d_out: Tensor, lse: Tensor, delta: Tensor, cu_q: Tensor, cu_kv: Tensor,
+    padded_cu_q: Tensor, padded_cu_kv: Tensor, max_seqlen_q: int, max_seqlen_kv: int, is_causal: bool, scale: float,
+) -> Tuple[Tensor, Tensor, Tensor]:
+    return _lib.attention_backward_varlen(q, k, v, d_out, lse, delta, cu_q, cu_kv, padded_cu_q, padded_cu_kv,
+                                          max_seqlen_q, max_seqlen_kv, is_causal, scale)
+
+
+@_attention_backward_varlen_op.register_fake
+def _(q, k, v, d_out, lse, delta, cu_q, cu_kv, padded_cu_q, padded_cu_kv, max_seqlen_q, max_seqlen_kv, is_causal, scale):
+    return torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+
+
 def _permuted_shape(x: Tensor, tile_shape: List[int], dilation: List[int]) -> List[int]:
     na_dim = x.dim() - 3
     groups, seqlen = 1, 1
@@ -261,6 +275,15 @@ def attention_backward(q, k, v, d_out, lse, delta, seqlen_q, seqlen_kv, is_causa
         return _attention_backward_op(q, k, v, d_out, lse, delta, int(seqlen_q), int(seqlen_kv), bool(is_causal),
                                       float(scale))
     return _lib.attention_backward(q, k, v, d_out, lse, delta, seqlen_q, seqlen_kv, is_causal, scale)
+
+
+def attention_backward_varlen(q, k, v, d_out, lse, delta, cu_q, cu_kv, padded_cu_q, padded_cu_kv, max_seqlen_q,
+                              max_seqlen_kv, is_causal, scale):
+    if _tracing():
+        return _attention_backward_varlen_op(q, k, v, d_out, lse, delta, cu_q, cu_kv, padded_cu_q, padded_cu_kv,
+                                             int(max_seqlen_q), int(max_seqlen_kv), bool(is_causal), float(scale))
+    return _lib.attention_backward_varlen(q, k, v, d_out, lse, delta, cu_q, cu_kv, padded_cu_q, padded_cu_kv,
+                                          max_seqlen_q, max_seqlen_kv, is_causal, scale)
 
 
 def token_permute(x, tile_shape, dilation, flip_tiled_dims, widen=False):

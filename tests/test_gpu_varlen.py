@@ -139,3 +139,32 @@ def test_varlen_backward(causal):
             assert torch.count_nonzero(k.grad[:, okv : okv + lkv]) == 0 and torch.count_nonzero(v.grad[:, okv : okv + lkv]) == 0
         oq += lq
         okv += lkv
+
+
+@pytest.mark.parametrize("head_dim,dtype", [(128, torch.float16), (32, torch.bfloat16)])
+def test_varlen_backward_equals_per_sequence_calls(head_dim, dtype):
+    # one set of launches for the packed batch gives, bit for bit, what the fixed-length backward
+    # gives sequence by sequence (same kernels, same 128-row tiles); lengths span several tiles
+    seqlens_q, seqlens_kv = [300, 128, 1, 513], [257, 640, 77, 130]
+    H, Hkv = 2, 1
+    tq, tkv = sum(seqlens_q), sum(seqlens_kv)
+    q = _rand((1, tq, H, head_dim), dtype, 60)
+    k = _rand((1, tkv, Hkv, head_dim), dtype, 61)
+    v = _rand((1, tkv, Hkv, head_dim), dtype, 62)
+    d_out = _rand((1, tq, H, head_dim), dtype, 63)
+    sq = torch.tensor(seqlens_q, dtype=torch.int32, device="cuda")
+    skv = torch.tensor(seqlens_kv, dtype=torch.int32, device="cuda")
+    for causal in (False, True):
+        qp, kp, vp = (t.clone().requires_grad_(True) for t in (q, k, v))
+        natten_amd.attention(qp, kp, vp, is_causal=causal, seqlens_Q=sq, seqlens_KV=skv).backward(d_out)
+        oq = okv = 0
+        for lq, lkv in zip(seqlens_q, seqlens_kv):
+            qs = q[:, oq : oq + lq].clone().requires_grad_(True)
+            ks = k[:, okv : okv + lkv].clone().requires_grad_(True)
+            vs = v[:, okv : okv + lkv].clone().requires_grad_(True)
+            natten_amd.attention(qs, ks, vs, is_causal=causal).backward(d_out[:, oq : oq + lq])
+            assert torch.equal(qp.grad[:, oq : oq + lq], qs.grad), (lq, lkv, causal)
+            assert torch.equal(kp.grad[:, okv : okv + lkv], ks.grad), (lq, lkv, causal)
+            assert torch.equal(vp.grad[:, okv : okv + lkv], vs.grad), (lq, lkv, causal)
+            oq += lq
+            okv += lkv

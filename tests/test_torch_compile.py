@@ -52,10 +52,18 @@ def test_compiled_equals_eager(name):
     assert torch.equal(out, ref_out) and torch.equal(lse, ref_lse)
 
 
+def _varlen_attention(q, k, v):
+    cu = torch.tensor([0, 40, 170, 300], dtype=torch.int32, device=q.device)
+    return natten_amd.attention(q, k, v, is_causal=True, cumulative_seqlen_Q=cu, cumulative_seqlen_KV=cu,
+                                max_seqlen_Q=130, max_seqlen_KV=130)
+
+
 GRAD_CASES = {
     "na2d": (lambda q, k, v: natten_amd.na2d(q, k, v, (5, 7), (2, 1), (1, 1), (False, True)), [(1, 20, 24, 2, 64)] * 3),
     "na3d padded head dim": (lambda q, k, v: natten_amd.na3d(q, k, v, (2, 5, 5)), [(1, 4, 8, 8, 2, 40)] * 3),
     "attention": (lambda q, k, v: natten_amd.attention(q, k, v, is_causal=True), [(2, 100, 4, 32)] * 3),
+    # sequence-packed: forward and backward must trace without reading the lengths on the host
+    "attention varlen": (_varlen_attention, [(1, 300, 2, 64)] * 3),
 }
 
 
