@@ -3,16 +3,20 @@
 // One kernel template, several roles.  A workgroup owns a "stationary" tile of 128 rows (one
 // row per lane and 32-row block, four waves) and streams 64-row tiles of the other side
 // through LDS:
-//   dQ role     : stationary = queries (operands Q, dO; result dQ), streamed = keys (K, V)
-//   dK, dV, dKV : stationary = keys    (operands K, V; results dK and / or dV), streamed = queries (Q, dO)
+//   dQ role          : stationary = queries (operands Q, dO; result dQ), streamed = keys (K, V)
+//   dKV, paired role : stationary = keys    (operands K, V; results dK and dV), streamed = queries (Q, dO)
 // Per streamed tile, with Y1/Y2 the streamed and X1/X2 the stationary operands:
 //   S^T  = Y1 X1^T,  dP^T = Y2 X2^T                     (32x32x16 MFMA, the lane owns a stationary row)
 //   P    = exp2(c S - log2e LSE) on unmasked pairs, 0 elsewhere;  dS = P (dP - delta)
 //   acc1^T += Y1^T dS^T   (dQ = scale * sum_k dS k  /  dK = scale * sum_q dS q)
 //   acc2^T += Y2^T P^T    (dV = sum_q P dO)
-// The dK and dV roles exist next to the combined one because at head dim 128 the combined
-// accumulators, stationary fragments and both products no longer fit the 256 vector registers
-// a matrix instruction can address directly.  LSE and delta = rowsum(dO * O) belong to the
+// In the dKV role one wave forms all of this for its 32 key rows.  At head dim 128 the
+// accumulators, stationary fragments and both products of that no longer fit the 256 vector
+// registers a matrix instruction can address directly; the paired role then splits the work
+// over two waves without recomputing anything: eight waves per workgroup, waves w and w + 4
+// share the 32 key rows of block w; wave w ("P wave") forms S^T, the probabilities and dV,
+// wave w + 4 ("dS wave") forms dP^T, takes the probabilities from LDS (fp16, one tile later),
+// and forms dS and dK.  LSE and delta = rowsum(dO * O) belong to the
 // query: per-lane scalars in the dQ role, a small per-tile LDS table in the others.  Nothing
 // is accumulated through memory, so the results are deterministic.
 //
@@ -68,15 +72,18 @@ struct FnaBwdParams {
   const int32_t* pcu_kv;
 };
 
-enum BwdRole : int { kBwdDQ = 0, kBwdDK = 1, kBwdDV = 2, kBwdDKV = 3 };
+enum BwdRole : int { kBwdDQ = 0, kBwdDKV = 1, kBwdPair = 2 };
 
 template <typename T, int D, int ROLE, bool VARLEN = false>
-__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
+__global__ void __launch_bounds__(ROLE == kBwdPair ? 512 : 256) __attribute__((amdgpu_waves_per_eu(2, 2)))
 fna_bwd_kernel(const FnaBwdParams p) {
   constexpr bool KV_STATIONARY = ROLE != kBwdDQ;
-  constexpr bool HAS_DS = ROLE != kBwdDV;                    // dP, dS and acc1 (dQ or dK)
-  constexpr bool HAS_PV = ROLE == kBwdDV || ROLE == kBwdDKV;  // acc2 (dV)
-  constexpr int NT = 256;
+  constexpr bool PAIR = ROLE == kBwdPair;
+  // what one wave's tile body forms (a P wave of the paired role is a dV wave that also hands on
+  // its probabilities; the dS waves have a body of their own)
+  constexpr bool HAS_DS = !PAIR;                      // dP, dS and acc1 (dQ or dK)
+  constexpr bool HAS_PV = ROLE == kBwdDKV || PAIR;  // acc2 (dV; dK in a dS wave)
+  constexpr int NT = PAIR ? 512 : 256;
   constexpr int AT = 128;  // stationary rows
   constexpr int BT = 64;   // streamed rows per tile
   constexpr int KSTEPS = D / 16;
@@ -93,12 +100,16 @@ fna_bwd_kernel(const FnaBwdParams p) {
   using M = Mma<T>;
   using vec8 = typename M::vec8;
   using vec2 = typename M::vec2;
+  typedef _Float16 h16x2_t __attribute__((ext_vector_type(2)));
 
   // One copy of Y1 and one of Y2 per stage, in the layout that serves row reads (S, dP) and
   // transpose reads (the accumulations) alike.
   // Stages: tiles are copied NS - 1 ahead.  Two stages at head dim 128 keep a workgroup under
   // half of the CU's LDS, so that two workgroups (two waves per SIMD) share a CU.
-  constexpr int NS = D == 128 ? 2 : 3;
+  // The paired role keeps a tile for two steps (the dS waves run one tile behind): three stages
+  // with copies one tile ahead.
+  constexpr int NS = (D == 128 && !PAIR) ? 2 : 3;
+  static_assert(!PAIR || D == 128, "the paired role is for head dim 128 (smaller ones fit the combined role)");
   __shared__ __attribute__((aligned(1024))) char sY1[NS * TILE_BYTES];
   __shared__ __attribute__((aligned(1024))) char sY2[NS * TILE_BYTES];
   __shared__ __attribute__((aligned(16))) uint32_t sTabA[NS * BT];
@@ -106,10 +117,15 @@ fna_bwd_kernel(const FnaBwdParams p) {
   __shared__ __attribute__((aligned(16))) float sLse[NS * BT];
   __shared__ __attribute__((aligned(16))) float sDelta[NS * BT];
   __shared__ __attribute__((aligned(16))) float sSpare[BT];
+  // paired role: probabilities from the P waves to the dS waves, fp16, [tile parity][row block]
+  // [sub-block][half of the 16 values][lane] x 16 bytes
+  __shared__ __attribute__((aligned(16))) char sX[PAIR ? 2 * 4 * NSB * 2 * 64 * 16 : 16];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int rw = PAIR ? (wave & 3) : wave;  // 32-row block of the stationary tile
+  const int part = PAIR ? (wave >> 2) : 0;  // paired role: 0 = P wave, 1 = dS wave
   const int l32 = lane & 31;
   const int g = lane >> 5;
 
@@ -236,7 +252,7 @@ fna_bwd_kernel(const FnaBwdParams p) {
   }
 
   // ---- this lane's stationary row -----------------------------------------------------------------
-  const int r_in = wave * 32 + l32;  // row inside the tile: dimension 0 fastest
+  const int r_in = rw * 32 + l32;  // row inside the tile: dimension 0 fastest
   int a_off[3];
   a_off[0] = r_in % a_tile[0];
   a_off[1] = (r_in / a_tile[0]) % a_tile[1];
@@ -266,8 +282,13 @@ fna_bwd_kernel(const FnaBwdParams p) {
   };
   auto store_results = [&](const f32x16_t (&a1)[DB], const f32x16_t (&a2)[DB], float scale1) {
     if constexpr (ROLE == kBwdDQ) store_rows(p.dq, a1, scale1);
-    if constexpr (ROLE == kBwdDK || ROLE == kBwdDKV) store_rows(p.dk, a1, scale1);
-    if constexpr (HAS_PV) store_rows(p.dv, a2, scale1 == 0.f ? 0.f : 1.f);
+    if constexpr (ROLE == kBwdDKV) store_rows(p.dk, a1, scale1);
+    if constexpr (PAIR) {
+      if (part) store_rows(p.dk, a2, scale1);  // a dS wave accumulates dK where a P wave accumulates dV
+      else store_rows(p.dv, a2, scale1 == 0.f ? 0.f : 1.f);
+    } else if constexpr (HAS_PV) {
+      store_rows(p.dv, a2, scale1 == 0.f ? 0.f : 1.f);
+    }
   };
 
   f32x16_t acc1[DB], acc2[DB];
@@ -283,7 +304,9 @@ fna_bwd_kernel(const FnaBwdParams p) {
   }
 
   // stationary operand fragments: row r_in, elements 16*ks + 8*g .. +7
-  const T* x1 = reinterpret_cast<const T*>(KV_STATIONARY ? p.k : p.q) + a_row * a_stride + int64_t(head_a) * D + g * 8;
+  // (paired role: K for the P waves, V for the dS waves)
+  const T* x1 = reinterpret_cast<const T*>(KV_STATIONARY ? ((PAIR && part) ? p.v : p.k) : p.q) + a_row * a_stride +
+                int64_t(head_a) * D + g * 8;
   const T* x2 = reinterpret_cast<const T*>(KV_STATIONARY ? p.v : p.d_out) + a_row * a_stride + int64_t(head_a) * D + g * 8;
   vec8 x1f[KSTEPS], x2f[HAS_DS ? KSTEPS : 1];
 #pragma unroll
@@ -438,12 +461,12 @@ fna_bwd_kernel(const FnaBwdParams p) {
     const int64_t row = p.fused ? batch_row0 + t.row0 : seq_row_b + t.row0;
     if constexpr (KV_STATIONARY) {
       // LSE / delta of the tile's 64 queries: one asynchronous 4-byte-per-lane copy each
-      // (wave 1, wave 2; wave 3 and, without delta, wave 2 make the same number of copies into a
+      // (wave 1, wave 2; the other waves but wave 0 make the same number of copies into a
       // spare row so that every wave counts the same number of outstanding copies per tile)
       const int64_t stat_row0 = p.fused ? (int64_t(bg / p.num_groups) * p.heads_q + t.head_b) * p.tokens + t.row0
                                         : stat_row_q + t.head_b * stat_head_stride + t.row0;
-      const float* src = (wave == 2 && HAS_DS ? p.delta : p.lse) + stat_row0;
-      float* dst = (wave == 1) ? &sLse[stage * BT] : (wave == 2 && HAS_DS) ? &sDelta[stage * BT] : &sSpare[0];
+      const float* src = (wave == 2 ? p.delta : p.lse) + stat_row0;
+      float* dst = (wave == 1) ? &sLse[stage * BT] : (wave == 2) ? &sDelta[stage * BT] : &sSpare[0];
       if (wave != 0) async_copy4_asm(src, stat_off, lds_address(dst));
     }
     const int64_t elem = row * b_stride + int64_t(t.head_b) * D;
@@ -493,8 +516,9 @@ fna_bwd_kernel(const FnaBwdParams p) {
   constexpr int NC = 2 * DB * W;                           // accumulation slots per sub-block
   constexpr int G = N1 + 2 * NC;
   constexpr int PF = 2;                                    // fragments read ahead
-  auto tile_body = [&](auto masked_tag, int stage, uint32_t addc, uint32_t subc) __attribute__((always_inline)) {
+  auto tile_body = [&](auto masked_tag, int stage, uint32_t addc, uint32_t subc, int exch) __attribute__((always_inline)) {
     constexpr bool MASKED = decltype(masked_tag)::value;
+    (void)exch;  // paired role: which of the two probability buffers this tile writes
     const char* y1 = sY1 + stage * TILE_BYTES;
     const char* y2 = sY2 + stage * TILE_BYTES;
 
@@ -525,6 +549,7 @@ fna_bwd_kernel(const FnaBwdParams p) {
     // when they are needed (the other wave covers the wait)
     u32x4_t ta, tb;
     f32x4_t ls4, dl4;
+    f32x4_t lsq[PAIR ? 4 : 1];  // paired role: the LSE values of a sub-block, read ahead of its products
     auto load_group = [&](auto gi_tag) {
       constexpr int gi = decltype(gi_tag)::value;  // sub-block * 4 + jj
       if constexpr (gi < 2 * 4) {
@@ -534,7 +559,8 @@ fna_bwd_kernel(const FnaBwdParams p) {
             ta = *reinterpret_cast<const u32x4_t*>(&sTabA[stage * BT + e0]);
             tb = *reinterpret_cast<const u32x4_t*>(&sTabB[stage * BT + e0]);
           }
-          ls4 = *reinterpret_cast<const f32x4_t*>(&sLse[stage * BT + e0]) * kLog2e;
+          if constexpr (PAIR) ls4 = lsq[gi % 4] * kLog2e;
+          else ls4 = *reinterpret_cast<const f32x4_t*>(&sLse[stage * BT + e0]) * kLog2e;
           if constexpr (HAS_DS) dl4 = *reinterpret_cast<const f32x4_t*>(&sDelta[stage * BT + e0]);
         } else if constexpr (MASKED) {
           ta = *reinterpret_cast<const u32x4_t*>(&sTabA[e0]);
@@ -542,6 +568,7 @@ fna_bwd_kernel(const FnaBwdParams p) {
       }
     };
     float held_p = 0.f, held_ds = 0.f;
+    uint32_t px[PAIR ? 8 : 1];  // paired role: the sub-block's probabilities as fp16 pairs
     auto elem = [&](auto sb_tag, auto r_tag) {
       constexpr int sb = decltype(sb_tag)::value, r = decltype(r_tag)::value;
       constexpr int i = r % 4;
@@ -568,6 +595,15 @@ fna_bwd_kernel(const FnaBwdParams p) {
           held_ds = ds;
         }
       } else {
+        if constexpr (PAIR) {
+          const h16x2_t h2 = {static_cast<_Float16>(held_p), static_cast<_Float16>(x)};
+          px[r / 2] = __builtin_bit_cast(uint32_t, h2);
+          if constexpr (r == 15) {
+            char* dst = sX + ((((exch * 4 + rw) * NSB + sb) * 2) * 64 + lane) * 16;
+            *reinterpret_cast<u32x4_t*>(dst) = u32x4_t{px[0], px[1], px[2], px[3]};
+            *reinterpret_cast<u32x4_t*>(dst + 64 * 16) = u32x4_t{px[4], px[5], px[6], px[7]};
+          }
+        }
         if constexpr (HAS_PV) {
           vec2 p2 = {static_cast<T>(held_p), static_cast<T>(x)};
           uint32_t pb = __builtin_bit_cast(uint32_t, p2);
@@ -596,6 +632,11 @@ fna_bwd_kernel(const FnaBwdParams p) {
       if constexpr (x + PF < G) fr[x + PF] = frag(std::integral_constant<int, x + PF>{});
       if constexpr (sl.prod) {
         constexpr int ks = sl.i / WP, which = sl.i % WP;
+        if constexpr (PAIR && sl.i == 0) {
+#pragma unroll
+          for (int jj = 0; jj < 4; ++jj)
+            lsq[jj] = *reinterpret_cast<const f32x4_t*>(&sLse[stage * BT + sb * 32 + 8 * jj + 4 * g]);
+        }
         f32x16_t zero;
 #pragma unroll
         for (int r = 0; r < 16; ++r) zero[r] = 0.f;
@@ -611,6 +652,108 @@ fna_bwd_kernel(const FnaBwdParams p) {
       }
       __builtin_amdgcn_sched_barrier(0);
     });
+  };
+
+  // ---- paired role: the dS waves ----------------------------------------------------------------
+  // produce: dP^T of the current tile, kept in registers until the next step;
+  // consume: dS of the previous tile from its dP^T, its delta and the P waves' probabilities,
+  // then dK += dS^T Q with that tile's Q (still in its stage).
+  f32x16_t held_dp[NSB];
+  auto pair_produce = [&](int stage) __attribute__((always_inline)) {
+    const char* y2 = sY2 + stage * TILE_BYTES;
+    constexpr int N = NSB * KSTEPS;
+    vec8 fr[N];
+    for_range<0, PF>([&](auto x_tag) {
+      constexpr int x = decltype(x_tag)::value;
+      fr[x] = row_frag(y2, x / KSTEPS, x % KSTEPS);
+    });
+    for_range<0, N>([&](auto x_tag) __attribute__((always_inline)) {
+      constexpr int x = decltype(x_tag)::value;
+      constexpr int sb = x / KSTEPS, ks = x % KSTEPS;
+      if constexpr (x + PF < N) fr[x + PF] = row_frag(y2, (x + PF) / KSTEPS, (x + PF) % KSTEPS);
+      f32x16_t zero;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) zero[r] = 0.f;
+      held_dp[sb] = M::run(fr[x], x1f[ks], ks == 0 ? zero : held_dp[sb]);
+      __builtin_amdgcn_sched_barrier(0);
+    });
+  };
+  auto pair_consume = [&](int stage, int exch) __attribute__((always_inline)) {
+    const char* y1 = sY1 + stage * TILE_BYTES;
+    vec8 dsf[NSB][2];
+#pragma unroll
+    for (int sb = 0; sb < NSB; ++sb) {
+      const char* src = sX + ((((exch * 4 + rw) * NSB + sb) * 2) * 64 + lane) * 16;
+      const u32x4_t lo = *reinterpret_cast<const u32x4_t*>(src);
+      const u32x4_t hi = *reinterpret_cast<const u32x4_t*>(src + 64 * 16);
+#pragma unroll
+      for (int jj = 0; jj < 4; ++jj) {
+        const f32x4_t dl4 = *reinterpret_cast<const f32x4_t*>(&sDelta[stage * BT + sb * 32 + 8 * jj + 4 * g]);
+#pragma unroll
+        for (int i2 = 0; i2 < 2; ++i2) {
+          const int r = 4 * jj + 2 * i2;  // this lane's values r and r + 1 of the sub-block
+          const uint32_t pw = (r < 8) ? lo[r / 2] : hi[r / 2 - 4];
+          const h16x2_t h2 = __builtin_bit_cast(h16x2_t, pw);
+          const float d0 = float(h2[0]) * (held_dp[sb][r] - dl4[2 * i2]);
+          const float d1 = float(h2[1]) * (held_dp[sb][r + 1] - dl4[2 * i2 + 1]);
+          vec2 d2 = {static_cast<T>(d0), static_cast<T>(d1)};
+          dsf[sb][r / 8][r % 8] = d2[0];
+          dsf[sb][r / 8][r % 8 + 1] = d2[1];
+        }
+      }
+    }
+    constexpr int NCB = 2 * DB;  // accumulation slots per sub-block
+    constexpr int N = NSB * NCB;
+    vec8 fr[N];
+    for_range<0, PF>([&](auto x_tag) {
+      constexpr int x = decltype(x_tag)::value;
+      fr[x] = tr_frag(y1, x / NCB, (x % NCB) / DB, x % DB);
+    });
+    for_range<0, N>([&](auto x_tag) __attribute__((always_inline)) {
+      constexpr int x = decltype(x_tag)::value;
+      constexpr int sb = x / NCB, h = (x % NCB) / DB, db = x % DB;
+      if constexpr (x + PF < N) {
+        constexpr int y = x + PF;
+        fr[y] = tr_frag(y1, y / NCB, (y % NCB) / DB, y % DB);
+      }
+      acc2[db] = M::run(fr[x], dsf[sb][h], acc2[db]);
+      __builtin_amdgcn_sched_barrier(0);
+    });
+  };
+  // One pass of the paired role over n_iter tiles: step `it` has the P waves on tile `it` and the
+  // dS waves forming dP of tile `it` after finishing tile it - 1; one more step drains the dS
+  // waves.  The barrier at the top of a step makes tile `it` (copied during step it - 1) and the
+  // probabilities of tile it - 1 visible, and frees the stage of tile it - 2 for the copy of
+  // tile it + 1.
+  auto run_pass_pair = [&](auto masked_tag, auto ds_wave_tag, int n_iter) __attribute__((always_inline)) {
+    constexpr bool MASKED = decltype(masked_tag)::value;
+    constexpr bool DS_WAVE = decltype(ds_wave_tag)::value;
+    if (n_iter <= 0) return;
+    start_walk(std::integral_constant<bool, !MASKED>{});
+    {
+      const Tile t = next_tile(std::integral_constant<bool, !MASKED>{}, 1 < n_iter);
+      issue(t, 0, MASKED);
+    }
+    // `tables`: wave 0, which builds the window tables of a masked tile, is a P wave
+    auto step_top = [&](int it, bool tables) __attribute__((always_inline)) {
+      wait_vmcnt<0>();
+      __syncthreads();
+      if (it + 1 < n_iter) {
+        const Tile t = next_tile(std::integral_constant<bool, !MASKED>{}, it + 2 < n_iter);
+        issue(t, (it + 1) % NS, tables);
+      }
+    };
+    for (int it = 0; it <= n_iter; ++it) {
+      step_top(it, MASKED && !DS_WAVE);
+      if constexpr (DS_WAVE) {
+        if (it > 0) pair_consume((it - 1) % NS, (it - 1) & 1);
+        if (it < n_iter) pair_produce(it % NS);
+      } else {
+        if (it < n_iter) tile_body(masked_tag, it % NS, 0u, 0u, it & 1);
+      }
+    }
+    wait_vmcnt<0>();
+    __syncthreads();  // stages and probability buffers are free for the next pass
   };
 
   // ---- pipeline: tile `it` is multiplied while tiles it+1 .. it+NS-1 are in flight ----------------
@@ -672,7 +815,7 @@ fna_bwd_kernel(const FnaBwdParams p) {
           subc |= uint32_t(511 + hi) << (10 * a);
         }
       }
-      tile_body(masked_tag, stage, addc, subc);
+      tile_body(masked_tag, stage, addc, subc, 0);
       if constexpr (NEED_ORIGIN) {
 #pragma unroll
         for (int a = 0; a < 3; ++a) {
@@ -685,8 +828,20 @@ fna_bwd_kernel(const FnaBwdParams p) {
     __syncthreads();  // the stages are free for the next pass
   };
   const int heads_walked = KV_STATIONARY ? rep : 1;
-  run_pass(std::true_type{}, (total - n_whole) * heads_walked);
-  run_pass(std::false_type{}, n_whole * heads_walked);
+  if constexpr (PAIR) {
+    // the two kinds of wave run separate copies of the passes (the same barriers in both), so
+    // that neither carries the other's registers
+    if (part == 0) {
+      run_pass_pair(std::true_type{}, std::false_type{}, (total - n_whole) * heads_walked);
+      run_pass_pair(std::false_type{}, std::false_type{}, n_whole * heads_walked);
+    } else {
+      run_pass_pair(std::true_type{}, std::true_type{}, (total - n_whole) * heads_walked);
+      run_pass_pair(std::false_type{}, std::true_type{}, n_whole * heads_walked);
+    }
+  } else {
+    run_pass(std::true_type{}, (total - n_whole) * heads_walked);
+    run_pass(std::false_type{}, n_whole * heads_walked);
+  }
 
   store_results(acc1, acc2, p.scale);
 }

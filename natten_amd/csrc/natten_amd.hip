@@ -430,16 +430,13 @@ static int launch_bwd(const FnaBwdParams& p, hipStream_t stream) {
   hipLaunchKernelGGL((fna_bwd_kernel<T, D, kBwdDQ, VARLEN>), dim3((unsigned)wg_q), dim3(256), 0, stream, p);
   if (int rc = check_launch("fna_backward (dQ)")) return rc;
   if constexpr (D == 128) {
-    // dK and dV separately: their accumulators, fragments and products together exceed the
-    // registers a matrix instruction addresses directly
-    hipLaunchKernelGGL((fna_bwd_kernel<T, D, kBwdDK, VARLEN>), dim3((unsigned)wg_kv), dim3(256), 0, stream, p);
-    if (int rc = check_launch("fna_backward (dK)")) return rc;
-    hipLaunchKernelGGL((fna_bwd_kernel<T, D, kBwdDV, VARLEN>), dim3((unsigned)wg_kv), dim3(256), 0, stream, p);
-    return check_launch("fna_backward (dV)");
+    // dK and dV by wave pairs (eight waves per workgroup): one wave's registers cannot hold the
+    // accumulators, fragments and products of both
+    hipLaunchKernelGGL((fna_bwd_kernel<T, D, kBwdPair, VARLEN>), dim3((unsigned)wg_kv), dim3(512), 0, stream, p);
   } else {
     hipLaunchKernelGGL((fna_bwd_kernel<T, D, kBwdDKV, VARLEN>), dim3((unsigned)wg_kv), dim3(256), 0, stream, p);
-    return check_launch("fna_backward (dK, dV)");
   }
+  return check_launch("fna_backward (dK, dV)");
 }
 
 template <typename T>
