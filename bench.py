@@ -218,7 +218,7 @@ def bench_backward(args, q, k, v, kernel, stride, dilation, causal, dt_name):
             "workload": WORKLOAD_NAMES[args.workload] + ", forward + backward",
             "backward_q_tile_shape": list(q_tile),
             "backward_kv_tile_shape": list(kv_tile),
-            "path": ("forward (one launch) + delta + dQ, dK, dV kernels on the original tensors" if fused else
+            "path": ("forward (one launch) + delta + dQ kernel + dK/dV kernel on the original tensors" if fused else
                      "forward + delta + token permutes + dQ and dK/dV kernels + unpermutes"),
         },
         "na_flop_per_step": 3.5 * fwd_flops,
