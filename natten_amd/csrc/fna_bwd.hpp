@@ -437,7 +437,8 @@ fna_bwd_kernel(const FnaBwdParams p) {
   const uint32_t lds_y1 = uint32_t(__builtin_amdgcn_readfirstlane(int(lds_address(sY1))));
   const uint32_t lds_y2 = uint32_t(__builtin_amdgcn_readfirstlane(int(lds_address(sY2))));
   const uint32_t stat_off = uint32_t(sub_pos(lane)) * 4u;  // byte offset of streamed row `lane` in lse / delta (head-major)
-  auto issue = [&](const Tile& t, int stage, bool masked) {
+  // the window tables of a masked streamed tile (key-stationary roles, wave 0)
+  auto build_tables = [&](const Tile& t, int stage, bool masked) {
     if constexpr (KV_STATIONARY) {
       if (wave == 0 && masked) {
         // per streamed query: its window relative to this workgroup's key tile
@@ -458,6 +459,9 @@ fna_bwd_kernel(const FnaBwdParams p) {
         sTabB[stage * BT + lane] = valid ? subc : 0u;
       }
     }
+  };
+  // the asynchronous copies of a streamed tile (and of its LSE / delta values) into a stage
+  auto issue_copies = [&](const Tile& t, int stage) {
     const int64_t row = p.fused ? batch_row0 + t.row0 : seq_row_b + t.row0;
     if constexpr (KV_STATIONARY) {
       // LSE / delta of the tile's 64 queries: one asynchronous 4-byte-per-lane copy each
@@ -478,6 +482,10 @@ fna_bwd_kernel(const FnaBwdParams p) {
       async_copy16_uniform(y1, off_u[i], lds_y1 + d);
       async_copy16_uniform(y2, off_u[i], lds_y2 + d);
     }
+  };
+  auto issue = [&](const Tile& t, int stage, bool masked) {
+    build_tables(t, stage, masked);
+    issue_copies(t, stage);
   };
 
   // lane-constant LDS read offsets (same fragment layouts as the forward kernel)
@@ -516,7 +524,7 @@ fna_bwd_kernel(const FnaBwdParams p) {
   constexpr int NC = 2 * DB * W;                           // accumulation slots per sub-block
   constexpr int G = N1 + 2 * NC;
   constexpr int PF = 2;                                    // fragments read ahead
-  auto tile_body = [&](auto masked_tag, int stage, uint32_t addc, uint32_t subc, int exch) __attribute__((always_inline)) {
+  auto tile_body = [&](auto masked_tag, int stage, uint32_t addc, uint32_t subc, int exch, auto&& after_slot) __attribute__((always_inline)) {
     constexpr bool MASKED = decltype(masked_tag)::value;
     (void)exch;  // paired role: which of the two probability buffers this tile writes
     const char* y1 = sY1 + stage * TILE_BYTES;
@@ -549,7 +557,6 @@ fna_bwd_kernel(const FnaBwdParams p) {
     // when they are needed (the other wave covers the wait)
     u32x4_t ta, tb;
     f32x4_t ls4, dl4;
-    f32x4_t lsq[PAIR ? 4 : 1];  // paired role: the LSE values of a sub-block, read ahead of its products
     auto load_group = [&](auto gi_tag) {
       constexpr int gi = decltype(gi_tag)::value;  // sub-block * 4 + jj
       if constexpr (gi < 2 * 4) {
@@ -559,8 +566,7 @@ fna_bwd_kernel(const FnaBwdParams p) {
             ta = *reinterpret_cast<const u32x4_t*>(&sTabA[stage * BT + e0]);
             tb = *reinterpret_cast<const u32x4_t*>(&sTabB[stage * BT + e0]);
           }
-          if constexpr (PAIR) ls4 = lsq[gi % 4] * kLog2e;
-          else ls4 = *reinterpret_cast<const f32x4_t*>(&sLse[stage * BT + e0]) * kLog2e;
+          ls4 = *reinterpret_cast<const f32x4_t*>(&sLse[stage * BT + e0]) * kLog2e;
           if constexpr (HAS_DS) dl4 = *reinterpret_cast<const f32x4_t*>(&sDelta[stage * BT + e0]);
         } else if constexpr (MASKED) {
           ta = *reinterpret_cast<const u32x4_t*>(&sTabA[e0]);
@@ -632,11 +638,6 @@ fna_bwd_kernel(const FnaBwdParams p) {
       if constexpr (x + PF < G) fr[x + PF] = frag(std::integral_constant<int, x + PF>{});
       if constexpr (sl.prod) {
         constexpr int ks = sl.i / WP, which = sl.i % WP;
-        if constexpr (PAIR && sl.i == 0) {
-#pragma unroll
-          for (int jj = 0; jj < 4; ++jj)
-            lsq[jj] = *reinterpret_cast<const f32x4_t*>(&sLse[stage * BT + sb * 32 + 8 * jj + 4 * g]);
-        }
         f32x16_t zero;
 #pragma unroll
         for (int r = 0; r < 16; ++r) zero[r] = 0.f;
@@ -650,6 +651,7 @@ fna_bwd_kernel(const FnaBwdParams p) {
         if constexpr (to_acc1) acc1[db] = M::run(fr[x], dsf[sb][h], acc1[db]);
         else acc2[db] = M::run(fr[x], pf[sb][h], acc2[db]);
       }
+      after_slot(x_tag);
       __builtin_amdgcn_sched_barrier(0);
     });
   };
@@ -730,26 +732,31 @@ fna_bwd_kernel(const FnaBwdParams p) {
     constexpr bool DS_WAVE = decltype(ds_wave_tag)::value;
     if (n_iter <= 0) return;
     start_walk(std::integral_constant<bool, !MASKED>{});
-    {
-      const Tile t = next_tile(std::integral_constant<bool, !MASKED>{}, 1 < n_iter);
-      issue(t, 0, MASKED);
-    }
-    // `tables`: wave 0, which builds the window tables of a masked tile, is a P wave
-    auto step_top = [&](int it, bool tables) __attribute__((always_inline)) {
+    Tile tn = next_tile(std::integral_constant<bool, !MASKED>{}, 1 < n_iter);
+    issue(tn, 0, MASKED && !DS_WAVE);  // wave 0, which builds the window tables, is a P wave
+    // The dS waves issue their copies of tile it + 1 right after the barrier (they begin a step
+    // with vector work); the P waves, which begin with matrix work, issue theirs after the
+    // products of the first sub-block, so that the eight waves do not all queue on the CU's
+    // address path while the matrix pipe idles.  (No branch around those copies: past the last
+    // tile the descriptor still names the last one, which is copied again into a stage nobody
+    // reads any more.)
+    for (int it = 0; it <= n_iter; ++it) {
       wait_vmcnt<0>();
       __syncthreads();
       if (it + 1 < n_iter) {
-        const Tile t = next_tile(std::integral_constant<bool, !MASKED>{}, it + 2 < n_iter);
-        issue(t, (it + 1) % NS, tables);
+        tn = next_tile(std::integral_constant<bool, !MASKED>{}, it + 2 < n_iter);
+        build_tables(tn, (it + 1) % NS, MASKED && !DS_WAVE);
       }
-    };
-    for (int it = 0; it <= n_iter; ++it) {
-      step_top(it, MASKED && !DS_WAVE);
       if constexpr (DS_WAVE) {
+        if (it + 1 < n_iter) issue_copies(tn, (it + 1) % NS);
         if (it > 0) pair_consume((it - 1) % NS, (it - 1) & 1);
         if (it < n_iter) pair_produce(it % NS);
       } else {
-        if (it < n_iter) tile_body(masked_tag, it % NS, 0u, 0u, it & 1);
+        if (it < n_iter) {
+          tile_body(masked_tag, it % NS, 0u, 0u, it & 1, [&](auto x_tag) {
+            if constexpr (decltype(x_tag)::value == NP - 1) issue_copies(tn, (it + 1) % NS);
+          });
+        }
       }
     }
     wait_vmcnt<0>();
@@ -815,7 +822,7 @@ fna_bwd_kernel(const FnaBwdParams p) {
           subc |= uint32_t(511 + hi) << (10 * a);
         }
       }
-      tile_body(masked_tag, stage, addc, subc, 0);
+      tile_body(masked_tag, stage, addc, subc, 0, [](auto) {});
       if constexpr (NEED_ORIGIN) {
 #pragma unroll
         for (int a = 0; a < 3; ++a) {
