@@ -220,9 +220,22 @@ def fna_forward(
     return out, lse
 
 
-def fused_layout_supported(qkv_shape, dilation, kv_tile_shape) -> bool:
-    """Whether fna_forward_fused accepts this problem: no KV tile may reach past the input."""
-    return all(X % (d * t) == 0 for X, d, t in zip(qkv_shape, dilation, kv_tile_shape))
+def _tile_span_fits(token_layout, dilation, tile_shape, row_bytes: int) -> bool:
+    """The kernels address the rows of a tile of the original tensors with 32-bit byte offsets
+    from the tile's first row: the tile must span less than 2^31 bytes."""
+    span, step = 0, 1
+    for X, d, t in zip(reversed(token_layout), reversed(dilation), reversed(tile_shape)):
+        span += (t - 1) * d * step
+        step *= X
+    return (span + 1) * row_bytes + 8192 < 2**31 - 1
+
+
+def fused_layout_supported(qkv_shape, dilation, kv_tile_shape, row_bytes: int = 0) -> bool:
+    """Whether fna_forward_fused accepts this problem: no KV tile may reach past the input, and
+    (given `row_bytes` = heads_kv * head_dim * 2) a KV tile spans less than 2^31 bytes of it."""
+    return all(X % (d * t) == 0 for X, d, t in zip(qkv_shape, dilation, kv_tile_shape)) and _tile_span_fits(
+        qkv_shape, dilation, kv_tile_shape, row_bytes
+    )
 
 
 def fna_forward_fused(
@@ -358,11 +371,14 @@ def fna_backward(
     return dq, dk, dv
 
 
-def backward_fused_layout_supported(token_layout, dilation, q_tile_shape, kv_tile_shape) -> bool:
-    """Whether the backward kernels can work on the original tensors: no padding on either side."""
-    return all(
-        X % (d * tq) == 0 and X % (d * tk) == 0
-        for X, d, tq, tk in zip(token_layout, dilation, q_tile_shape, kv_tile_shape)
+def backward_fused_layout_supported(token_layout, dilation, q_tile_shape, kv_tile_shape, row_bytes: int = 0) -> bool:
+    """Whether the backward kernels can work on the original tensors: no padding on either side,
+    and (given `row_bytes` = heads_q * head_dim * 2) tiles that span less than 2^31 bytes."""
+    return (
+        all(X % (d * tq) == 0 and X % (d * tk) == 0
+            for X, d, tq, tk in zip(token_layout, dilation, q_tile_shape, kv_tile_shape))
+        and _tile_span_fits(token_layout, dilation, q_tile_shape, row_bytes)
+        and _tile_span_fits(token_layout, dilation, kv_tile_shape, row_bytes)
     )
 
 

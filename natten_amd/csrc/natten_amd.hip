@@ -572,6 +572,14 @@ int natten_amd_fna_backward_fused(const void* q, const void* k, const void* v, c
                                is_causal, q_tile_shape, kv_tile_shape))
     return rc;
   if (int rc = check_common(what, q, k, v, dq, lse, batch, int(tokens), int(tokens), heads_q, heads_kv, head_dim)) return rc;
+  // per-lane byte offsets inside a tile are 32-bit
+  long long span_q = 0, span_kv = 0;
+  for (int a = 0; a < 3; ++a) {
+    span_q += (long long)(f.q_tile[a] - 1) * f.dil[a] * f.tok_stride[a];
+    span_kv += (long long)(f.kv_tile[a] - 1) * f.dil[a] * f.tok_stride[a];
+  }
+  if ((span_q + 1) * heads_q * head_dim * 2 + 8192 >= 0x7fffffffLL || (span_kv + 1) * heads_kv * head_dim * 2 + 8192 >= 0x7fffffffLL)
+    return fail("%s: a tile spans more than 2^31 bytes of the tensors; use the token-permuted entry point", what);
   if (prod3(f.q_tile) != 128 || prod3(f.kv_tile) != 128)
     return fail("%s: Q and KV tiles must hold 128 tokens each, got %d and %d", what, prod3(f.q_tile), prod3(f.kv_tile));
   FnaBwdParams p;

@@ -154,7 +154,8 @@ def amd_fna_generic(
         )
     use_fp8 = fp8_ok and fp8_matmul is not False
     widen = is_fp8(in_dtype) and not use_fp8
-    fusable = (not widen) and _lib.fused_layout_supported(query.shape[1 : 1 + na_dim], dilation, kv_tile_shape)
+    fusable = (not widen) and _lib.fused_layout_supported(query.shape[1 : 1 + na_dim], dilation, kv_tile_shape,
+                                                          row_bytes=key.shape[-2] * d_pad * 2)
     if fused and not fusable:
         raise ValueError(
             "natten_amd: the fused path needs operands that are not widened and an input extent that is a multiple of "
@@ -241,7 +242,8 @@ class AmdFnaFunction(torch.autograd.Function):
         )
         delta = torch_ops.compute_delta(output, d_output)
         na_dim = len(kernel_size)
-        fusable = _lib.backward_fused_layout_supported(query.shape[1 : 1 + na_dim], dilation, q_tile, kv_tile)
+        fusable = _lib.backward_fused_layout_supported(query.shape[1 : 1 + na_dim], dilation, q_tile, kv_tile,
+                                                       row_bytes=query.shape[-2] * query.shape[-1] * 2)
         if fusable and ctx.fused is not False:
             # the kernels gather and scatter their tiles themselves: no permuted copies
             dq, dk, dv = torch_ops.fna_backward_fused(

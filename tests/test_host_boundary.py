@@ -134,3 +134,36 @@ def test_query_range_matches_brute_force():
                 assert (first, last) == (hits[0], hits[-1]), (L, k, s, c, j0, j1)
             else:
                 assert first > last, (L, k, s, c, j0, j1)
+
+
+def test_route_predicates_keep_32_bit_tile_offsets():
+    # the kernels that gather tiles from the original tensors use 32-bit byte offsets inside a
+    # tile: a tile that spans 2^31 bytes or more must take the token-permuted route
+    row_bytes = 24 * 128 * 2
+    assert _lib.fused_layout_supported((32, 48, 80), (1, 1, 1), (1, 8, 8), row_bytes=row_bytes)
+    assert _lib.backward_fused_layout_supported((32, 48, 80), (1, 1, 1), (2, 8, 8), (2, 8, 8), row_bytes=row_bytes)
+    # 128 planes of 512 x 512 tokens: a (128, 1, 1) tile spans 127 planes = 204 GB
+    big = (128, 512, 512)
+    assert _lib.fused_layout_supported(big, (1, 1, 1), (1, 8, 8), row_bytes=row_bytes)
+    assert not _lib.fused_layout_supported(big, (1, 1, 1), (64, 1, 1), row_bytes=row_bytes)
+    assert not _lib.backward_fused_layout_supported(big, (1, 1, 1), (128, 1, 1), (2, 8, 8), row_bytes=row_bytes)
+    assert not _lib.backward_fused_layout_supported(big, (1, 1, 1), (2, 8, 8), (128, 1, 1), row_bytes=row_bytes)
+    assert _lib.backward_fused_layout_supported(big, (1, 1, 1), (2, 8, 8), (2, 8, 8), row_bytes=row_bytes)
+    # extents that are not multiples of dilation x tile are refused as before
+    assert not _lib.fused_layout_supported((20, 24), (1, 1), (8, 8), row_bytes=1024)
+
+
+def test_backward_entry_point_rejects_tiles_beyond_32_bit_offsets():
+    # argument validation happens before anything touches a device: fake (aligned, non-null)
+    # pointers are never dereferenced on this path
+    import ctypes as C
+
+    L = _lib.lib()
+    i32 = lambda xs: (C.c_int32 * 3)(*xs)
+    ptr = 0x10000
+    rc = L.natten_amd_fna_backward_fused(
+        ptr, ptr, ptr, ptr, ptr, ptr, ptr, ptr, ptr, _lib.DTYPE_CODES[__import__("torch").bfloat16], 3, 1, 24, 24, 128,
+        i32((128, 512, 512)), i32((3, 3, 3)), i32((1, 1, 1)), i32((1, 1, 1)), i32((0, 0, 0)), i32((128, 1, 1)),
+        i32((2, 8, 8)), C.c_float(0.1), None,
+    )
+    assert rc != 0 and b"2^31 bytes" in L.natten_amd_last_error()
