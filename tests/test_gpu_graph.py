@@ -1,4 +1,4 @@
-"""The forward under HIP graph capture: the entry points allocate nothing and launch on the
+"""The forward, and a whole training step, under HIP graph capture: the entry points allocate nothing and launch on the
 caller's stream, so a captured call replays correctly.  Each replay (with new inputs copied into
 the captured tensors, and eager work and synchronisations in between) is compared with the
 eager result bit for bit."""
@@ -35,3 +35,42 @@ def test_forward_replays_from_a_graph(shape, kernel, causal):
             ref_out, ref_lse = fn()   # eager work between the replays
             torch.cuda.synchronize()
             assert torch.equal(out, ref_out) and torch.equal(lse, ref_lse), f"replay {i} differs from the eager call"
+
+
+@pytest.mark.parametrize("shape,kernel,causal,head_dim", [
+    ((16, 16), (5, 5), (False, True), 64),     # backward on the original tensors, dQ + combined dK/dV role
+    ((16, 32), (7, 9), (True, False), 128),    # the same with the paired dK/dV role
+    ((20, 24), (5, 7), (False, False), 64),    # permutes + backward kernels + unpermutes
+])
+def test_training_step_replays_from_a_graph(shape, kernel, causal, head_dim):
+    # forward and backward captured together; the gradients of every replay (new inputs copied
+    # into the captured tensors) equal those of the eager step bit for bit
+    gen = torch.Generator().manual_seed(1)
+    mk = lambda: torch.randn((1, *shape, 2, head_dim), generator=gen).to(torch.bfloat16).cuda()
+    q, k, v = (mk().requires_grad_(True) for _ in range(3))
+    d_out = mk()
+
+    def step(a, b, c):
+        natten_amd.na2d(a, b, c, kernel, is_causal=causal).backward(d_out)
+
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        for _ in range(2):  # warm-up outside the capture
+            step(q, k, v)
+    torch.cuda.current_stream().wait_stream(side)
+    for t in (q, k, v):
+        t.grad = None  # the captured backward allocates the gradients from the graph's pool
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step(q, k, v)
+    for i in range(3):
+        with torch.no_grad():
+            for t in (q, k, v, d_out):
+                t.copy_(mk())
+        graph.replay()
+        torch.cuda.synchronize()
+        eager = [t.detach().clone().requires_grad_(True) for t in (q, k, v)]
+        step(*eager)   # eager work between the replays
+        torch.cuda.synchronize()
+        for name, a, b in zip("qkv", (q, k, v), eager):
+            assert torch.equal(a.grad, b.grad), f"replay {i}: d{name} differs from the eager step"
