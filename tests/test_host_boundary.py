@@ -167,3 +167,22 @@ def test_backward_entry_point_rejects_tiles_beyond_32_bit_offsets():
         i32((2, 8, 8)), C.c_float(0.1), None,
     )
     assert rc != 0 and b"2^31 bytes" in L.natten_amd_last_error()
+
+
+def test_every_entry_point_rejects_null_arguments_before_touching_a_device():
+    # argument validation comes first in every entry point: all-zero arguments (null pointers,
+    # zero sizes) give an error code and a message, without any device call
+    import ctypes as C
+
+    L = _lib.lib()
+    skipped = {"natten_amd_abi_version", "natten_amd_last_error", "natten_amd_fna_supported_tiles"}
+    checked = 0
+    for name, (_, arg_types) in _lib._SIGNATURES.items():
+        if name in skipped:
+            continue
+        zeros = [None if a is C.c_void_p else (0.0 if a is C.c_float else 0) for a in arg_types]
+        rc = getattr(L, name)(*zeros)
+        assert rc != 0, f"{name} accepted null arguments"
+        assert L.natten_amd_last_error(), f"{name} returned an error without a message"
+        checked += 1
+    assert checked >= 14
