@@ -40,6 +40,11 @@ WORKLOADS = {
 MEASURED_TRAFFIC_BYTES = {
     ("c4", (2, 8, 8), (1, 8, 8)): 2.82e10,
 }
+# The same for the two backward launches together (dQ role 20.3 GB read + 0.7 GB written, paired
+# dK / dV role 63.7 GB + 1.9 GB), keyed by (workload, backward q tile, backward kv tile).
+MEASURED_BACKWARD_TRAFFIC_BYTES = {
+    ("c4", (2, 8, 8), (2, 8, 8)): 8.66e10,
+}
 
 WORKLOAD_NAMES = {
     "c4": "na3d bf16 B=1 H=24 30x48x80 D=128 k=(18,24,24) s=(1,8,8) causal=(T,F,F) +LSE",
@@ -231,7 +236,7 @@ def bench_backward(args, q, k, v, kernel, stride, dilation, causal, dt_name):
             "peak": peak,
             "unit": "TFLOP/s",
             "frac": achieved / peak,
-            "traffic": None,
+            "traffic": MEASURED_BACKWARD_TRAFFIC_BYTES.get((args.workload, tuple(q_tile), tuple(kv_tile))),
             "algorithmic_flop": 2.5 * fwd_flops,
         },
         "cpu_baseline": None,
