@@ -70,6 +70,10 @@ struct FnaBwdParams {
   const int32_t* cu_kv;
   const int32_t* pcu_q;   // [batch + 1] cumulative padded lengths (row offsets into the tensors)
   const int32_t* pcu_kv;
+  // Workgroup order of the key-stationary launch.  0: every XCD takes one contiguous eighth of
+  // the (batch, head, tile) space.  > 0: runs of this many consecutive tiles are dealt round-robin
+  // to the XCDs (the grid is then a whole number of rounds of 8 runs).
+  int kv_wg_run;
 };
 
 enum BwdRole : int { kBwdDQ = 0, kBwdDKV = 1, kBwdPair = 2 };
@@ -143,11 +147,20 @@ fna_bwd_kernel(const FnaBwdParams p) {
   // ---- workgroup -> (batch * group, head, stationary tile) --------------------------------------
   // Workgroup ids go round-robin to the 8 XCDs; each XCD takes one contiguous eighth of the
   // (batch, head, tile) space, so that the workgroups resident on an XCD are neighbouring tiles
-  // of one head and find each other's streamed tiles in that XCD's L2.
+  // of one head and find each other's streamed tiles in that XCD's L2.  The paired role, with
+  // half as many workgroups resident, does better with short runs dealt round-robin: the XCDs
+  // then work on neighbouring runs of one head at a time and meet in the memory-side cache.
   const int num_a = a_tiled[0] * a_tiled[1] * a_tiled[2];
   const int total_wg = p.batch * heads_a * num_a;
-  const int chunk = (total_wg + kNumXcd - 1) / kNumXcd;
-  const int lin = (int(blockIdx.x) % kNumXcd) * chunk + int(blockIdx.x) / kNumXcd;
+  const int wg_run = KV_STATIONARY ? p.kv_wg_run : 0;
+  int lin;
+  if (wg_run > 0) {
+    const int local = int(blockIdx.x) / kNumXcd;
+    lin = ((local / wg_run) * kNumXcd + int(blockIdx.x) % kNumXcd) * wg_run + local % wg_run;
+  } else {
+    const int chunk = (total_wg + kNumXcd - 1) / kNumXcd;
+    lin = (int(blockIdx.x) % kNumXcd) * chunk + int(blockIdx.x) / kNumXcd;
+  }
   if (lin >= total_wg) return;
   // Within a head the tiles are taken with dimension 0 slowest: the workgroups running side by
   // side are then neighbours in the faster dimensions at the same dimension-0 position and

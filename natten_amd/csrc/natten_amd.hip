@@ -421,11 +421,29 @@ int natten_amd_attention_forward_varlen(const void* q, const void* k, const void
 
 extern "C++" {
 template <typename T, int D, bool VARLEN>
-static int launch_bwd(const FnaBwdParams& p, hipStream_t stream) {
+static int launch_bwd(const FnaBwdParams& params, hipStream_t stream) {
+  FnaBwdParams p = params;
   // grids are padded to a multiple of the 8 XCDs: each XCD takes a contiguous eighth of the tiles
   auto grid = [](long long wgs) { return (wgs + kNumXcd - 1) / kNumXcd * kNumXcd; };
   const long long wg_q = grid((long long)p.batch * p.heads_q * prod3(p.q_tiled));
-  const long long wg_kv = grid((long long)p.batch * p.heads_kv * prod3(p.kv_tiled));
+  long long wg_kv = grid((long long)p.batch * p.heads_kv * prod3(p.kv_tiled));
+  if constexpr (D == 128) {
+    // paired role (one workgroup per CU, 32 resident per XCD): runs of about 32 key tiles, a whole
+    // number of dimension-0 slabs or an even part of one, dealt round-robin to the XCDs
+    const int slab = p.kv_tiled[1] * p.kv_tiled[2];
+    int run;
+    if (slab >= 32) {
+      const int parts = (slab + 16) / 32;
+      run = (slab + parts - 1) / parts;
+    } else {
+      int rows = (32 + slab / 2) / slab;
+      if (rows > p.kv_tiled[0]) rows = p.kv_tiled[0];
+      run = slab * rows;
+    }
+    p.kv_wg_run = run;
+    const long long runs = ((long long)p.batch * p.heads_kv * prod3(p.kv_tiled) + run - 1) / run;
+    wg_kv = (runs + kNumXcd - 1) / kNumXcd * kNumXcd * run;
+  }
   if (wg_q > 0x7fffffffLL || wg_kv > 0x7fffffffLL) return fail("fna_backward: problem needs more than 2^31 workgroups");
   hipLaunchKernelGGL((fna_bwd_kernel<T, D, kBwdDQ, VARLEN>), dim3((unsigned)wg_q), dim3(256), 0, stream, p);
   if (int rc = check_launch("fna_backward (dQ)")) return rc;
