@@ -131,21 +131,29 @@ class AmdFmhaFunction(torch.autograd.Function):
         return dq[:, :sq, :, :head_dim], dk[:, :skv, :, :head_dim], dv[:, :skv, :, :head_dim], None, None
 
 
-def _padded_packing(cu: Tensor, rows: int) -> Tuple[Tensor, Tensor, int]:
+def _padded_packing(cu: Tensor, rows: int) -> Tuple[Tensor, Tensor, Tensor, int]:
     """A packing of the same sequences with every sequence padded to a multiple of 128 rows, from
     device arithmetic only (no copy to the host): (padded cumulative lengths [sequences + 1] int32,
-    padded row of every packed row [rows] int64, row count of the padded packing).  The row count
-    is an upper bound the host can know: rows + 127 per sequence, rounded up to 128."""
+    padded row of every packed row [rows] int64, which packed rows belong to a sequence [rows]
+    bool, row count of the padded packing).  The row count is an upper bound the host can know:
+    rows + 127 per sequence, rounded up to 128."""
     num_seqs = cu.numel() - 1
     cu = cu.to(torch.int32)
     padded_len = (cu[1:] - cu[:-1] + 127) // 128 * 128
     padded_cu = torch.cat([cu.new_zeros(1), torch.cumsum(padded_len, 0).to(torch.int32)])
     row = torch.arange(rows, device=cu.device, dtype=torch.int32)
-    # the sequence of a packed row (empty sequences own no row; rows past the last sequence, which a
-    # consistent caller does not have, count to the last one and stay inside the bound)
+    # the sequence of a packed row (empty sequences own no row; rows past the last sequence belong
+    # to none: they count to the last one, which keeps them inside the bound, and their gradients
+    # are set to zero afterwards)
     seq = torch.searchsorted(cu[1:].contiguous(), row, right=True).clamp_(max=num_seqs - 1)
     dest = (padded_cu[seq] + (row - cu[seq])).long()
-    return padded_cu, dest, -(-(rows + 127 * num_seqs) // 128) * 128
+    return padded_cu, dest, row < cu[-1], -(-(rows + 127 * num_seqs) // 128) * 128
+
+
+def _from_padded_packing(x: Tensor, dest: Tensor, owned: Tensor) -> Tensor:
+    """The rows of the packed layout back from the padded packing; rows of no sequence are zero."""
+    rows = x.index_select(1, dest)
+    return torch.where(owned.view(1, -1, *([1] * (x.dim() - 2))), rows, torch.zeros_like(rows))
 
 
 def _to_padded_packing(x: Tensor, dest: Tensor, padded_rows: int) -> Tensor:
@@ -185,8 +193,8 @@ class AmdFmhaVarlenFunction(torch.autograd.Function):
             # no sequence has both queries and keys: the output does not depend on the operands
             return (torch.zeros_like(query), torch.zeros_like(key), torch.zeros_like(value)) + (None,) * 6
         delta = torch_ops.compute_delta(o, do)
-        pcu_q, dest_q, rows_q = _padded_packing(cu_q, q.shape[1])
-        pcu_kv, dest_kv, rows_kv = _padded_packing(cu_kv, k.shape[1])
+        pcu_q, dest_q, owned_q, rows_q = _padded_packing(cu_q, q.shape[1])
+        pcu_kv, dest_kv, owned_kv, rows_kv = _padded_packing(cu_kv, k.shape[1])
         dq, dk, dv = torch_ops.attention_backward_varlen(
             _to_padded_packing(q, dest_q, rows_q), _to_padded_packing(k, dest_kv, rows_kv),
             _to_padded_packing(v, dest_kv, rows_kv), _to_padded_packing(do, dest_q, rows_q),
@@ -194,5 +202,6 @@ class AmdFmhaVarlenFunction(torch.autograd.Function):
             cu_q.to(torch.int32).contiguous(), cu_kv.to(torch.int32).contiguous(), pcu_q, pcu_kv, max_q, max_kv,
             is_causal, scale,
         )
-        dq, dk, dv = dq.index_select(1, dest_q), dk.index_select(1, dest_kv), dv.index_select(1, dest_kv)
+        dq = _from_padded_packing(dq, dest_q, owned_q)
+        dk, dv = _from_padded_packing(dk, dest_kv, owned_kv), _from_padded_packing(dv, dest_kv, owned_kv)
         return (dq[..., :head_dim], dk[..., :head_dim], dv[..., :head_dim]) + (None,) * 6

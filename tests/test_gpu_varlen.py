@@ -168,3 +168,17 @@ def test_varlen_backward_equals_per_sequence_calls(head_dim, dtype):
             assert torch.equal(vp.grad[:, okv : okv + lkv], vs.grad), (lq, lkv, causal)
             oq += lq
             okv += lkv
+
+
+def test_gradients_of_rows_outside_every_sequence_are_zero():
+    # cumulative lengths that stop short of the packed tensors, forward and backward
+    q, k, v = (_rand((1, 100, 2, 64), torch.bfloat16, s).requires_grad_(True) for s in (1, 2, 3))
+    d_out = _rand((1, 100, 2, 64), torch.bfloat16, 4)
+    cu = torch.tensor([0, 30, 80], dtype=torch.int32, device="cuda")
+    natten_amd.attention(q, k, v, cumulative_seqlen_Q=cu, cumulative_seqlen_KV=cu, max_seqlen_Q=50,
+                         max_seqlen_KV=50).backward(d_out)
+    for t in (q, k, v):
+        assert torch.isfinite(t.grad).all() and torch.count_nonzero(t.grad[:, 80:]) == 0
+    ref = O.attention_backward(to_np(q[:, 30:80]), to_np(k[:, 30:80]), to_np(v[:, 30:80]), to_np(d_out[:, 30:80]))
+    for name, t, r in zip(("dq", "dk", "dv"), (q, k, v), ref):
+        assert_close(name, to_np(t.grad[:, 30:80]), r, atol=2e-2, rtol=2e-2)
