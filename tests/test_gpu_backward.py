@@ -231,3 +231,33 @@ def test_layer_trains():
     for name, prm in layer.named_parameters():
         assert prm.grad is not None and torch.isfinite(prm.grad).all(), name
         assert prm.grad.abs().max() > 0, name
+
+
+def _pairs(B, H, shape, k):
+    n = 1
+    for x in shape:
+        n *= x
+    w = 1
+    for x in k:
+        w *= x
+    return B * H * n * w
+
+
+@pytest.mark.parametrize("na_dim", [1, 2, 3])
+def test_reference_problem_lists_backward(na_dim):
+    # the hand-picked problems of the reference's test-suite (tests/problems.py), forward + backward
+    # as tests/test_blackwell_fna.py runs them, each non-causal and causal along its first
+    # dimension; the largest ones (more than 6e7 query-key pairs for the float64 oracle) are
+    # left to the sampled checks of tests/test_gpu_configs.py
+    from tests import problems
+
+    cases = {1: problems.NA_1D, 2: problems.NA_2D, 3: problems.NA_3D}[na_dim]
+    ran = 0
+    for i, (B, H, Hkv, D, shape, k, s, d) in enumerate(cases):
+        if _pairs(B, H, shape, k) > 6e7:
+            continue
+        dtype = torch.bfloat16 if i % 2 == 0 else torch.float16
+        for causal in ((False,) * na_dim, (True,) + (False,) * (na_dim - 1)):
+            run_backward(B, H, Hkv, D, shape, k, s, d, causal, dtype, seed=100 + i)
+            ran += 1
+    assert ran >= 16
