@@ -74,3 +74,39 @@ def test_training_step_replays_from_a_graph(shape, kernel, causal, head_dim):
         torch.cuda.synchronize()
         for name, a, b in zip("qkv", (q, k, v), eager):
             assert torch.equal(a.grad, b.grad), f"replay {i}: d{name} differs from the eager step"
+
+
+def test_varlen_training_step_replays_from_a_graph():
+    # sequence-packed attention: the backward builds its padded packing with device index
+    # arithmetic (cumsum, searchsorted, index_copy_), all of which must replay correctly
+    gen = torch.Generator().manual_seed(2)
+    mk = lambda: torch.randn((1, 300, 2, 64), generator=gen).to(torch.bfloat16).cuda()
+    q, k, v = (mk().requires_grad_(True) for _ in range(3))
+    d_out = mk()
+    cu = torch.tensor([0, 40, 170, 300], dtype=torch.int32, device="cuda")
+
+    def step(a, b, c):
+        natten_amd.attention(a, b, c, is_causal=True, cumulative_seqlen_Q=cu, cumulative_seqlen_KV=cu,
+                             max_seqlen_Q=130, max_seqlen_KV=130).backward(d_out)
+
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            step(q, k, v)
+    torch.cuda.current_stream().wait_stream(side)
+    for t in (q, k, v):
+        t.grad = None
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step(q, k, v)
+    for i in range(3):
+        with torch.no_grad():
+            for t in (q, k, v, d_out):
+                t.copy_(mk())
+        graph.replay()
+        torch.cuda.synchronize()
+        eager = [t.detach().clone().requires_grad_(True) for t in (q, k, v)]
+        step(*eager)
+        torch.cuda.synchronize()
+        for name, a, b in zip("qkv", (q, k, v), eager):
+            assert torch.equal(a.grad, b.grad), f"replay {i}: d{name} differs from the eager step"
