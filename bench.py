@@ -290,16 +290,17 @@ def main():
     else:
         q, k, v = (x.to(dtype) for x in (q, k, v))
     na = {1: natten_amd.na1d, 2: natten_amd.na2d, 3: natten_amd.na3d}[n]
-    q_tile = tuple(int(x) for x in args.q_tile.split(",")) if args.q_tile else None
-    kv_tile = tuple(int(x) for x in args.kv_tile.split(",")) if args.kv_tile else None
-    q_tile, kv_tile = check_fna_forward_config(q, kernel, stride, dilation, causal, q_tile, kv_tile)
-
     if args.backward:
+        # --q-tile / --kv-tile then name the backward tiles; the forward of the step uses its defaults
         if quantised:
             print("bench.py: there is no backward pass for 8-bit float operands.", file=sys.stderr)
             sys.exit(2)
         bench_backward(args, q, k, v, kernel, stride, dilation, causal, dt_name)
         return
+
+    q_tile = tuple(int(x) for x in args.q_tile.split(",")) if args.q_tile else None
+    kv_tile = tuple(int(x) for x in args.kv_tile.split(",")) if args.kv_tile else None
+    q_tile, kv_tile = check_fna_forward_config(q, kernel, stride, dilation, causal, q_tile, kv_tile)
 
     def step():
         if quantised:
