@@ -6,8 +6,11 @@ One step = one na3d/na2d forward through the public API on inputs already reside
 a single launch that gathers its tiles from the original tensors when the problem allows it
 (all benchmark workloads do), else token permute of Q/K/V, kernel, unpermute of O and LSE.  Prints ONE JSON line: whole-path throughput in effective
 NA TFLOP/s (4 * B * H * D * sum_q |window(q)| per step), the fused kernel's roofline figures from
-HIP-event timing of kernel-only launches, and a CPU baseline (the C oracle on a bounded sample
-of the same workload's queries, timed on this box's host cores).
+HIP events over the timed steps, and a CPU baseline: the PyTorch call the reference's CPU path makes
+(flex_attention with the neighborhood block mask, oracle/flex_cpu.py) timed on this box's host
+cores, on the workload itself where the dense N x N mask fits in memory and on a labelled cropped
+proxy where it does not; the C oracle's rate on a sample of the workload's queries is reported
+beside it (and checks the GPU result on that sample).
 """
 
 from __future__ import annotations
@@ -33,18 +36,68 @@ WORKLOADS = {
     "c2d": (2, 8, (64, 64), 64, (13, 13), (1, 1), (2, 2), (False, False), "bf16", 1.0),
     # e4m3 operands with per-head absmax scales, bf16 output; multiplied by the 8-bit matrix instruction
     "c5": (1, 16, (16, 64, 64), 128, (8, 16, 16), (4, 8, 8), (1, 2, 2), (False, False, False), "e4m3", 1.0),
+    # the shapes the reference publishes runtimes for (docs/profiler.md:853-876, :925-951, :654-755; fp16, batch 1)
+    "hunyuan_na": (1, 24, (30, 48, 80), 128, (18, 24, 24), (1, 1, 1), (1, 1, 1), (False, False, False), "fp16", 1.0),
+    "hunyuan_gna": (1, 24, (30, 48, 80), 128, (18, 24, 24), (16, 8, 8), (1, 1, 1), (False, False, False), "fp16", 1.0),
+    "flux_na": (1, 24, (256, 256), 128, (80, 80), (1, 1), (1, 1), (False, False), "fp16", 1.0),
+    "flux_gna": (1, 24, (256, 256), 128, (80, 80), (16, 16), (1, 1), (False, False), "fp16", 1.0),
 }
-# HBM-side traffic of one fused-kernel launch, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# and calibrated on the permute kernel (a copy of known size); the summary of that run is kept with the profiles.
-# Keyed by (workload, q_tile_shape, kv_tile_shape); other combinations report null.
-MEASURED_TRAFFIC_BYTES = {
-    ("c4", (2, 8, 8), (1, 8, 8)): 2.82e10,
+# Published forward runtimes of the reference's Blackwell FNA kernel on a B200 for those shapes
+# (kernel only / with token permute; docs/sample-outputs/profiler-*-blackwell-fna-b200.txt): other
+# hardware, context only, never a baseline for `vs_baseline`.
+REFERENCE_B200_MS = {
+    "hunyuan_na": (42.243, 47.353),
+    "hunyuan_gna": (13.010, 18.538),
+    "flux_na": (8.692, 10.931),
+    "flux_gna": (4.114, 6.389),
 }
-# The same for the two backward launches together (dQ role 20.3 GB read + 0.7 GB written, paired
-# dK / dV role 63.7 GB + 1.9 GB), keyed by (workload, backward q tile, backward kv tile).
-MEASURED_BACKWARD_TRAFFIC_BYTES = {
-    ("c4", (2, 8, 8), (2, 8, 8)): 8.66e10,
+# Cropped proxies for the CPU baseline where the reference's CPU path (dense N x N mask and scores)
+# does not fit in memory: same kernel / stride / dilation / causal / head dim on a smaller layout
+# and fewer heads.  name -> (layout, heads); workloads not listed run as they are (c3: one head at a time).
+CPU_PROXY = {
+    "c4": ((20, 24, 24), 2),
+    "c5": ((8, 32, 32), 2),
+    "hunyuan_na": ((20, 24, 24), 2),
+    "hunyuan_gna": ((20, 24, 24), 2),
+    "flux_na": ((96, 96), 2),
+    "flux_gna": ((96, 96), 2),
 }
+# HBM-side traffic of a launch (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, calibrated on a copy of known
+# size) is read from the profile summaries, which carry one line per measurement:
+#   traffic: workload=c4 pass=forward q_tile=2,8,8 kv_tile=1,8,8 bytes=2.82e10 kernel_digest=<hex>
+# and is reported only while `kernel_digest` equals the digest of the kernel sources this run uses;
+# after any change to those sources the bench prints null until the counters are collected again.
+KERNEL_SOURCES = ["fna_fwd.hpp", "fna_fwd_fp8.hpp", "fna_bwd.hpp", "na_math.hpp", "natten_amd.hip"]
+
+
+def kernel_digest():
+    import hashlib
+
+    h = hashlib.sha256()
+    for name in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, "natten_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic(workload, which, q_tile, kv_tile):
+    """Bytes per launch from profiles/*.md for this workload, pass and tiles, or None when no
+    measurement of the current kernel sources is on file."""
+    import glob
+    import re
+
+    want = {"workload": workload, "pass": which, "q_tile": ",".join(map(str, q_tile)),
+            "kv_tile": ",".join(map(str, kv_tile)), "kernel_digest": kernel_digest()}
+    for path in sorted(glob.glob(os.path.join(ROOT, "profiles", "*.md"))):
+        with open(path) as f:
+            for line in f:
+                if not line.lstrip().startswith("traffic:"):
+                    continue
+                kv = dict(re.findall(r"(\w+)=(\S+)", line))
+                if all(kv.get(key) == val for key, val in want.items()) and "bytes" in kv:
+                    return {"bytes": float(kv["bytes"]), "source": os.path.relpath(path, ROOT)}
+    return None
+
 
 WORKLOAD_NAMES = {
     "c4": "na3d bf16 B=1 H=24 30x48x80 D=128 k=(18,24,24) s=(1,8,8) causal=(T,F,F) +LSE",
@@ -52,6 +105,10 @@ WORKLOAD_NAMES = {
     "c2": "na2d bf16 B=2 H=8 64x64 D=64 k=(13,13)",
     "c2d": "na2d bf16 B=2 H=8 64x64 D=64 k=(13,13) d=(2,2)",
     "c5": "na3d e4m3 (per-head scales, bf16 out) B=1 H=16 16x64x64 D=128 k=(8,16,16) s=(4,8,8) d=(1,2,2)",
+    "hunyuan_na": "na3d fp16 B=1 H=24 30x48x80 D=128 k=(18,24,24)",
+    "hunyuan_gna": "na3d fp16 B=1 H=24 30x48x80 D=128 k=(18,24,24) s=(16,8,8)",
+    "flux_na": "na2d fp16 B=1 H=24 256x256 D=128 k=(80,80)",
+    "flux_gna": "na2d fp16 B=1 H=24 256x256 D=128 k=(80,80) s=(16,16)",
 }
 
 
@@ -74,8 +131,9 @@ def count_attended(layout, k, s, d, c):
     return total
 
 
-def cpu_baseline(q, k, v, kernel, stride, dilation, causal, out_gpu, lse_gpu, seconds_target=15.0, tol=1e-2):
-    """C oracle on a bounded sample of this workload's queries, all heads, host cores."""
+def c_oracle_sample(q, k, v, kernel, stride, dilation, causal, out_gpu, lse_gpu, seconds_target=6.0, tol=1e-2):
+    """C oracle on a bounded sample of this workload's queries (all heads) on the host cores: its
+    rate, and the GPU result checked against it on that sample."""
     import numpy as np
 
     from oracle import c_oracle
@@ -112,9 +170,83 @@ def cpu_baseline(q, k, v, kernel, stride, dilation, causal, out_gpu, lse_gpu, se
         "unit": "TFLOP/s",
         "cores": threads,
         "kind": "port",
-        "sample": f"C oracle (float64), {nq} random queries x {H} heads of this workload, {dt:.1f} s wall",
-        "parity_on_sample": {"ok": ok, "max_abs_err_out": err_o, "max_abs_err_lse": err_l, "atol_rtol": tol},
+        "sample": f"C oracle (float64 window walk), {nq} random queries x {H} heads of this workload, {dt:.1f} s wall",
+        "gpu_parity_on_sample": {"ok": ok, "max_abs_err_out": err_o, "max_abs_err_lse": err_l, "atol_rtol": tol},
     }
+
+
+def cpu_baseline(workload, q, k, v, kernel, stride, dilation, causal, dt_name, std, timed_runs=2):
+    """The reference's CPU path, timed on this box's host cores: torch.nn.attention.flex_attention
+    with the neighborhood block mask on CPU tensors (the one PyTorch call `flex_fna_generic` makes
+    without tile shapes, src/natten/backends/flex.py:126-137, :538-547; restated in
+    oracle/flex_cpu.py).  Eager flex on the CPU materialises N x N masks and scores: the workload
+    runs as it is when that fits, one head at a time when only that fits, and otherwise the call is
+    reported as not fitting and a cropped proxy (same window parameters, smaller layout, two heads)
+    is timed instead, labelled as such, and checked against the C oracle."""
+    import warnings
+
+    import numpy as np
+    import torch
+
+    from oracle import c_oracle
+    from oracle.flex_cpu import flex_na_cpu
+
+    B, H, D = q.shape[0], q.shape[-2], q.shape[-1]
+    n = q.dim() - 3
+    layout = tuple(int(x) for x in q.shape[1 : 1 + n])
+    N = int(np.prod(layout))
+    cpu_dtype = {"bf16": torch.bfloat16, "fp16": torch.float16, "e4m3": torch.bfloat16}[dt_name]
+    info = {"unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+            "call": "torch.nn.attention.flex_attention + create_block_mask(BLOCK_SIZE=(64, 64), device='cpu') on "
+                    "[B, H, N, D] CPU tensors, return_lse=True, FORCE_USE_FLEX_ATTENTION: the call of the reference's "
+                    "CPU path (flex-fna backend), with its mask_mod restated",
+            "os_cpu_count": os.cpu_count(), "torch_num_threads": torch.get_num_threads()}
+    proxy = CPU_PROXY.get(workload)
+    if proxy is not None:
+        p_layout, p_heads = proxy
+        info["fits"] = False
+        info["reason"] = (f"N = {N} tokens: the dense N x N boolean mask alone is {N * N / 1e9:.1f} GB and the float32 "
+                          f"scores {4.0 * N * N / 1e9:.1f} GB per head")
+        gen = torch.Generator().manual_seed(0)
+        cq, ck, cv = ((torch.randn((1, *p_layout, p_heads, D), generator=gen) * std).to(cpu_dtype) for _ in range(3))
+        heads_timed, layout_timed = p_heads, p_layout
+        sample = (f"cropped proxy: same kernel_size / stride / dilation / is_causal / head_dim on "
+                  f"{'x'.join(map(str, p_layout))}, B=1, H={p_heads}, {cpu_dtype}".replace("torch.", ""))
+    else:
+        info["fits"] = True
+        per_head = N > 8192  # float32 scores of all heads at once would not fit: one head per call
+        cq, ck, cv = (t[:1].to("cpu", cpu_dtype) for t in (q, k, v)) if per_head else (t.to("cpu", cpu_dtype) for t in (q, k, v))
+        if per_head:
+            cq, ck, cv = (t[..., :1, :].contiguous() for t in (cq, ck, cv))
+        heads_timed, layout_timed = cq.shape[-2], layout
+        sample = ("the workload itself" if not per_head else
+                  f"the workload one head at a time: 1 of {B * H} (batch, head) pairs timed")
+    attended = count_attended(layout_timed, kernel, stride, dilation, causal)
+    flops = 4.0 * cq.shape[0] * heads_timed * D * attended
+    times = []
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        with torch.no_grad():
+            for i in range(1 + timed_runs):  # first run untimed: warm-up
+                t0 = time.perf_counter()
+                ref_out, ref_lse = flex_na_cpu(cq, ck, cv, kernel, stride, dilation, causal)
+                if i:
+                    times.append(time.perf_counter() - t0)
+    med = float(np.median(times))
+    info["value"] = flops / med / 1e12
+    info["seconds_per_call"] = med
+    info["sample"] = f"{sample}; 1 warm-up + {timed_runs} timed calls, median"
+    # the flex result against the C oracle on the same inputs (rows of the first head pair)
+    rng = np.random.default_rng(1)
+    Np = int(np.prod(layout_timed))
+    tok = rng.integers(0, Np, size=64)
+    o_ref, l_ref, _ = c_oracle.na_rows(cq.float().numpy(), ck.float().numpy(), cv.float().numpy(), kernel, stride,
+                                       dilation, causal, None, np.zeros(64, dtype=np.int32), tok, 8)
+    got_o = ref_out.reshape(cq.shape[0], Np, heads_timed, D)[0, torch_idx(tok)].float().numpy()
+    got_l = ref_lse.reshape(cq.shape[0], Np, heads_timed)[0, torch_idx(tok)].float().numpy()
+    info["flex_vs_c_oracle"] = {"max_abs_err_out": float(np.abs(got_o - o_ref).max()),
+                                "max_abs_err_lse": float(np.abs(got_l - l_ref).max())}
+    return info
 
 
 def torch_idx(a):
@@ -236,7 +368,8 @@ def bench_backward(args, q, k, v, kernel, stride, dilation, causal, dt_name):
             "peak": peak,
             "unit": "TFLOP/s",
             "frac": achieved / peak,
-            "traffic": MEASURED_BACKWARD_TRAFFIC_BYTES.get((args.workload, tuple(q_tile), tuple(kv_tile))),
+            "traffic": (measured_traffic(args.workload, "backward", q_tile, kv_tile) or {}).get("bytes"),
+            "kernel_digest": kernel_digest(),
             "algorithmic_flop": 2.5 * fwd_flops,
         },
         "cpu_baseline": None,
@@ -309,16 +442,24 @@ def main():
         return na(q, k, v, kernel, stride, dilation, causal, q_tile_shape=q_tile, kv_tile_shape=kv_tile,
                   return_lse=True)
 
+    # One loop gives both figures: the host clock around the K steps (bracketed by synchronisation)
+    # and HIP events recorded on the launch stream (torch's current stream) before the first and
+    # after the last of the same K steps.
+    ev0 = torch.cuda.Event(enable_timing=True)
+    ev1 = torch.cuda.Event(enable_timing=True)
     with torch.no_grad():
         for _ in range(args.warmup):
             out, lse = step()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
+        ev0.record()
         for _ in range(args.steps):
             out, lse = step()
+        ev1.record()
         torch.cuda.synchronize()
         t1 = time.perf_counter()
     ms_per_step = (t1 - t0) * 1e3 / args.steps
+    step_events_ms = ev0.elapsed_time(ev1) / args.steps
     flops = 4.0 * B * H * D * count_attended(layout, kernel, stride, dilation, causal)
     tflops_e2e = flops / (ms_per_step * 1e-3) / 1e12
 
@@ -368,7 +509,10 @@ def main():
             torch.cuda.synchronize()
             return e0.elapsed_time(e1) / iters
 
-        kernel_ms = timed(kern, args.steps)
+        # the step is this one launch when the one-launch route applies: its duration is then the
+        # event time of the timed steps themselves; otherwise the kernel is timed on its own
+        kernel_ms = step_events_ms if fused else timed(kern, args.steps)
+        kernel_alone_ms = timed(kern, args.steps)
         kernel_permuted_ms = timed(kern_permuted, args.steps)
         op, lp = kern_permuted()
         perm_ms = timed(lambda: token_permute_operation(tp_in, q_tile, dilation), args.steps)
@@ -378,6 +522,7 @@ def main():
     peak = PEAK_TFLOPS[dt_name]
     dense_flops = 4.0 * B * H * D * float(q.numel() // (B * H * D)) ** 2
 
+    traffic = measured_traffic(args.workload, "forward", q_tile, kv_tile) if fused else None
     result = {
         "metric": "FNA fwd ms + effective TFLOP/s (% MFMA peak), na3d bf16 D=128, 1 GPU",
         "value": tflops_e2e,
@@ -401,7 +546,11 @@ def main():
         "na_flop_per_step": flops,
         "dense_over_na_flop": dense_flops / flops,
         "kernel_ms": kernel_ms,
+        "kernel_ms_source": ("HIP events around the timed steps (one launch per step)" if fused else
+                             "HIP events around kernel-only launches"),
+        "kernel_direct_call_ms": kernel_alone_ms,
         "kernel_on_permuted_operands_ms": kernel_permuted_ms,
+        "e2e_permuted_route_ms": 3 * perm_ms + kernel_permuted_ms + unperm_ms,
         "token_permute": {
             "permute_q_ms": perm_ms,
             "unpermute_o_ms": unperm_ms,
@@ -415,7 +564,9 @@ def main():
             "peak": peak,
             "unit": "TFLOP/s",
             "frac": achieved / peak,
-            "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, tuple(q_tile), tuple(kv_tile))),
+            "traffic": traffic["bytes"] if traffic else None,
+            "traffic_source": traffic["source"] if traffic else None,
+            "kernel_digest": kernel_digest(),
             "algorithmic_bytes": (4 * q.numel() * (1 if quantised else q.element_size())
                                   + (q.numel() if quantised else 0) + lse.numel() * 4),
         },
@@ -433,8 +584,14 @@ def main():
     if not args.no_cpu_baseline:
         # 16-bit operands: atol = rtol = 1e-2; 8-bit matrix path (P rounded to e4m3, relative error
         # up to 2^-4 per probability): atol = rtol = 2^-4
-        result["cpu_baseline"] = cpu_baseline(q, k, v, kernel, stride, dilation, causal, out, lse,
-                                              tol=2.0**-4 if quantised else 1e-2)
+        result["cpu_baseline"] = cpu_baseline(args.workload, q, k, v, kernel, stride, dilation, causal, dt_name, std)
+        result["cpu_baseline"]["c_oracle"] = c_oracle_sample(q, k, v, kernel, stride, dilation, causal, out, lse,
+                                                             tol=2.0**-4 if quantised else 1e-2)
+    if args.workload in REFERENCE_B200_MS:
+        ref_k, ref_e2e = REFERENCE_B200_MS[args.workload]
+        result["reference_published_b200"] = {
+            "kernel_ms": ref_k, "with_token_permute_ms": ref_e2e,
+            "note": "the reference's Blackwell FNA kernel on an NVIDIA B200 (its docs/profiler.md): other hardware, context only"}
     print(json.dumps(result), flush=True)
 
 

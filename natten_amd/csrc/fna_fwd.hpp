@@ -64,6 +64,7 @@ struct FnaParams {
   // key rows cu_kv[b] .. cu_kv[b+1]-1; q_tiled[0] then counts the Q tiles of the longest one.
   const int32_t* cu_q;   // [batch + 1]
   const int32_t* cu_kv;  // [batch + 1]
+  int total_q, total_kv;  // rows of the packed operands: offsets that do not fit them are not followed
 };
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
@@ -314,6 +315,9 @@ fna_fwd_kernel(const FnaParams p) {
       const int q0 = p.cu_q[bg], kv0 = p.cu_kv[bg];
       seqlen_q = p.cu_q[bg + 1] - q0;
       seqlen_kv = p.cu_kv[bg + 1] - kv0;
+      // a malformed cumulative array (negative, decreasing, past the end) must not become an address
+      if (q0 < 0 || kv0 < 0 || seqlen_q < 0 || seqlen_kv < 0 || q0 > p.total_q - seqlen_q || kv0 > p.total_kv - seqlen_kv)
+        return;
       q_seq_row0 = q0;
       kv_seq_row0 = kv0;
       ksz[0] = seqlen_kv;

@@ -413,6 +413,8 @@ int natten_amd_attention_forward_varlen(const void* q, const void* k, const void
   p.v_scale = v_scale;
   p.cu_q = cumulative_seqlen_q;
   p.cu_kv = cumulative_seqlen_kv;
+  p.total_q = total_seqlen_q;
+  p.total_kv = total_seqlen_kv;
   set_wg_layout(p, 1);
   return dispatch_dtype(p, dtype, head_dim, QT, KVT, static_cast<hipStream_t>(stream));
 }

@@ -151,8 +151,16 @@ def neighborhood_attention_generic(
 
     scale = scale or query.shape[-1] ** -0.5
     final_dtype = out_dtype or query.dtype
-    # 8-bit float operands: partial results stay in bf16 until after the merge
-    work_dtype = torch.bfloat16 if is_fp8(query.dtype) else final_dtype
+    # Partial results before a merge: bf16 for 8-bit float operands; the operands' own type when
+    # gradients are wanted (the merge's backward writes the merged output and LSE into the very
+    # tensors the partial attentions saved, so those must reach it uncast); else the final type.
+    needs_grad = torch.is_grad_enabled() and any(
+        t is not None and t.requires_grad for t in (query, key, value, additional_keys, additional_values)
+    )
+    if is_fp8(query.dtype):
+        work_dtype = torch.bfloat16
+    else:
+        work_dtype = query.dtype if needs_grad else final_dtype
     output, lse = amd_fna_generic(
         query, key, value, kernel_size=kernel_size, stride=stride, dilation=dilation, is_causal=is_causal,
         scale=scale, q_tile_shape=q_tile_shape, kv_tile_shape=kv_tile_shape, return_lse=True,

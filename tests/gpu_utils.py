@@ -48,3 +48,55 @@ def assert_close(name, got, ref, atol=ATOL, rtol=RTOL):
 
 def tuplify(x, n):
     return tuple([x] * n) if isinstance(x, (int, bool)) else tuple(x)
+
+
+def stratified_tokens(shape, kernel_size, stride, dilation, is_causal, n_samples, rng):
+    """Row-major token indices of `n_samples` query positions chosen to hit every class of window:
+    all corners; per dimension the first and last `kernel_size * dilation` coordinates (clamped
+    windows of every dilation group at both borders), the first and last coordinates of a causal
+    dimension, the coordinates either side of a stride-group boundary; the rest uniform."""
+    n = len(shape)
+    edge = []
+    for X, k, s, d, c in zip(shape, kernel_size, stride, dilation, is_causal):
+        w = min(X, k * d)
+        e = set(range(w)) | set(range(X - w, X))
+        step = s * d
+        for b in range(step, X, step):  # last query of a stride group and the first of the next
+            e.update(x for x in range(b - d, b + d) if 0 <= x < X)
+        edge.append(np.array(sorted(e)))
+    coords = [np.array(c) for c in itertools.product(*[(0, X - 1) for X in shape])]
+    while len(coords) < n_samples:
+        kind = len(coords) % 3
+        c = np.empty(n, dtype=np.int64)
+        for a in range(n):
+            use_edge = kind == 0 or (kind == 1 and rng.integers(0, 2) == 0)
+            c[a] = rng.choice(edge[a]) if use_edge else rng.integers(0, shape[a])
+        coords.append(c)
+    coords = np.stack(coords[:max(n_samples, 1)])
+    return np.ravel_multi_index(tuple(coords.T), shape)
+
+
+def sampled_check(q, k, v, out, lse, kernel, stride, dilation, causal, n_samples, seed, batches=None,
+                  atol=ATOL, rtol=RTOL, scale=None, tag=""):
+    """Checks `out`, `lse` at a stratified sample of query positions (all heads of each) against the
+    C oracle.  `batches`: the batch entries to draw from (each is handed to the oracle on its own,
+    so that a many-gigabyte batch never has to exist as float32 on the host)."""
+    B = q.shape[0]
+    n = q.dim() - 3
+    shape = tuple(q.shape[1 : 1 + n])
+    N = int(np.prod(shape))
+    H, D = q.shape[-2], q.shape[-1]
+    kernel, stride, dilation, causal = (tuplify(x, n) for x in (kernel, stride, dilation, causal))
+    rng = np.random.default_rng(seed)
+    batches = list(range(B)) if batches is None else list(batches)
+    per = -(-n_samples // len(batches))
+    for b in batches:
+        tok = stratified_tokens(shape, kernel, stride, dilation, causal, per, rng)
+        bat = np.zeros(len(tok), dtype=np.int32)
+        ref_o, ref_l, _ = c_oracle.na_rows(to_np(q[b : b + 1]), to_np(k[b : b + 1]), to_np(v[b : b + 1]), kernel,
+                                           stride, dilation, causal, scale, bat, tok, threads=16)
+        ti = torch.as_tensor(tok, device=out.device)
+        got_o = to_np(out[b].reshape(N, H, out.shape[-1])[ti])
+        got_l = to_np(lse[b].reshape(N, H)[ti])
+        assert_close(f"sampled out {tag} batch {b}", got_o, ref_o, atol, rtol)
+        assert_close(f"sampled lse {tag} batch {b}", got_l, ref_l, atol, rtol)

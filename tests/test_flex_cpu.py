@@ -1,0 +1,133 @@
+"""CPU checks of the reference-CPU-path restatement (oracle/flex_cpu.py) and of the two small
+copies of the window arithmetic outside the oracle (the tile chooser's and the benchmark's FLOP count).
+
+The mask predicate handed to flex_attention follows the centre-clamp form of the reference's
+src/natten/backends/flex.py:333-407; the oracle's mask follows the start / end form of
+csrc/include/natten/cuda/reference/mask.hpp:59-91.  They must agree on every (query, key) pair."""
+
+import itertools
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import na_oracle as O
+from oracle.flex_cpu import flex_na_cpu, na_mask_mod
+
+CASES = [
+    ((23,), (5,), (2,), (1,), (False,)),
+    ((23,), (6,), (3,), (2,), (True,)),
+    ((40,), (7,), (7,), (3,), (False,)),
+    ((9, 11), (3, 4), (1, 2), (2, 1), (False, True)),
+    ((12, 10), (5, 5), (5, 2), (1, 2), (True, False)),
+    ((7, 8, 9), (3, 2, 4), (2, 1, 3), (1, 2, 2), (True, False, False)),
+    ((6, 6, 10), (6, 3, 5), (1, 3, 4), (1, 1, 2), (False, True, True)),
+]
+
+
+@pytest.mark.parametrize("shape,kernel,stride,dilation,causal", CASES)
+def test_mask_mod_equals_oracle_mask(shape, kernel, stride, dilation, causal):
+    N = int(np.prod(shape))
+    mod = na_mask_mod(shape, kernel, stride, dilation, causal)
+    qi = torch.arange(N).view(N, 1).expand(N, N)
+    ki = torch.arange(N).view(1, N).expand(N, N)
+    got = mod(torch.zeros((), dtype=torch.int64), torch.zeros((), dtype=torch.int64), qi, ki).numpy()
+    ref = O.na_mask_dense(shape, kernel, stride, dilation, causal)
+    assert got.shape == ref.shape and np.array_equal(got, ref)
+
+
+def test_mask_mod_random_sweep():
+    rng = np.random.default_rng(7)
+    for _ in range(60):
+        n = int(rng.integers(1, 4))
+        shape = tuple(int(rng.integers(4, {1: 60, 2: 14, 3: 8}[n])) for _ in range(n))
+        k = tuple(int(rng.integers(2, x + 1)) for x in shape)
+        s = tuple(int(rng.integers(1, kk + 1)) for kk in k)
+        d = tuple(int(rng.integers(1, x // kk + 1)) for x, kk in zip(shape, k))
+        c = tuple(bool(rng.integers(0, 2)) for _ in range(n))
+        N = int(np.prod(shape))
+        mod = na_mask_mod(shape, k, s, d, c)
+        qi = torch.arange(N).view(N, 1).expand(N, N)
+        ki = torch.arange(N).view(1, N).expand(N, N)
+        got = mod(None, None, qi, ki).numpy()
+        assert np.array_equal(got, O.na_mask_dense(shape, k, s, d, c)), (shape, k, s, d, c)
+
+
+def test_flex_call_matches_dense_oracle_config1():
+    # the first benchmark configuration as written: na1d fp32 on CPU, B=1, heads=2, L=256, D=32, k=7, seed 0
+    torch.manual_seed(0)
+    q, k, v = (torch.randn(1, 256, 2, 32) for _ in range(3))
+    out, lse = flex_na_cpu(q, k, v, (7,), (1,), (1,), (False,))
+    ref_o, ref_l = O.na_forward(q.numpy(), k.numpy(), v.numpy(), (7,), (1,), (1,), (False,))
+    assert np.abs(out.numpy() - ref_o).max() < 1e-4 and np.abs(lse.numpy() - ref_l).max() < 1e-4
+
+
+def test_flex_call_matches_dense_oracle_2d_gqa():
+    torch.manual_seed(1)
+    q = torch.randn(2, 10, 12, 4, 16)
+    k, v = torch.randn(2, 10, 12, 2, 16), torch.randn(2, 10, 12, 2, 16)
+    args = ((5, 4), (2, 3), (2, 1), (True, False))
+    out, lse = flex_na_cpu(q, k, v, *args)
+    ref_o, ref_l = O.na_forward(q.numpy(), k.numpy(), v.numpy(), *args)
+    assert np.abs(out.numpy() - ref_o).max() < 1e-4 and np.abs(lse.numpy() - ref_l).max() < 1e-4
+
+
+# ---- the window arithmetic outside the oracle ---------------------------------------------------------
+
+
+def test_tile_chooser_window_equals_oracle_exhaustively():
+    from natten_amd.tile_config import _win
+
+    for L in range(2, 34):
+        for k in range(2, L + 1):
+            for s in range(1, k + 1):
+                for causal in (False, True):
+                    for i in range(L):
+                        st = int(O.window_start(i, k, s, L, causal))
+                        en = int(O.window_end(i, st, k, L, causal))
+                        assert _win(i, k, s, L, causal) == (st, en), (L, k, s, causal, i)
+
+
+def test_benchmark_flop_count_equals_oracle():
+    import bench
+
+    for L in range(2, 28):
+        for k in range(2, L + 1):
+            for s in (1, 2, 3, k):
+                if s > k:
+                    continue
+                for d in range(1, L // k + 1):
+                    for causal in (False, True):
+                        assert bench.count_attended((L,), (k,), (s,), (d,), (causal,)) == \
+                            O.count_attended((L,), (k,), (s,), (d,), (causal,)), (L, k, s, d, causal)
+    rng = np.random.default_rng(3)
+    for _ in range(40):
+        n = int(rng.integers(2, 4))
+        shape = tuple(int(rng.integers(4, 12)) for _ in range(n))
+        k = tuple(int(rng.integers(2, x + 1)) for x in shape)
+        s = tuple(int(rng.integers(1, kk + 1)) for kk in k)
+        d = tuple(int(rng.integers(1, x // kk + 1)) for x, kk in zip(shape, k))
+        c = tuple(bool(rng.integers(0, 2)) for _ in range(n))
+        ref = int(O.na_mask_dense(shape, k, s, d, c).sum())
+        assert bench.count_attended(shape, k, s, d, c) == ref == O.count_attended(shape, k, s, d, c)
+    # the five benchmark configurations (FLOP = 4 B H D x this count)
+    for name, flop in (("c2", 2.8353e9), ("c3", 1.3744e11), ("c4", 1.0518e13), ("c5", 1.0995e12)):
+        B, H, layout, D, kernel, stride, dilation, causal, _, _ = bench.WORKLOADS[name]
+        got = 4.0 * B * H * D * bench.count_attended(layout, kernel, stride, dilation, causal)
+        assert abs(got - flop) / flop < 1e-3, (name, got)
+
+
+def test_traffic_is_only_reported_for_the_current_kernel_sources(tmp_path, monkeypatch):
+    import bench
+
+    digest = bench.kernel_digest()
+    prof = tmp_path / "profiles"
+    prof.mkdir()
+    (prof / "x.md").write_text(
+        f"traffic: workload=c4 pass=forward q_tile=2,8,8 kv_tile=1,8,8 bytes=1.5e10 kernel_digest={digest}\n"
+        "traffic: workload=c3 pass=forward q_tile=8,16 kv_tile=8,8 bytes=7e8 kernel_digest=0123456789abcdef\n")
+    monkeypatch.setattr(bench, "ROOT", str(tmp_path))
+    monkeypatch.setattr(bench, "kernel_digest", lambda: digest)
+    assert bench.measured_traffic("c4", "forward", (2, 8, 8), (1, 8, 8))["bytes"] == 1.5e10
+    assert bench.measured_traffic("c4", "forward", (4, 8, 8), (1, 8, 8)) is None
+    assert bench.measured_traffic("c3", "forward", (8, 16), (8, 8)) is None  # measured on other sources

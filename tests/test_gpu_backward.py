@@ -186,8 +186,9 @@ def test_backward_argument_errors():
         natten_amd.na2d(q8, q8, q8, 3)
 
 
+@pytest.mark.parametrize("out_dtype", [None, torch.float32])
 @pytest.mark.parametrize("na_dim,D", [(1, 64), (2, 48), (3, 128)])
-def test_backward_with_additional_keys_values(na_dim, D):
+def test_backward_with_additional_keys_values(na_dim, D, out_dtype):
     # the merge hands both partial attentions the merged output and LSE, so that their backward
     # passes add up to the backward of attention over the joint context (reference
     # src/natten/attn_merge.py:130-190); checked against the dense oracle on the concatenated keys
@@ -202,8 +203,11 @@ def test_backward_with_additional_keys_values(na_dim, D):
     d_out = torch.randn(q.shape, generator=gen).to(dtype).cuda()
     for t in (q, kk, v, ak, av):
         t.requires_grad_(True)
-    out = NA[na_dim](q, kk, v, ks, is_causal=causal, additional_keys=ak, additional_values=av)
-    out.backward(d_out)
+    # with an output type other than the operands' the partial results must still reach the merge
+    # uncast (the merge's backward writes into the tensors the partial attentions saved)
+    out = NA[na_dim](q, kk, v, ks, is_causal=causal, additional_keys=ak, additional_values=av, out_dtype=out_dtype)
+    assert out.dtype == (out_dtype or dtype)
+    out.backward(d_out.to(out.dtype))
     N = int(np.prod(shape))
     B, H = q.shape[0], q.shape[-2]
     mask = np.concatenate([O.na_mask_dense(shape, ks, 1, 1, causal), np.ones((N, 37), dtype=bool)], axis=1)

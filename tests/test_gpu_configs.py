@@ -12,28 +12,9 @@ import torch
 
 import natten_amd
 from oracle import c_oracle
-from tests.gpu_utils import assert_close, make_qkv, oracle_full, to_np
+from tests.gpu_utils import assert_close, make_qkv, oracle_full, sampled_check, to_np
 
 pytestmark = pytest.mark.gpu
-
-
-def _sampled_check(q, k, v, out, lse, kernel, stride, dilation, causal, n_samples, seed):
-    B = q.shape[0]
-    n = q.dim() - 3
-    N = int(np.prod(q.shape[1 : 1 + n]))
-    H, D = q.shape[-2], q.shape[-1]
-    rng = np.random.default_rng(seed)
-    tok = rng.integers(0, N, size=n_samples)
-    # always include the corners, where windows are clamped
-    tok[:2] = (0, N - 1)
-    bat = rng.integers(0, B, size=n_samples)
-    ref_o, ref_l, _ = c_oracle.na_rows(to_np(q), to_np(k), to_np(v), kernel, stride, dilation, causal, None, bat, tok,
-                                       threads=8)
-    ti, bi = torch.as_tensor(tok), torch.as_tensor(bat)
-    got_o = to_np(out.reshape(B, N, H, D)[bi, ti])
-    got_l = to_np(lse.reshape(B, N, H)[bi, ti])
-    assert_close("sampled out", got_o, ref_o)
-    assert_close("sampled lse", got_l, ref_l)
 
 
 def _properties(fn, q, k, v, args, out, lse):
@@ -66,7 +47,7 @@ def test_config3_full_size_sampled():
     args = ((32, 32), (16, 16), (1, 1))
     with torch.no_grad():
         out, lse = natten_amd.na2d(q, k, v, *args, return_lse=True)
-    _sampled_check(q, k, v, out, lse, *args, (False, False), n_samples=200, seed=1)
+    sampled_check(q, k, v, out, lse, *args, (False, False), n_samples=2000, seed=1)
     _properties(natten_amd.na2d, q, k, v, args, out, lse)
 
 
@@ -75,10 +56,34 @@ def test_config4_full_size_sampled():
     args = ((18, 24, 24), (1, 8, 8), (1, 1, 1), (True, False, False))
     with torch.no_grad():
         out, lse = natten_amd.na3d(q, k, v, *args, return_lse=True)
-    _sampled_check(q, k, v, out, lse, *args, n_samples=64, seed=2)
+    sampled_check(q, k, v, out, lse, *args, n_samples=2000, seed=2)
     _properties(natten_amd.na3d, q, k, v, args, out, lse)
     # causal in time: the first frame attends only itself, so its LSE is below the last frame's
     assert (lse[0, 0].mean() < lse[0, -1].mean()).item()
+
+
+def test_tensors_above_4_gib_both_routes():
+    """The fourth configuration with batch 8: every tensor is 5.7 GB, so row offsets pass 2^31 and
+    2^32 bytes.  The kernels address a tile as a 64-bit base plus 32-bit per-lane offsets; the first
+    and the last batch entry (the one beyond 4 GiB) are sampled against the oracle on both routes
+    (one launch on the original tensors; permute + kernel + unpermute), which must agree bit for bit."""
+    from natten_amd.fna import amd_fna_generic
+
+    B, shape, H, D = 8, (30, 48, 80), 24, 128
+    gen = torch.Generator(device="cuda").manual_seed(11)
+    q, k, v = (torch.randn((B, *shape, H, D), generator=gen, device="cuda", dtype=torch.bfloat16) for _ in range(3))
+    assert q.numel() * q.element_size() > 2**32
+    args = ((18, 24, 24), (1, 8, 8), (1, 1, 1), (True, False, False))
+    with torch.no_grad():
+        out, lse = natten_amd.na3d(q, k, v, *args, return_lse=True)
+        sampled_check(q, k, v, out, lse, *args, n_samples=400, seed=3, batches=(0, B - 1), tag="one launch")
+        assert torch.isfinite(out).all() and torch.isfinite(lse).all()
+        out2, lse2 = amd_fna_generic(q, k, v, *args, return_lse=True, fused=False)
+    assert torch.equal(out, out2) and torch.equal(lse, lse2), "the two routes differ above 4 GiB"
+    # every batch entry is an independent problem: entry 7 alone gives the same bits
+    with torch.no_grad():
+        out7, lse7 = natten_amd.na3d(q[7:], k[7:], v[7:], *args, return_lse=True)
+    assert torch.equal(out7, out[7:]) and torch.equal(lse7, lse[7:])
 
 
 def test_permute_round_trip_full_size():

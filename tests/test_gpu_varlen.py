@@ -113,6 +113,25 @@ def test_rows_outside_every_sequence_are_zero():
     assert_close("lse", to_np(lse[:, 30:80]), ref_l)
 
 
+def test_malformed_cumulative_lengths_are_not_followed():
+    # cumulative arrays the tensors cannot hold (past the end, decreasing, negative): the kernel
+    # leaves the rows of such a sequence untouched (zeros) instead of forming addresses from
+    # them; the well-formed sequence in the same launch is computed as usual
+    from natten_amd import _lib
+
+    q, k, v = (_rand((1, 100, 2, 64), torch.bfloat16, s) for s in (4, 5, 6))
+    good = torch.tensor([0, 40], dtype=torch.int32, device="cuda")
+    for bad_tail in ([5000], [-7], [20]):
+        cu_q = torch.tensor([0, 40] + bad_tail, dtype=torch.int32, device="cuda")
+        cu_kv = torch.tensor([0, 40, 100], dtype=torch.int32, device="cuda")
+        for a, b in ((cu_q, cu_kv), (cu_kv, cu_q)):
+            out, lse = _lib.attention_forward_varlen(q, k, v, a, b, 60, 60, False, 0.125)
+            torch.cuda.synchronize()
+            ref_o, ref_l = _lib.attention_forward_varlen(q, k, v, good, good, 60, 60, False, 0.125)
+            assert torch.equal(out[:, :40], ref_o[:, :40]) and torch.equal(lse[:, :40], ref_l[:, :40])
+            assert torch.count_nonzero(out[:, 40:]) == 0 and torch.count_nonzero(lse[:, 40:]) == 0
+
+
 @pytest.mark.parametrize("causal", [False, True])
 def test_varlen_backward(causal):
     # gradients of the packed call against the backward oracle evaluated per sequence
