@@ -572,8 +572,22 @@ fna_fwd_kernel(const FnaParams p) {
   issue_tile_load(kbase, ld_koff, sK0, cur.row0);
   issue_tile_load(vbase, ld_voff, sV0, cur.row0);
 
+  float sm_scale = p.scale, out_scale = 1.f;
+  if (p.q_scale) sm_scale *= p.q_scale[head];
+  if (p.k_scale) sm_scale *= p.k_scale[head_kv];
+  if (p.v_scale) out_scale = p.v_scale[head_kv];
+  const float c_log2 = sm_scale * 1.4426950408889634f;
+
   // ---- per-lane setup: this lane's query rows, their windows, Q fragments ---------------------
-  int wst[MQ][3], wen[MQ][3];
+  // coordinates of this lane's query in row block mb (recomputed where a masked tile needs the
+  // query's window: keeping the window in registers for the whole loop costs more than that)
+  auto query_coord = [&](int mb, int (&c)[3]) __attribute__((always_inline)) {
+    int r = (wave * MQ + mb) * 32 + l32;  // row-major index inside the tile
+    c[2] = q_first[2] + r % p.q_tile[2];
+    r /= p.q_tile[2];
+    c[1] = q_first[1] + r % p.q_tile[1];
+    c[0] = q_first[0] + r / p.q_tile[1];
+  };
   int q_row[MQ];     // this lane's row of the permuted sequence / token offset in the group (fused), or -1
   vec8 qf[MQ][KSTEPS];
 #pragma unroll
@@ -596,8 +610,6 @@ fna_fwd_kernel(const FnaParams p) {
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
       const int c = q_first[a] + off[a];
-      wst[mb][a] = na_window_start(c, ksz[a], p.stride[a], extent[a], p.causal[a] != 0);
-      wen[mb][a] = na_window_end(c, wst[mb][a], ksz[a], extent[a], p.causal[a] != 0);
       if (p.fused) {
         valid = valid && (c < extent[a]);
         row += c * tok_step[a];
@@ -607,7 +619,20 @@ fna_fwd_kernel(const FnaParams p) {
     q_row[mb] = valid ? row : -1;
     const T* qrow = qbase + int64_t(row_c) * q_row_stride + g * 8;
 #pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) qf[mb][ks] = *reinterpret_cast<const vec8*>(qrow + ks * 16);
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+      const vec8 raw = *reinterpret_cast<const vec8*>(qrow + ks * 16);
+      // The query row carries the softmax scale (in the exp2 domain) into the matrix product, so
+      // that the logits leave the matrix pipe ready for exp2: q' = round(q * scale * log2(e)).
+      // Rounding q' to the operand type moves a logit by about 2^-9 (bf16) / 2^-12 (fp16) of
+      // |q||k| scale / sqrt(D) -- the size of the operands' own rounding; values are clamped to
+      // the type's finite range (only fp16 has one that a finite product can leave).
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        float x = float(raw[e]) * c_log2;
+        if constexpr (std::is_same<T, _Float16>::value) x = fminf(fmaxf(x, -65504.f), 65504.f);
+        qf[mb][ks][e] = static_cast<T>(x);
+      }
+    }
   }
 
   f32x16_t acc[MQ][DB];
@@ -621,11 +646,6 @@ fna_fwd_kernel(const FnaParams p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[mb][db][r] = 0.f;
   }
-  float sm_scale = p.scale, out_scale = 1.f;
-  if (p.q_scale) sm_scale *= p.q_scale[head];
-  if (p.k_scale) sm_scale *= p.k_scale[head_kv];
-  if (p.v_scale) out_scale = p.v_scale[head_kv];
-  const float c_log2 = sm_scale * 1.4426950408889634f;
 
   // lane-constant LDS read offsets
   int k_off[KSTEPS];  // K operand: row l32 (+32*sb), chunk 2*ks+g
@@ -664,9 +684,12 @@ fna_fwd_kernel(const FnaParams p) {
     return __builtin_bit_cast(vec8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
   };
 
+  // Logits are kept in the exp2 domain and relative to the row's running maximum: the matrix
+  // product starts from the accumulator value -m (sixteen registers per row block that only
+  // change when the maximum moves), so the probabilities are exp2 of what the matrix pipe returns.
   f32x16_t S_a[MQ][NSB], S_b[MQ][NSB];  // logits of the current / coming tile, swapping roles every iteration
   vec8 pf[MQ][NSB][2];
-  float msc[MQ];                // running maxima in the exp2 domain (0 while -inf)
+  f32x16_t c_init[MQ];          // -(running maximum), 0 while it is -inf: accumulator input of S = K Q^T
   float psum[MQ][2];
 
   // Element e of the current tile's probabilities: row block e % MQ, logit v = e / MQ of the lane
@@ -676,7 +699,7 @@ fna_fwd_kernel(const FnaParams p) {
   auto exp_elem = [&](const f32x16_t (&S_cur)[MQ][NSB], int e) {
     const int mb = e % MQ, v = e / MQ;
     const int sb = v / 16, r = v % 16;
-    float x = fast_exp2(S_cur[mb][sb][r] * c_log2 - msc[mb]);
+    float x = fast_exp2(S_cur[mb][sb][r]);
     psum[mb][r & 1] += x;
     if (r % 2 == 0) {
       pin(x);
@@ -700,7 +723,7 @@ fna_fwd_kernel(const FnaParams p) {
   };
 
   // element mask of a PARTIAL tile for row block mb
-  auto apply_mask = [&](f32x16_t (&S)[NSB], const int (&ws)[3], const int (&we)[3], const int (&origin)[3]) {
+  auto apply_mask = [&](f32x16_t (&S)[NSB], const int (&ws)[3], const int (&we)[3], const int (&origin)[3]) __attribute__((always_inline)) {
     // window of this lane's query relative to the tile origin, clamped to the tile
     uint32_t addc = 0, subc = 0;
 #pragma unroll
@@ -724,26 +747,36 @@ fna_fwd_kernel(const FnaParams p) {
       }
   };
 
-  // adopts the maximum `mx` of the lane's half row of the coming tile: the running maximum is
-  // only moved (and O, the row sum rescaled) when some row of the wave outgrew it by 2^8
-  auto update_max = [&](int mb, float mx) {
+  // adopts the maximum `mx` of the lane's half row of the coming tile (relative to the running
+  // maximum, like the logits `S` themselves): the running maximum is only moved (and the logits of
+  // that tile, O and the row sum shifted / rescaled) when some row of the wave outgrew it by 2^8
+  auto update_max = [&](int mb, float mx, f32x16_t (&S)[NSB]) __attribute__((always_inline)) {
     mx = cross_half_max(mx);
-    const bool grow = (mx - m_run[mb]) * c_log2 > kLazyRescaleLog2;  // also true while m_run == -inf and mx finite
+    const bool first = (m_run[mb] == -INFINITY) && (mx != -INFINITY);
+    const bool grow = first || (mx > kLazyRescaleLog2);
     if (__any(grow)) {
-      const float m_new = fmaxf(m_run[mb], mx);
-      const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-      const float alpha = fast_exp2((m_run[mb] - m_use) * c_log2);  // m_run == -inf -> 0
-      m_run[mb] = m_new;
+      // rows still at -inf take their first maximum as it is (it may be negative) and have
+      // nothing accumulated yet; the others only grow
+      const bool was_inf = m_run[mb] == -INFINITY;
+      const float shift = was_inf ? ((mx == -INFINITY) ? 0.f : mx) : fmaxf(mx, 0.f);
+      const float alpha = was_inf ? 1.f : fast_exp2(-shift);
+      if (mx != -INFINITY) m_run[mb] = (was_inf ? 0.f : m_run[mb]) + shift;
       l_run[mb] *= alpha;
 #pragma unroll
       for (int db = 0; db < DB; ++db)
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[mb][db][r] *= alpha;
+#pragma unroll
+      for (int sb = 0; sb < NSB; ++sb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) S[sb][r] -= shift;
+      const float c = (m_run[mb] == -INFINITY) ? 0.f : -m_run[mb];
+#pragma unroll
+      for (int r = 0; r < 16; ++r) c_init[mb][r] = c;
     }
-    msc[mb] = ((m_run[mb] == -INFINITY) ? 0.f : m_run[mb]) * c_log2;
   };
   // masks (PARTIAL tiles) and maxima of a whole tile of logits, outside the slots
-  auto finish_logits = [&](f32x16_t (&S)[MQ][NSB], const bool t_full, const bool t_skip, const int (&t_origin)[3], bool have_max, const float (&mx_in)[MQ]) {
+  auto finish_logits = [&](f32x16_t (&S)[MQ][NSB], const bool t_full, const bool t_skip, const int (&t_origin)[3], bool have_max, const float (&mx_in)[MQ]) __attribute__((always_inline)) {
 #pragma unroll
     for (int mb = 0; mb < MQ; ++mb) {
       float mx = mx_in[mb];
@@ -755,14 +788,23 @@ fna_fwd_kernel(const FnaParams p) {
 #pragma unroll
           for (int r = 0; r < 16; ++r) S[mb][sb][r] = -INFINITY;
       } else if (!t_full || !have_max) {
-        if (!t_full) apply_mask(S[mb], wst[mb], wen[mb], t_origin);
+        if (!t_full) {
+          int qc[3], ws[3], we[3];
+          query_coord(mb, qc);
+#pragma unroll
+          for (int a = 0; a < 3; ++a) {
+            ws[a] = na_window_start(qc[a], ksz[a], p.stride[a], extent[a], p.causal[a] != 0);
+            we[a] = na_window_end(qc[a], ws[a], ksz[a], extent[a], p.causal[a] != 0);
+          }
+          apply_mask(S[mb], ws, we, t_origin);
+        }
         mx = -INFINITY;
 #pragma unroll
         for (int sb = 0; sb < NSB; ++sb)
 #pragma unroll
           for (int r = 0; r < 16; ++r) mx = fmaxf(mx, S[mb][sb][r]);
       }
-      update_max(mb, mx);
+      update_max(mb, mx, S[mb]);
     }
   };
 
@@ -776,7 +818,9 @@ fna_fwd_kernel(const FnaParams p) {
   __syncthreads();  // K(0), V(0) and the coordinate table are in LDS
   if (1 < total_tiles) issue_tile_load(kbase, ld_koff, sK1, nxt.row0);
 #pragma unroll
-  for (int mb = 0; mb < MQ; ++mb) msc[mb] = 0.f;
+  for (int mb = 0; mb < MQ; ++mb)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) c_init[mb][r] = 0.f;
   {
 #pragma unroll
     for (int mb = 0; mb < MQ; ++mb)
@@ -834,10 +878,7 @@ fna_fwd_kernel(const FnaParams p) {
 #pragma unroll
         for (int mb = 0; mb < MQ; ++mb) {
           if constexpr (s % KSTEPS == 0) {
-            f32x16_t zero;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) zero[r] = 0.f;
-            S_nxt[mb][s / KSTEPS] = M::run(kf[s], qf[mb][s % KSTEPS], zero);
+            S_nxt[mb][s / KSTEPS] = M::run(kf[s], qf[mb][s % KSTEPS], c_init[mb]);
           } else {
             S_nxt[mb][s / KSTEPS] = M::run(kf[s], qf[mb][s % KSTEPS], S_nxt[mb][s / KSTEPS]);
           }
@@ -965,7 +1006,7 @@ fna_fwd_kernel(const FnaParams p) {
           *reinterpret_cast<tx4*>(orow + db * 32 + 8 * j + 4 * g) = o4;
         }
       if (g == 0) {
-        const float lse = (l > 0.f) ? (m_run[mb] * sm_scale + __logf(l)) : -INFINITY;
+        const float lse = (l > 0.f) ? (m_run[mb] * 0.6931471805599453f + __logf(l)) : -INFINITY;
         p.lse[(q_row_base + row) * p.heads_q + head] = lse;
       }
     }
