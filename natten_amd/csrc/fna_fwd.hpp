@@ -92,6 +92,14 @@ struct Mma<__bf16> {
   static __device__ __forceinline__ f32x16_t run(vec8 a, vec8 b, f32x16_t c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
+  // a * b + c into registers of its own (c stays live and untouched).  Written as assembly: from
+  // the builtin the compiler first copies c into the destination (sixteen moves) and accumulates
+  // in place.  The two wait states cover a dependent matrix instruction issued right behind it.
+  static __device__ __forceinline__ f32x16_t run_from(vec8 a, vec8 b, const f32x16_t& c) {
+    f32x16_t d;
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %3\n\ts_nop 1" : "=&v"(d) : "v"(a), "v"(b), "v"(c));
+    return d;
+  }
   // c + a.x + a.y
   static __device__ __forceinline__ float add2(vec2 a, float c) {
     const vec2 one = {static_cast<__bf16>(1.0f), static_cast<__bf16>(1.0f)};
@@ -105,6 +113,11 @@ struct Mma<_Float16> {
   using vec2 = f16x2_t;
   static __device__ __forceinline__ f32x16_t run(vec8 a, vec8 b, f32x16_t c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ f32x16_t run_from(vec8 a, vec8 b, const f32x16_t& c) {
+    f32x16_t d;
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %3\n\ts_nop 1" : "=&v"(d) : "v"(a), "v"(b), "v"(c));
+    return d;
   }
   static __device__ __forceinline__ float add2(vec2 a, float c) {
     const vec2 one = {static_cast<_Float16>(1.0f), static_cast<_Float16>(1.0f)};
@@ -774,6 +787,9 @@ fna_fwd_kernel(const FnaParams p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) c_init[mb][r] = c;
     }
+    // one home for the sixteen registers on both paths (otherwise the compiler keeps a second
+    // copy of them alive and copies one to the other in every iteration)
+    asm volatile("" : "+v"(c_init[mb]));
   };
   // masks (PARTIAL tiles) and maxima of a whole tile of logits, outside the slots
   auto finish_logits = [&](f32x16_t (&S)[MQ][NSB], const bool t_full, const bool t_skip, const int (&t_origin)[3], bool have_max, const float (&mx_in)[MQ]) __attribute__((always_inline)) {
@@ -878,7 +894,7 @@ fna_fwd_kernel(const FnaParams p) {
 #pragma unroll
         for (int mb = 0; mb < MQ; ++mb) {
           if constexpr (s % KSTEPS == 0) {
-            S_nxt[mb][s / KSTEPS] = M::run(kf[s], qf[mb][s % KSTEPS], c_init[mb]);
+            S_nxt[mb][s / KSTEPS] = M::run_from(kf[s], qf[mb][s % KSTEPS], c_init[mb]);
           } else {
             S_nxt[mb][s / KSTEPS] = M::run(kf[s], qf[mb][s % KSTEPS], S_nxt[mb][s / KSTEPS]);
           }
