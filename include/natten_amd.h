@@ -80,7 +80,19 @@ const char* natten_amd_last_error(void);
  * type; tiles must be 128 x 64 tokens.  A more accurate, slower route for the same operands:
  * widen them to bf16 while permuting (natten_amd_token_permute_widen, exact) and call this
  * function with dtype BF16 and the scales.
+ *
+ * run_persistent (the reference's `run_persistent` argument, blackwell_fna.h:52, scheduler
+ * csrc/include/natten/cuda/fmha_blackwell/kernel/fmha_tile_scheduler.hpp:146-149): non-zero
+ * launches as many workgroups as the device keeps resident, which take Q tiles from per-XCD work
+ * queues until none is left, instead of one workgroup per Q tile; results are bit-identical.
+ * The queues are counters in `workspace`: device memory owned by the caller, 64-byte aligned,
+ * at least natten_amd_fna_forward_workspace_bytes() bytes, cleared by the launch itself (by a
+ * kernel, so the call may be captured in a graph) and free for reuse once the work queued on
+ * `stream` by this call has run.  Two calls must not use one workspace concurrently.  Tile
+ * pairs other than 128 x 64 tokens and 8-bit operands ignore the flag.  run_persistent == 0:
+ * workspace may be NULL.
  */
+uint64_t natten_amd_fna_forward_workspace_bytes(void);
 int natten_amd_fna_forward(const void* q, const void* k, const void* v, void* out, float* lse,
                            int dtype, int na_dim, int batch, int seqlen_q, int seqlen_kv,
                            int heads_q, int heads_kv, int head_dim, const int32_t* q_shape,
@@ -89,6 +101,7 @@ int natten_amd_fna_forward(const void* q, const void* k, const void* v, void* ou
                            const int32_t* dilation, const int32_t* is_causal,
                            const int32_t* q_tile_shape, const int32_t* kv_tile_shape, float scale,
                            const float* q_scale, const float* k_scale, const float* v_scale,
+                           int run_persistent, void* workspace, uint64_t workspace_bytes,
                            void* stream);
 
 /*
@@ -100,7 +113,8 @@ int natten_amd_fna_forward(const void* q, const void* k, const void* v, void* ou
  * disappear; results are bit-identical to the permuted path with the same tile shapes.
  * Requires qkv_shape[a] to be a multiple of dilation[a] * kv_tile_shape[a] in every dimension
  * (no KV tile may reach past the input); returns an error otherwise, and the caller uses the
- * permuted path.  dtype, tiles, head_dim and scales as in natten_amd_fna_forward.
+ * permuted path.  dtype, tiles, head_dim, scales, run_persistent and workspace as in
+ * natten_amd_fna_forward.
  */
 int natten_amd_fna_forward_fused(const void* q, const void* k, const void* v, void* out,
                                  float* lse, int dtype, int na_dim, int batch, int heads_q,
@@ -109,7 +123,8 @@ int natten_amd_fna_forward_fused(const void* q, const void* k, const void* v, vo
                                  const int32_t* dilation, const int32_t* is_causal,
                                  const int32_t* q_tile_shape, const int32_t* kv_tile_shape,
                                  float scale, const float* q_scale, const float* k_scale,
-                                 const float* v_scale, void* stream);
+                                 const float* v_scale, int run_persistent, void* workspace,
+                                 uint64_t workspace_bytes, void* stream);
 
 /*
  * Supported tile sizes (tokens per tile).  Writes up to `capacity` pairs

@@ -19,7 +19,7 @@ from torch import Tensor
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libnatten_amd.so")
 
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 DTYPE_CODES = {
     torch.float16: 0,
@@ -46,11 +46,14 @@ _SIGNATURES = {
         + [ctypes.c_int] * 8
         + [ctypes.c_void_p] * 9
         + [ctypes.c_float]
-        + [ctypes.c_void_p] * 4,
+        + [ctypes.c_void_p] * 3
+        + [ctypes.c_int, ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p],
     ),
+    "natten_amd_fna_forward_workspace_bytes": (ctypes.c_uint64, []),
     "natten_amd_fna_forward_fused": (
         ctypes.c_int,
-        [ctypes.c_void_p] * 5 + [ctypes.c_int] * 6 + [ctypes.c_void_p] * 7 + [ctypes.c_float] + [ctypes.c_void_p] * 4,
+        [ctypes.c_void_p] * 5 + [ctypes.c_int] * 6 + [ctypes.c_void_p] * 7 + [ctypes.c_float] + [ctypes.c_void_p] * 3
+        + [ctypes.c_int, ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p],
     ),
     "natten_amd_attention_forward": (
         ctypes.c_int,
@@ -195,10 +198,13 @@ def fna_forward(
     kernel_size, stride, dilation, is_causal, scale: float,
     q_shape, kv_shape, qkv_shape, q_tile_shape, kv_tile_shape,
     q_scale: Optional[Tensor] = None, k_scale: Optional[Tensor] = None, v_scale: Optional[Tensor] = None,
+    run_persistent: bool = False,
 ) -> Tuple[Tensor, Tensor]:
     """Token-permuted q [B*G, SQ, H, D], k/v [B*G, SK, Hkv, D] -> (out, lse float32 [B*G, SQ, H]).
 
-    q_scale [H], k_scale / v_scale [Hkv]: optional float32 per-head dequantisation scales."""
+    q_scale [H], k_scale / v_scale [Hkv]: optional float32 per-head dequantisation scales.
+    run_persistent: work-queue launch (as many workgroups as stay resident pull Q tiles from
+    per-XCD queues kept in a small workspace) instead of a workgroup per Q tile; same results."""
     L = lib()
     _require_gpu(q, k, v)
     if q.dtype not in (torch.float16, torch.bfloat16) + FP8_DTYPES:
@@ -214,10 +220,21 @@ def fna_forward(
             DTYPE_CODES[q.dtype], na_dim, q.shape[0], q.shape[1], k.shape[1], q.shape[2], k.shape[2], q.shape[3],
             _i32(q_shape), _i32(kv_shape), _i32(qkv_shape), _i32(kernel_size), _i32(stride), _i32(dilation),
             _i32([1 if c else 0 for c in is_causal]), _i32(q_tile_shape), _i32(kv_tile_shape),
-            float(scale), *scales, _stream(q),
+            float(scale), *scales, *_queue_workspace(q, run_persistent), _stream(q),
         )
     _check(rc)
     return out, lse
+
+
+def _queue_workspace(like: Tensor, run_persistent: bool):
+    """(flag, pointer, bytes) of the work-queue launch's workspace, allocated by the caller side as
+    the reference's wrappers allocate theirs (src/natten/_libnatten/torch_wrappers.py:688-693)."""
+    if not run_persistent:
+        return 0, None, 0
+    nbytes = int(lib().natten_amd_fna_forward_workspace_bytes())
+    # the launch clears it; torch's allocator hands the block out again only to later work of this stream
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=like.device)
+    return 1, ws.data_ptr(), nbytes
 
 
 def _tile_span_fits(token_layout, dilation, tile_shape, row_bytes: int) -> bool:
@@ -242,6 +259,7 @@ def fna_forward_fused(
     q: Tensor, k: Tensor, v: Tensor,
     kernel_size, stride, dilation, is_causal, scale: float, q_tile_shape, kv_tile_shape,
     q_scale: Optional[Tensor] = None, k_scale: Optional[Tensor] = None, v_scale: Optional[Tensor] = None,
+    run_persistent: bool = False,
 ) -> Tuple[Tensor, Tensor]:
     """Original-layout q [B, *X, H, D], k/v [B, *X, Hkv, D] -> (out like q, lse float32 [B, *X, H])."""
     L = lib()
@@ -259,7 +277,7 @@ def fna_forward_fused(
             DTYPE_CODES[q.dtype], na_dim, q.shape[0], q.shape[-2], k.shape[-2], q.shape[-1],
             _i32(qkv_shape), _i32(kernel_size), _i32(stride), _i32(dilation),
             _i32([1 if c else 0 for c in is_causal]), _i32(q_tile_shape), _i32(kv_tile_shape),
-            float(scale), *scales, _stream(q),
+            float(scale), *scales, *_queue_workspace(q, run_persistent), _stream(q),
         )
     _check(rc)
     return out, lse

@@ -266,9 +266,10 @@ struct FnaSmem {
 // accumulation registers) and reads every K / V fragment from LDS once for two MFMAs.
 // RAGGED: seqlen_kv is not a multiple of KVT (dense attention on unpadded sequences); the tile
 // copies then clamp their rows and are issued at the top of an iteration instead of one per slot.
+// The work of one workgroup on one Q tile; `pid` is the position of that tile in the launch order
+// (what blockIdx.x is when every Q tile has a workgroup of its own).
 template <typename T, int D, int NWAVES, int MQ, bool RAGGED, int KVT>
-__global__ void __launch_bounds__(NWAVES * 64) __attribute__((amdgpu_waves_per_eu(MQ == 1 ? 2 : 1, MQ == 1 ? 2 : 1)))
-fna_fwd_kernel(const FnaParams p) {
+static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const int pid) {
   constexpr int NT = NWAVES * 64;
   constexpr int QT = NWAVES * MQ * 32;
   constexpr int KSTEPS = D / 16;
@@ -303,7 +304,6 @@ fna_fwd_kernel(const FnaParams p) {
   // ---- workgroup id -> (batch*group, head, Q tile); groups of Q tiles are dealt to XCDs ------
   int bg, head, qtile_rm;
   {
-    const int pid = blockIdx.x;
     const int xcd = pid % kNumXcd;
     const int local = pid / kNumXcd;
     const int group = (local / p.wg_group) * kNumXcd + xcd;
@@ -1027,6 +1027,57 @@ fna_fwd_kernel(const FnaParams p) {
       }
     }
   }
+}
+
+template <typename T, int D, int NWAVES, int MQ, bool RAGGED, int KVT>
+__global__ void __launch_bounds__(NWAVES * 64) __attribute__((amdgpu_waves_per_eu(MQ == 1 ? 2 : 1, MQ == 1 ? 2 : 1)))
+fna_fwd_kernel(const FnaParams p) {
+  fna_fwd_tile<T, D, NWAVES, MQ, RAGGED, KVT>(p, int(blockIdx.x));
+}
+
+// Work-queue launch: as many workgroups as the chip keeps resident, each taking Q tiles until
+// none is left.  Workgroup i runs on XCD i % 8 (the dispatcher deals workgroups to XCDs in turn),
+// and launch position `local * 8 + x` is what the one-tile-per-workgroup launch runs on XCD x:
+// every XCD has a queue of its own (`queues[16 * x]`, one counter per 64-byte line) over its
+// `per_xcd` positions in the same order, so the tiles resident on an XCD share K/V in its L2 as
+// before; a workgroup whose queue has run dry takes from the other XCDs' queues, which evens
+// out the tail.  The counters must be zero at launch.  Every workgroup ends after at most
+// `8 * per_xcd + 8` counter increments in total, whatever the other workgroups do.
+constexpr int kQueueStride = 16;  // uint32 counters per 64-byte line
+constexpr int kQueueWords = kNumXcd * kQueueStride;
+
+template <typename T, int D, int NWAVES, int MQ, bool RAGGED, int KVT>
+__global__ void __launch_bounds__(NWAVES * 64) __attribute__((amdgpu_waves_per_eu(MQ == 1 ? 2 : 1, MQ == 1 ? 2 : 1)))
+fna_fwd_queue_kernel(const FnaParams p, uint32_t* __restrict__ queues, const int per_xcd) {
+  __shared__ int s_next;
+  const int home = int(blockIdx.x) % kNumXcd;
+  int victim = 0;  // queues tried so far: home first, then the others in turn
+  // thread 0 takes the next position from the queues (-1: all are empty)
+  auto take = [&]() {
+    while (victim < kNumXcd) {
+      const int x = (home + victim) % kNumXcd;
+      const uint32_t local = atomicAdd(&queues[x * kQueueStride], 1u);
+      if (local < uint32_t(per_xcd)) return int(local) * kNumXcd + x;
+      ++victim;  // that queue is empty for good
+    }
+    return -1;
+  };
+  int mine = threadIdx.x == 0 ? take() : 0;
+  for (;;) {
+    __syncthreads();  // everyone has read s_next, and is done with the LDS of the previous tile
+    if (threadIdx.x == 0) s_next = mine;
+    __syncthreads();
+    const int pid = s_next;
+    if (pid < 0) break;
+    // the position after this one is fetched while this one is worked on
+    if (threadIdx.x == 0) mine = take();
+    fna_fwd_tile<T, D, NWAVES, MQ, RAGGED, KVT>(p, pid);
+  }
+}
+
+// clears the queue counters (a kernel rather than a memset so that callers may capture the launch pair in a graph)
+__global__ void fna_queue_clear_kernel(uint32_t* queues) {
+  if (threadIdx.x < kQueueWords) queues[threadIdx.x] = 0;
 }
 
 }  // namespace natten_amd

@@ -67,14 +67,36 @@ struct TileConfig {
 const TileConfig kTileConfigs[] = {{128, 64}, {256, 64}, {64, 64}};
 constexpr int kNumTileConfigs = sizeof(kTileConfigs) / sizeof(kTileConfigs[0]);
 
+// Workgroups a work-queue launch starts: two per compute unit (what the kernel's LDS and register
+// use keep resident), a multiple of the XCD count; the device's figure is read once.
+int resident_workgroups() {
+  static int cached[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 512;
+  if (cached[dev] == 0) {
+    int cus = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1) cus = 256;
+    cached[dev] = (2 * cus / kNumXcd) * kNumXcd;
+    if (cached[dev] < kNumXcd) cached[dev] = kNumXcd;
+  }
+  return cached[dev];
+}
+
+// `queues` != nullptr: work-queue launch (kQueueWords zero-initialised counters are cleared and used).
 template <typename T, int D, int NWAVES, int MQ, bool RAGGED, int KVT>
-int launch_fna(const FnaParams& p, hipStream_t stream) {
+int launch_fna(const FnaParams& p, hipStream_t stream, uint32_t* queues = nullptr) {
   constexpr int QT = NWAVES * MQ * 32;
-  auto kernel = fna_fwd_kernel<T, D, NWAVES, MQ, RAGGED, KVT>;
   if ((p.seqlen_q + QT - 1) / QT != p.num_q_tiles) return fail("fna_forward: internal tile count mismatch");
   const long long wgs = (long long)((p.total_groups + kNumXcd - 1) / kNumXcd) * kNumXcd * p.wg_group;
   if (wgs > 0x7fffffffLL) return fail("fna_forward: problem needs more than 2^31 workgroups");
-  hipLaunchKernelGGL(kernel, dim3((unsigned)wgs), dim3(NWAVES * 64), 0, stream, p);
+  if (queues != nullptr) {
+    const long long resident = resident_workgroups();
+    hipLaunchKernelGGL(fna_queue_clear_kernel, dim3(1), dim3(kQueueWords), 0, stream, queues);
+    hipLaunchKernelGGL((fna_fwd_queue_kernel<T, D, NWAVES, MQ, RAGGED, KVT>), dim3((unsigned)(wgs < resident ? wgs : resident)),
+                       dim3(NWAVES * 64), 0, stream, p, queues, int(wgs / kNumXcd));
+    return check_launch("fna_forward (work queue)");
+  }
+  hipLaunchKernelGGL((fna_fwd_kernel<T, D, NWAVES, MQ, RAGGED, KVT>), dim3((unsigned)wgs), dim3(NWAVES * 64), 0, stream, p);
   return check_launch("fna_forward");
 }
 
@@ -89,32 +111,34 @@ int launch_fna_fp8(const FnaParams& p, hipStream_t stream) {
 }
 
 template <typename T, int D>
-int dispatch_tiles(const FnaParams& p, int qt, int kvt, hipStream_t stream) {
+int dispatch_tiles(const FnaParams& p, int qt, int kvt, hipStream_t stream, uint32_t* queues) {
   if (p.seqlen_kv % kvt != 0 || p.cu_q != nullptr) {
     // key sequences that end inside a tile: dense attention on unpadded or packed sequences only
     if (qt == 128 && kvt == 64) return launch_fna<T, D, 4, 1, true, 64>(p, stream);
     return fail("fna_forward: seqlen_kv (%d) must be a multiple of the KV tile (%d tokens)", p.seqlen_kv, kvt);
   }
-  if (qt == 128 && kvt == 64) return launch_fna<T, D, 4, 1, false, 64>(p, stream);
+  // the work-queue launch exists for the default tile pair; the others launch a workgroup per Q tile
+  if (qt == 128 && kvt == 64) return launch_fna<T, D, 4, 1, false, 64>(p, stream, queues);
   if (qt == 256 && kvt == 64) return launch_fna<T, D, 8, 1, false, 64>(p, stream);
   if (qt == 64 && kvt == 64) return launch_fna<T, D, 2, 1, false, 64>(p, stream);
   return fail("fna_forward: no kernel for Q tile of %d and KV tile of %d tokens", qt, kvt);
 }
 
 template <typename T>
-int dispatch_head_dim(const FnaParams& p, int head_dim, int qt, int kvt, hipStream_t stream) {
+int dispatch_head_dim(const FnaParams& p, int head_dim, int qt, int kvt, hipStream_t stream, uint32_t* queues) {
   switch (head_dim) {
-    case 32: return dispatch_tiles<T, 32>(p, qt, kvt, stream);
-    case 64: return dispatch_tiles<T, 64>(p, qt, kvt, stream);
-    case 128: return dispatch_tiles<T, 128>(p, qt, kvt, stream);
+    case 32: return dispatch_tiles<T, 32>(p, qt, kvt, stream, queues);
+    case 64: return dispatch_tiles<T, 64>(p, qt, kvt, stream, queues);
+    case 128: return dispatch_tiles<T, 128>(p, qt, kvt, stream, queues);
   }
   return fail("fna_forward: head_dim must be 32, 64 or 128, got %d", head_dim);
 }
 
-int dispatch_dtype(const FnaParams& p, int dtype, int head_dim, int qt, int kvt, hipStream_t stream) {
+int dispatch_dtype(const FnaParams& p, int dtype, int head_dim, int qt, int kvt, hipStream_t stream,
+                   uint32_t* queues = nullptr) {
   switch (dtype) {
-    case NATTEN_AMD_F16: return dispatch_head_dim<_Float16>(p, head_dim, qt, kvt, stream);
-    case NATTEN_AMD_BF16: return dispatch_head_dim<__bf16>(p, head_dim, qt, kvt, stream);
+    case NATTEN_AMD_F16: return dispatch_head_dim<_Float16>(p, head_dim, qt, kvt, stream, queues);
+    case NATTEN_AMD_BF16: return dispatch_head_dim<__bf16>(p, head_dim, qt, kvt, stream, queues);
   }
   if (dtype == NATTEN_AMD_F8E4M3 || dtype == NATTEN_AMD_F8E5M2) {
     // 8-bit float operands, bf16 output: one kernel configuration
@@ -188,11 +212,25 @@ int fill_fna_params(const char* what, FnaParams& p, int na_dim, const int* q_sha
   p.tok_stride[0] = p.qkv_shape[2] * p.qkv_shape[1];
   return 0;
 }
+
+// The queue counters of a work-queue launch inside the caller's workspace (nullptr: launch a
+// workgroup per Q tile).  rc != 0 on a workspace that cannot hold them.
+int queue_workspace(const char* what, int run_persistent, void* workspace, uint64_t workspace_bytes, uint32_t** queues) {
+  *queues = nullptr;
+  if (!run_persistent) return 0;
+  if (!workspace || workspace_bytes < uint64_t(kQueueWords) * 4 || (reinterpret_cast<uintptr_t>(workspace) & 63))
+    return fail("%s: run_persistent needs a 64-byte aligned device workspace of at least %d bytes (got %p, %llu bytes)", what,
+                kQueueWords * 4, workspace, (unsigned long long)workspace_bytes);
+  *queues = static_cast<uint32_t*>(workspace);
+  return 0;
+}
 }  // namespace
 
 extern "C" {
 
-int natten_amd_abi_version(void) { return 6; }
+int natten_amd_abi_version(void) { return 7; }
+
+uint64_t natten_amd_fna_forward_workspace_bytes(void) { return uint64_t(kQueueWords) * 4; }
 
 const char* natten_amd_last_error(void) { return g_error; }
 
@@ -218,9 +256,11 @@ int natten_amd_fna_forward(const void* q, const void* k, const void* v, void* ou
                            const int32_t* kernel_size, const int32_t* stride, const int32_t* dilation,
                            const int32_t* is_causal, const int32_t* q_tile_shape, const int32_t* kv_tile_shape,
                            float scale, const float* q_scale, const float* k_scale, const float* v_scale,
-                           void* stream) {
+                           int run_persistent, void* workspace, uint64_t workspace_bytes, void* stream) {
   g_error[0] = 0;
   if (na_dim < 1 || na_dim > 3) return fail("fna_forward: na_dim must be 1, 2 or 3, got %d", na_dim);
+  uint32_t* queues;
+  if (int rc = queue_workspace("fna_forward", run_persistent, workspace, workspace_bytes, &queues)) return rc;
   if (int rc = check_common("fna_forward", q, k, v, out, lse, batch, seqlen_q, seqlen_kv, heads_q, heads_kv, head_dim))
     return rc;
   if (!q_shape || !kv_shape || !qkv_shape || !kernel_size || !stride || !dilation || !is_causal || !q_tile_shape ||
@@ -255,7 +295,7 @@ int natten_amd_fna_forward(const void* q, const void* k, const void* v, void* ou
   p.k_scale = k_scale;
   p.v_scale = v_scale;
   set_wg_layout(p, 1);
-  return dispatch_dtype(p, dtype, head_dim, prod3(p.q_tile), prod3(p.kv_tile), static_cast<hipStream_t>(stream));
+  return dispatch_dtype(p, dtype, head_dim, prod3(p.q_tile), prod3(p.kv_tile), static_cast<hipStream_t>(stream), queues);
 }
 
 int natten_amd_fna_forward_fused(const void* q, const void* k, const void* v, void* out, float* lse, int dtype,
@@ -263,9 +303,12 @@ int natten_amd_fna_forward_fused(const void* q, const void* k, const void* v, vo
                                  const int32_t* qkv_shape, const int32_t* kernel_size, const int32_t* stride,
                                  const int32_t* dilation, const int32_t* is_causal, const int32_t* q_tile_shape,
                                  const int32_t* kv_tile_shape, float scale, const float* q_scale,
-                                 const float* k_scale, const float* v_scale, void* stream) {
+                                 const float* k_scale, const float* v_scale, int run_persistent, void* workspace,
+                                 uint64_t workspace_bytes, void* stream) {
   g_error[0] = 0;
   if (na_dim < 1 || na_dim > 3) return fail("fna_forward_fused: na_dim must be 1, 2 or 3, got %d", na_dim);
+  uint32_t* queues;
+  if (int rc = queue_workspace("fna_forward_fused", run_persistent, workspace, workspace_bytes, &queues)) return rc;
   if (!qkv_shape || !kernel_size || !stride || !dilation || !is_causal || !q_tile_shape || !kv_tile_shape)
     return fail("fna_forward_fused: null shape argument");
   int qs[3] = {1, 1, 1}, ks[3] = {1, 1, 1};
@@ -314,7 +357,7 @@ int natten_amd_fna_forward_fused(const void* q, const void* k, const void* v, vo
   p.fused = 1;
   p.tokens = int(tokens);
   set_wg_layout(p, 1);
-  return dispatch_dtype(p, dtype, head_dim, prod3(p.q_tile), prod3(p.kv_tile), static_cast<hipStream_t>(stream));
+  return dispatch_dtype(p, dtype, head_dim, prod3(p.q_tile), prod3(p.kv_tile), static_cast<hipStream_t>(stream), queues);
 }
 
 int natten_amd_attention_forward(const void* q, const void* k, const void* v, void* out, float* lse, int dtype,

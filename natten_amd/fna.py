@@ -106,8 +106,12 @@ def amd_fna_generic(
     fp8_matmul: Optional[bool] = None,
     backward_q_tile_shape=None,
     backward_kv_tile_shape=None,
+    run_persistent_kernel: bool = False,
 ) -> Union[Tensor, Tuple[Tensor, Tensor]]:
-    """`fused` selects the one-launch path that gathers tiles from the original tensors (None:
+    """`run_persistent_kernel`: work-queue launch of the forward kernel (resident workgroups pull
+    Q tiles from per-XCD queues) instead of a workgroup per Q tile; bit-identical results.
+
+    `fused` selects the one-launch path that gathers tiles from the original tensors (None:
     whenever the problem allows it); otherwise tokens are permuted, multiplied and unpermuted
     by separate kernels, as the reference does.  Both give bit-identical results.
 
@@ -133,7 +137,7 @@ def amd_fna_generic(
         )
         output, lse = AmdFnaFunction.apply(
             query, key, value, kernel_size, stride, dilation, is_causal, scale, q_tile_shape, kv_tile_shape,
-            bwd_q_tile, bwd_kv_tile, fused,
+            bwd_q_tile, bwd_kv_tile, fused, bool(run_persistent_kernel),
         )
         if out_dtype is not None and output.dtype != out_dtype:
             output = output.to(out_dtype)
@@ -169,6 +173,7 @@ def amd_fna_generic(
             q_scale=resolve_scale(q_scale, query.shape[-2], query.device, "q_scale"),
             k_scale=resolve_scale(k_scale, key.shape[-2], query.device, "k_scale"),
             v_scale=resolve_scale(v_scale, key.shape[-2], query.device, "v_scale"),
+            run_persistent=bool(run_persistent_kernel),
         )
         if d_pad != head_dim:
             output = output[..., :head_dim].contiguous()
@@ -188,7 +193,7 @@ def amd_fna_generic(
     out_perm, lse_perm = torch_ops.fna_forward(
         q_perm, k_perm, v_perm, kernel_size, stride, dilation, is_causal, scale,
         q_shape, kv_shape, qkv_shape, q_tile_shape, kv_tile_shape,
-        q_scale=q_scale, k_scale=k_scale, v_scale=v_scale,
+        q_scale=q_scale, k_scale=k_scale, v_scale=v_scale, run_persistent=bool(run_persistent_kernel),
     )
 
     output = token_unpermute_operation(out_perm, qkv_shape, q_tile_shape, dilation, flip_tiled_dims=True)
@@ -218,11 +223,11 @@ class AmdFnaFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, query, key, value, kernel_size, stride, dilation, is_causal, scale, q_tile_shape, kv_tile_shape,
-                bwd_q_tile_shape, bwd_kv_tile_shape, fused):
+                bwd_q_tile_shape, bwd_kv_tile_shape, fused, run_persistent_kernel=False):
         with torch.no_grad():
             output, lse = amd_fna_generic(
                 query, key, value, kernel_size, stride, dilation, is_causal, scale, q_tile_shape, kv_tile_shape,
-                return_lse=True, fused=fused,
+                return_lse=True, fused=fused, run_persistent_kernel=run_persistent_kernel,
             )
         ctx.save_for_backward(query, key, value, output, lse)
         ctx.na_args = (kernel_size, stride, dilation, is_causal, scale, bwd_q_tile_shape, bwd_kv_tile_shape)
@@ -252,7 +257,7 @@ class AmdFnaFunction(torch.autograd.Function):
             )
             if d_pad != head_dim:
                 dq, dk, dv = (t[..., :head_dim].contiguous() for t in (dq, dk, dv))
-            return (dq, dk, dv) + (None,) * 10
+            return (dq, dk, dv) + (None,) * 11
 
         def perm(x, tile):
             return token_permute_operation(x.contiguous(), tile, dilation, flip_tiled_dims=True)
@@ -272,4 +277,4 @@ class AmdFnaFunction(torch.autograd.Function):
         dv = token_unpermute_operation(dv_perm, qkv_shape, kv_tile, dilation, flip_tiled_dims=True)
         if d_pad != head_dim:
             dq, dk, dv = (t[..., :head_dim].contiguous() for t in (dq, dk, dv))
-        return (dq, dk, dv) + (None,) * 10
+        return (dq, dk, dv) + (None,) * 11

@@ -28,15 +28,16 @@ def _fna_forward_op(
     q: Tensor, k: Tensor, v: Tensor, kernel_size: List[int], stride: List[int], dilation: List[int],
     is_causal: List[bool], scale: float, q_shape: List[int], kv_shape: List[int], qkv_shape: List[int],
     q_tile_shape: List[int], kv_tile_shape: List[int], q_scale: Optional[Tensor], k_scale: Optional[Tensor],
-    v_scale: Optional[Tensor],
+    v_scale: Optional[Tensor], run_persistent: bool,
 ) -> Tuple[Tensor, Tensor]:
     return _lib.fna_forward(q, k, v, kernel_size, stride, dilation, is_causal, scale, q_shape, kv_shape, qkv_shape,
-                            q_tile_shape, kv_tile_shape, q_scale=q_scale, k_scale=k_scale, v_scale=v_scale)
+                            q_tile_shape, kv_tile_shape, q_scale=q_scale, k_scale=k_scale, v_scale=v_scale,
+                            run_persistent=run_persistent)
 
 
 @_fna_forward_op.register_fake
 def _(q, k, v, kernel_size, stride, dilation, is_causal, scale, q_shape, kv_shape, qkv_shape, q_tile_shape,
-      kv_tile_shape, q_scale, k_scale, v_scale):
+      kv_tile_shape, q_scale, k_scale, v_scale, run_persistent):
     return q.new_empty(q.shape, dtype=_out_dtype(q)), q.new_empty(q.shape[:-1], dtype=torch.float32)
 
 
@@ -44,14 +45,16 @@ def _(q, k, v, kernel_size, stride, dilation, is_causal, scale, q_shape, kv_shap
 def _fna_forward_fused_op(
     q: Tensor, k: Tensor, v: Tensor, kernel_size: List[int], stride: List[int], dilation: List[int],
     is_causal: List[bool], scale: float, q_tile_shape: List[int], kv_tile_shape: List[int],
-    q_scale: Optional[Tensor], k_scale: Optional[Tensor], v_scale: Optional[Tensor],
+    q_scale: Optional[Tensor], k_scale: Optional[Tensor], v_scale: Optional[Tensor], run_persistent: bool,
 ) -> Tuple[Tensor, Tensor]:
     return _lib.fna_forward_fused(q, k, v, kernel_size, stride, dilation, is_causal, scale, q_tile_shape,
-                                  kv_tile_shape, q_scale=q_scale, k_scale=k_scale, v_scale=v_scale)
+                                  kv_tile_shape, q_scale=q_scale, k_scale=k_scale, v_scale=v_scale,
+                                  run_persistent=run_persistent)
 
 
 @_fna_forward_fused_op.register_fake
-def _(q, k, v, kernel_size, stride, dilation, is_causal, scale, q_tile_shape, kv_tile_shape, q_scale, k_scale, v_scale):
+def _(q, k, v, kernel_size, stride, dilation, is_causal, scale, q_tile_shape, kv_tile_shape, q_scale, k_scale, v_scale,
+      run_persistent):
     return q.new_empty(q.shape, dtype=_out_dtype(q)), q.new_empty(q.shape[:-1], dtype=torch.float32)
 
 
@@ -208,23 +211,25 @@ def _ints(t) -> List[int]:
 # ---- what the drivers call -------------------------------------------------------------------------
 
 def fna_forward(q, k, v, kernel_size, stride, dilation, is_causal, scale, q_shape, kv_shape, qkv_shape, q_tile_shape,
-                kv_tile_shape, q_scale=None, k_scale=None, v_scale=None):
+                kv_tile_shape, q_scale=None, k_scale=None, v_scale=None, run_persistent=False):
     if _tracing():
         return _fna_forward_op(q, k, v, _ints(kernel_size), _ints(stride), _ints(dilation),
                                [bool(c) for c in is_causal], float(scale), _ints(q_shape), _ints(kv_shape),
-                               _ints(qkv_shape), _ints(q_tile_shape), _ints(kv_tile_shape), q_scale, k_scale, v_scale)
+                               _ints(qkv_shape), _ints(q_tile_shape), _ints(kv_tile_shape), q_scale, k_scale, v_scale,
+                               bool(run_persistent))
     return _lib.fna_forward(q, k, v, kernel_size, stride, dilation, is_causal, scale, q_shape, kv_shape, qkv_shape,
-                            q_tile_shape, kv_tile_shape, q_scale=q_scale, k_scale=k_scale, v_scale=v_scale)
+                            q_tile_shape, kv_tile_shape, q_scale=q_scale, k_scale=k_scale, v_scale=v_scale,
+                            run_persistent=run_persistent)
 
 
 def fna_forward_fused(q, k, v, kernel_size, stride, dilation, is_causal, scale, q_tile_shape, kv_tile_shape,
-                      q_scale=None, k_scale=None, v_scale=None):
+                      q_scale=None, k_scale=None, v_scale=None, run_persistent=False):
     if _tracing():
         return _fna_forward_fused_op(q, k, v, _ints(kernel_size), _ints(stride), _ints(dilation),
                                      [bool(c) for c in is_causal], float(scale), _ints(q_tile_shape),
-                                     _ints(kv_tile_shape), q_scale, k_scale, v_scale)
+                                     _ints(kv_tile_shape), q_scale, k_scale, v_scale, bool(run_persistent))
     return _lib.fna_forward_fused(q, k, v, kernel_size, stride, dilation, is_causal, scale, q_tile_shape, kv_tile_shape,
-                                  q_scale=q_scale, k_scale=k_scale, v_scale=v_scale)
+                                  q_scale=q_scale, k_scale=k_scale, v_scale=v_scale, run_persistent=run_persistent)
 
 
 def attention_forward(q, k, v, is_causal, scale, q_scale=None, k_scale=None, v_scale=None):

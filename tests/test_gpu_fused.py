@@ -75,3 +75,70 @@ def test_fused_with_dequantisation_scales():
     ref_o, ref_l = oracle_full(qd, kd, vd, *args)
     assert_close("out", to_np(out_f), ref_o, atol=2e-2, rtol=1e-2)
     assert_close("lse", to_np(lse_f), ref_l)
+
+
+# ---- work-queue launch (run_persistent_kernel) ------------------------------------------------------
+
+QUEUE_CASES = [
+    # shape, kernel, stride, dilation, causal, heads, heads_kv, D  (default 128 x 64 token tiles)
+    ((2000,), (65,), (8,), (3,), (True,), 2, 1, 64),
+    ((40, 48), (9, 11), (2, 1), (1, 2), (False, False), 4, 2, 128),
+    ((37, 29), (7, 5), (1, 1), (1, 1), (True, False), 2, 2, 32),          # token-permuted route (odd extents)
+    ((10, 16, 24), (6, 8, 8), (1, 8, 4), (1, 1, 1), (True, False, False), 3, 3, 128),
+    ((8, 16, 16), (8, 16, 16), (1, 1, 1), (1, 1, 1), (True, False, False), 1, 1, 64),
+]
+
+
+@pytest.mark.parametrize("case", QUEUE_CASES)
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_work_queue_launch_equals_one_workgroup_per_tile(case, dtype):
+    # resident workgroups pulling Q tiles from per-XCD queues compute the same bits as a workgroup
+    # per Q tile, on both operand layouts; twice in a row (the queues are cleared by every launch)
+    shape, k, s, d, causal, H, Hkv, D = case
+    q, kk, v = make_qkv(3, shape, H, Hkv, D, dtype, seed=11)
+    with torch.no_grad():
+        ref = amd_fna_generic(q, kk, v, k, s, d, causal, return_lse=True, run_persistent_kernel=False)
+        for _ in range(2):
+            got = amd_fna_generic(q, kk, v, k, s, d, causal, return_lse=True, run_persistent_kernel=True)
+            assert torch.equal(got[0], ref[0]) and torch.equal(got[1], ref[1])
+        got = amd_fna_generic(q, kk, v, k, s, d, causal, return_lse=True, run_persistent_kernel=True, fused=False)
+        assert torch.equal(got[0], ref[0]) and torch.equal(got[1], ref[1])
+    ref_o, ref_l = oracle_full(q, kk, v, k, s, d, causal)
+    assert_close("out", to_np(got[0]), ref_o)
+    assert_close("lse", to_np(got[1]), ref_l)
+
+
+def test_work_queue_launch_many_more_tiles_than_workgroups():
+    # 24 x 900 Q tiles against 512 resident workgroups, non-causal and causal, through the public API
+    q, kk, v = make_qkv(1, (30, 48, 80), 4, 4, 128, torch.float16, seed=5)
+    for causal in ((False, False, False), (True, False, False)):
+        args = ((18, 24, 24), (16, 8, 8), (1, 1, 1), causal)
+        with torch.no_grad():
+            a = natten_amd.na3d(q, kk, v, *args, return_lse=True, run_persistent_kernel=True)
+            b = natten_amd.na3d(q, kk, v, *args, return_lse=True, run_persistent_kernel=False)
+            c = natten_amd.na3d(q, kk, v, *args, return_lse=True)  # the default picks one of the two
+        assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+        assert torch.equal(c[0], b[0]) and torch.equal(c[1], b[1])
+
+
+def test_work_queue_launch_replays_from_a_graph():
+    # the launch clears its queues with a kernel, so the pair can be captured; replays with new
+    # inputs and eager work in between give the eager bits every time
+    q, kk, v = make_qkv(2, (32, 48), 2, 2, 64, torch.bfloat16, seed=9)
+    args = ((9, 7), (2, 1), (1, 1), (False, False))
+    sq, sk, sv = q.clone(), kk.clone(), v.clone()
+    stream = torch.cuda.Stream()
+    with torch.no_grad(), torch.cuda.stream(stream):
+        amd_fna_generic(sq, sk, sv, *args, return_lse=True, run_persistent_kernel=True)  # warm up outside the capture
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=stream):
+            out, lse = amd_fna_generic(sq, sk, sv, *args, return_lse=True, run_persistent_kernel=True)
+    for seed in (1, 2, 3):
+        nq, nk, nv = make_qkv(2, (32, 48), 2, 2, 64, torch.bfloat16, seed=seed)
+        sq.copy_(nq), sk.copy_(nk), sv.copy_(nv)
+        g.replay()
+        torch.cuda.synchronize()
+        with torch.no_grad():
+            eo, el = amd_fna_generic(nq, nk, nv, *args, return_lse=True, run_persistent_kernel=False)
+        assert torch.equal(out, eo) and torch.equal(lse, el), f"replay {seed}"

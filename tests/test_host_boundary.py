@@ -175,7 +175,8 @@ def test_every_entry_point_rejects_null_arguments_before_touching_a_device():
     import ctypes as C
 
     L = _lib.lib()
-    skipped = {"natten_amd_abi_version", "natten_amd_last_error", "natten_amd_fna_supported_tiles"}
+    skipped = {"natten_amd_abi_version", "natten_amd_last_error", "natten_amd_fna_supported_tiles",
+               "natten_amd_fna_forward_workspace_bytes"}
     checked = 0
     for name, (_, arg_types) in _lib._SIGNATURES.items():
         if name in skipped:
@@ -186,3 +187,21 @@ def test_every_entry_point_rejects_null_arguments_before_touching_a_device():
         assert L.natten_amd_last_error(), f"{name} returned an error without a message"
         checked += 1
     assert checked >= 14
+
+
+def test_work_queue_launch_needs_a_workspace():
+    # run_persistent without a workspace, with one that is too small, or misaligned: refused with
+    # a message before any device call (the other arguments are not even looked at)
+    import ctypes as C
+
+    L = _lib.lib()
+    need = L.natten_amd_fna_forward_workspace_bytes()
+    assert need == 512
+    for name in ("natten_amd_fna_forward", "natten_amd_fna_forward_fused"):
+        arg_types = _lib._SIGNATURES[name][1]
+        for ws, nbytes in ((None, 0), (4096, need - 1), (4096 + 32, need)):
+            args = [None if a is C.c_void_p else (0.0 if a is C.c_float else 0) for a in arg_types]
+            args[6] = 1  # na_dim
+            args[-4], args[-3], args[-2] = 1, ws, nbytes
+            assert getattr(L, name)(*args) != 0
+            assert b"workspace" in L.natten_amd_last_error(), L.natten_amd_last_error()
