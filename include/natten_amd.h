@@ -127,6 +127,29 @@ int natten_amd_fna_forward_fused(const void* q, const void* k, const void* v, vo
                                  uint64_t workspace_bytes, void* stream);
 
 /*
+ * natten_amd_fna_forward_fused with run_persistent = 1 for callers that cannot allocate device
+ * memory (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc):
+ * it has no counterpart in the reference.  The queue counters live in a 512-byte array inside
+ * the library's device image instead of a workspace, and the call allocates and frees nothing
+ * (no hipMalloc / hipFree, no allocating library routine).  Operands, results and arguments
+ * are those of natten_amd_fna_forward_fused; limits: fp16 / bf16 operands, Q tiles of 128 and
+ * KV tiles of 64 tokens (the work-queue kernel's), at most 2^31 - 4096 Q tiles over all
+ * (batch, head) pairs; anything else is refused with an error.  Results are bit-identical to
+ * natten_amd_fna_forward_fused.  Every call on a GPU shares that GPU's array (the launch clears
+ * it first, with a kernel): calls that overlap in time on one GPU -- on different streams or
+ * from different threads -- race on the queues and must not be made; calls queued on one
+ * stream are fine.
+ */
+int natten_amd_fna_forward_fused_static(const void* q, const void* k, const void* v, void* out,
+                                        float* lse, int dtype, int na_dim, int batch, int heads_q,
+                                        int heads_kv, int head_dim, const int32_t* qkv_shape,
+                                        const int32_t* kernel_size, const int32_t* stride,
+                                        const int32_t* dilation, const int32_t* is_causal,
+                                        const int32_t* q_tile_shape, const int32_t* kv_tile_shape,
+                                        float scale, const float* q_scale, const float* k_scale,
+                                        const float* v_scale, void* stream);
+
+/*
  * Supported tile sizes (tokens per tile).  Writes up to `capacity` pairs
  * (q_tile_size, kv_tile_size) for the given dtype / head_dim and returns how many exist.
  */

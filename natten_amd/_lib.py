@@ -55,6 +55,10 @@ _SIGNATURES = {
         [ctypes.c_void_p] * 5 + [ctypes.c_int] * 6 + [ctypes.c_void_p] * 7 + [ctypes.c_float] + [ctypes.c_void_p] * 3
         + [ctypes.c_int, ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p],
     ),
+    "natten_amd_fna_forward_fused_static": (
+        ctypes.c_int,
+        [ctypes.c_void_p] * 5 + [ctypes.c_int] * 6 + [ctypes.c_void_p] * 7 + [ctypes.c_float] + [ctypes.c_void_p] * 4,
+    ),
     "natten_amd_attention_forward": (
         ctypes.c_int,
         [ctypes.c_void_p] * 5 + [ctypes.c_int] * 8 + [ctypes.c_float] + [ctypes.c_void_p] * 4,
@@ -281,6 +285,35 @@ def fna_forward_fused(
         )
     _check(rc)
     return out, lse
+
+
+def fna_forward_fused_static(
+    q: Tensor, k: Tensor, v: Tensor, out: Tensor, lse: Tensor,
+    kernel_size, stride, dilation, is_causal, scale: float, q_tile_shape, kv_tile_shape,
+) -> None:
+    """fna_forward_fused as a work-queue launch whose queues live in the library's own device
+    image: the call allocates nothing, so the caller passes the results' buffers too
+    (out like q, lse float32 [B, *X, H]).  For callers that cannot allocate; calls that overlap
+    in time on one GPU must not be made."""
+    L = lib()
+    _require_gpu(q, k, v, out, lse)
+    if q.dtype not in (torch.float16, torch.bfloat16):
+        raise NotImplementedError(f"natten_amd fna_forward_fused_static does not support {q.dtype}.")
+    if out.shape != q.shape or out.dtype != q.dtype or not out.is_contiguous():
+        raise ValueError("out must be a contiguous tensor of q's shape and dtype.")
+    if lse.shape != q.shape[:-1] or lse.dtype != torch.float32 or not lse.is_contiguous():
+        raise ValueError("lse must be a contiguous float32 tensor of q's shape without the last dimension.")
+    na_dim = len(kernel_size)
+    qkv_shape = [int(x) for x in q.shape[1 : 1 + na_dim]]
+    with torch.cuda.device(q.device):
+        rc = L.natten_amd_fna_forward_fused_static(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
+            DTYPE_CODES[q.dtype], na_dim, q.shape[0], q.shape[-2], k.shape[-2], q.shape[-1],
+            _i32(qkv_shape), _i32(kernel_size), _i32(stride), _i32(dilation),
+            _i32([1 if c else 0 for c in is_causal]), _i32(q_tile_shape), _i32(kv_tile_shape),
+            float(scale), None, None, None, _stream(q),
+        )
+    _check(rc)
 
 
 def attention_forward(

@@ -9,6 +9,7 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <mutex>
 #include <type_traits>
 
 #include "fna_bwd.hpp"
@@ -20,6 +21,14 @@
 #include "tokperm.hpp"
 
 using namespace natten_amd;
+
+// Queue counters of natten_amd_fna_forward_fused_static, the entry point for callers that cannot
+// allocate: every GPU the library runs on holds this array (512 bytes) until the process ends.
+// The name is a host-side stand-in, not a device address: host code only ever uses the
+// per-device address hipGetSymbolAddress returns for it (static_scratch()).  No `used`
+// attribute: the compiler gives the device-side symbol external binding because host code names
+// it, and with the attribute it stays local, where the runtime's lookup by name cannot find it.
+static __device__ __align__(256) uint32_t scratch[kQueueWords];
 
 namespace {
 
@@ -298,17 +307,14 @@ int natten_amd_fna_forward(const void* q, const void* k, const void* v, void* ou
   return dispatch_dtype(p, dtype, head_dim, prod3(p.q_tile), prod3(p.kv_tile), static_cast<hipStream_t>(stream), queues);
 }
 
-int natten_amd_fna_forward_fused(const void* q, const void* k, const void* v, void* out, float* lse, int dtype,
-                                 int na_dim, int batch, int heads_q, int heads_kv, int head_dim,
-                                 const int32_t* qkv_shape, const int32_t* kernel_size, const int32_t* stride,
-                                 const int32_t* dilation, const int32_t* is_causal, const int32_t* q_tile_shape,
-                                 const int32_t* kv_tile_shape, float scale, const float* q_scale,
-                                 const float* k_scale, const float* v_scale, int run_persistent, void* workspace,
-                                 uint64_t workspace_bytes, void* stream) {
-  g_error[0] = 0;
-  if (na_dim < 1 || na_dim > 3) return fail("fna_forward_fused: na_dim must be 1, 2 or 3, got %d", na_dim);
-  uint32_t* queues;
-  if (int rc = queue_workspace("fna_forward_fused", run_persistent, workspace, workspace_bytes, &queues)) return rc;
+namespace {
+// natten_amd_fna_forward_fused after its workspace has been resolved (`queues` == nullptr: a workgroup per Q tile)
+int fna_forward_fused_impl(const void* q, const void* k, const void* v, void* out, float* lse, int dtype, int na_dim,
+                           int batch, int heads_q, int heads_kv, int head_dim, const int32_t* qkv_shape,
+                           const int32_t* kernel_size, const int32_t* stride, const int32_t* dilation,
+                           const int32_t* is_causal, const int32_t* q_tile_shape, const int32_t* kv_tile_shape,
+                           float scale, const float* q_scale, const float* k_scale, const float* v_scale,
+                           uint32_t* queues, void* stream) {
   if (!qkv_shape || !kernel_size || !stride || !dilation || !is_causal || !q_tile_shape || !kv_tile_shape)
     return fail("fna_forward_fused: null shape argument");
   int qs[3] = {1, 1, 1}, ks[3] = {1, 1, 1};
@@ -358,6 +364,87 @@ int natten_amd_fna_forward_fused(const void* q, const void* k, const void* v, vo
   p.tokens = int(tokens);
   set_wg_layout(p, 1);
   return dispatch_dtype(p, dtype, head_dim, prod3(p.q_tile), prod3(p.kv_tile), static_cast<hipStream_t>(stream), queues);
+}
+}  // namespace
+
+int natten_amd_fna_forward_fused(const void* q, const void* k, const void* v, void* out, float* lse, int dtype,
+                                 int na_dim, int batch, int heads_q, int heads_kv, int head_dim,
+                                 const int32_t* qkv_shape, const int32_t* kernel_size, const int32_t* stride,
+                                 const int32_t* dilation, const int32_t* is_causal, const int32_t* q_tile_shape,
+                                 const int32_t* kv_tile_shape, float scale, const float* q_scale,
+                                 const float* k_scale, const float* v_scale, int run_persistent, void* workspace,
+                                 uint64_t workspace_bytes, void* stream) {
+  g_error[0] = 0;
+  if (na_dim < 1 || na_dim > 3) return fail("fna_forward_fused: na_dim must be 1, 2 or 3, got %d", na_dim);
+  uint32_t* queues;
+  if (int rc = queue_workspace("fna_forward_fused", run_persistent, workspace, workspace_bytes, &queues)) return rc;
+  return fna_forward_fused_impl(q, k, v, out, lse, dtype, na_dim, batch, heads_q, heads_kv, head_dim, qkv_shape,
+                                kernel_size, stride, dilation, is_causal, q_tile_shape, kv_tile_shape, scale, q_scale,
+                                k_scale, v_scale, queues, stream);
+}
+
+namespace {
+// Device address of `scratch` on the current device, looked up once per device (each GPU holds
+// its own copy of the array at its own address); nullptr + error message on failure.
+uint32_t* static_scratch(const char* what) {
+  constexpr int kMaxDevices = 64;
+  static uint32_t* ptrs[kMaxDevices] = {};
+  static std::mutex lock;
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    fail("%s: cannot identify the current device (%s, device %d)", what, hipGetErrorString(e), dev);
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> guard(lock);
+  if (ptrs[dev] == nullptr) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || ptr == nullptr) {
+      fail("%s: hipGetSymbolAddress(scratch) failed on device %d: %s", what, dev, hipGetErrorString(e));
+      return nullptr;
+    }
+    ptrs[dev] = static_cast<uint32_t*>(ptr);
+  }
+  return ptrs[dev];
+}
+}  // namespace
+
+int natten_amd_fna_forward_fused_static(const void* q, const void* k, const void* v, void* out, float* lse, int dtype,
+                                        int na_dim, int batch, int heads_q, int heads_kv, int head_dim,
+                                        const int32_t* qkv_shape, const int32_t* kernel_size, const int32_t* stride,
+                                        const int32_t* dilation, const int32_t* is_causal,
+                                        const int32_t* q_tile_shape, const int32_t* kv_tile_shape, float scale,
+                                        const float* q_scale, const float* k_scale, const float* v_scale,
+                                        void* stream) {
+  g_error[0] = 0;
+  const char* what = "fna_forward_fused_static";
+  if (na_dim < 1 || na_dim > 3) return fail("%s: na_dim must be 1, 2 or 3, got %d", what, na_dim);
+  if (!qkv_shape || !q_tile_shape || !kv_tile_shape) return fail("%s: null shape argument", what);
+  // only the work-queue kernel uses the scratch array: 16-bit operands, 128 x 64 token tiles
+  if (dtype != NATTEN_AMD_F16 && dtype != NATTEN_AMD_BF16)
+    return fail("%s: the work-queue kernel takes fp16 / bf16 operands, got dtype code %d", what, dtype);
+  long long qt = 1, kvt = 1, q_tiles = 1;
+  for (int a = 0; a < na_dim; ++a) {
+    if (q_tile_shape[a] < 1 || kv_tile_shape[a] < 1 || qkv_shape[a] < 1 || !dilation || dilation[a] < 1)
+      return fail("%s: invalid parameter along dimension %d", what, a);
+    qt *= q_tile_shape[a];
+    kvt *= kv_tile_shape[a];
+    const long long ext = (qkv_shape[a] + dilation[a] - 1) / dilation[a];
+    q_tiles *= (ext + q_tile_shape[a] - 1) / q_tile_shape[a] * dilation[a];
+  }
+  if (qt != 128 || kvt != 64)
+    return fail("%s: the work-queue kernel exists for Q tiles of 128 and KV tiles of 64 tokens, got %lld and %lld", what, qt,
+                kvt);
+  // the queues hold 32-bit positions: at most 2^28 Q tiles per queue (2^31 in all); the array itself never grows
+  if (batch < 1 || heads_q < 1 || q_tiles * batch * heads_q > (1LL << 31) - 4096)
+    return fail("%s: %lld Q tiles x %d x %d exceed the 2^31 positions the static queues can count", what, q_tiles, batch,
+                heads_q);
+  uint32_t* queues = static_scratch(what);
+  if (queues == nullptr) return 1;
+  return fna_forward_fused_impl(q, k, v, out, lse, dtype, na_dim, batch, heads_q, heads_kv, head_dim, qkv_shape,
+                                kernel_size, stride, dilation, is_causal, q_tile_shape, kv_tile_shape, scale, q_scale,
+                                k_scale, v_scale, queues, stream);
 }
 
 int natten_amd_attention_forward(const void* q, const void* k, const void* v, void* out, float* lse, int dtype,
