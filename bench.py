@@ -41,6 +41,9 @@ WORKLOADS = {
     "hunyuan_gna": (1, 24, (30, 48, 80), 128, (18, 24, 24), (16, 8, 8), (1, 1, 1), (False, False, False), "fp16", 1.0),
     "flux_na": (1, 24, (256, 256), 128, (80, 80), (1, 1), (1, 1), (False, False), "fp16", 1.0),
     "flux_gna": (1, 24, (256, 256), 128, (80, 80), (16, 16), (1, 1), (False, False), "fp16", 1.0),
+    # extents that no tile shape divides (and an uneven dilation in time): the one-launch route clamps
+    # its gathers; compare `ms_per_step` with `e2e_permuted_route_ms`
+    "odd3d": (1, 24, (29, 46, 78), 128, (9, 24, 24), (1, 8, 8), (2, 1, 1), (False, False, False), "bf16", 1.0),
 }
 # Published forward runtimes of the reference's Blackwell FNA kernel on a B200 for those shapes
 # (kernel only / with token permute; docs/sample-outputs/profiler-*-blackwell-fna-b200.txt): other
@@ -61,6 +64,7 @@ CPU_PROXY = {
     "hunyuan_gna": ((20, 24, 24), 2),
     "flux_na": ((96, 96), 2),
     "flux_gna": ((96, 96), 2),
+    "odd3d": ((19, 25, 27), 2),
 }
 # HBM-side traffic of a launch (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, calibrated on a copy of known
 # size) is read from the profile summaries, which carry one line per measurement:
@@ -109,6 +113,7 @@ WORKLOAD_NAMES = {
     "hunyuan_gna": "na3d fp16 B=1 H=24 30x48x80 D=128 k=(18,24,24) s=(16,8,8)",
     "flux_na": "na2d fp16 B=1 H=24 256x256 D=128 k=(80,80)",
     "flux_gna": "na2d fp16 B=1 H=24 256x256 D=128 k=(80,80) s=(16,16)",
+    "odd3d": "na3d bf16 B=1 H=24 29x46x78 D=128 k=(9,24,24) s=(1,8,8) d=(2,1,1)",
 }
 
 
@@ -481,7 +486,8 @@ def main():
             tp_in = q
         scale = D**-0.5
 
-        fused = _lib.fused_layout_supported(layout, dilation, kv_tile)
+        fused = _lib.fused_layout_supported(layout, dilation, kv_tile, q_tile_shape=q_tile,
+                                            dtype=None if quantised else dtype)
 
         def kern_permuted():
             return _lib.fna_forward(qp, kp, vp, kernel, stride, dilation, causal, scale, q_shape, kv_shape,

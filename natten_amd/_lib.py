@@ -251,12 +251,26 @@ def _tile_span_fits(token_layout, dilation, tile_shape, row_bytes: int) -> bool:
     return (span + 1) * row_bytes + 8192 < 2**31 - 1
 
 
-def fused_layout_supported(qkv_shape, dilation, kv_tile_shape, row_bytes: int = 0) -> bool:
-    """Whether fna_forward_fused accepts this problem: no KV tile may reach past the input, and
-    (given `row_bytes` = heads_kv * head_dim * 2) a KV tile spans less than 2^31 bytes of it."""
-    return all(X % (d * t) == 0 for X, d, t in zip(qkv_shape, dilation, kv_tile_shape)) and _tile_span_fits(
-        qkv_shape, dilation, kv_tile_shape, row_bytes
-    )
+def fused_layout_supported(qkv_shape, dilation, kv_tile_shape, row_bytes: int = 0, q_tile_shape=None,
+                           dtype: Optional[torch.dtype] = None) -> bool:
+    """Whether fna_forward_fused accepts this problem.  Always: (given `row_bytes` = heads_kv *
+    head_dim * 2) a KV tile spans less than 2^31 bytes of the input.  When every extent is a multiple
+    of dilation x KV tile no KV tile reaches past its dilation group.  Otherwise (`q_tile_shape`
+    and `dtype` given) the operands must be fp16 / bf16, and if some dilation group is narrower than
+    the KV tile in a dimension the tiles must be 128 x 64 tokens (the one instance that clamps)."""
+    if not _tile_span_fits(qkv_shape, dilation, kv_tile_shape, row_bytes):
+        return False
+    if all(X % (d * t) == 0 for X, d, t in zip(qkv_shape, dilation, kv_tile_shape)):
+        return True
+    if q_tile_shape is None or dtype not in (torch.float16, torch.bfloat16):
+        return False
+    if all(X // d >= t for X, d, t in zip(qkv_shape, dilation, kv_tile_shape)):
+        return True
+    q_tokens = kv_tokens = 1
+    for tq, tk in zip(q_tile_shape, kv_tile_shape):
+        q_tokens *= tq
+        kv_tokens *= tk
+    return q_tokens == 128 and kv_tokens == 64
 
 
 def fna_forward_fused(

@@ -57,6 +57,12 @@ struct FnaParams {
   // (every dilation group's extent must be a multiple of the KV tile in each dimension, so
   // that no KV tile reaches past the input).
   int fused;
+  // fused == 1 only: some KV tile would reach past a dilation group's extent (extents that are
+  // not multiples of dilation x KV tile).  1: every group is at least one KV tile wide in every
+  // dimension; such a tile is then gathered from where it ends at the group's last position, and its
+  // leading keys (which the tile before it already delivered) are masked.  2: the RAGGED instance,
+  // which gathers the tile where it is and clamps the rows that fall outside the group.
+  int edge;
   int tok_stride[3];  // tokens per unit step of an original coordinate: X1*X2, X2, 1
   int tokens;         // X0 * X1 * X2
   // Sequence-packed dense attention (RAGGED instances only; null otherwise): `batch` sequences
@@ -500,20 +506,33 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
     const char* src;  // first row of the tile (this head)
     uint32_t lds0;    // LDS byte address of this wave's first chunk
     int row0;
-    bool inside;      // the whole tile lies inside the sequence
+    int lim[3];       // original layout: positions of the tile that lie inside the dilation group, per dimension
+    bool inside;      // the whole tile lies inside the sequence / the dilation group
   };
-  auto make_copy = [&](const T* base, char* dst, int kv_row0) {
+  auto make_copy = [&](const T* base, char* dst, int kv_row0, const int (&origin)[3]) {
     TileCopy c;
     kv_row0 = __builtin_amdgcn_readfirstlane(kv_row0);  // uniform by construction; keeps the base in scalar registers
     c.src = reinterpret_cast<const char*>(base) + int64_t(kv_row0) * kv_row_stride * 2 - (RAGGED ? 0 : kImmBias);
     c.lds0 = lds_address(dst) + uint32_t(wave * PER * 1024);
     c.row0 = kv_row0;
-    c.inside = kv_row0 + KVT <= seqlen_kv;
+    c.inside = true;
+    if constexpr (RAGGED) {
+      if (p.fused) {
+#pragma unroll
+        for (int a = 0; a < 3; ++a) {
+          c.lim[a] = na_min(extent[a] - origin[a], p.kv_tile[a]);
+          c.inside = c.inside && (c.lim[a] == p.kv_tile[a]);
+        }
+      } else {
+        c.inside = kv_row0 + KVT <= seqlen_kv;
+      }
+    }
     return c;
   };
-  // issues copy I (0 <= I < PER) of a tile
-  auto copy_one = [&](auto i_tag, const TileCopy& c, const uint32_t (&off)[NOFF]) {
+  // issues copy I (0 <= I < PER) of a tile; V_LAYOUT selects the LDS swizzle of the operand
+  auto copy_one = [&](auto i_tag, const TileCopy& c, const uint32_t (&off)[NOFF], auto v_tag) {
     constexpr int I = decltype(i_tag)::value;
+    constexpr bool V_LAYOUT = decltype(v_tag)::value;
     if constexpr (I < PER) {
       if (CHUNKS % (NT * PER) == 0 || (wave * PER + I) * 64 < CHUNKS) {
         constexpr int IMM = (I % 4) * 1024;
@@ -521,10 +540,28 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
         uint32_t voff = off[I % 4];
         if constexpr (RAGGED) {
           if (!c.inside) {
-            // last, partial tile of an unpadded sequence: rows past the end are masked; read the
-            // last valid row instead so that no out-of-bounds address is formed
-            const int over = na_max(c.row0 + ld_row[I % 4] + (I / 4) * ROWS_PER_4 - (seqlen_kv - 1), 0);
-            voff -= uint32_t(over) * uint32_t(kv_row_stride * 2);
+            if (p.fused) {
+              // a tile that reaches past its dilation group (original layout): positions beyond
+              // the group's extent are masked; gather the group's last row along that dimension
+              // instead, so that no address outside the tensor is formed.  The LDS placement
+              // (and with it the order of every sum) stays that of the whole tile.
+              const int P = (wave * PER + I) * 64 + lane;
+              const int r = P / CPR, slot = P % CPR;
+              int t0 = r % p.kv_tile[0];
+              const int r1 = r / p.kv_tile[0];
+              int t1 = r1 % p.kv_tile[1], t2 = r1 / p.kv_tile[1];
+              t0 = na_min(t0, c.lim[0] - 1);
+              t1 = na_min(t1, c.lim[1] - 1);
+              t2 = na_min(t2, c.lim[2] - 1);
+              const uint32_t pos = uint32_t(t0 * tok_step[0] + t1 * tok_step[1] + t2 * tok_step[2]);
+              voff = pos * uint32_t(kv_row_stride * 2) + uint32_t((V_LAYOUT ? L::v_slot(r, slot) : L::k_slot(r, slot)) * 16);
+              src = c.src;
+            } else {
+              // last, partial tile of an unpadded sequence: rows past the end are masked; read the
+              // last valid row instead so that no out-of-bounds address is formed
+              const int over = na_max(c.row0 + ld_row[I % 4] + (I / 4) * ROWS_PER_4 - (seqlen_kv - 1), 0);
+              voff -= uint32_t(over) * uint32_t(kv_row_stride * 2);
+            }
           }
           // the clamped per-lane offset may be smaller than the immediate: take the immediate
           // off the uniform base instead
@@ -535,23 +572,24 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
     }
   };
   static_assert(PER <= 8, "tile copy is written for at most eight copies per thread");
-  auto issue_tile_load = [&](const T* base, const uint32_t (&off)[NOFF], char* dst, int kv_row0) {
-    const TileCopy c = make_copy(base, dst, kv_row0);
-    copy_one(std::integral_constant<int, 0>{}, c, off);
-    copy_one(std::integral_constant<int, 1>{}, c, off);
-    copy_one(std::integral_constant<int, 2>{}, c, off);
-    copy_one(std::integral_constant<int, 3>{}, c, off);
-    copy_one(std::integral_constant<int, 4>{}, c, off);
-    copy_one(std::integral_constant<int, 5>{}, c, off);
-    copy_one(std::integral_constant<int, 6>{}, c, off);
-    copy_one(std::integral_constant<int, 7>{}, c, off);
+  auto issue_tile_load = [&](const T* base, const uint32_t (&off)[NOFF], char* dst, int kv_row0, const int (&origin)[3],
+                             auto v_tag) {
+    const TileCopy c = make_copy(base, dst, kv_row0, origin);
+    copy_one(std::integral_constant<int, 0>{}, c, off, v_tag);
+    copy_one(std::integral_constant<int, 1>{}, c, off, v_tag);
+    copy_one(std::integral_constant<int, 2>{}, c, off, v_tag);
+    copy_one(std::integral_constant<int, 3>{}, c, off, v_tag);
+    copy_one(std::integral_constant<int, 4>{}, c, off, v_tag);
+    copy_one(std::integral_constant<int, 5>{}, c, off, v_tag);
+    copy_one(std::integral_constant<int, 6>{}, c, off, v_tag);
+    copy_one(std::integral_constant<int, 7>{}, c, off, v_tag);
   };
 
   // KV tile stream: dimension 2 fastest, dimension 0 slowest.  The load stream runs up to two
   // tiles ahead of the softmax, so tile descriptors are produced in order and handed down.
   struct TileInfo {
     int row0;       // first row of the tile in the permuted KV sequence / token offset of its origin (fused)
-    int origin[3];  // coordinate of its first token
+    int origin[3];  // coordinate of its first token (a tile moved back from the group's edge: of the first one gathered)
     bool full;      // every key of the tile is attended by every query of this wave
     bool skip;      // no key of the tile is attended by any query of this wave
   };
@@ -562,10 +600,12 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
     t.skip = false;
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
-      t.origin[a] = (box_tile0[a] + itc[a]) * p.kv_tile[a];
-      const int end = t.origin[a] + p.kv_tile[a];
-      t.full = t.full && (t.origin[a] >= wave_full_lo[a]) && (end <= wave_full_hi[a]);
-      t.skip = t.skip || (end <= wave_lo[a]) || (t.origin[a] >= wave_hi[a]);
+      const int org = (box_tile0[a] + itc[a]) * p.kv_tile[a];
+      const int end = org + p.kv_tile[a];
+      t.full = t.full && (org >= wave_full_lo[a]) && (end <= wave_full_hi[a]);  // never when end > extent
+      t.skip = t.skip || (end <= wave_lo[a]) || (org >= wave_hi[a]);
+      // a tile that would reach past the group is moved back to end at the group's last position
+      t.origin[a] = (p.edge == 1) ? na_min(org, extent[a] - p.kv_tile[a]) : org;
     }
     t.row0 = p.fused ? t.origin[0] * tok_step[0] + t.origin[1] * tok_step[1] + t.origin[2] * tok_step[2]
                      : ((box_tile0[0] + itc[0]) + p.kv_tiled[0] * ((box_tile0[1] + itc[1]) + p.kv_tiled[1] * (box_tile0[2] + itc[2]))) * KVT;
@@ -582,8 +622,10 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
   using Stage0 = std::integral_constant<int, 0>;
   using Stage1 = std::integral_constant<int, 1>;
   TileInfo cur = next_tile();  // tile 0
-  issue_tile_load(kbase, ld_koff, sK0, cur.row0);
-  issue_tile_load(vbase, ld_voff, sV0, cur.row0);
+  using KLayout = std::false_type;
+  using VLayout = std::true_type;
+  issue_tile_load(kbase, ld_koff, sK0, cur.row0, cur.origin, KLayout{});
+  issue_tile_load(vbase, ld_voff, sV0, cur.row0, cur.origin, VLayout{});
 
   float sm_scale = p.scale, out_scale = 1.f;
   if (p.q_scale) sm_scale *= p.q_scale[head];
@@ -741,7 +783,10 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
     uint32_t addc = 0, subc = 0;
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
-      const int lo = na_min(na_max(ws[a] - origin[a], 0), p.kv_tile[a]);
+      // a tile moved back from the group's edge starts before its place in the tiling (the next
+      // multiple of the tile extent): the keys up to there belong to the tile before it
+      const int lead = na_ceil_div(origin[a], p.kv_tile[a]) * p.kv_tile[a] - origin[a];
+      const int lo = na_min(na_max(ws[a] - origin[a], lead), p.kv_tile[a]);
       const int hi = na_min(na_max(we[a] - origin[a], 0), p.kv_tile[a]);
       addc |= uint32_t(512 - lo) << (10 * a);
       subc |= uint32_t(511 + hi) << (10 * a);
@@ -832,7 +877,7 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
   TileInfo nxt = next_tile();  // tile 1 (a descriptor past the box is never used)
   wait_vmcnt<0>();
   __syncthreads();  // K(0), V(0) and the coordinate table are in LDS
-  if (1 < total_tiles) issue_tile_load(kbase, ld_koff, sK1, nxt.row0);
+  if (1 < total_tiles) issue_tile_load(kbase, ld_koff, sK1, nxt.row0, nxt.origin, KLayout{});
 #pragma unroll
   for (int mb = 0; mb < MQ; ++mb)
 #pragma unroll
@@ -872,11 +917,12 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
     const TileInfo t2 = next_tile();
     // Past the end of the box the spread copies re-read the current tile into the free stage
     // (never used), which keeps the slots below free of control flow.
-    const TileCopy ck = make_copy(kbase, sK_cur, (j + 2 < total_tiles) ? t2.row0 : cur.row0);
-    const TileCopy cv = make_copy(vbase, sV_nxt, (j + 1 < total_tiles) ? nxt.row0 : cur.row0);
+    // (the spread copies only exist without RAGGED, where a tile's origin is not looked at)
+    const TileCopy ck = make_copy(kbase, sK_cur, (j + 2 < total_tiles) ? t2.row0 : cur.row0, cur.origin);
+    const TileCopy cv = make_copy(vbase, sV_nxt, (j + 1 < total_tiles) ? nxt.row0 : cur.row0, cur.origin);
     if constexpr (!SPREAD) {
-      if (j + 2 < total_tiles) issue_tile_load(kbase, ld_koff, sK_cur, t2.row0);
-      if (j + 1 < total_tiles) issue_tile_load(vbase, ld_voff, sV_nxt, nxt.row0);
+      if (j + 2 < total_tiles) issue_tile_load(kbase, ld_koff, sK_cur, t2.row0, t2.origin, KLayout{});
+      if (j + 1 < total_tiles) issue_tile_load(vbase, ld_voff, sV_nxt, nxt.row0, nxt.origin, VLayout{});
     }
 
     // -- G1 ------------------------------------------------------------------------------------
@@ -915,8 +961,8 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
         constexpr int c_lo = (s * 2 * PER * 2) / N_QK, c_hi = ((s + 1) * 2 * PER * 2) / N_QK;
         for_range<c_lo, c_hi - c_lo>([&](auto c_tag) {
           constexpr int c = decltype(c_tag)::value;
-          if constexpr (c < PER) copy_one(std::integral_constant<int, c>{}, ck, ld_koff);
-          else if constexpr (c < 2 * PER) copy_one(std::integral_constant<int, c - PER>{}, cv, ld_voff);
+          if constexpr (c < PER) copy_one(std::integral_constant<int, c>{}, ck, ld_koff, KLayout{});
+          else if constexpr (c < 2 * PER) copy_one(std::integral_constant<int, c - PER>{}, cv, ld_voff, VLayout{});
         });
       }
       __builtin_amdgcn_sched_barrier(0);

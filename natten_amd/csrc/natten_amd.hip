@@ -121,7 +121,7 @@ int launch_fna_fp8(const FnaParams& p, hipStream_t stream) {
 
 template <typename T, int D>
 int dispatch_tiles(const FnaParams& p, int qt, int kvt, hipStream_t stream, uint32_t* queues) {
-  if (p.seqlen_kv % kvt != 0 || p.cu_q != nullptr) {
+  if (p.seqlen_kv % kvt != 0 || p.cu_q != nullptr || p.edge == 2) {
     // key sequences that end inside a tile: dense attention on unpadded or packed sequences only
     if (qt == 128 && kvt == 64) return launch_fna<T, D, 4, 1, true, 64>(p, stream);
     return fail("fna_forward: seqlen_kv (%d) must be a multiple of the KV tile (%d tokens)", p.seqlen_kv, kvt);
@@ -319,19 +319,34 @@ int fna_forward_fused_impl(const void* q, const void* k, const void* v, void* ou
     return fail("fna_forward_fused: null shape argument");
   int qs[3] = {1, 1, 1}, ks[3] = {1, 1, 1};
   long long tokens = 1;
+  // Extents that are not multiples of dilation x KV tile: some KV tile would reach past its
+  // dilation group.  1: every group is at least a KV tile wide everywhere, any kernel instance will
+  // do (such tiles are gathered from one tile extent before the group's end).  2: a group is
+  // narrower than the KV tile somewhere, only the instance that clamps its gathers will do.
+  int edge = 0;
   for (int a = 0; a < na_dim; ++a) {
     if (qkv_shape[a] < 1 || dilation[a] < 1 || q_tile_shape[a] < 1 || kv_tile_shape[a] < 1)
       return fail("fna_forward_fused: invalid parameter along dimension %d", a);
-    // every dilation group must have the same extent, a multiple of the KV tile: no KV tile
-    // may reach past the input, because the kernel gathers whole tiles without bounds checks
-    if (qkv_shape[a] % dilation[a] != 0 || (qkv_shape[a] / dilation[a]) % kv_tile_shape[a] != 0)
-      return fail("fna_forward_fused: the input extent %d along dimension %d is not a multiple of dilation * KV tile "
-                  "(%d * %d); use the token-permuted entry point",
-                  qkv_shape[a], a, dilation[a], kv_tile_shape[a]);
-    const int ext = qkv_shape[a] / dilation[a];
+    // dilation groups may differ in extent by one; the padded per-group layouts cover the largest
+    const int ext = na_ceil_div(qkv_shape[a], dilation[a]);
+    if (qkv_shape[a] % dilation[a] != 0 || ext % kv_tile_shape[a] != 0) edge = edge > 1 ? edge : 1;
+    if (qkv_shape[a] / dilation[a] < kv_tile_shape[a]) edge = 2;
     qs[a] = na_ceil_div(ext, q_tile_shape[a]) * q_tile_shape[a];
-    ks[a] = ext;
+    ks[a] = na_ceil_div(ext, kv_tile_shape[a]) * kv_tile_shape[a];
     tokens *= qkv_shape[a];
+  }
+  if (edge != 0) {
+    long long qt = 1, kvt = 1;
+    for (int a = 0; a < na_dim; ++a) {
+      qt *= q_tile_shape[a];
+      kvt *= kv_tile_shape[a];
+    }
+    if (dtype != NATTEN_AMD_F16 && dtype != NATTEN_AMD_BF16)
+      return fail("fna_forward_fused: an input extent that is not a multiple of dilation * KV tile in every dimension "
+                  "needs fp16 / bf16 operands (got dtype code %d); use the token-permuted entry point", dtype);
+    if (edge == 2 && (qt != 128 || kvt != 64))
+      return fail("fna_forward_fused: a dilation group narrower than the KV tile needs tiles of 128 x 64 tokens (got "
+                  "%lld x %lld); use the token-permuted entry point", qt, kvt);
   }
   if (tokens > 0x7fffffffLL) return fail("fna_forward_fused: more than 2^31 tokens per batch");
   if (int rc = check_common("fna_forward_fused", q, k, v, out, lse, batch, prod3(qs), prod3(ks), heads_q, heads_kv,
@@ -361,6 +376,7 @@ int fna_forward_fused_impl(const void* q, const void* k, const void* v, void* ou
   p.k_scale = k_scale;
   p.v_scale = v_scale;
   p.fused = 1;
+  p.edge = edge;
   p.tokens = int(tokens);
   set_wg_layout(p, 1);
   return dispatch_dtype(p, dtype, head_dim, prod3(p.q_tile), prod3(p.kv_tile), static_cast<hipStream_t>(stream), queues);

@@ -159,10 +159,12 @@ def amd_fna_generic(
     use_fp8 = fp8_ok and fp8_matmul is not False
     widen = is_fp8(in_dtype) and not use_fp8
     fusable = (not widen) and _lib.fused_layout_supported(query.shape[1 : 1 + na_dim], dilation, kv_tile_shape,
-                                                          row_bytes=key.shape[-2] * d_pad * 2)
+                                                          row_bytes=key.shape[-2] * d_pad * 2,
+                                                          q_tile_shape=q_tile_shape, dtype=in_dtype)
     if fused and not fusable:
         raise ValueError(
-            "natten_amd: the fused path needs operands that are not widened and an input extent that is a multiple of "
+            "natten_amd: the fused path needs operands that are not widened and, unless they are fp16 / bf16 with tiles of "
+            "128 x 64 tokens, an input extent that is a multiple of "
             f"dilation * KV tile in every dimension; got {tuple(query.shape[1:1 + na_dim])}, {dilation=}, "
             f"{kv_tile_shape=}, {in_dtype}."
         )

@@ -100,3 +100,23 @@ def sampled_check(q, k, v, out, lse, kernel, stride, dilation, causal, n_samples
         got_l = to_np(lse[b].reshape(N, H)[ti])
         assert_close(f"sampled out {tag} batch {b}", got_o, ref_o, atol, rtol)
         assert_close(f"sampled lse {tag} batch {b}", got_l, ref_l, atol, rtol)
+
+
+def routes_agree_bit_for_bit(shape, dilation, kv_tile) -> bool:
+    """Whether the one-launch route and the permuted route place every key at the same position of
+    its KV tile (then all sums run in the same order and the results are bit-identical).  Not so
+    when an extent is no multiple of dilation x KV tile while every dilation group is at least a
+    tile wide: the one-launch route then gathers the last tile of such a dimension from one tile
+    extent before the group's end (its leading keys masked) instead of padding it."""
+    if all(X % (d * t) == 0 for X, d, t in zip(shape, dilation, kv_tile)):
+        return True
+    return not all(X // d >= t for X, d, t in zip(shape, dilation, kv_tile))
+
+
+def assert_routes_agree(tag, a, b, shape, dilation, kv_tile):
+    """Outputs / LSEs of the two routes: bit-equal where the key placement is the same, else equal up
+    to the order of summation (a few units in the last place of the 16-bit result)."""
+    if routes_agree_bit_for_bit(shape, dilation, kv_tile):
+        assert torch.equal(a, b), "the two routes differ: " + tag
+    else:
+        assert_close("routes " + tag, to_np(a), to_np(b), atol=4e-3, rtol=8e-3)

@@ -17,7 +17,7 @@ import natten_amd
 from natten_amd.tile_config import get_all_backward_tile_shapes
 from oracle import c_oracle
 from oracle import na_oracle as O
-from tests.gpu_utils import assert_close, make_qkv, to_np, tuplify
+from tests.gpu_utils import assert_close, make_qkv, routes_agree_bit_for_bit, to_np, tuplify
 
 pytestmark = pytest.mark.gpu
 
@@ -50,8 +50,17 @@ def run_backward(B, H, Hkv, D, shape, k, s, d, causal, dtype, bq=None, bkv=None,
         q2, k2, v2 = (t.detach().clone().requires_grad_(True) for t in (q, kk, v))
         amd_fna_generic(q2, k2, v2, k, s, d, causal, backward_q_tile_shape=bq, backward_kv_tile_shape=bkv,
                         fused=False).backward(d_out)
+        # (the forward results the backward starts from are only bit-equal between the routes where
+        # both place the keys alike in their tiles; elsewhere they agree up to summation order)
+        from natten_amd.tile_config import check_fna_forward_config
+
+        _, fwd_kt = check_fna_forward_config(q, k, s, d, causal, None, None)
+        exact = routes_agree_bit_for_bit(shape, d, fwd_kt)
         for name, a, b in zip(("dq", "dk", "dv"), (q.grad, kk.grad, v.grad), (q2.grad, k2.grad, v2.grad)):
-            assert torch.equal(a, b), f"original-layout and permuted backward differ in {name}: {tag}"
+            if exact:
+                assert torch.equal(a, b), f"original-layout and permuted backward differ in {name}: {tag}"
+            else:
+                assert_close(f"routes {name} {tag}", to_np(a), to_np(b), atol=TOL[dtype] / 2, rtol=TOL[dtype] / 2)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])

@@ -7,7 +7,8 @@ import torch
 import natten_amd
 from natten_amd import _lib
 from natten_amd.fna import amd_fna_generic
-from tests.gpu_utils import assert_close, make_qkv, oracle_full, to_np
+from tests.gpu_utils import (assert_close, assert_routes_agree, make_qkv, oracle_full, routes_agree_bit_for_bit,
+                             sampled_check, to_np)
 
 pytestmark = pytest.mark.gpu
 
@@ -43,20 +44,76 @@ def test_fused_equals_permuted_and_oracle(case, dtype):
     assert_close("lse", to_np(lse_f), ref_l)
 
 
-def test_fused_rejects_inputs_that_kv_tiles_overrun():
-    q, kk, v = make_qkv(1, (20, 24), 2, 2, 64, torch.bfloat16, seed=1)
-    args = ((5, 7), (1, 1), (1, 1), (False, False))
-    assert not _lib.fused_layout_supported((20, 24), (1, 1), (8, 8))
+def test_fused_rejects_what_no_kernel_instance_gathers():
+    # a dilation group narrower than the KV tile needs the instance that clamps its gathers, which
+    # exists for tiles of 128 x 64 tokens: other tile pairs take the permuted route
+    q, kk, v = make_qkv(1, (20, 6), 2, 2, 64, torch.bfloat16, seed=1)
+    args = ((5, 3), (1, 1), (1, 1), (False, False))
+    assert not _lib.fused_layout_supported((20, 6), (1, 1), (8, 8))
+    assert not _lib.fused_layout_supported((20, 6), (1, 1), (8, 8), q_tile_shape=(8, 8), dtype=torch.bfloat16)
+    assert _lib.fused_layout_supported((20, 6), (1, 1), (8, 8), q_tile_shape=(16, 8), dtype=torch.bfloat16)
+    assert _lib.fused_layout_supported((20, 24), (1, 1), (8, 8), q_tile_shape=(8, 8), dtype=torch.bfloat16)
+    assert not _lib.fused_layout_supported((20, 24), (1, 1), (8, 8), q_tile_shape=(8, 8), dtype=torch.float8_e4m3fn)
     with pytest.raises(ValueError):
-        amd_fna_generic(q, kk, v, *args, q_tile_shape=(16, 8), kv_tile_shape=(8, 8), fused=True)
+        amd_fna_generic(q, kk, v, *args, q_tile_shape=(8, 8), kv_tile_shape=(8, 8), fused=True)
     with pytest.raises(RuntimeError):
-        _lib.fna_forward_fused(q, kk, v, *args, 0.125, (16, 8), (8, 8))
-    # the default picks the permuted path and still matches the oracle
+        _lib.fna_forward_fused(q, kk, v, *args, 0.125, (8, 8), (8, 8))
+    # the default picks the permuted path there and still matches the oracle
     with torch.no_grad():
-        out, lse = natten_amd.na2d(q, kk, v, *args, q_tile_shape=(16, 8), kv_tile_shape=(8, 8), return_lse=True)
+        out, lse = natten_amd.na2d(q, kk, v, *args, q_tile_shape=(8, 8), kv_tile_shape=(8, 8), return_lse=True)
     ref_o, ref_l = oracle_full(q, kk, v, *args)
     assert_close("out", to_np(out), ref_o)
     assert_close("lse", to_np(lse), ref_l)
+
+
+EDGE_CASES = [
+    # shape, kernel, stride, dilation, heads, heads_kv, D, q_tile, kv_tile: extents that are not
+    # multiples of dilation x KV tile (the reference's odd-sized problems among them)
+    ((125,), (15,), (1,), (1,), 2, 2, 64, (128,), (64,)),
+    ((125,), (3,), (1,), (1,), 1, 1, 32, (128,), (64,)),
+    ((257,), (8,), (7,), (5,), 2, 1, 64, (128,), (64,)),
+    ((84, 19), (7, 3), (1, 1), (1, 1), 1, 1, 32, (16, 8), (8, 8)),
+    ((84, 19), (7, 3), (1, 1), (5, 1), 1, 1, 32, (16, 8), (8, 8)),
+    ((19, 29), (8, 8), (1, 1), (2, 3), 1, 1, 128, (8, 16), (8, 8)),
+    ((67, 80), (12, 7), (8, 4), (5, 11), 1, 1, 128, (16, 8), (4, 16)),
+    ((5, 25), (5, 16), (1, 16), (1, 1), 2, 1, 48, (4, 32), (4, 16)),
+    ((33, 33), (24, 16), (1, 1), (1, 1), 1, 1, 128, (8, 16), (8, 8)),
+    ((13, 11, 9), (3, 4, 3), (2, 3, 3), (3, 2, 2), 1, 1, 32, (2, 8, 8), (1, 8, 8)),
+    ((18, 37, 12), (14, 16, 12), (12, 8, 1), (1, 2, 1), 1, 1, 64, (4, 8, 4), (2, 8, 4)),
+    ((57, 20, 88), (20, 4, 6), (1, 1, 1), (2, 1, 1), 1, 1, 72, (2, 4, 16), (2, 4, 8)),
+    # the other tile sizes (every group at least a tile wide)
+    ((84, 19), (7, 3), (1, 1), (1, 1), 2, 1, 64, (8, 8), (8, 8)),
+    ((30, 27, 21), (5, 9, 7), (1, 3, 1), (2, 1, 1), 1, 1, 128, (4, 8, 8), (1, 8, 8)),
+]
+
+
+@pytest.mark.parametrize("case", EDGE_CASES)
+def test_fused_on_extents_that_tiles_do_not_divide(case):
+    # one launch on the original tensors whatever the extents, within tolerance of the oracle,
+    # non-causal and causal.  Where a dilation group is narrower than the KV tile the kernel clamps
+    # its gathers, every key keeps its place in the tile and the result is bit-equal to permute +
+    # kernel + unpermute; elsewhere the last tile of a dimension is gathered from one tile extent
+    # before the group's end and the two routes agree up to the order of summation
+    shape, k, s, d, H, Hkv, D, qt, kt = case
+    n = len(shape)
+    assert not all(X % (dd * t) == 0 for X, dd, t in zip(shape, d, kt))
+    for ci, causal in enumerate([(False,) * n, (True,) + (False,) * (n - 1), (True,) * n]):
+        dtype = [torch.bfloat16, torch.float16][ci % 2]
+        q, kk, v = make_qkv(2, shape, H, Hkv, D, dtype, seed=13 + ci)
+        with torch.no_grad():
+            out_f, lse_f = amd_fna_generic(q, kk, v, k, s, d, causal, q_tile_shape=qt, kv_tile_shape=kt,
+                                           return_lse=True, fused=True)
+            out_p, lse_p = amd_fna_generic(q, kk, v, k, s, d, causal, q_tile_shape=qt, kv_tile_shape=kt,
+                                           return_lse=True, fused=False)
+        tag = f"{shape} k={k} s={s} d={d} c={causal}"
+        assert_routes_agree("output " + tag, out_f, out_p, shape, d, kt)
+        assert_routes_agree("LSE " + tag, lse_f, lse_p, shape, d, kt)
+        if int(torch.tensor(shape).prod()) <= 40000:
+            ref_o, ref_l = oracle_full(q, kk, v, k, s, d, causal)
+            assert_close("out " + tag, to_np(out_f), ref_o)
+            assert_close("lse " + tag, to_np(lse_f), ref_l)
+        else:
+            sampled_check(q, kk, v, out_f, lse_f, k, s, d, causal, 400, seed=ci, tag=tag)
 
 
 def test_fused_with_dequantisation_scales():
@@ -101,8 +158,9 @@ def test_work_queue_launch_equals_one_workgroup_per_tile(case, dtype):
         for _ in range(2):
             got = amd_fna_generic(q, kk, v, k, s, d, causal, return_lse=True, run_persistent_kernel=True)
             assert torch.equal(got[0], ref[0]) and torch.equal(got[1], ref[1])
+        perm = amd_fna_generic(q, kk, v, k, s, d, causal, return_lse=True, run_persistent_kernel=False, fused=False)
         got = amd_fna_generic(q, kk, v, k, s, d, causal, return_lse=True, run_persistent_kernel=True, fused=False)
-        assert torch.equal(got[0], ref[0]) and torch.equal(got[1], ref[1])
+        assert torch.equal(got[0], perm[0]) and torch.equal(got[1], perm[1])
     ref_o, ref_l = oracle_full(q, kk, v, k, s, d, causal)
     assert_close("out", to_np(got[0]), ref_o)
     assert_close("lse", to_np(got[1]), ref_l)

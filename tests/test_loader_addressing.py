@@ -139,3 +139,61 @@ def test_full_tile_copy_addresses(D, nwaves, case):
                 assert (wave * per * 1024) + (i // 4) * 4096 + (i % 4) * 1024 + lane * 16 == P * 16
                 covered.add(P)
             assert covered == set(range(chunks))
+
+
+EDGE_CASES = [
+    # (layout X, dilation, kv_tile): some extent is not a multiple of dilation x KV tile
+    ((57, 20, 88), (2, 1, 1), (2, 4, 8)),
+    ((84, 19, 1), (1, 1, 1), (8, 8, 1)),
+    ((84, 19, 1), (5, 1, 1), (8, 8, 1)),
+    ((125, 1, 1), (1, 1, 1), (64, 1, 1)),
+    ((19, 29, 1), (2, 3, 1), (8, 8, 1)),       # group extents (10|9, 10|9): smaller than no tile, uneven groups
+    ((5, 25, 1), (1, 1, 1), (4, 16, 1)),       # extent 5 over tiles of 4
+    ((3, 7, 9), (1, 2, 2), (4, 4, 4)),         # every group extent smaller than the tile
+    ((13, 11, 9), (3, 2, 2), (1, 8, 8)),
+]
+
+
+@pytest.mark.parametrize("D", [32, 128])
+@pytest.mark.parametrize("case", EDGE_CASES)
+def test_edge_tile_gathers_stay_inside_the_group(D, case):
+    """The instance that clamps (original layout, RAGGED): for every dilation group and every KV tile
+    that starts inside the group's extent, each lane's address is that of the row the LDS position
+    stands for, with coordinates past the group's extent replaced by the group's last one -- so it
+    lies inside the tensor, and inside the group."""
+    nwaves, kvt = 4, 64
+    cpr, chunks, per = _geometry(D, nwaves, kvt)
+    X, dil, kv_tile = case
+    assert kv_tile[0] * kv_tile[1] * kv_tile[2] == kvt
+    strides = (X[1] * X[2], X[2], 1)
+    tok_step = tuple(d * s for d, s in zip(dil, strides))
+    n_tokens = X[0] * X[1] * X[2]
+    heads_kv = 2
+    stride2 = heads_kv * D * 2
+    total_bytes = n_tokens * stride2
+    for group in itertools.product(*[range(d) for d in dil]):
+        ext = tuple(-(-(x - g) // d) for x, g, d in zip(X, group, dil))
+        group_tok = sum(g * s for g, s in zip(group, strides))
+        for origin in itertools.product(*[range(0, e, t) for e, t in zip(ext, kv_tile)]):
+            lim = tuple(min(e - o, t) for e, o, t in zip(ext, origin, kv_tile))
+            assert all(l >= 1 for l in lim)
+            inside = lim == tuple(kv_tile)
+            tile_base = (group_tok + sum(o * st for o, st in zip(origin, tok_step))) * stride2
+            for wave, i, lane in itertools.product(range(nwaves), range(per), range(64)):
+                imm = (i % 4) * 1024
+                P = (wave * per + i) * 64 + lane
+                r, slot = P // cpr, P % cpr
+                t = (r % kv_tile[0], (r // kv_tile[0]) % kv_tile[1], r // (kv_tile[0] * kv_tile[1]))
+                if inside:
+                    continue  # the unclamped arithmetic, covered above
+                tc = tuple(min(a, l - 1) for a, l in zip(t, lim))
+                voff = U32(sum(a * st for a, st in zip(tc, tok_step))) * U32(stride2) + U32(_slots(D, r, slot)[0] * 16)
+                src = tile_base - imm
+                addr = src + int(voff) + imm
+                assert 0 <= addr and addr + 16 <= total_bytes, (case, group, origin, wave, i, lane)
+                # the token it names belongs to this group and lies inside its extent
+                tok = (addr // stride2)
+                crd = (tok // strides[0], (tok // strides[1]) % X[1], tok % X[2])
+                assert all(c % d == g for c, d, g in zip(crd, dil, group))
+                assert all(c // d == o + a for c, d, o, a in zip(crd, dil, origin, tc))
+                assert (wave * per * 1024) + (i // 4) * 4096 + imm + lane * 16 == P * 16

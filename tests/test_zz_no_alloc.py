@@ -43,7 +43,11 @@ def test_static_scratch_entry_point_refuses_what_the_work_queue_kernel_does_not_
     out, lse = torch.empty_like(q), torch.empty(q.shape[:-1], dtype=torch.float32, device=q.device)
     with pytest.raises(RuntimeError, match="Q tiles of 128"):
         _lib.fna_forward_fused_static(q, kk, v, out, lse, (5, 5), (1, 1), (1, 1), (False, False), 0.125, (16, 16), (8, 8))
-    with pytest.raises(RuntimeError, match="multiple of dilation"):
-        q15, k15, v15, o15 = (t[:, :15].contiguous() for t in (q, kk, v, out))
-        _lib.fna_forward_fused_static(q15, k15, v15, o15, lse[:, :15].contiguous(), (5, 5), (1, 1), (1, 1), (False, False),
-                                      0.125, (8, 16), (8, 8))
+    with pytest.raises(RuntimeError, match="fp16 / bf16"):
+        L = _lib.lib()
+        q8 = q.to(torch.float8_e4m3fn)
+        rc = L.natten_amd_fna_forward_fused_static(
+            q8.data_ptr(), q8.data_ptr(), q8.data_ptr(), out.data_ptr(), lse.data_ptr(), _lib.DTYPE_CODES[q8.dtype], 2, 1, 2,
+            2, 64, _lib._i32([16, 32]), _lib._i32([5, 5]), _lib._i32([1, 1]), _lib._i32([1, 1]), _lib._i32([0, 0]),
+            _lib._i32([8, 16]), _lib._i32([8, 8]), 0.125, None, None, None, None)
+        _lib._check(rc)
