@@ -8,39 +8,56 @@
 
 namespace natten_amd {
 
-template <typename T>
-__device__ __forceinline__ float merge_load(const T* p) { return static_cast<float>(*p); }
+// sigmoid(l1 - l0) and the merged LSE of one row, written to stay finite for any pair
+__device__ __forceinline__ void merge_row_scalars(float a, float b, float& sig, float& lse) {
+  const float d = b - a;
+  if (d <= 0.f) {
+    const float e = __expf(d);
+    sig = e / (1.f + e);
+    lse = a + log1pf(e);
+  } else {
+    const float e = __expf(-d);
+    sig = 1.f / (1.f + e);
+    lse = b + log1pf(e);
+  }
+  if (a == -INFINITY && b == -INFINITY) {
+    sig = 0.f;
+    lse = -INFINITY;
+  }
+}
 
-// One wave-row mapping: each thread handles one (row, 8-element slice) pair; the row's scalars
-// are recomputed per thread (cheap) so no cross-lane traffic is needed.
-template <typename T>
+// VEC elements per thread (16 bytes of a 16-bit payload, 16 or 32 of a float one): a thread owns
+// one (row, VEC-element slice) pair, reads the row's two LSEs once and moves its slice with one
+// access per operand; the thread of a row's first slice writes the merged LSE.  VEC == 1 is the
+// form for head dims or pointers that do not allow the wide accesses.
+template <typename T, int VEC>
 __global__ void __launch_bounds__(256) merge_kernel(const T* __restrict__ o0, const float* __restrict__ l0,
                                                     const T* __restrict__ o1, const float* __restrict__ l1,
                                                     T* out, float* lse_out, int64_t rows, int head_dim) {
-  const int64_t total = rows * head_dim;
+  typedef T tvec __attribute__((ext_vector_type(VEC)));
+  const int slices = head_dim / VEC;
+  const int64_t total = rows * slices;
   for (int64_t idx = int64_t(blockIdx.x) * 256 + threadIdx.x; idx < total; idx += int64_t(gridDim.x) * 256) {
-    const int64_t row = idx / head_dim;
-    const int col = int(idx - row * head_dim);
-    const float a = l0[row], b = l1[row];
-    // sigmoid(b - a) and logsigmoid(a - b) = -log(1 + exp(b - a)), written to stay finite
-    const float d = b - a;
+    const int64_t row = idx / slices;
+    const int slice = int(idx - row * slices);
     float sig, lse;
-    if (d <= 0.f) {
-      const float e = __expf(d);
-      sig = e / (1.f + e);
-      lse = a + log1pf(e);
+    merge_row_scalars(l0[row], l1[row], sig, lse);
+    const int64_t at = row * head_dim + int64_t(slice) * VEC;
+    if constexpr (VEC == 1) {
+      const float x0 = static_cast<float>(o0[at]), x1 = static_cast<float>(o1[at]);
+      out[at] = static_cast<T>(x0 - sig * (x0 - x1));
     } else {
-      const float e = __expf(-d);
-      sig = 1.f / (1.f + e);
-      lse = b + log1pf(e);
+      const tvec a = *reinterpret_cast<const tvec*>(o0 + at);
+      const tvec b = *reinterpret_cast<const tvec*>(o1 + at);
+      tvec r;
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) {
+        const float x0 = static_cast<float>(a[i]), x1 = static_cast<float>(b[i]);
+        r[i] = static_cast<T>(x0 - sig * (x0 - x1));
+      }
+      *reinterpret_cast<tvec*>(out + at) = r;
     }
-    if (a == -INFINITY && b == -INFINITY) {
-      sig = 0.f;
-      lse = -INFINITY;
-    }
-    const float x0 = static_cast<float>(o0[idx]), x1 = static_cast<float>(o1[idx]);
-    out[idx] = static_cast<T>(x0 - sig * (x0 - x1));
-    if (col == 0) lse_out[row] = lse;
+    if (slice == 0) lse_out[row] = lse;
   }
 }
 

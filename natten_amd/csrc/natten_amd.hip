@@ -998,6 +998,17 @@ static int tokperm_common(const char* what, bool unpermute, int widen, const voi
     hipLaunchKernelGGL((tokperm_widen_kernel<false>), dim3(unsigned(blocks)), dim3(256), 0, s, p);
     return check_launch(what);
   }
+  if (vec == 16 && p.row_bytes >= 256) {
+    // a wave per token row
+    const int64_t rows = int64_t(batch) * p.num_groups * p.perm_len;
+    int64_t wgs = (rows + 3) / 4;
+    if (wgs > 256 * 32) wgs = 256 * 32;
+    if (unpermute)
+      hipLaunchKernelGGL(tokperm_rows_kernel<true>, dim3(unsigned(wgs)), dim3(256), 0, s, p);
+    else
+      hipLaunchKernelGGL(tokperm_rows_kernel<false>, dim3(unsigned(wgs)), dim3(256), 0, s, p);
+    return check_launch(what);
+  }
   switch (vec) {
     case 16: NA_TOKPERM_LAUNCH(16); break;
     case 4: NA_TOKPERM_LAUNCH(4); break;
@@ -1039,28 +1050,30 @@ int natten_amd_merge_attentions(const void* o0, const float* lse0, const void* o
   if (!o0 || !lse0 || !o1 || !lse1 || !out || !lse_out) return fail("merge_attentions: null pointer argument");
   if (rows < 1 || head_dim < 1) return fail("merge_attentions: rows and head_dim must be positive");
   if (lse_out == lse0 || lse_out == lse1) return fail("merge_attentions: lse_out must not alias an input");
-  const int64_t total = rows * head_dim;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  // eight elements per thread where head dim and alignment allow 16-byte accesses
+  const uintptr_t align = reinterpret_cast<uintptr_t>(o0) | reinterpret_cast<uintptr_t>(o1) | reinterpret_cast<uintptr_t>(out);
+  const bool wide = head_dim % 8 == 0 && align % (dtype == NATTEN_AMD_F32 ? 32 : 16) == 0;
+  const int64_t total = rows * (wide ? head_dim / 8 : head_dim);
   int64_t blocks = (total + 255) / 256;
   if (blocks > 256 * 64) blocks = 256 * 64;
-  hipStream_t s = static_cast<hipStream_t>(stream);
+#define NA_MERGE_LAUNCH(T, VEC)                                                                                     \
+  hipLaunchKernelGGL((merge_kernel<T, VEC>), dim3(unsigned(blocks)), dim3(256), 0, s, static_cast<const T*>(o0), lse0, \
+                     static_cast<const T*>(o1), lse1, static_cast<T*>(out), lse_out, rows, head_dim)
   switch (dtype) {
     case NATTEN_AMD_F16:
-      hipLaunchKernelGGL(merge_kernel<_Float16>, dim3(unsigned(blocks)), dim3(256), 0, s,
-                         static_cast<const _Float16*>(o0), lse0, static_cast<const _Float16*>(o1), lse1,
-                         static_cast<_Float16*>(out), lse_out, rows, head_dim);
+      if (wide) NA_MERGE_LAUNCH(_Float16, 8); else NA_MERGE_LAUNCH(_Float16, 1);
       break;
     case NATTEN_AMD_BF16:
-      hipLaunchKernelGGL(merge_kernel<__bf16>, dim3(unsigned(blocks)), dim3(256), 0, s, static_cast<const __bf16*>(o0),
-                         lse0, static_cast<const __bf16*>(o1), lse1, static_cast<__bf16*>(out), lse_out, rows,
-                         head_dim);
+      if (wide) NA_MERGE_LAUNCH(__bf16, 8); else NA_MERGE_LAUNCH(__bf16, 1);
       break;
     case NATTEN_AMD_F32:
-      hipLaunchKernelGGL(merge_kernel<float>, dim3(unsigned(blocks)), dim3(256), 0, s, static_cast<const float*>(o0),
-                         lse0, static_cast<const float*>(o1), lse1, static_cast<float*>(out), lse_out, rows, head_dim);
+      if (wide) NA_MERGE_LAUNCH(float, 8); else NA_MERGE_LAUNCH(float, 1);
       break;
     default:
       return fail("merge_attentions: unsupported dtype code %d", dtype);
   }
+#undef NA_MERGE_LAUNCH
   return check_launch("merge_attentions");
 }
 

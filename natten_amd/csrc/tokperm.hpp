@@ -98,6 +98,42 @@ __global__ void __launch_bounds__(256) tokperm_kernel(const TokPermParams p) {
   }
 }
 
+// The same copy for rows of at least 256 bytes in 16-byte chunks: a wave takes one token row at
+// a time, so the row's index arithmetic (a dozen 64-bit divisions) runs once per row on the
+// scalar unit instead of once per 16 bytes on every lane, and its lanes move up to four chunks
+// each per step (loads first, then stores).  Permuted rows are written / read exactly once and
+// never needed again soon: their stores bypass the cache hierarchy's reuse tracking (non-temporal).
+template <bool UNPERMUTE>
+__global__ void __launch_bounds__(256) tokperm_rows_kernel(const TokPermParams p) {
+  typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+  const int chunks = int(p.row_bytes / 16);
+  const int64_t rows = int64_t(p.batch) * p.num_groups * p.perm_len;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(int(threadIdx.x >> 6));
+  const int64_t n_waves = int64_t(gridDim.x) * 4;
+  for (int64_t tok = int64_t(blockIdx.x) * 4 + wave; tok < rows; tok += n_waves) {
+    int64_t orig_tok;
+    const bool inside = tokperm_decode(p, tok, orig_tok);  // wave-uniform
+    if (UNPERMUTE && !inside) continue;
+    const u4* src = reinterpret_cast<const u4*>(p.src + (UNPERMUTE ? tok : orig_tok) * p.row_bytes);
+    u4* dst = reinterpret_cast<u4*>(p.dst + (UNPERMUTE ? orig_tok : tok) * p.row_bytes);
+    for (int c0 = 0; c0 < chunks; c0 += 256) {
+      u4 val[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int c = c0 + u * 64 + lane;
+        val[u] = u4{0, 0, 0, 0};
+        if (c < chunks && (UNPERMUTE || inside)) val[u] = __builtin_nontemporal_load(src + c);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int c = c0 + u * 64 + lane;
+        if (c < chunks) __builtin_nontemporal_store(val[u], dst + c);
+      }
+    }
+  }
+}
+
 // Token permute that also widens 8-bit floating point to bf16 (exact: every e4m3 / e5m2 value is
 // a bf16 value).  row_bytes counts SOURCE bytes (one per element, a multiple of 8); the
 // destination row holds twice as many.  Each thread converts 8 elements: 8 bytes in, 16 out.
