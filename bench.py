@@ -71,14 +71,19 @@ CPU_PROXY = {
 #   traffic: workload=c4 pass=forward q_tile=2,8,8 kv_tile=1,8,8 bytes=2.82e10 kernel_digest=<hex>
 # and is reported only while `kernel_digest` equals the digest of the kernel sources this run uses;
 # after any change to those sources the bench prints null until the counters are collected again.
-KERNEL_SOURCES = ["fna_fwd.hpp", "fna_fwd_fp8.hpp", "fna_bwd.hpp", "na_math.hpp", "natten_amd.hip"]
+KERNEL_SOURCES = {
+    # kernels and launch geometry of each pass (the C entry points around them do not touch the traffic)
+    "forward": ["fna_fwd.hpp", "na_math.hpp"],
+    "forward_fp8": ["fna_fwd.hpp", "fna_fwd_fp8.hpp", "na_math.hpp"],
+    "backward": ["fna_fwd.hpp", "fna_bwd.hpp", "na_math.hpp"],
+}
 
 
-def kernel_digest():
+def kernel_digest(which="forward"):
     import hashlib
 
     h = hashlib.sha256()
-    for name in KERNEL_SOURCES:
+    for name in KERNEL_SOURCES[which]:
         with open(os.path.join(ROOT, "natten_amd", "csrc", name), "rb") as f:
             h.update(f.read())
     return h.hexdigest()[:16]
@@ -91,7 +96,7 @@ def measured_traffic(workload, which, q_tile, kv_tile):
     import re
 
     want = {"workload": workload, "pass": which, "q_tile": ",".join(map(str, q_tile)),
-            "kv_tile": ",".join(map(str, kv_tile)), "kernel_digest": kernel_digest()}
+            "kv_tile": ",".join(map(str, kv_tile)), "kernel_digest": kernel_digest(which)}
     for path in sorted(glob.glob(os.path.join(ROOT, "profiles", "*.md"))):
         with open(path) as f:
             for line in f:
@@ -374,7 +379,7 @@ def bench_backward(args, q, k, v, kernel, stride, dilation, causal, dt_name):
             "unit": "TFLOP/s",
             "frac": achieved / peak,
             "traffic": (measured_traffic(args.workload, "backward", q_tile, kv_tile) or {}).get("bytes"),
-            "kernel_digest": kernel_digest(),
+            "kernel_digest": kernel_digest("backward"),
             "algorithmic_flop": 2.5 * fwd_flops,
         },
         "cpu_baseline": None,
@@ -489,6 +494,14 @@ def main():
         fused = _lib.fused_layout_supported(layout, dilation, kv_tile, q_tile_shape=q_tile,
                                             dtype=None if quantised else dtype)
 
+        from natten_amd.functional import _use_work_queue
+
+        # the launch kind the public call above picked (work queue or a workgroup per Q tile)
+        n_q_tiles = B * H
+        for X, d_, t_ in zip(layout, dilation, q_tile):
+            n_q_tiles *= -(-(-(-X // d_)) // t_) * d_
+        kscales["run_persistent"] = _use_work_queue(None, causal, n_q_tiles)
+
         def kern_permuted():
             return _lib.fna_forward(qp, kp, vp, kernel, stride, dilation, causal, scale, q_shape, kv_shape,
                                     qkv_shape, q_tile, kv_tile, **kscales)
@@ -499,7 +512,8 @@ def main():
                 return _lib.fna_forward_fused(q8, k8, v8, kernel, stride, dilation, causal, scale, q_tile, kv_tile,
                                               **kscales)
             if fused:
-                return _lib.fna_forward_fused(q, k, v, kernel, stride, dilation, causal, scale, q_tile, kv_tile)
+                return _lib.fna_forward_fused(q, k, v, kernel, stride, dilation, causal, scale, q_tile, kv_tile,
+                                              **kscales)
             return kern_permuted()
 
         def timed(fn, iters):
@@ -528,7 +542,8 @@ def main():
     peak = PEAK_TFLOPS[dt_name]
     dense_flops = 4.0 * B * H * D * float(q.numel() // (B * H * D)) ** 2
 
-    traffic = measured_traffic(args.workload, "forward", q_tile, kv_tile) if fused else None
+    which = "forward_fp8" if quantised else "forward"
+    traffic = measured_traffic(args.workload, which, q_tile, kv_tile) if fused else None
     result = {
         "metric": "FNA fwd ms + effective TFLOP/s (% MFMA peak), na3d bf16 D=128, 1 GPU",
         "value": tflops_e2e,
@@ -548,6 +563,7 @@ def main():
             "kv_tile_shape": list(kv_tile),
             "path": ("one launch: fused FNA kernel gathering tiles from the original tensors" if fused else
                      "token permute (Q,K,V) + fused FNA kernel + token unpermute (O, LSE)"),
+            "launch": "work queue (resident workgroups pull Q tiles)" if kscales["run_persistent"] else "one workgroup per Q tile",
         },
         "na_flop_per_step": flops,
         "dense_over_na_flop": dense_flops / flops,
@@ -572,7 +588,7 @@ def main():
             "frac": achieved / peak,
             "traffic": traffic["bytes"] if traffic else None,
             "traffic_source": traffic["source"] if traffic else None,
-            "kernel_digest": kernel_digest(),
+            "kernel_digest": kernel_digest(which),
             "algorithmic_bytes": (4 * q.numel() * (1 if quantised else q.element_size())
                                   + (q.numel() if quantised else 0) + lse.numel() * 4),
         },

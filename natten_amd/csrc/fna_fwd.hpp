@@ -1126,4 +1126,24 @@ __global__ void fna_queue_clear_kernel(uint32_t* queues) {
   if (threadIdx.x < kQueueWords) queues[threadIdx.x] = 0;
 }
 
+// ---- host side of the launch geometry (kept with the kernels: the two must agree) -----------------
+
+// Workgroup layout: Q tiles are enumerated with dimension 0 slowest; a group is a run of about
+// as many consecutive Q tiles as one XCD keeps resident (32 CUs x 2 workgroups), made of whole
+// dimension-0 slabs when possible, so that the tiles resident on an XCD overlap in their KV boxes.
+// `tiles_per_wg` Q tiles share a workgroup (consecutive tiles of the enumeration) and an XCD keeps
+// about 64 Q tiles resident either way (32 CUs x 2 single-tile workgroups or x 1 two-tile workgroup).
+inline void set_wg_layout(FnaParams& p, int tiles_per_wg = 1) {
+  p.num_q_tiles = p.q_tiled[0] * p.q_tiled[1] * p.q_tiled[2];
+  const int slab = p.q_tiled[1] * p.q_tiled[2];
+  int rows = (64 + slab / 2) / slab;
+  if (rows < 1) rows = 1;
+  if (rows > p.q_tiled[0]) rows = p.q_tiled[0];
+  const int units = (p.num_q_tiles + tiles_per_wg - 1) / tiles_per_wg;
+  p.wg_group = (slab * rows + tiles_per_wg - 1) / tiles_per_wg;
+  if (p.wg_group > units) p.wg_group = units;
+  p.groups_per_bh = (units + p.wg_group - 1) / p.wg_group;
+  p.total_groups = p.batch * p.heads_q * p.groups_per_bh;
+}
+
 }  // namespace natten_amd

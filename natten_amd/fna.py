@@ -106,10 +106,11 @@ def amd_fna_generic(
     fp8_matmul: Optional[bool] = None,
     backward_q_tile_shape=None,
     backward_kv_tile_shape=None,
-    run_persistent_kernel: bool = False,
+    run_persistent_kernel: Optional[bool] = False,
 ) -> Union[Tensor, Tuple[Tensor, Tensor]]:
     """`run_persistent_kernel`: work-queue launch of the forward kernel (resident workgroups pull
-    Q tiles from per-XCD queues) instead of a workgroup per Q tile; bit-identical results.
+    Q tiles from per-XCD queues) instead of a workgroup per Q tile; bit-identical results.  None:
+    whichever was measured faster for this kind of problem (`functional._use_work_queue`).
 
     `fused` selects the one-launch path that gathers tiles from the original tensors (None:
     whenever the problem allows it); otherwise tokens are permuted, multiplied and unpermuted
@@ -131,6 +132,13 @@ def amd_fna_generic(
     head_dim = query.shape[-1]
     scale = scale or head_dim**-0.5
     d_pad = padded_head_dim(head_dim)
+    if run_persistent_kernel is None:
+        from .functional import _use_work_queue
+
+        tiles = query.shape[0] * query.shape[-2]
+        for X, d, t in zip(query.shape[1 : 1 + na_dim], dilation, q_tile_shape):
+            tiles *= -(-(-(-X // d)) // t) * d
+        run_persistent_kernel = _use_work_queue(None, is_causal, tiles)
     if torch.is_grad_enabled() and (query.requires_grad or key.requires_grad or value.requires_grad):
         bwd_q_tile, bwd_kv_tile = check_fna_backward_config(
             query, kernel_size, stride, dilation, is_causal, backward_q_tile_shape, backward_kv_tile_shape

@@ -167,7 +167,7 @@ def neighborhood_attention_generic(
         q_scale=q_scale, k_scale=k_scale, v_scale=v_scale,
         out_dtype=work_dtype if has_additional_attention else final_dtype, fp8_matmul=fp8_matmul,
         backward_q_tile_shape=backward_q_tile_shape, backward_kv_tile_shape=backward_kv_tile_shape,
-        run_persistent_kernel=_use_work_queue(run_persistent_kernel, is_causal),
+        run_persistent_kernel=run_persistent_kernel,
     )
 
     if has_additional_attention:
@@ -185,14 +185,17 @@ def neighborhood_attention_generic(
     return (output, lse) if return_lse else output
 
 
-def _use_work_queue(run_persistent_kernel: Optional[bool], is_causal) -> bool:
-    """`run_persistent_kernel` as given, or the measured default: the work-queue launch (resident
+def _use_work_queue(run_persistent_kernel: Optional[bool], is_causal, num_q_tiles: int = 1 << 30) -> bool:
+    """`run_persistent_kernel` as given, or the measured default.  The work-queue launch (resident
     workgroups pull Q tiles from per-XCD queues) is 1.5-14 % faster than a workgroup per Q tile on
-    the non-causal shapes measured and 2-3.5 % slower when dimension 0 is causal (Q tiles of
-    very different lengths), so that case launches a workgroup per tile.  Results are bit-identical."""
+    the large non-causal shapes measured, 2-3.5 % slower when dimension 0 is causal (Q tiles of
+    very different lengths), and its second launch (the one that clears the queues) costs more than
+    it gains on problems of a few thousand Q tiles or less: those cases launch a workgroup per
+    tile.  `num_q_tiles`: Q tiles over all batch entries, dilation groups and heads.  Results are
+    bit-identical either way."""
     if run_persistent_kernel is not None:
         return bool(run_persistent_kernel)
-    return not bool(is_causal[0])
+    return (not bool(is_causal[0])) and num_q_tiles >= 8192
 
 
 def _make_na(na_dim: int, name: str):

@@ -127,7 +127,7 @@ def test_traffic_is_only_reported_for_the_current_kernel_sources(tmp_path, monke
         f"traffic: workload=c4 pass=forward q_tile=2,8,8 kv_tile=1,8,8 bytes=1.5e10 kernel_digest={digest}\n"
         "traffic: workload=c3 pass=forward q_tile=8,16 kv_tile=8,8 bytes=7e8 kernel_digest=0123456789abcdef\n")
     monkeypatch.setattr(bench, "ROOT", str(tmp_path))
-    monkeypatch.setattr(bench, "kernel_digest", lambda: digest)
+    monkeypatch.setattr(bench, "kernel_digest", lambda which="forward": digest)
     assert bench.measured_traffic("c4", "forward", (2, 8, 8), (1, 8, 8))["bytes"] == 1.5e10
     assert bench.measured_traffic("c4", "forward", (4, 8, 8), (1, 8, 8)) is None
     assert bench.measured_traffic("c3", "forward", (8, 16), (8, 8)) is None  # measured on other sources
