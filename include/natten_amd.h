@@ -150,6 +150,16 @@ int natten_amd_fna_forward_fused_static(const void* q, const void* k, const void
                                         const float* v_scale, void* stream);
 
 /*
+ * Host arithmetic only (no device call): the window [*start, *end) of key coordinates that query
+ * coordinate `query` attends along one dimension of a dilation group of `extent` tokens --
+ * csrc/include/natten/cuda/fna_blackwell/collective/fna_fusion.hpp:88-123 (get_win_start /
+ * get_win_end), evaluated with the same routine the forward kernels' set-up uses (the stride's
+ * division replaced by a multiply and a shift), so that tests can pin it against the oracle.
+ */
+int natten_amd_window(int query, int kernel_size, int stride, int extent, int is_causal,
+                      int32_t* start, int32_t* end);
+
+/*
  * Supported tile sizes (tokens per tile).  Writes up to `capacity` pairs
  * (q_tile_size, kv_tile_size) for the given dtype / head_dim and returns how many exist.
  */

@@ -19,7 +19,7 @@ from torch import Tensor
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libnatten_amd.so")
 
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 DTYPE_CODES = {
     torch.float16: 0,
@@ -36,6 +36,7 @@ _load_error: Optional[str] = None
 _SIGNATURES = {
     "natten_amd_abi_version": (ctypes.c_int, []),
     "natten_amd_last_error": (ctypes.c_char_p, []),
+    "natten_amd_window": (ctypes.c_int, [ctypes.c_int] * 5 + [ctypes.c_void_p] * 2),
     "natten_amd_fna_supported_tiles": (
         ctypes.c_int,
         [ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int],
@@ -383,6 +384,15 @@ def attention_forward_varlen(
         )
     _check(rc)
     return out, lse
+
+
+def window(query: int, kernel_size: int, stride: int, extent: int, is_causal: bool) -> Tuple[int, int]:
+    """[start, end) of the key coordinates a query coordinate attends along one dimension (host
+    arithmetic only, the routine of the forward kernels' set-up)."""
+    st, en = ctypes.c_int32(), ctypes.c_int32()
+    _check(lib().natten_amd_window(int(query), int(kernel_size), int(stride), int(extent), int(bool(is_causal)),
+                                   ctypes.addressof(st), ctypes.addressof(en)))
+    return st.value, en.value
 
 
 def query_range(key_first: int, key_last: int, kernel_size: int, stride: int, extent: int, num_queries: int,

@@ -71,6 +71,12 @@ struct FnaParams {
   const int32_t* cu_q;   // [batch + 1]
   const int32_t* cu_kv;  // [batch + 1]
   int total_q, total_kv;  // rows of the packed operands: offsets that do not fit them are not followed
+  // Derived by finish_fna_params(): what the per-workgroup set-up would otherwise divide for.
+  // Tile extents are powers of two (log2 below); the other divisors get multiply-shift pairs.
+  int q_tile_lg[3], kv_tile_lg[3];
+  int ext_base[3], ext_rem[3];  // qkv_shape / dil and qkv_shape % dil: extent of dilation group g = base + (g < rem)
+  NaDiv d_stride[3], d_dil[3], d_q_tiled[3];
+  NaDiv d_wg_group, d_groups_per_bh, d_heads_q, d_q_per_kv, d_num_groups;
 };
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
@@ -300,6 +306,10 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
   __shared__ __attribute__((aligned(1024))) char sK1[TILE_BYTES];
   __shared__ __attribute__((aligned(1024))) char sV1[TILE_BYTES];
   __shared__ __attribute__((aligned(16))) uint32_t sTab[KVT];
+  // Per-dimension geometry the element mask of a PARTIAL tile needs (twelve words per dimension, see
+  // kGeo* below).  Kept in LDS and read where a masked tile is met: in scalar registers for the
+  // whole loop these thirty-odd values would push the loop's own scalars out to spill lanes.
+  __shared__ __attribute__((aligned(16))) int sGeo[3][12];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -310,24 +320,25 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
   // ---- workgroup id -> (batch*group, head, Q tile); groups of Q tiles are dealt to XCDs ------
   int bg, head, qtile_rm;
   {
-    const int xcd = pid % kNumXcd;
-    const int local = pid / kNumXcd;
-    const int group = (local / p.wg_group) * kNumXcd + xcd;
-    const int within = local % p.wg_group;
+    const int xcd = int(uint32_t(pid) % kNumXcd);
+    const int local = int(uint32_t(pid) / kNumXcd);
+    const int run = na_div(local, p.d_wg_group);
+    const int group = run * kNumXcd + xcd;
+    const int within = local - run * p.wg_group;
     if (group >= p.total_groups) return;
-    const int bh = group / p.groups_per_bh;
-    qtile_rm = (group % p.groups_per_bh) * p.wg_group + within;
+    const int bh = na_div(group, p.d_groups_per_bh);
+    qtile_rm = (group - bh * p.groups_per_bh) * p.wg_group + within;
     if (qtile_rm >= p.num_q_tiles) return;
-    bg = bh / p.heads_q;
-    head = bh % p.heads_q;
+    bg = na_div(bh, p.d_heads_q);
+    head = bh - bg * p.heads_q;
   }
-  const int head_kv = head / (p.heads_q / p.heads_kv);
+  const int head_kv = na_div(head, p.d_q_per_kv);
 
   // sequence lengths, window and row range of this batch entry: launch constants, except for
   // sequence-packed dense attention, where every batch entry is a sequence of its own
   int seqlen_q = p.seqlen_q, seqlen_kv = p.seqlen_kv;
   int ksz[3] = {p.ksize[0], p.ksize[1], p.ksize[2]};
-  int shp[3] = {p.qkv_shape[0], p.qkv_shape[1], p.qkv_shape[2]};
+  int ext0 = p.ext_base[0];  // extent of dimension 0 before dilation groups (a sequence's own length when packed)
   int64_t q_seq_row0 = int64_t(bg) * p.seqlen_q, kv_seq_row0 = int64_t(bg) * p.seqlen_kv;
   if constexpr (RAGGED) {
     if (p.cu_q != nullptr) {
@@ -340,7 +351,7 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
       q_seq_row0 = q0;
       kv_seq_row0 = kv0;
       ksz[0] = seqlen_kv;
-      shp[0] = seqlen_kv;
+      ext0 = seqlen_kv;  // (packed sequences are not dilated)
       // Q tiles are counted for the longest sequence: the ones past the end of this one have nothing to do
       int t0 = qtile_rm;
       if (p.causal[0]) t0 = p.q_tiled[0] - 1 - t0;
@@ -366,34 +377,37 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
   // qtile_rm enumerates Q tiles with dimension 0 slowest; causal dimension 0 is walked from
   // the far end so that the Q tiles with the longest KV loops start first.
   int extent[3], q_first[3], box_tile0[3], box_n[3];
+  const int b_orig = na_div(bg, p.d_num_groups);  // batch entry before the dilation groups were folded in
   int qtile_idx;  // position of the tile in the permuted sequence (dimension 0 fastest)
   int tok_step[3];  // fused layout: tokens per unit step of a coordinate inside a dilation group
   int group_tok = 0;  // fused layout: token of the dilation group's first element
   {
-    int gl = bg % p.num_groups;
+    int gl = bg - b_orig * p.num_groups;
     int tc[3];
-    int t = qtile_rm;
-    tc[2] = t % p.q_tiled[2];
-    t /= p.q_tiled[2];
-    tc[1] = t % p.q_tiled[1];
-    tc[0] = t / p.q_tiled[1];
+    const int t01 = na_div(qtile_rm, p.d_q_tiled[2]);
+    tc[2] = qtile_rm - t01 * p.q_tiled[2];
+    tc[0] = na_div(t01, p.d_q_tiled[1]);
+    tc[1] = t01 - tc[0] * p.q_tiled[1];
     if (p.causal[0]) tc[0] = p.q_tiled[0] - 1 - tc[0];
     qtile_idx = tc[0] + p.q_tiled[0] * (tc[1] + p.q_tiled[1] * tc[2]);
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
-      const int gi = gl % p.dil[a];
-      gl /= p.dil[a];
-      extent[a] = na_group_extent(shp[a], p.dil[a], gi);
+      const int rest = na_div(gl, p.d_dil[a]);
+      const int gi = gl - rest * p.dil[a];
+      gl = rest;
+      // dilation group gi holds one more token than the last groups when gi < X % d (reference
+      // fna_fusion.hpp:250-256, without its divisions: 0 <= gi < d decides the quotient there)
+      extent[a] = (a == 0 ? ext0 : p.ext_base[a]) + (gi < p.ext_rem[a] ? 1 : 0);
       tok_step[a] = p.dil[a] * p.tok_stride[a];
       group_tok += gi * p.tok_stride[a];
-      q_first[a] = tc[a] * p.q_tile[a];
+      q_first[a] = tc[a] << p.q_tile_lg[a];
       const int qf = q_first[a], ql = qf + p.q_tile[a] - 1;
       const bool c = p.causal[a] != 0;
-      const int st_f = na_window_start(qf, ksz[a], p.stride[a], extent[a], c);
-      const int st_l = na_window_start(ql, ksz[a], p.stride[a], extent[a], c);
+      const int st_f = na_window_start(qf, ksz[a], p.stride[a], p.d_stride[a], extent[a], c);
+      const int st_l = na_window_start(ql, ksz[a], p.stride[a], p.d_stride[a], extent[a], c);
       const int en_l = na_window_end(ql, st_l, ksz[a], extent[a], c);
-      box_tile0[a] = st_f / p.kv_tile[a];
-      box_n[a] = na_ceil_div(en_l, p.kv_tile[a]) - box_tile0[a];
+      box_tile0[a] = st_f >> p.kv_tile_lg[a];
+      box_n[a] = ((en_l + p.kv_tile[a] - 1) >> p.kv_tile_lg[a]) - box_tile0[a];
     }
   }
   const int total_tiles = box_n[0] * box_n[1] * box_n[2];
@@ -409,14 +423,14 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
   int wave_lo[3], wave_hi[3], wave_full_lo[3], wave_full_hi[3];
   {
     const int i0 = wave * (MQ * 32), i1 = i0 + MQ * 32 - 1;
-    const int t12 = p.q_tile[1] * p.q_tile[2];
+    const int lg2 = p.q_tile_lg[2], lg12 = p.q_tile_lg[1] + p.q_tile_lg[2];
     int f[3], l[3];
-    f[0] = i0 / t12;
-    f[1] = (i0 / p.q_tile[2]) % p.q_tile[1];
-    f[2] = i0 % p.q_tile[2];
-    l[0] = i1 / t12;
-    l[1] = (i1 / p.q_tile[2]) % p.q_tile[1];
-    l[2] = i1 % p.q_tile[2];
+    f[0] = i0 >> lg12;
+    f[1] = (i0 >> lg2) & (p.q_tile[1] - 1);
+    f[2] = i0 & (p.q_tile[2] - 1);
+    l[0] = i1 >> lg12;
+    l[1] = (i1 >> lg2) & (p.q_tile[1] - 1);
+    l[2] = i1 & (p.q_tile[2] - 1);
     if (f[0] != l[0]) {
       f[1] = 0;
       l[1] = p.q_tile[1] - 1;
@@ -430,9 +444,9 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
       // rows past the end of an unpadded sequence (dense attention) are clamped like the loads
       const int qmin = q_first[a] + f[a], qmax = q_first[a] + na_min(l[a], p.q_tile[a] - 1);
       const bool c = p.causal[a] != 0;
-      const int st_min = na_window_start(qmin, ksz[a], p.stride[a], extent[a], c);
+      const int st_min = na_window_start(qmin, ksz[a], p.stride[a], p.d_stride[a], extent[a], c);
       const int en_min = na_window_end(qmin, st_min, ksz[a], extent[a], c);
-      const int st_max = na_window_start(qmax, ksz[a], p.stride[a], extent[a], c);
+      const int st_max = na_window_start(qmax, ksz[a], p.stride[a], p.d_stride[a], extent[a], c);
       const int en_max = na_window_end(qmax, st_max, ksz[a], extent[a], c);
       wave_lo[a] = st_min;
       wave_hi[a] = en_max;
@@ -441,31 +455,45 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
     }
   }
 
+  enum { kGeoQFirst, kGeoKernel, kGeoStride, kGeoExtent, kGeoDivMul, kGeoDivShift, kGeoCausal, kGeoQMask, kGeoQLog2,
+         kGeoKvTile, kGeoKvLog2 };
+  if (tid < 3) {
+    const int a = tid;
+    sGeo[a][kGeoQFirst] = q_first[a];
+    sGeo[a][kGeoKernel] = ksz[a];
+    sGeo[a][kGeoStride] = p.stride[a];
+    sGeo[a][kGeoExtent] = extent[a];
+    sGeo[a][kGeoDivMul] = int(p.d_stride[a].mul);
+    sGeo[a][kGeoDivShift] = int(p.d_stride[a].shift);
+    sGeo[a][kGeoCausal] = p.causal[a];
+    sGeo[a][kGeoQMask] = p.q_tile[a] - 1;
+    sGeo[a][kGeoQLog2] = p.q_tile_lg[a];
+    sGeo[a][kGeoKvTile] = p.kv_tile[a];
+    sGeo[a][kGeoKvLog2] = p.kv_tile_lg[a];
+  }
   // in-tile coordinates of every KV position, packed in 10-bit fields
   for (int i = tid; i < KVT; i += NT) {
-    int r = i;
-    const int t0 = r % p.kv_tile[0];
-    r /= p.kv_tile[0];
-    const int t1 = r % p.kv_tile[1];
-    r /= p.kv_tile[1];
-    sTab[i] = uint32_t(t0) | (uint32_t(t1) << 10) | (uint32_t(r) << 20);
+    const int t0 = i & (p.kv_tile[0] - 1);
+    const int r1 = i >> p.kv_tile_lg[0];
+    const int t1 = r1 & (p.kv_tile[1] - 1);
+    sTab[i] = uint32_t(t0) | (uint32_t(t1) << 10) | (uint32_t(r1 >> p.kv_tile_lg[1]) << 20);
   }
 
   const int64_t q_row_stride = int64_t(p.heads_q) * D;
   const int64_t kv_row_stride = int64_t(p.heads_kv) * D;
   // first row of this (batch, dilation group): rows are then addressed by permuted row index
   // (permuted layout) or by token offset inside the group (fused layout)
-  const int64_t q_row_base = p.fused ? int64_t(bg / p.num_groups) * p.tokens + group_tok : q_seq_row0;
-  const int64_t kv_row_base = p.fused ? int64_t(bg / p.num_groups) * p.tokens + group_tok : kv_seq_row0;
+  const int64_t q_row_base = p.fused ? int64_t(b_orig) * p.tokens + group_tok : q_seq_row0;
+  const int64_t kv_row_base = p.fused ? int64_t(b_orig) * p.tokens + group_tok : kv_seq_row0;
   const T* qbase = reinterpret_cast<const T*>(p.q) + q_row_base * q_row_stride + int64_t(head) * D;
   const T* kbase = reinterpret_cast<const T*>(p.k) + kv_row_base * kv_row_stride + int64_t(head_kv) * D;
   const T* vbase = reinterpret_cast<const T*>(p.v) + kv_row_base * kv_row_stride + int64_t(head_kv) * D;
   // row (permuted) or token offset (fused) of position `r` (dimension 0 fastest) of a KV tile
   auto kv_tile_pos = [&](int r) {
     if (!p.fused) return r;
-    const int t0 = r % p.kv_tile[0];
-    r /= p.kv_tile[0];
-    return t0 * tok_step[0] + (r % p.kv_tile[1]) * tok_step[1] + (r / p.kv_tile[1]) * tok_step[2];
+    const int t0 = r & (p.kv_tile[0] - 1);
+    r >>= p.kv_tile_lg[0];
+    return t0 * tok_step[0] + (r & (p.kv_tile[1] - 1)) * tok_step[1] + (r >> p.kv_tile_lg[1]) * tok_step[2];
   };
 
   // ---- async tile loads -------------------------------------------------------------------------
@@ -547,9 +575,9 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
               // (and with it the order of every sum) stays that of the whole tile.
               const int P = (wave * PER + I) * 64 + lane;
               const int r = P / CPR, slot = P % CPR;
-              int t0 = r % p.kv_tile[0];
-              const int r1 = r / p.kv_tile[0];
-              int t1 = r1 % p.kv_tile[1], t2 = r1 / p.kv_tile[1];
+              int t0 = r & (p.kv_tile[0] - 1);
+              const int r1 = r >> p.kv_tile_lg[0];
+              int t1 = r1 & (p.kv_tile[1] - 1), t2 = r1 >> p.kv_tile_lg[1];
               t0 = na_min(t0, c.lim[0] - 1);
               t1 = na_min(t1, c.lim[1] - 1);
               t2 = na_min(t2, c.lim[2] - 1);
@@ -634,25 +662,16 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
   const float c_log2 = sm_scale * 1.4426950408889634f;
 
   // ---- per-lane setup: this lane's query rows, their windows, Q fragments ---------------------
-  // coordinates of this lane's query in row block mb (recomputed where a masked tile needs the
-  // query's window: keeping the window in registers for the whole loop costs more than that)
-  auto query_coord = [&](int mb, int (&c)[3]) __attribute__((always_inline)) {
-    int r = (wave * MQ + mb) * 32 + l32;  // row-major index inside the tile
-    c[2] = q_first[2] + r % p.q_tile[2];
-    r /= p.q_tile[2];
-    c[1] = q_first[1] + r % p.q_tile[1];
-    c[0] = q_first[0] + r / p.q_tile[1];
-  };
   int q_row[MQ];     // this lane's row of the permuted sequence / token offset in the group (fused), or -1
   vec8 qf[MQ][KSTEPS];
 #pragma unroll
   for (int mb = 0; mb < MQ; ++mb) {
     int r = (wave * MQ + mb) * 32 + l32;  // row-major index inside the tile
     int off[3];
-    off[2] = r % p.q_tile[2];
-    r /= p.q_tile[2];
-    off[1] = r % p.q_tile[1];
-    off[0] = r / p.q_tile[1];
+    off[2] = r & (p.q_tile[2] - 1);
+    r >>= p.q_tile_lg[2];
+    off[1] = r & (p.q_tile[1] - 1);
+    off[0] = r >> p.q_tile_lg[1];
     int row = qtile_idx * QT + off[0] + p.q_tile[0] * (off[1] + p.q_tile[1] * off[2]);
     bool valid = row < seqlen_q;
     int row_c = na_min(row, seqlen_q - 1);
@@ -777,17 +796,30 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
     return x < 0 ? 0 : (n > N_ELEMS ? N_ELEMS : n);
   };
 
-  // element mask of a PARTIAL tile for row block mb
-  auto apply_mask = [&](f32x16_t (&S)[NSB], const int (&ws)[3], const int (&we)[3], const int (&origin)[3]) __attribute__((always_inline)) {
-    // window of this lane's query relative to the tile origin, clamped to the tile
+  // element mask of a PARTIAL tile for row block mb: the lane's query coordinates and window are
+  // worked out here, from the geometry in LDS (a masked tile is the exception)
+  auto apply_mask = [&](f32x16_t (&S)[NSB], int mb, const int (&origin)[3]) __attribute__((always_inline)) {
     uint32_t addc = 0, subc = 0;
+    int r = (wave * MQ + mb) * 32 + l32;  // row-major index of the query inside the Q tile
 #pragma unroll
-    for (int a = 0; a < 3; ++a) {
-      // a tile moved back from the group's edge starts before its place in the tiling (the next
+    for (int a = 2; a >= 0; --a) {
+      typedef int i32x4 __attribute__((ext_vector_type(4)));
+      const i32x4 g0 = *reinterpret_cast<const i32x4*>(&sGeo[a][0]);
+      const i32x4 g1 = *reinterpret_cast<const i32x4*>(&sGeo[a][4]);
+      const i32x4 g2 = *reinterpret_cast<const i32x4*>(&sGeo[a][8]);
+      const int qc = g0[kGeoQFirst] + (r & g1[kGeoQMask - 4]);
+      r >>= g2[kGeoQLog2 - 8];
+      const int kt = g2[kGeoKvTile - 8], kt_lg = g2[kGeoKvLog2 - 8];
+      const bool causal = g1[kGeoCausal - 4] != 0;
+      const NaDiv sd = {uint32_t(g1[kGeoDivMul - 4]), uint32_t(g1[kGeoDivShift - 4])};
+      const int ws = na_window_start(qc, g0[kGeoKernel], g0[kGeoStride], sd, g0[kGeoExtent], causal);
+      const int we = na_window_end(qc, ws, g0[kGeoKernel], g0[kGeoExtent], causal);
+      // window of this lane's query relative to the tile origin, clamped to the tile.  A tile
+      // moved back from the group's edge starts before its place in the tiling (the next
       // multiple of the tile extent): the keys up to there belong to the tile before it
-      const int lead = na_ceil_div(origin[a], p.kv_tile[a]) * p.kv_tile[a] - origin[a];
-      const int lo = na_min(na_max(ws[a] - origin[a], lead), p.kv_tile[a]);
-      const int hi = na_min(na_max(we[a] - origin[a], 0), p.kv_tile[a]);
+      const int lead = (((origin[a] + kt - 1) >> kt_lg) << kt_lg) - origin[a];
+      const int lo = na_min(na_max(ws - origin[a], lead), kt);
+      const int hi = na_min(na_max(we - origin[a], 0), kt);
       addc |= uint32_t(512 - lo) << (10 * a);
       subc |= uint32_t(511 + hi) << (10 * a);
     }
@@ -849,16 +881,7 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
 #pragma unroll
           for (int r = 0; r < 16; ++r) S[mb][sb][r] = -INFINITY;
       } else if (!t_full || !have_max) {
-        if (!t_full) {
-          int qc[3], ws[3], we[3];
-          query_coord(mb, qc);
-#pragma unroll
-          for (int a = 0; a < 3; ++a) {
-            ws[a] = na_window_start(qc[a], ksz[a], p.stride[a], extent[a], p.causal[a] != 0);
-            we[a] = na_window_end(qc[a], ws[a], ksz[a], extent[a], p.causal[a] != 0);
-          }
-          apply_mask(S[mb], ws, we, t_origin);
-        }
+        if (!t_full) apply_mask(S[mb], mb, t_origin);
         mx = -INFINITY;
 #pragma unroll
         for (int sb = 0; sb < NSB; ++sb)
@@ -1144,6 +1167,29 @@ inline void set_wg_layout(FnaParams& p, int tiles_per_wg = 1) {
   if (p.wg_group > units) p.wg_group = units;
   p.groups_per_bh = (units + p.wg_group - 1) / p.wg_group;
   p.total_groups = p.batch * p.heads_q * p.groups_per_bh;
+  // what the kernels' set-up would otherwise divide for (every forward launch comes through here)
+  for (int a = 0; a < 3; ++a) {
+    p.q_tile_lg[a] = p.kv_tile_lg[a] = 0;
+    while ((1 << p.q_tile_lg[a]) < p.q_tile[a]) ++p.q_tile_lg[a];
+    while ((1 << p.kv_tile_lg[a]) < p.kv_tile[a]) ++p.kv_tile_lg[a];
+    p.ext_base[a] = p.qkv_shape[a] / p.dil[a];
+    p.ext_rem[a] = p.qkv_shape[a] % p.dil[a];
+    p.d_stride[a] = na_make_div(p.stride[a]);
+    p.d_dil[a] = na_make_div(p.dil[a]);
+    p.d_q_tiled[a] = na_make_div(p.q_tiled[a]);
+  }
+  p.d_wg_group = na_make_div(p.wg_group);
+  p.d_groups_per_bh = na_make_div(p.groups_per_bh);
+  p.d_heads_q = na_make_div(p.heads_q);
+  p.d_q_per_kv = na_make_div(p.heads_q / p.heads_kv);
+  p.d_num_groups = na_make_div(p.num_groups);
+}
+
+// tile extents must be powers of two (every factorisation of the supported token counts is)
+inline bool fna_tiles_are_powers_of_two(const FnaParams& p) {
+  for (int a = 0; a < 3; ++a)
+    if ((p.q_tile[a] & (p.q_tile[a] - 1)) || (p.kv_tile[a] & (p.kv_tile[a] - 1))) return false;
+  return true;
 }
 
 }  // namespace natten_amd

@@ -35,6 +35,41 @@ NA_HD int na_window_end(int i, int start, int k, int L, bool causal) {
   return causal ? na_min(i + 1, L) : start + k;
 }
 
+// Division by a launch constant without a divide: floor(n / d) = (mul * n) >> shift (64-bit product)
+// for every 0 <= n < 2^31 and 1 <= d < 2^31, with shift = 31 + ceil(log2 d) and
+// mul = floor(2^shift / d) + 1 < 2^32 + 1 (the error mul * d - 2^shift lies in (0, d], which is at most
+// 2^(shift - 31): small enough not to carry into the quotient for dividends below 2^31).
+// The kernels' per-workgroup set-up divides by strides, dilations and tile counts dozens of
+// times; a hardware integer division costs about thirty instructions, this three.
+struct NaDiv {
+  uint32_t mul;
+  uint32_t shift;
+};
+
+inline NaDiv na_make_div(int d) {
+  int lg = 0;
+  while ((int64_t(1) << lg) < d) ++lg;
+  NaDiv f;
+  f.shift = uint32_t(31 + lg);
+  f.mul = uint32_t(((uint64_t(1) << f.shift) / uint64_t(d)) + 1);  // d == 2^lg gives 2^31 + 1, the largest value
+  return f;
+}
+
+NA_HD int na_div(int n, NaDiv f) { return int((uint64_t(f.mul) * uint64_t(uint32_t(n))) >> f.shift); }
+
+// na_window_start with the stride's division precomputed (s_div = na_make_div(s))
+NA_HD int na_window_start(int i, int k, int s, NaDiv s_div, int L, bool causal) {
+  const int wl = int(uint32_t(k) >> 1);
+  const int wr = wl + int(uint32_t(k) & 1u) - 1;
+  const int group_first = na_div(i, s_div) * s;
+  if (causal) {
+    const int leader = na_min(group_first + s - 1, L - 1);
+    return na_max(leader - wl - wr, 0);
+  }
+  const int leader = na_min(group_first + int(uint32_t(s) >> 1), L - 1);
+  return na_max(leader - wl, 0) + ((leader + wr >= L) ? (L - wr - leader - 1) : 0);
+}
+
 // Number of tokens of dilation group g along a dimension of extent X.
 NA_HD int na_group_extent(int X, int d, int g) { return X / d + 1 - ((g + (d - X % d)) / d); }
 

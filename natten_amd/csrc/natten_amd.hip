@@ -77,6 +77,7 @@ int resident_workgroups() {
 template <typename T, int D, int NWAVES, int MQ, bool RAGGED, int KVT>
 int launch_fna(const FnaParams& p, hipStream_t stream, uint32_t* queues = nullptr) {
   constexpr int QT = NWAVES * MQ * 32;
+  if (!fna_tiles_are_powers_of_two(p)) return fail("fna_forward: tile extents must be powers of two");
   if ((p.seqlen_q + QT - 1) / QT != p.num_q_tiles) return fail("fna_forward: internal tile count mismatch");
   const long long wgs = (long long)((p.total_groups + kNumXcd - 1) / kNumXcd) * kNumXcd * p.wg_group;
   if (wgs > 0x7fffffffLL) return fail("fna_forward: problem needs more than 2^31 workgroups");
@@ -219,11 +220,22 @@ int queue_workspace(const char* what, int run_persistent, void* workspace, uint6
 
 extern "C" {
 
-int natten_amd_abi_version(void) { return 7; }
+int natten_amd_abi_version(void) { return 8; }
 
 uint64_t natten_amd_fna_forward_workspace_bytes(void) { return uint64_t(kQueueWords) * 4; }
 
 const char* natten_amd_last_error(void) { return g_error; }
+
+int natten_amd_window(int query, int kernel_size, int stride, int extent, int is_causal, int32_t* start, int32_t* end) {
+  g_error[0] = 0;
+  if (!start || !end) return fail("window: null pointer argument");
+  if (query < 0 || kernel_size < 1 || stride < 1 || extent < 1)
+    return fail("window: query >= 0, kernel_size, stride and extent >= 1 expected");
+  // the arithmetic the kernels' set-up runs: stride division by multiply and shift
+  *start = na_window_start(query, kernel_size, stride, na_make_div(stride), extent, is_causal != 0);
+  *end = na_window_end(query, *start, kernel_size, extent, is_causal != 0);
+  return 0;
+}
 
 int natten_amd_fna_supported_tiles(int dtype, int head_dim, int32_t* q_sizes, int32_t* kv_sizes, int capacity) {
   if (dtype == NATTEN_AMD_F8E4M3 || dtype == NATTEN_AMD_F8E5M2) {

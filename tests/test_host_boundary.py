@@ -205,3 +205,27 @@ def test_work_queue_launch_needs_a_workspace():
             args[-4], args[-3], args[-2] = 1, ws, nbytes
             assert getattr(L, name)(*args) != 0
             assert b"workspace" in L.natten_amd_last_error(), L.natten_amd_last_error()
+
+
+def test_kernel_window_arithmetic_equals_oracle():
+    # natten_amd_window runs the routine of the kernels' set-up (stride division by multiply and
+    # shift); against the oracle's window for every query of every small problem, and for large
+    # coordinates and strides at random
+    from oracle import na_oracle as O
+
+    for L in range(1, 40):
+        for k in range(1, L + 1):
+            for s in range(1, k + 1):
+                for causal in (False, True):
+                    for i in range(L + 3):  # queries past the extent (padding) get a window too
+                        st = int(O.window_start(i, k, s, L, causal))
+                        assert _lib.window(i, k, s, L, causal) == (st, int(O.window_end(i, st, k, L, causal)))
+    rng = np.random.default_rng(5)
+    for _ in range(3000):
+        L = int(rng.integers(1, 2**30))
+        k = int(rng.integers(1, L + 1))
+        s = int(rng.integers(1, k + 1))
+        i = int(rng.integers(0, L))
+        causal = bool(rng.integers(0, 2))
+        st = int(O.window_start(i, k, s, L, causal))
+        assert _lib.window(i, k, s, L, causal) == (st, int(O.window_end(i, st, k, L, causal))), (i, k, s, L, causal)
