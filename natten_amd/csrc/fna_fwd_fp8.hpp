@@ -72,19 +72,22 @@ fna_fwd_fp8_kernel(const FnaParams p) {
   // ---- workgroup id -> (batch*group, head, Q tile); groups of Q tiles are dealt to XCDs ------
   int bg, head, qtile_rm;
   {
-    const int pid = blockIdx.x;
-    const int xcd = pid % kNumXcd;
-    const int local = pid / kNumXcd;
-    const int group = (local / p.wg_group) * kNumXcd + xcd;
-    const int within = local % p.wg_group;
+    // (divisions by launch constants are multiply-shift pairs and shifts, as in fna_fwd_kernel)
+    const uint32_t pid = blockIdx.x;
+    const int xcd = int(pid % kNumXcd);
+    const int local = int(pid / kNumXcd);
+    const int run = na_div(local, p.d_wg_group);
+    const int group = run * kNumXcd + xcd;
+    const int within = local - run * p.wg_group;
     if (group >= p.total_groups) return;
-    const int bh = group / p.groups_per_bh;
-    qtile_rm = (group % p.groups_per_bh) * p.wg_group + within;
+    const int bh = na_div(group, p.d_groups_per_bh);
+    qtile_rm = (group - bh * p.groups_per_bh) * p.wg_group + within;
     if (qtile_rm >= p.num_q_tiles) return;
-    bg = bh / p.heads_q;
-    head = bh % p.heads_q;
+    bg = na_div(bh, p.d_heads_q);
+    head = bh - bg * p.heads_q;
   }
-  const int head_kv = head / (p.heads_q / p.heads_kv);
+  const int head_kv = na_div(head, p.d_q_per_kv);
+  const int b_orig = na_div(bg, p.d_num_groups);  // batch entry before the dilation groups were folded in
 
   // ---- workgroup-uniform setup: dilation group, Q tile origin, KV tile box -------------------
   // qtile_rm enumerates Q tiles with dimension 0 slowest; causal dimension 0 is walked from
@@ -94,30 +97,30 @@ fna_fwd_fp8_kernel(const FnaParams p) {
   int tok_step[3];  // fused layout: tokens per unit step of a coordinate inside a dilation group
   int group_tok = 0;  // fused layout: token of the dilation group's first element
   {
-    int gl = bg % p.num_groups;
+    int gl = bg - b_orig * p.num_groups;
     int tc[3];
-    int t = qtile_rm;
-    tc[2] = t % p.q_tiled[2];
-    t /= p.q_tiled[2];
-    tc[1] = t % p.q_tiled[1];
-    tc[0] = t / p.q_tiled[1];
+    const int t01 = na_div(qtile_rm, p.d_q_tiled[2]);
+    tc[2] = qtile_rm - t01 * p.q_tiled[2];
+    tc[0] = na_div(t01, p.d_q_tiled[1]);
+    tc[1] = t01 - tc[0] * p.q_tiled[1];
     if (p.causal[0]) tc[0] = p.q_tiled[0] - 1 - tc[0];
     qtile_idx = tc[0] + p.q_tiled[0] * (tc[1] + p.q_tiled[1] * tc[2]);
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
-      const int gi = gl % p.dil[a];
-      gl /= p.dil[a];
-      extent[a] = na_group_extent(p.qkv_shape[a], p.dil[a], gi);
+      const int rest = na_div(gl, p.d_dil[a]);
+      const int gi = gl - rest * p.dil[a];
+      gl = rest;
+      extent[a] = p.ext_base[a] + (gi < p.ext_rem[a] ? 1 : 0);  // dilation group gi: one more token while gi < X % d
       tok_step[a] = p.dil[a] * p.tok_stride[a];
       group_tok += gi * p.tok_stride[a];
-      q_first[a] = tc[a] * p.q_tile[a];
+      q_first[a] = tc[a] << p.q_tile_lg[a];
       const int qf = q_first[a], ql = qf + p.q_tile[a] - 1;
       const bool c = p.causal[a] != 0;
-      const int st_f = na_window_start(qf, p.ksize[a], p.stride[a], extent[a], c);
-      const int st_l = na_window_start(ql, p.ksize[a], p.stride[a], extent[a], c);
+      const int st_f = na_window_start(qf, p.ksize[a], p.stride[a], p.d_stride[a], extent[a], c);
+      const int st_l = na_window_start(ql, p.ksize[a], p.stride[a], p.d_stride[a], extent[a], c);
       const int en_l = na_window_end(ql, st_l, p.ksize[a], extent[a], c);
-      box_tile0[a] = st_f / p.kv_tile[a];
-      box_n[a] = na_ceil_div(en_l, p.kv_tile[a]) - box_tile0[a];
+      box_tile0[a] = st_f >> p.kv_tile_lg[a];
+      box_n[a] = ((en_l + p.kv_tile[a] - 1) >> p.kv_tile_lg[a]) - box_tile0[a];
     }
   }
   const int total_tiles = box_n[0] * box_n[1] * box_n[2];
@@ -133,14 +136,14 @@ fna_fwd_fp8_kernel(const FnaParams p) {
   int wave_lo[3], wave_hi[3], wave_full_lo[3], wave_full_hi[3];
   {
     const int i0 = wave * 32, i1 = i0 + 31;
-    const int t12 = p.q_tile[1] * p.q_tile[2];
+    const int lg2 = p.q_tile_lg[2], lg12 = p.q_tile_lg[1] + p.q_tile_lg[2];
     int f[3], l[3];
-    f[0] = i0 / t12;
-    f[1] = (i0 / p.q_tile[2]) % p.q_tile[1];
-    f[2] = i0 % p.q_tile[2];
-    l[0] = i1 / t12;
-    l[1] = (i1 / p.q_tile[2]) % p.q_tile[1];
-    l[2] = i1 % p.q_tile[2];
+    f[0] = i0 >> lg12;
+    f[1] = (i0 >> lg2) & (p.q_tile[1] - 1);
+    f[2] = i0 & (p.q_tile[2] - 1);
+    l[0] = i1 >> lg12;
+    l[1] = (i1 >> lg2) & (p.q_tile[1] - 1);
+    l[2] = i1 & (p.q_tile[2] - 1);
     if (f[0] != l[0]) {
       f[1] = 0;
       l[1] = p.q_tile[1] - 1;
@@ -154,9 +157,9 @@ fna_fwd_fp8_kernel(const FnaParams p) {
       // rows past the end of an unpadded sequence (dense attention) are clamped like the loads
       const int qmin = q_first[a] + f[a], qmax = q_first[a] + na_min(l[a], p.q_tile[a] - 1);
       const bool c = p.causal[a] != 0;
-      const int st_min = na_window_start(qmin, p.ksize[a], p.stride[a], extent[a], c);
+      const int st_min = na_window_start(qmin, p.ksize[a], p.stride[a], p.d_stride[a], extent[a], c);
       const int en_min = na_window_end(qmin, st_min, p.ksize[a], extent[a], c);
-      const int st_max = na_window_start(qmax, p.ksize[a], p.stride[a], extent[a], c);
+      const int st_max = na_window_start(qmax, p.ksize[a], p.stride[a], p.d_stride[a], extent[a], c);
       const int en_max = na_window_end(qmax, st_max, p.ksize[a], extent[a], c);
       wave_lo[a] = st_min;
       wave_hi[a] = en_max;
@@ -167,12 +170,10 @@ fna_fwd_fp8_kernel(const FnaParams p) {
 
   // in-tile coordinates of every KV position, packed in 10-bit fields
   for (int i = tid; i < KVT; i += NT) {
-    int r = i;
-    const int t0 = r % p.kv_tile[0];
-    r /= p.kv_tile[0];
-    const int t1 = r % p.kv_tile[1];
-    r /= p.kv_tile[1];
-    sTab[i] = uint32_t(t0) | (uint32_t(t1) << 10) | (uint32_t(r) << 20);
+    const int t0 = i & (p.kv_tile[0] - 1);
+    const int r1 = i >> p.kv_tile_lg[0];
+    const int t1 = r1 & (p.kv_tile[1] - 1);
+    sTab[i] = uint32_t(t0) | (uint32_t(t1) << 10) | (uint32_t(r1 >> p.kv_tile_lg[1]) << 20);
   }
 
   const int64_t q_row_stride = int64_t(p.heads_q) * D;
@@ -180,17 +181,17 @@ fna_fwd_fp8_kernel(const FnaParams p) {
   // (row strides are in bytes: one byte per element)
   // first row of this (batch, dilation group): rows are then addressed by permuted row index
   // (permuted layout) or by token offset inside the group (fused layout)
-  const int64_t q_row_base = p.fused ? int64_t(bg / p.num_groups) * p.tokens + group_tok : int64_t(bg) * p.seqlen_q;
-  const int64_t kv_row_base = p.fused ? int64_t(bg / p.num_groups) * p.tokens + group_tok : int64_t(bg) * p.seqlen_kv;
+  const int64_t q_row_base = p.fused ? int64_t(b_orig) * p.tokens + group_tok : int64_t(bg) * p.seqlen_q;
+  const int64_t kv_row_base = p.fused ? int64_t(b_orig) * p.tokens + group_tok : int64_t(bg) * p.seqlen_kv;
   const uint8_t* qbase = static_cast<const uint8_t*>(p.q) + q_row_base * q_row_stride + int64_t(head) * D;
   const uint8_t* kbase = static_cast<const uint8_t*>(p.k) + kv_row_base * kv_row_stride + int64_t(head_kv) * D;
   const uint8_t* vbase = static_cast<const uint8_t*>(p.v) + kv_row_base * kv_row_stride + int64_t(head_kv) * D;
   // row (permuted) or token offset (fused) of position `r` (dimension 0 fastest) of a KV tile
   auto kv_tile_pos = [&](int r) {
     if (!p.fused) return r;
-    const int t0 = r % p.kv_tile[0];
-    r /= p.kv_tile[0];
-    return t0 * tok_step[0] + (r % p.kv_tile[1]) * tok_step[1] + (r / p.kv_tile[1]) * tok_step[2];
+    const int t0 = r & (p.kv_tile[0] - 1);
+    r >>= p.kv_tile_lg[0];
+    return t0 * tok_step[0] + (r & (p.kv_tile[1] - 1)) * tok_step[1] + (r >> p.kv_tile_lg[1]) * tok_step[2];
   };
 
 
@@ -274,10 +275,10 @@ fna_fwd_fp8_kernel(const FnaParams p) {
   {
     int r = wave * 32 + l32;  // row-major index inside the tile
     int off[3];
-    off[2] = r % p.q_tile[2];
-    r /= p.q_tile[2];
-    off[1] = r % p.q_tile[1];
-    off[0] = r / p.q_tile[1];
+    off[2] = r & (p.q_tile[2] - 1);
+    r >>= p.q_tile_lg[2];
+    off[1] = r & (p.q_tile[1] - 1);
+    off[0] = r >> p.q_tile_lg[1];
     int row = qtile_idx * QT + off[0] + p.q_tile[0] * (off[1] + p.q_tile[1] * off[2]);
     bool valid = row < p.seqlen_q;
     int row_c = na_min(row, p.seqlen_q - 1);
@@ -289,7 +290,7 @@ fna_fwd_fp8_kernel(const FnaParams p) {
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
       const int c = q_first[a] + off[a];
-      wst[a] = na_window_start(c, p.ksize[a], p.stride[a], extent[a], p.causal[a] != 0);
+      wst[a] = na_window_start(c, p.ksize[a], p.stride[a], p.d_stride[a], extent[a], p.causal[a] != 0);
       wen[a] = na_window_end(c, wst[a], p.ksize[a], extent[a], p.causal[a] != 0);
       if (p.fused) {
         valid = valid && (c < extent[a]);

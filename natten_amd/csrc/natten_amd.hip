@@ -95,6 +95,7 @@ int launch_fna(const FnaParams& p, hipStream_t stream, uint32_t* queues = nullpt
 template <bool E5M2, int D>
 int launch_fna_fp8(const FnaParams& p, hipStream_t stream) {
   constexpr int QT = 128;
+  if (!fna_tiles_are_powers_of_two(p)) return fail("fna_forward: tile extents must be powers of two");
   if ((p.seqlen_q + QT - 1) / QT != p.num_q_tiles) return fail("fna_forward: internal tile count mismatch");
   const long long wgs = (long long)((p.total_groups + kNumXcd - 1) / kNumXcd) * kNumXcd * p.wg_group;
   if (wgs > 0x7fffffffLL) return fail("fna_forward: problem needs more than 2^31 workgroups");
