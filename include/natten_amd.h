@@ -115,6 +115,14 @@ int natten_amd_fna_forward(const void* q, const void* k, const void* v, void* ou
  * (no KV tile may reach past the input); returns an error otherwise, and the caller uses the
  * permuted path.  dtype, tiles, head_dim, scales, run_persistent and workspace as in
  * natten_amd_fna_forward.
+ *
+ * anchor_kv_tiles != 0: the KV tiles of a Q tile are laid out from the first key of its window
+ * box (per dimension) instead of from multiples of the KV tile extent -- there is no permuted
+ * layout to follow here -- so no tile lies partly before the window: fewer tiles are visited
+ * whenever window starts are not multiples of the tile extent (stride 1, or strides that do not
+ * divide the tile).  Needs every dilation group at least one KV tile wide in every dimension and
+ * is ignored otherwise.  Sums run in a different order than with anchor_kv_tiles == 0, which is
+ * bit-identical to the permuted path where the tiles divide the extents.
  */
 int natten_amd_fna_forward_fused(const void* q, const void* k, const void* v, void* out,
                                  float* lse, int dtype, int na_dim, int batch, int heads_q,
@@ -123,8 +131,8 @@ int natten_amd_fna_forward_fused(const void* q, const void* k, const void* v, vo
                                  const int32_t* dilation, const int32_t* is_causal,
                                  const int32_t* q_tile_shape, const int32_t* kv_tile_shape,
                                  float scale, const float* q_scale, const float* k_scale,
-                                 const float* v_scale, int run_persistent, void* workspace,
-                                 uint64_t workspace_bytes, void* stream);
+                                 const float* v_scale, int anchor_kv_tiles, int run_persistent,
+                                 void* workspace, uint64_t workspace_bytes, void* stream);
 
 /*
  * natten_amd_fna_forward_fused with run_persistent = 1 for callers that cannot allocate device
@@ -135,7 +143,7 @@ int natten_amd_fna_forward_fused(const void* q, const void* k, const void* v, vo
  * are those of natten_amd_fna_forward_fused; limits: fp16 / bf16 operands, Q tiles of 128 and
  * KV tiles of 64 tokens (the work-queue kernel's), at most 2^31 - 4096 Q tiles over all
  * (batch, head) pairs; anything else is refused with an error.  Results are bit-identical to
- * natten_amd_fna_forward_fused.  Every call on a GPU shares that GPU's array (the launch clears
+ * natten_amd_fna_forward_fused with anchor_kv_tiles = 1.  Every call on a GPU shares that GPU's array (the launch clears
  * it first, with a kernel): calls that overlap in time on one GPU -- on different streams or
  * from different threads -- race on the queues and must not be made; calls queued on one
  * stream are fine.

@@ -19,7 +19,7 @@ from torch import Tensor
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libnatten_amd.so")
 
-ABI_VERSION = 8
+ABI_VERSION = 9
 
 DTYPE_CODES = {
     torch.float16: 0,
@@ -54,7 +54,7 @@ _SIGNATURES = {
     "natten_amd_fna_forward_fused": (
         ctypes.c_int,
         [ctypes.c_void_p] * 5 + [ctypes.c_int] * 6 + [ctypes.c_void_p] * 7 + [ctypes.c_float] + [ctypes.c_void_p] * 3
-        + [ctypes.c_int, ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p],
+        + [ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p],
     ),
     "natten_amd_fna_forward_fused_static": (
         ctypes.c_int,
@@ -278,9 +278,11 @@ def fna_forward_fused(
     q: Tensor, k: Tensor, v: Tensor,
     kernel_size, stride, dilation, is_causal, scale: float, q_tile_shape, kv_tile_shape,
     q_scale: Optional[Tensor] = None, k_scale: Optional[Tensor] = None, v_scale: Optional[Tensor] = None,
-    run_persistent: bool = False,
+    run_persistent: bool = False, anchored_tiles: bool = True,
 ) -> Tuple[Tensor, Tensor]:
-    """Original-layout q [B, *X, H, D], k/v [B, *X, Hkv, D] -> (out like q, lse float32 [B, *X, H])."""
+    """Original-layout q [B, *X, H, D], k/v [B, *X, Hkv, D] -> (out like q, lse float32 [B, *X, H]).
+    anchored_tiles: lay the KV tiles of a Q tile out from the first key of its window instead of
+    from multiples of the tile extent (fewer tiles; sums run in another order than on the permuted path)."""
     L = lib()
     _require_gpu(q, k, v)
     if q.dtype not in (torch.float16, torch.bfloat16) + FP8_DTYPES:
@@ -296,7 +298,7 @@ def fna_forward_fused(
             DTYPE_CODES[q.dtype], na_dim, q.shape[0], q.shape[-2], k.shape[-2], q.shape[-1],
             _i32(qkv_shape), _i32(kernel_size), _i32(stride), _i32(dilation),
             _i32([1 if c else 0 for c in is_causal]), _i32(q_tile_shape), _i32(kv_tile_shape),
-            float(scale), *scales, *_queue_workspace(q, run_persistent), _stream(q),
+            float(scale), *scales, 1 if anchored_tiles else 0, *_queue_workspace(q, run_persistent), _stream(q),
         )
     _check(rc)
     return out, lse

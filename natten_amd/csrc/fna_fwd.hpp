@@ -63,6 +63,11 @@ struct FnaParams {
   // leading keys (which the tile before it already delivered) are masked.  2: the RAGGED instance,
   // which gathers the tile where it is and clamps the rows that fall outside the group.
   int edge;
+  // fused == 1 only: KV tiles are laid out from the first key of the Q tile's window box (per
+  // dimension) instead of from multiples of the tile extent, which saves the part of a tile that
+  // would lie before the window; a tile that then reaches past the group is moved back as under
+  // edge == 1 (every dilation group must be at least one KV tile wide in every dimension).
+  int anchor;
   int tok_stride[3];  // tokens per unit step of an original coordinate: X1*X2, X2, 1
   int tokens;         // X0 * X1 * X2
   // Sequence-packed dense attention (RAGGED instances only; null otherwise): `batch` sequences
@@ -376,7 +381,7 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
   // ---- workgroup-uniform setup: dilation group, Q tile origin, KV tile box -------------------
   // qtile_rm enumerates Q tiles with dimension 0 slowest; causal dimension 0 is walked from
   // the far end so that the Q tiles with the longest KV loops start first.
-  int extent[3], q_first[3], box_tile0[3], box_n[3];
+  int extent[3], q_first[3], box_org[3], box_n[3];  // box_org: coordinate of the box's first KV tile
   const int b_orig = na_div(bg, p.d_num_groups);  // batch entry before the dilation groups were folded in
   int qtile_idx;  // position of the tile in the permuted sequence (dimension 0 fastest)
   int tok_step[3];  // fused layout: tokens per unit step of a coordinate inside a dilation group
@@ -406,8 +411,8 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
       const int st_f = na_window_start(qf, ksz[a], p.stride[a], p.d_stride[a], extent[a], c);
       const int st_l = na_window_start(ql, ksz[a], p.stride[a], p.d_stride[a], extent[a], c);
       const int en_l = na_window_end(ql, st_l, ksz[a], extent[a], c);
-      box_tile0[a] = st_f >> p.kv_tile_lg[a];
-      box_n[a] = ((en_l + p.kv_tile[a] - 1) >> p.kv_tile_lg[a]) - box_tile0[a];
+      box_org[a] = p.anchor ? st_f : ((st_f >> p.kv_tile_lg[a]) << p.kv_tile_lg[a]);
+      box_n[a] = (en_l - box_org[a] + p.kv_tile[a] - 1) >> p.kv_tile_lg[a];
     }
   }
   const int total_tiles = box_n[0] * box_n[1] * box_n[2];
@@ -456,7 +461,7 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
   }
 
   enum { kGeoQFirst, kGeoKernel, kGeoStride, kGeoExtent, kGeoDivMul, kGeoDivShift, kGeoCausal, kGeoQMask, kGeoQLog2,
-         kGeoKvTile, kGeoKvLog2 };
+         kGeoKvTile, kGeoKvLog2, kGeoBoxOrg };
   if (tid < 3) {
     const int a = tid;
     sGeo[a][kGeoQFirst] = q_first[a];
@@ -470,6 +475,7 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
     sGeo[a][kGeoQLog2] = p.q_tile_lg[a];
     sGeo[a][kGeoKvTile] = p.kv_tile[a];
     sGeo[a][kGeoKvLog2] = p.kv_tile_lg[a];
+    sGeo[a][kGeoBoxOrg] = box_org[a];
   }
   // in-tile coordinates of every KV position, packed in 10-bit fields
   for (int i = tid; i < KVT; i += NT) {
@@ -628,15 +634,17 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
     t.skip = false;
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
-      const int org = (box_tile0[a] + itc[a]) * p.kv_tile[a];
+      const int org = box_org[a] + (itc[a] << p.kv_tile_lg[a]);
       const int end = org + p.kv_tile[a];
       t.full = t.full && (org >= wave_full_lo[a]) && (end <= wave_full_hi[a]);  // never when end > extent
       t.skip = t.skip || (end <= wave_lo[a]) || (org >= wave_hi[a]);
       // a tile that would reach past the group is moved back to end at the group's last position
-      t.origin[a] = (p.edge == 1) ? na_min(org, extent[a] - p.kv_tile[a]) : org;
+      t.origin[a] = (p.edge == 1 || p.anchor) ? na_min(org, extent[a] - p.kv_tile[a]) : org;
     }
     t.row0 = p.fused ? t.origin[0] * tok_step[0] + t.origin[1] * tok_step[1] + t.origin[2] * tok_step[2]
-                     : ((box_tile0[0] + itc[0]) + p.kv_tiled[0] * ((box_tile0[1] + itc[1]) + p.kv_tiled[1] * (box_tile0[2] + itc[2]))) * KVT;
+                     : (((box_org[0] >> p.kv_tile_lg[0]) + itc[0]) +
+                        p.kv_tiled[0] * (((box_org[1] >> p.kv_tile_lg[1]) + itc[1]) +
+                                         p.kv_tiled[1] * ((box_org[2] >> p.kv_tile_lg[2]) + itc[2]))) * KVT;
     if (++itc[2] == box_n[2]) {
       itc[2] = 0;
       if (++itc[1] == box_n[1]) {
@@ -815,9 +823,10 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
       const int ws = na_window_start(qc, g0[kGeoKernel], g0[kGeoStride], sd, g0[kGeoExtent], causal);
       const int we = na_window_end(qc, ws, g0[kGeoKernel], g0[kGeoExtent], causal);
       // window of this lane's query relative to the tile origin, clamped to the tile.  A tile
-      // moved back from the group's edge starts before its place in the tiling (the next
-      // multiple of the tile extent): the keys up to there belong to the tile before it
-      const int lead = (((origin[a] + kt - 1) >> kt_lg) << kt_lg) - origin[a];
+      // moved back from the group's edge starts before its place in the tiling (the box origin
+      // plus a multiple of the tile extent): the keys up to there belong to the tile before it
+      const int from_box = origin[a] - g2[kGeoBoxOrg - 8];
+      const int lead = (((from_box + kt - 1) >> kt_lg) << kt_lg) - from_box;
       const int lo = na_min(na_max(ws - origin[a], lead), kt);
       const int hi = na_min(na_max(we - origin[a], 0), kt);
       addc |= uint32_t(512 - lo) << (10 * a);

@@ -92,7 +92,7 @@ fna_fwd_fp8_kernel(const FnaParams p) {
   // ---- workgroup-uniform setup: dilation group, Q tile origin, KV tile box -------------------
   // qtile_rm enumerates Q tiles with dimension 0 slowest; causal dimension 0 is walked from
   // the far end so that the Q tiles with the longest KV loops start first.
-  int extent[3], q_first[3], box_tile0[3], box_n[3];
+  int extent[3], q_first[3], box_org[3], box_n[3];  // box_org: coordinate of the box's first KV tile
   int qtile_idx;  // position of the tile in the permuted sequence (dimension 0 fastest)
   int tok_step[3];  // fused layout: tokens per unit step of a coordinate inside a dilation group
   int group_tok = 0;  // fused layout: token of the dilation group's first element
@@ -119,8 +119,9 @@ fna_fwd_fp8_kernel(const FnaParams p) {
       const int st_f = na_window_start(qf, p.ksize[a], p.stride[a], p.d_stride[a], extent[a], c);
       const int st_l = na_window_start(ql, p.ksize[a], p.stride[a], p.d_stride[a], extent[a], c);
       const int en_l = na_window_end(ql, st_l, p.ksize[a], extent[a], c);
-      box_tile0[a] = st_f >> p.kv_tile_lg[a];
-      box_n[a] = ((en_l + p.kv_tile[a] - 1) >> p.kv_tile_lg[a]) - box_tile0[a];
+      // original layout: tiles may be laid out from the window's first key (see FnaParams::anchor)
+      box_org[a] = p.anchor ? st_f : ((st_f >> p.kv_tile_lg[a]) << p.kv_tile_lg[a]);
+      box_n[a] = (en_l - box_org[a] + p.kv_tile[a] - 1) >> p.kv_tile_lg[a];
     }
   }
   const int total_tiles = box_n[0] * box_n[1] * box_n[2];
@@ -244,13 +245,17 @@ fna_fwd_fp8_kernel(const FnaParams p) {
     t.skip = false;
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
-      t.origin[a] = (box_tile0[a] + itc[a]) * p.kv_tile[a];
-      const int end = t.origin[a] + p.kv_tile[a];
-      t.full = t.full && (t.origin[a] >= wave_full_lo[a]) && (end <= wave_full_hi[a]);
-      t.skip = t.skip || (end <= wave_lo[a]) || (t.origin[a] >= wave_hi[a]);
+      const int org = box_org[a] + (itc[a] << p.kv_tile_lg[a]);
+      const int end = org + p.kv_tile[a];
+      t.full = t.full && (org >= wave_full_lo[a]) && (end <= wave_full_hi[a]);  // never when end > extent
+      t.skip = t.skip || (end <= wave_lo[a]) || (org >= wave_hi[a]);
+      // a tile that would reach past the group is moved back to end at the group's last position
+      t.origin[a] = p.anchor ? na_min(org, extent[a] - p.kv_tile[a]) : org;
     }
     t.row0 = p.fused ? t.origin[0] * tok_step[0] + t.origin[1] * tok_step[1] + t.origin[2] * tok_step[2]
-                     : ((box_tile0[0] + itc[0]) + p.kv_tiled[0] * ((box_tile0[1] + itc[1]) + p.kv_tiled[1] * (box_tile0[2] + itc[2]))) * KVT;
+                     : (((box_org[0] >> p.kv_tile_lg[0]) + itc[0]) +
+                        p.kv_tiled[0] * (((box_org[1] >> p.kv_tile_lg[1]) + itc[1]) +
+                                         p.kv_tiled[1] * ((box_org[2] >> p.kv_tile_lg[2]) + itc[2]))) * KVT;
     if (++itc[2] == box_n[2]) {
       itc[2] = 0;
       if (++itc[1] == box_n[1]) {
@@ -376,7 +381,11 @@ fna_fwd_fp8_kernel(const FnaParams p) {
     uint32_t addc = 0, subc = 0;
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
-      const int lo = na_min(na_max(wst[a] - origin[a], 0), p.kv_tile[a]);
+      // a tile moved back from the group's edge starts before its place in the tiling: the keys up
+      // to there belong to the tile before it
+      const int from_box = origin[a] - box_org[a];
+      const int lead = (((from_box + p.kv_tile[a] - 1) >> p.kv_tile_lg[a]) << p.kv_tile_lg[a]) - from_box;
+      const int lo = na_min(na_max(wst[a] - origin[a], lead), p.kv_tile[a]);
       const int hi = na_min(na_max(wen[a] - origin[a], 0), p.kv_tile[a]);
       addc |= uint32_t(512 - lo) << (10 * a);
       subc |= uint32_t(511 + hi) << (10 * a);

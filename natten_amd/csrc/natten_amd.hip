@@ -221,7 +221,7 @@ int queue_workspace(const char* what, int run_persistent, void* workspace, uint6
 
 extern "C" {
 
-int natten_amd_abi_version(void) { return 8; }
+int natten_amd_abi_version(void) { return 9; }
 
 uint64_t natten_amd_fna_forward_workspace_bytes(void) { return uint64_t(kQueueWords) * 4; }
 
@@ -309,7 +309,7 @@ int fna_forward_fused_impl(const void* q, const void* k, const void* v, void* ou
                            const int32_t* kernel_size, const int32_t* stride, const int32_t* dilation,
                            const int32_t* is_causal, const int32_t* q_tile_shape, const int32_t* kv_tile_shape,
                            float scale, const float* q_scale, const float* k_scale, const float* v_scale,
-                           uint32_t* queues, void* stream) {
+                           int anchor_kv_tiles, uint32_t* queues, void* stream) {
   if (!qkv_shape || !kernel_size || !stride || !dilation || !is_causal || !q_tile_shape || !kv_tile_shape)
     return fail("fna_forward_fused: null shape argument");
   int qs[3] = {1, 1, 1}, ks[3] = {1, 1, 1};
@@ -372,6 +372,10 @@ int fna_forward_fused_impl(const void* q, const void* k, const void* v, void* ou
   p.v_scale = v_scale;
   p.fused = 1;
   p.edge = edge;
+  // tiles laid out from the window's first key: needs every dilation group at least a KV tile wide
+  p.anchor = (anchor_kv_tiles != 0 && edge != 2) ? 1 : 0;
+  for (int a = 0; a < na_dim; ++a)
+    if (qkv_shape[a] / dilation[a] < kv_tile_shape[a]) p.anchor = 0;
   p.tokens = int(tokens);
   set_wg_layout(p, 1);
   return dispatch_dtype(p, dtype, head_dim, prod3(p.q_tile), prod3(p.kv_tile), static_cast<hipStream_t>(stream), queues);
@@ -383,15 +387,15 @@ int natten_amd_fna_forward_fused(const void* q, const void* k, const void* v, vo
                                  const int32_t* qkv_shape, const int32_t* kernel_size, const int32_t* stride,
                                  const int32_t* dilation, const int32_t* is_causal, const int32_t* q_tile_shape,
                                  const int32_t* kv_tile_shape, float scale, const float* q_scale,
-                                 const float* k_scale, const float* v_scale, int run_persistent, void* workspace,
-                                 uint64_t workspace_bytes, void* stream) {
+                                 const float* k_scale, const float* v_scale, int anchor_kv_tiles, int run_persistent,
+                                 void* workspace, uint64_t workspace_bytes, void* stream) {
   g_error[0] = 0;
   if (na_dim < 1 || na_dim > 3) return fail("fna_forward_fused: na_dim must be 1, 2 or 3, got %d", na_dim);
   uint32_t* queues;
   if (int rc = queue_workspace("fna_forward_fused", run_persistent, workspace, workspace_bytes, &queues)) return rc;
   return fna_forward_fused_impl(q, k, v, out, lse, dtype, na_dim, batch, heads_q, heads_kv, head_dim, qkv_shape,
                                 kernel_size, stride, dilation, is_causal, q_tile_shape, kv_tile_shape, scale, q_scale,
-                                k_scale, v_scale, queues, stream);
+                                k_scale, v_scale, anchor_kv_tiles, queues, stream);
 }
 
 namespace {
@@ -455,7 +459,7 @@ int natten_amd_fna_forward_fused_static(const void* q, const void* k, const void
   if (queues == nullptr) return 1;
   return fna_forward_fused_impl(q, k, v, out, lse, dtype, na_dim, batch, heads_q, heads_kv, head_dim, qkv_shape,
                                 kernel_size, stride, dilation, is_causal, q_tile_shape, kv_tile_shape, scale, q_scale,
-                                k_scale, v_scale, queues, stream);
+                                k_scale, v_scale, /*anchor_kv_tiles=*/1, queues, stream);
 }
 
 int natten_amd_attention_forward(const void* q, const void* k, const void* v, void* out, float* lse, int dtype,

@@ -107,10 +107,16 @@ def amd_fna_generic(
     backward_q_tile_shape=None,
     backward_kv_tile_shape=None,
     run_persistent_kernel: Optional[bool] = False,
+    anchored_tiles: bool = True,
 ) -> Union[Tensor, Tuple[Tensor, Tensor]]:
     """`run_persistent_kernel`: work-queue launch of the forward kernel (resident workgroups pull
     Q tiles from per-XCD queues) instead of a workgroup per Q tile; bit-identical results.  None:
     whichever was measured faster for this kind of problem (`functional._use_work_queue`).
+
+    `anchored_tiles` (one-launch path only): KV tiles are laid out from the first key of a Q tile's
+    window instead of from multiples of the tile extent, so that no tile lies partly before the
+    window (fewer tiles whenever window starts are not multiples of the tile extent); False keeps
+    the permuted path's tiling, and with it bit-identical results to that path.
 
     `fused` selects the one-launch path that gathers tiles from the original tensors (None:
     whenever the problem allows it); otherwise tokens are permuted, multiplied and unpermuted
@@ -145,7 +151,7 @@ def amd_fna_generic(
         )
         output, lse = AmdFnaFunction.apply(
             query, key, value, kernel_size, stride, dilation, is_causal, scale, q_tile_shape, kv_tile_shape,
-            bwd_q_tile, bwd_kv_tile, fused, bool(run_persistent_kernel),
+            bwd_q_tile, bwd_kv_tile, fused, bool(run_persistent_kernel), bool(anchored_tiles),
         )
         if out_dtype is not None and output.dtype != out_dtype:
             output = output.to(out_dtype)
@@ -183,7 +189,7 @@ def amd_fna_generic(
             q_scale=resolve_scale(q_scale, query.shape[-2], query.device, "q_scale"),
             k_scale=resolve_scale(k_scale, key.shape[-2], query.device, "k_scale"),
             v_scale=resolve_scale(v_scale, key.shape[-2], query.device, "v_scale"),
-            run_persistent=bool(run_persistent_kernel),
+            run_persistent=bool(run_persistent_kernel), anchored_tiles=bool(anchored_tiles),
         )
         if d_pad != head_dim:
             output = output[..., :head_dim].contiguous()
@@ -233,11 +239,12 @@ class AmdFnaFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, query, key, value, kernel_size, stride, dilation, is_causal, scale, q_tile_shape, kv_tile_shape,
-                bwd_q_tile_shape, bwd_kv_tile_shape, fused, run_persistent_kernel=False):
+                bwd_q_tile_shape, bwd_kv_tile_shape, fused, run_persistent_kernel=False, anchored_tiles=True):
         with torch.no_grad():
             output, lse = amd_fna_generic(
                 query, key, value, kernel_size, stride, dilation, is_causal, scale, q_tile_shape, kv_tile_shape,
                 return_lse=True, fused=fused, run_persistent_kernel=run_persistent_kernel,
+                anchored_tiles=anchored_tiles,
             )
         ctx.save_for_backward(query, key, value, output, lse)
         ctx.na_args = (kernel_size, stride, dilation, is_causal, scale, bwd_q_tile_shape, bwd_kv_tile_shape)
@@ -267,7 +274,7 @@ class AmdFnaFunction(torch.autograd.Function):
             )
             if d_pad != head_dim:
                 dq, dk, dv = (t[..., :head_dim].contiguous() for t in (dq, dk, dv))
-            return (dq, dk, dv) + (None,) * 11
+            return (dq, dk, dv) + (None,) * 12
 
         def perm(x, tile):
             return token_permute_operation(x.contiguous(), tile, dilation, flip_tiled_dims=True)
@@ -287,4 +294,4 @@ class AmdFnaFunction(torch.autograd.Function):
         dv = token_unpermute_operation(dv_perm, qkv_shape, kv_tile, dilation, flip_tiled_dims=True)
         if d_pad != head_dim:
             dq, dk, dv = (t[..., :head_dim].contiguous() for t in (dq, dk, dv))
-        return (dq, dk, dv) + (None,) * 11
+        return (dq, dk, dv) + (None,) * 12

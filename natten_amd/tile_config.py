@@ -45,17 +45,21 @@ def _win(i: int, k: int, s: int, L: int, causal: bool) -> Tuple[int, int]:
 
 
 @functools.lru_cache(maxsize=4096)
-def _dim_cost(L: int, k: int, s: int, causal: bool, tq: int, tk: int) -> Tuple[int, int]:
+def _dim_cost(L: int, k: int, s: int, causal: bool, tq: int, tk: int, anchored: bool = False) -> Tuple[int, int]:
     """(visited pairs, fully-unmasked pairs) along one dimension of extent L for Q tile extent tq
-    and KV tile extent tk; the totals of a multi-dimensional problem are products of these."""
+    and KV tile extent tk; the totals of a multi-dimensional problem are products of these.
+    `anchored`: the KV tiles of a Q tile start at its window's first key (the one-launch forward
+    on the original tensors) instead of at multiples of tk."""
     visited = full = 0
     for q0 in range(0, _ceil_div(L, tq) * tq, tq):
         st_f, en_f = _win(q0, k, s, L, causal)
         st_l, en_l = _win(q0 + tq - 1, k, s, L, causal)
-        t0, t1 = st_f // tk, _ceil_div(en_l, tk)
-        visited += (t1 - t0) * tk * tq
-        for t in range(t0, t1):
-            if t * tk >= st_l and (t + 1) * tk <= en_f:
+        org = st_f if anchored and L >= tk else (st_f // tk) * tk
+        n = _ceil_div(en_l - org, tk)
+        visited += n * tk * tq
+        for t in range(n):
+            lo = org + t * tk
+            if lo >= st_l and lo + tk <= en_f and lo + tk <= L:
                 full += tk * tq
     return visited, full
 
@@ -75,21 +79,25 @@ def _factorisations(total: int, n: int) -> List[DimensionType]:
 @functools.lru_cache(maxsize=1024)
 def choose_tile_shapes(
     token_layout: DimensionType, kernel_size: DimensionType, stride: DimensionType, dilation: DimensionType,
-    is_causal: Tuple[bool, ...], q_size: int, kv_size: int,
+    is_causal: Tuple[bool, ...], q_size: int, kv_size: int, anchored: bool = False,
 ) -> Tuple[DimensionType, DimensionType]:
     n = len(token_layout)
     ext = tuple(_ceil_div(x, d) for x, d in zip(token_layout, dilation))
     best, best_cost = None, None
     for qt in _factorisations(q_size, n):
         for kt in _factorisations(kv_size, n):
-            visited = full = 1
-            for a in range(n):
-                v, f = _dim_cost(ext[a], kernel_size[a], stride[a], is_causal[a], qt[a], kt[a])
-                visited *= v
-                full *= f
-            cost = visited + 0.3 * (visited - full)
-            # ties: prefer tiles that are long in the last (memory-contiguous) dimensions
-            key = (cost, tuple(-x for x in reversed(qt)), tuple(-x for x in reversed(kt)))
+            costs = []
+            for anch in ((True, False) if anchored else (False,)):
+                visited = full = 1
+                for a in range(n):
+                    v, f = _dim_cost(ext[a], kernel_size[a], stride[a], is_causal[a], qt[a], kt[a], anch)
+                    visited *= v
+                    full *= f
+                costs.append(visited + 0.3 * (visited - full))
+            # ties (anchored tiles make many shapes equal): the cost with tiles at multiples of their
+            # extent, which is what the token-permuted route pays; then tiles that are long in the
+            # last (memory-contiguous) dimensions
+            key = (*costs, tuple(-x for x in reversed(qt)), tuple(-x for x in reversed(kt)))
             if best_cost is None or key < best_cost:
                 best, best_cost = (qt, kt), key
     assert best is not None
@@ -108,7 +116,9 @@ def check_fna_forward_config(
         raise ValueError("`q_tile_shape` and `kv_tile_shape` must be given together or not at all.")
     if q_tile_shape is None:
         q_size, kv_size = TILE_SIZES[0]
-        return choose_tile_shapes(layout, tuple(kernel_size), tuple(stride), tuple(dilation), tuple(is_causal), q_size, kv_size)
+        # the forward runs on the original tensors wherever it can, with KV tiles laid out from each window's first key
+        return choose_tile_shapes(layout, tuple(kernel_size), tuple(stride), tuple(dilation), tuple(is_causal), q_size,
+                                  kv_size, True)
     from .checks import check_tile_shape
 
     q_tile_shape = check_tile_shape(q_tile_shape, na_dim, "q_tile_shape")

@@ -46,15 +46,16 @@ def _fna_forward_fused_op(
     q: Tensor, k: Tensor, v: Tensor, kernel_size: List[int], stride: List[int], dilation: List[int],
     is_causal: List[bool], scale: float, q_tile_shape: List[int], kv_tile_shape: List[int],
     q_scale: Optional[Tensor], k_scale: Optional[Tensor], v_scale: Optional[Tensor], run_persistent: bool,
+    anchored_tiles: bool,
 ) -> Tuple[Tensor, Tensor]:
     return _lib.fna_forward_fused(q, k, v, kernel_size, stride, dilation, is_causal, scale, q_tile_shape,
                                   kv_tile_shape, q_scale=q_scale, k_scale=k_scale, v_scale=v_scale,
-                                  run_persistent=run_persistent)
+                                  run_persistent=run_persistent, anchored_tiles=anchored_tiles)
 
 
 @_fna_forward_fused_op.register_fake
 def _(q, k, v, kernel_size, stride, dilation, is_causal, scale, q_tile_shape, kv_tile_shape, q_scale, k_scale, v_scale,
-      run_persistent):
+      run_persistent, anchored_tiles):
     return q.new_empty(q.shape, dtype=_out_dtype(q)), q.new_empty(q.shape[:-1], dtype=torch.float32)
 
 
@@ -223,13 +224,15 @@ def fna_forward(q, k, v, kernel_size, stride, dilation, is_causal, scale, q_shap
 
 
 def fna_forward_fused(q, k, v, kernel_size, stride, dilation, is_causal, scale, q_tile_shape, kv_tile_shape,
-                      q_scale=None, k_scale=None, v_scale=None, run_persistent=False):
+                      q_scale=None, k_scale=None, v_scale=None, run_persistent=False, anchored_tiles=True):
     if _tracing():
         return _fna_forward_fused_op(q, k, v, _ints(kernel_size), _ints(stride), _ints(dilation),
                                      [bool(c) for c in is_causal], float(scale), _ints(q_tile_shape),
-                                     _ints(kv_tile_shape), q_scale, k_scale, v_scale, bool(run_persistent))
+                                     _ints(kv_tile_shape), q_scale, k_scale, v_scale, bool(run_persistent),
+                                     bool(anchored_tiles))
     return _lib.fna_forward_fused(q, k, v, kernel_size, stride, dilation, is_causal, scale, q_tile_shape, kv_tile_shape,
-                                  q_scale=q_scale, k_scale=k_scale, v_scale=v_scale, run_persistent=run_persistent)
+                                  q_scale=q_scale, k_scale=k_scale, v_scale=v_scale, run_persistent=run_persistent,
+                                  anchored_tiles=anchored_tiles)
 
 
 def attention_forward(q, k, v, is_causal, scale, q_scale=None, k_scale=None, v_scale=None):

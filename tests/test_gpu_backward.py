@@ -47,20 +47,26 @@ def run_backward(B, H, Hkv, D, shape, k, s, d, causal, dtype, bq=None, bkv=None,
         # padding, token-permuted copies otherwise), the permuted route must agree bit for bit
         from natten_amd.fna import amd_fna_generic
 
-        q2, k2, v2 = (t.detach().clone().requires_grad_(True) for t in (q, kk, v))
-        amd_fna_generic(q2, k2, v2, k, s, d, causal, backward_q_tile_shape=bq, backward_kv_tile_shape=bkv,
-                        fused=False).backward(d_out)
-        # (the forward results the backward starts from are only bit-equal between the routes where
-        # both place the keys alike in their tiles; elsewhere they agree up to summation order)
         from natten_amd.tile_config import check_fna_forward_config
 
+        grads = []
+        for route in (dict(anchored_tiles=False), dict(fused=False)):
+            q2, k2, v2 = (t.detach().clone().requires_grad_(True) for t in (q, kk, v))
+            amd_fna_generic(q2, k2, v2, k, s, d, causal, backward_q_tile_shape=bq, backward_kv_tile_shape=bkv,
+                            **route).backward(d_out)
+            grads.append((q2.grad, k2.grad, v2.grad))
+        # (the forward results the backward starts from are only bit-equal between the routes where
+        # both place the keys alike in their tiles; elsewhere they agree up to summation order)
         _, fwd_kt = check_fna_forward_config(q, k, s, d, causal, None, None)
         exact = routes_agree_bit_for_bit(shape, d, fwd_kt)
-        for name, a, b in zip(("dq", "dk", "dv"), (q.grad, kk.grad, v.grad), (q2.grad, k2.grad, v2.grad)):
+        for name, a, b, c in zip(("dq", "dk", "dv"), grads[0], grads[1], (q.grad, kk.grad, v.grad)):
             if exact:
                 assert torch.equal(a, b), f"original-layout and permuted backward differ in {name}: {tag}"
             else:
-                assert_close(f"routes {name} {tag}", to_np(a), to_np(b), atol=TOL[dtype] / 2, rtol=TOL[dtype] / 2)
+                assert_close(f"routes {name} {tag}", to_np(a), to_np(b), atol=TOL[dtype], rtol=TOL[dtype])
+            # and the default (KV tiles of the forward laid out from the window's first key): two
+            # roundings of the same gradient, a unit of the last place apart at most
+            assert_close(f"default route {name} {tag}", to_np(c), to_np(b), atol=1.5 * TOL[dtype], rtol=TOL[dtype])
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])

@@ -198,13 +198,17 @@ def test_fp8_matmul_fused_equals_permuted(dtype, D):
     kw = dict(q_tile_shape=(2, 8, 8), kv_tile_shape=(2, 4, 8), return_lse=True, q_scale=sq, k_scale=sk, v_scale=sv,
               out_dtype=torch.bfloat16, fp8_matmul=True)
     with torch.no_grad():
-        out_f, lse_f = amd_fna_generic(q8, k8, v8, *args, fused=True, **kw)
+        out_f, lse_f = amd_fna_generic(q8, k8, v8, *args, fused=True, anchored_tiles=False, **kw)
         out_p, lse_p = amd_fna_generic(q8, k8, v8, *args, fused=False, **kw)
+        out_a, lse_a = amd_fna_generic(q8, k8, v8, *args, fused=True, anchored_tiles=True, **kw)
     assert torch.equal(out_f, out_p) and torch.equal(lse_f, lse_p)
     qd, kd, vd = dequantise(q8, sq), dequantise(k8, sk), dequantise(v8, sv)
     ref_o, ref_l = c_oracle.na_forward(to_np(qd), to_np(kd), to_np(vd), *args, None)
     check_out("out", True, to_np(out_f), ref_o, vd)
     assert_close("lse", to_np(lse_f), ref_l)
+    # KV tiles laid out from the window's first key (the default on the original tensors)
+    check_out("out, anchored tiles", True, to_np(out_a), ref_o, vd)
+    assert_close("lse, anchored tiles", to_np(lse_a), ref_l)
 
 
 def test_fp8_matmul_rejects_unsupported_shapes():

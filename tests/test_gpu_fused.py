@@ -34,14 +34,19 @@ def test_fused_equals_permuted_and_oracle(case, dtype):
     assert _lib.fused_layout_supported(shape, d, kt)
     with torch.no_grad():
         out_f, lse_f = amd_fna_generic(q, kk, v, k, s, d, causal, q_tile_shape=qt, kv_tile_shape=kt, return_lse=True,
-                                       fused=True)
+                                       fused=True, anchored_tiles=False)
         out_p, lse_p = amd_fna_generic(q, kk, v, k, s, d, causal, q_tile_shape=qt, kv_tile_shape=kt, return_lse=True,
                                        fused=False)
+        out_a, lse_a = amd_fna_generic(q, kk, v, k, s, d, causal, q_tile_shape=qt, kv_tile_shape=kt, return_lse=True,
+                                       fused=True, anchored_tiles=True)
     assert torch.equal(out_f, out_p)
     assert torch.equal(lse_f, lse_p)
     ref_o, ref_l = oracle_full(q, kk, v, k, s, d, causal)
     assert_close("out", to_np(out_f), ref_o)
     assert_close("lse", to_np(lse_f), ref_l)
+    # KV tiles laid out from the window's first key: other tiles, same attention
+    assert_close("out, anchored tiles", to_np(out_a), ref_o)
+    assert_close("lse, anchored tiles", to_np(lse_a), ref_l)
 
 
 def test_fused_rejects_what_no_kernel_instance_gathers():
@@ -102,10 +107,14 @@ def test_fused_on_extents_that_tiles_do_not_divide(case):
         q, kk, v = make_qkv(2, shape, H, Hkv, D, dtype, seed=13 + ci)
         with torch.no_grad():
             out_f, lse_f = amd_fna_generic(q, kk, v, k, s, d, causal, q_tile_shape=qt, kv_tile_shape=kt,
-                                           return_lse=True, fused=True)
+                                           return_lse=True, fused=True, anchored_tiles=False)
             out_p, lse_p = amd_fna_generic(q, kk, v, k, s, d, causal, q_tile_shape=qt, kv_tile_shape=kt,
                                            return_lse=True, fused=False)
+            out_a, lse_a = amd_fna_generic(q, kk, v, k, s, d, causal, q_tile_shape=qt, kv_tile_shape=kt,
+                                           return_lse=True, fused=True, anchored_tiles=True)
         tag = f"{shape} k={k} s={s} d={d} c={causal}"
+        assert_close("anchored tiles, output " + tag, to_np(out_a), to_np(out_f), atol=4e-3, rtol=8e-3)
+        assert_close("anchored tiles, LSE " + tag, to_np(lse_a), to_np(lse_f), atol=4e-3, rtol=8e-3)
         assert_routes_agree("output " + tag, out_f, out_p, shape, d, kt)
         assert_routes_agree("LSE " + tag, lse_f, lse_p, shape, d, kt)
         if int(torch.tensor(shape).prod()) <= 40000:
@@ -123,7 +132,8 @@ def test_fused_with_dequantisation_scales():
     sv = torch.tensor([2.0, 0.5], device="cuda")
     args = ((5, 5), (1, 1), (1, 1), (False, False))
     with torch.no_grad():
-        out_f, lse_f = amd_fna_generic(q, kk, v, *args, return_lse=True, q_scale=sq, k_scale=sk, v_scale=sv, fused=True)
+        out_f, lse_f = amd_fna_generic(q, kk, v, *args, return_lse=True, q_scale=sq, k_scale=sk, v_scale=sv, fused=True,
+                                       anchored_tiles=False)
         out_p, lse_p = amd_fna_generic(q, kk, v, *args, return_lse=True, q_scale=sq, k_scale=sk, v_scale=sv, fused=False)
     assert torch.equal(out_f, out_p) and torch.equal(lse_f, lse_p)
     qd = q.float() * sq.view(1, 1, 1, -1, 1)
@@ -154,7 +164,7 @@ def test_work_queue_launch_equals_one_workgroup_per_tile(case, dtype):
     shape, k, s, d, causal, H, Hkv, D = case
     q, kk, v = make_qkv(3, shape, H, Hkv, D, dtype, seed=11)
     with torch.no_grad():
-        ref = amd_fna_generic(q, kk, v, k, s, d, causal, return_lse=True, run_persistent_kernel=False)
+        ref = amd_fna_generic(q, kk, v, k, s, d, causal, return_lse=True, run_persistent_kernel=False)  # anchored tiles
         for _ in range(2):
             got = amd_fna_generic(q, kk, v, k, s, d, causal, return_lse=True, run_persistent_kernel=True)
             assert torch.equal(got[0], ref[0]) and torch.equal(got[1], ref[1])
