@@ -494,13 +494,10 @@ def main():
         fused = _lib.fused_layout_supported(layout, dilation, kv_tile, q_tile_shape=q_tile,
                                             dtype=None if quantised else dtype)
 
-        from natten_amd.functional import _use_work_queue
+        from natten_amd.functional import work_queue_default
 
         # the launch kind the public call above picked (work queue or a workgroup per Q tile)
-        n_q_tiles = B * H
-        for X, d_, t_ in zip(layout, dilation, q_tile):
-            n_q_tiles *= -(-(-(-X // d_)) // t_) * d_
-        kscales["run_persistent"] = _use_work_queue(None, causal, n_q_tiles)
+        kscales["run_persistent"] = work_queue_default(B, H, layout, kernel, stride, dilation, causal, q_tile, kv_tile)
 
         def kern_permuted():
             return _lib.fna_forward(qp, kp, vp, kernel, stride, dilation, causal, scale, q_shape, kv_shape,

@@ -89,7 +89,7 @@ const char* natten_amd_last_error(void);
  * at least natten_amd_fna_forward_workspace_bytes() bytes, cleared by the launch itself (by a
  * kernel, so the call may be captured in a graph) and free for reuse once the work queued on
  * `stream` by this call has run.  Two calls must not use one workspace concurrently.  Tile
- * pairs other than 128 x 64 tokens and 8-bit operands ignore the flag.  run_persistent == 0:
+ * pairs other than 128 x 64 tokens ignore the flag.  run_persistent == 0:
  * workspace may be NULL.
  */
 uint64_t natten_amd_fna_forward_workspace_bytes(void);

@@ -1124,33 +1124,72 @@ fna_fwd_kernel(const FnaParams p) {
 constexpr int kQueueStride = 16;  // uint32 counters per 64-byte line
 constexpr int kQueueWords = kNumXcd * kQueueStride;
 
+// The launch parameters of a work-queue kernel, read anew for every tile.  Left to itself the compiler
+// hoists the set-up's reads of launch parameters (and what it derives from them) out of the loop
+// over tiles and keeps them in scalar registers across the tile's main loop, whose own scalars then
+// go to spill lanes.  A pointer to the kernel argument segment (the parameter block is the first
+// argument) that passes through an empty asm statement per tile is a new value each time: the reads
+// stay where the tile makes them, still as scalar loads from constant memory.
+typedef const FnaParams __attribute__((address_space(4)))* FnaKernargPtr;
+static __device__ __forceinline__ FnaKernargPtr fna_kernarg_params() {
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Wold-style-cast"
+  return (FnaKernargPtr)__builtin_amdgcn_kernarg_segment_ptr();
+#pragma clang diagnostic pop
+}
+static __device__ __forceinline__ const FnaParams& fna_params_for_this_tile(FnaKernargPtr& args) {
+  asm volatile("" : "+s"(args));
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Wold-style-cast"
+  return *(const FnaParams*)args;
+#pragma clang diagnostic pop
+}
+
+// The loop of a resident workgroup: `tile(pid)` is run for every launch position the workgroup
+// pulls, first from the queue of its own XCD, then from the others'.  Thread 0 fetches the position
+// after the current one while the other waves start on the current tile.  All queue state lives in
+// LDS: nothing of it occupies a register while a tile is worked on.
+template <typename Tile>
+static __device__ __forceinline__ void fna_queue_loop(uint32_t* __restrict__ queues, const int per_xcd, Tile&& tile) {
+  __shared__ int s_pos[2];   // s_pos[i & 1]: position of the workgroup's i-th tile (-1: none is left)
+  __shared__ int s_victim;   // queues found empty so far: the home queue first, then the others in turn
+  const int home = int(blockIdx.x) % kNumXcd;
+  auto queue_of = [&](int victim) __attribute__((always_inline)) {
+    return &queues[((home + victim) % kNumXcd) * kQueueStride];
+  };
+  // thread 0: the next position (-1: every queue is empty)
+  auto take = [&]() __attribute__((always_inline)) {
+    int victim = s_victim;
+    uint32_t ticket = atomicAdd(queue_of(victim), 1u);
+    while (ticket >= uint32_t(per_xcd)) {  // that queue is empty for good
+      if (++victim == kNumXcd) break;
+      ticket = atomicAdd(queue_of(victim), 1u);
+    }
+    s_victim = victim;
+    return victim == kNumXcd ? -1 : int(ticket) * kNumXcd + (home + victim) % kNumXcd;
+  };
+  if (threadIdx.x == 0) {
+    s_victim = 0;
+    s_pos[0] = take();
+  }
+  for (int i = 0;; i ^= 1) {
+    // s_pos[i] is written, everyone has read s_pos[i ^ 1] and is done with the LDS of the previous tile
+    __syncthreads();
+    const int pid = __builtin_amdgcn_readfirstlane(s_pos[i]);
+    if (pid < 0) break;
+    if (threadIdx.x == 0) s_pos[i ^ 1] = take();
+    tile(pid);
+  }
+}
+
 template <typename T, int D, int NWAVES, int MQ, bool RAGGED, int KVT>
 __global__ void __launch_bounds__(NWAVES * 64) __attribute__((amdgpu_waves_per_eu(MQ == 1 ? 2 : 1, MQ == 1 ? 2 : 1)))
 fna_fwd_queue_kernel(const FnaParams p, uint32_t* __restrict__ queues, const int per_xcd) {
-  __shared__ int s_next;
-  const int home = int(blockIdx.x) % kNumXcd;
-  int victim = 0;  // queues tried so far: home first, then the others in turn
-  // thread 0 takes the next position from the queues (-1: all are empty)
-  auto take = [&]() {
-    while (victim < kNumXcd) {
-      const int x = (home + victim) % kNumXcd;
-      const uint32_t local = atomicAdd(&queues[x * kQueueStride], 1u);
-      if (local < uint32_t(per_xcd)) return int(local) * kNumXcd + x;
-      ++victim;  // that queue is empty for good
-    }
-    return -1;
-  };
-  int mine = threadIdx.x == 0 ? take() : 0;
-  for (;;) {
-    __syncthreads();  // everyone has read s_next, and is done with the LDS of the previous tile
-    if (threadIdx.x == 0) s_next = mine;
-    __syncthreads();
-    const int pid = s_next;
-    if (pid < 0) break;
-    // the position after this one is fetched while this one is worked on
-    if (threadIdx.x == 0) mine = take();
-    fna_fwd_tile<T, D, NWAVES, MQ, RAGGED, KVT>(p, pid);
-  }
+  FnaKernargPtr args = fna_kernarg_params();
+  fna_queue_loop(queues, per_xcd, [&](int pid) __attribute__((always_inline)) {
+    fna_fwd_tile<T, D, NWAVES, MQ, RAGGED, KVT>(fna_params_for_this_tile(args), pid);
+  });
+  (void)p;
 }
 
 // clears the queue counters (a kernel rather than a memset so that callers may capture the launch pair in a graph)

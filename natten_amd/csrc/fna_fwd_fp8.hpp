@@ -34,9 +34,9 @@ constexpr float kFp8LazyRescaleLog2 = 2.0f; // so that 2^6 * 2^2 = 256 stays bel
 // One 32-row query block per wave, 64-key tiles, two waves per SIMD.  D = 64 or 128.
 // LDS tile: 64 rows of D bytes, 16-byte chunks XOR-swizzled by (row / rows-per-256-bytes); the
 // rows of a V tile are stored in the order the P fragment holds its keys (see v_key_of_lds_row).
+// `pid`: the launch position (the workgroup id of a launch with one workgroup per Q tile).
 template <bool E5M2, int D, int NWAVES>
-__global__ void __launch_bounds__(NWAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
-fna_fwd_fp8_kernel(const FnaParams p) {
+static __device__ __forceinline__ void fna_fwd_fp8_tile(const FnaParams& p, const uint32_t pid) {
   constexpr int KVT = 64;
   constexpr int NT = NWAVES * 64;
   constexpr int QT = NWAVES * 32;
@@ -73,7 +73,6 @@ fna_fwd_fp8_kernel(const FnaParams p) {
   int bg, head, qtile_rm;
   {
     // (divisions by launch constants are multiply-shift pairs and shifts, as in fna_fwd_kernel)
-    const uint32_t pid = blockIdx.x;
     const int xcd = int(pid % kNumXcd);
     const int local = int(pid / kNumXcd);
     const int run = na_div(local, p.d_wg_group);
@@ -571,6 +570,23 @@ fna_fwd_fp8_kernel(const FnaParams p) {
       }
     }
   }
+}
+
+template <bool E5M2, int D, int NWAVES>
+__global__ void __launch_bounds__(NWAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
+fna_fwd_fp8_kernel(const FnaParams p) {
+  fna_fwd_fp8_tile<E5M2, D, NWAVES>(p, blockIdx.x);
+}
+
+// Work-queue form (see fna_fwd_queue_kernel).
+template <bool E5M2, int D, int NWAVES>
+__global__ void __launch_bounds__(NWAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
+fna_fwd_fp8_queue_kernel(const FnaParams p, uint32_t* __restrict__ queues, const int per_xcd) {
+  FnaKernargPtr args = fna_kernarg_params();
+  fna_queue_loop(queues, per_xcd, [&](int pid) __attribute__((always_inline)) {
+    fna_fwd_fp8_tile<E5M2, D, NWAVES>(fna_params_for_this_tile(args), uint32_t(pid));
+  });
+  (void)p;
 }
 
 }  // namespace natten_amd

@@ -93,12 +93,19 @@ int launch_fna(const FnaParams& p, hipStream_t stream, uint32_t* queues = nullpt
 }
 
 template <bool E5M2, int D>
-int launch_fna_fp8(const FnaParams& p, hipStream_t stream) {
+int launch_fna_fp8(const FnaParams& p, hipStream_t stream, uint32_t* queues) {
   constexpr int QT = 128;
   if (!fna_tiles_are_powers_of_two(p)) return fail("fna_forward: tile extents must be powers of two");
   if ((p.seqlen_q + QT - 1) / QT != p.num_q_tiles) return fail("fna_forward: internal tile count mismatch");
   const long long wgs = (long long)((p.total_groups + kNumXcd - 1) / kNumXcd) * kNumXcd * p.wg_group;
   if (wgs > 0x7fffffffLL) return fail("fna_forward: problem needs more than 2^31 workgroups");
+  if (queues != nullptr) {
+    const long long resident = resident_workgroups();
+    hipLaunchKernelGGL(fna_queue_clear_kernel, dim3(1), dim3(kQueueWords), 0, stream, queues);
+    hipLaunchKernelGGL((fna_fwd_fp8_queue_kernel<E5M2, D, 4>), dim3((unsigned)(wgs < resident ? wgs : resident)), dim3(256), 0,
+                       stream, p, queues, int(wgs / kNumXcd));
+    return check_launch("fna_forward (work queue)");
+  }
   hipLaunchKernelGGL((fna_fwd_fp8_kernel<E5M2, D, 4>), dim3((unsigned)wgs), dim3(256), 0, stream, p);
   return check_launch("fna_forward");
 }
@@ -143,8 +150,9 @@ int dispatch_dtype(const FnaParams& p, int dtype, int head_dim, int qt, int kvt,
     if (head_dim != 64 && head_dim != 128)
       return fail("fna_forward: 8-bit float operands need head_dim 64 or 128, got %d", head_dim);
     const bool e5m2 = dtype == NATTEN_AMD_F8E5M2;
-    if (head_dim == 128) return e5m2 ? launch_fna_fp8<true, 128>(p, stream) : launch_fna_fp8<false, 128>(p, stream);
-    return e5m2 ? launch_fna_fp8<true, 64>(p, stream) : launch_fna_fp8<false, 64>(p, stream);
+    if (head_dim == 128)
+      return e5m2 ? launch_fna_fp8<true, 128>(p, stream, queues) : launch_fna_fp8<false, 128>(p, stream, queues);
+    return e5m2 ? launch_fna_fp8<true, 64>(p, stream, queues) : launch_fna_fp8<false, 64>(p, stream, queues);
   }
   return fail("fna_forward: unsupported dtype code %d", dtype);
 }

@@ -111,7 +111,7 @@ def amd_fna_generic(
 ) -> Union[Tensor, Tuple[Tensor, Tensor]]:
     """`run_persistent_kernel`: work-queue launch of the forward kernel (resident workgroups pull
     Q tiles from per-XCD queues) instead of a workgroup per Q tile; bit-identical results.  None:
-    whichever was measured faster for this kind of problem (`functional._use_work_queue`).
+    whichever was measured faster for this kind of problem (`functional.work_queue_default`).
 
     `anchored_tiles` (one-launch path only): KV tiles are laid out from the first key of a Q tile's
     window instead of from multiples of the tile extent, so that no tile lies partly before the
@@ -139,12 +139,11 @@ def amd_fna_generic(
     scale = scale or head_dim**-0.5
     d_pad = padded_head_dim(head_dim)
     if run_persistent_kernel is None:
-        from .functional import _use_work_queue
+        from .functional import work_queue_default
 
-        tiles = query.shape[0] * query.shape[-2]
-        for X, d, t in zip(query.shape[1 : 1 + na_dim], dilation, q_tile_shape):
-            tiles *= -(-(-(-X // d)) // t) * d
-        run_persistent_kernel = _use_work_queue(None, is_causal, tiles)
+        run_persistent_kernel = work_queue_default(
+            query.shape[0], query.shape[-2], query.shape[1 : 1 + na_dim], kernel_size, stride, dilation, is_causal,
+            q_tile_shape, kv_tile_shape)
     if torch.is_grad_enabled() and (query.requires_grad or key.requires_grad or value.requires_grad):
         bwd_q_tile, bwd_kv_tile = check_fna_backward_config(
             query, kernel_size, stride, dilation, is_causal, backward_q_tile_shape, backward_kv_tile_shape

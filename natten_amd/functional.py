@@ -185,17 +185,32 @@ def neighborhood_attention_generic(
     return (output, lse) if return_lse else output
 
 
-def _use_work_queue(run_persistent_kernel: Optional[bool], is_causal, num_q_tiles: int = 1 << 30) -> bool:
+def _use_work_queue(run_persistent_kernel: Optional[bool], is_causal, num_q_tiles: int = 1 << 30,
+                    kv_tiles_per_q_tile: int = 1 << 10) -> bool:
     """`run_persistent_kernel` as given, or the measured default.  The work-queue launch (resident
-    workgroups pull Q tiles from per-XCD queues) is 1.5-14 % faster than a workgroup per Q tile on
+    workgroups pull Q tiles from per-XCD queues) is 1-7 % faster than a workgroup per Q tile on
     the large non-causal shapes measured, 2-3.5 % slower when dimension 0 is causal (Q tiles of
-    very different lengths), and its second launch (the one that clears the queues) costs more than
-    it gains on problems of a few thousand Q tiles or less: those cases launch a workgroup per
-    tile.  `num_q_tiles`: Q tiles over all batch entries, dilation groups and heads.  Results are
-    bit-identical either way."""
+    very different lengths), and no gain on 2 048 Q tiles x 16 KV tiles or less, where its second
+    launch (the one that clears the queues) costs what the queue gains: those cases launch a
+    workgroup per tile.  `num_q_tiles`: Q tiles over all batch entries, dilation groups and heads;
+    `kv_tiles_per_q_tile`: KV tiles a Q tile visits (an estimate).  Results are bit-identical
+    either way."""
     if run_persistent_kernel is not None:
         return bool(run_persistent_kernel)
-    return (not bool(is_causal[0])) and num_q_tiles >= 8192
+    return (not bool(is_causal[0])) and num_q_tiles >= 2048 and num_q_tiles * kv_tiles_per_q_tile >= 65536
+
+
+def work_queue_default(batch: int, heads: int, token_layout, kernel_size, stride, dilation, is_causal, q_tile_shape,
+                       kv_tile_shape) -> bool:
+    """The launch kind the ops pick when `run_persistent_kernel` is None, from the problem's tile counts."""
+    tiles, visits = batch * heads, 1
+    for X, k, s, d, qt, kt in zip(token_layout, kernel_size, stride, dilation, q_tile_shape, kv_tile_shape):
+        extent = -(-X // d)
+        tiles *= -(-extent // qt) * d
+        # keys the queries of one Q tile attend along this dimension: a window per stride group the tile spans
+        box = min(extent, k + (-(-qt // s) - 1) * s)
+        visits *= -(-box // kt)
+    return _use_work_queue(None, is_causal, tiles, visits)
 
 
 def _make_na(na_dim: int, name: str):

@@ -201,7 +201,12 @@ def test_fp8_matmul_fused_equals_permuted(dtype, D):
         out_f, lse_f = amd_fna_generic(q8, k8, v8, *args, fused=True, anchored_tiles=False, **kw)
         out_p, lse_p = amd_fna_generic(q8, k8, v8, *args, fused=False, **kw)
         out_a, lse_a = amd_fna_generic(q8, k8, v8, *args, fused=True, anchored_tiles=True, **kw)
+        # work-queue launch of the 8-bit kernel: the same bits as a workgroup per Q tile, on both layouts
+        out_aq, lse_aq = amd_fna_generic(q8, k8, v8, *args, fused=True, run_persistent_kernel=True, **kw)
+        out_pq, lse_pq = amd_fna_generic(q8, k8, v8, *args, fused=False, run_persistent_kernel=True, **kw)
     assert torch.equal(out_f, out_p) and torch.equal(lse_f, lse_p)
+    assert torch.equal(out_aq, out_a) and torch.equal(lse_aq, lse_a)
+    assert torch.equal(out_pq, out_p) and torch.equal(lse_pq, lse_p)
     qd, kd, vd = dequantise(q8, sq), dequantise(k8, sk), dequantise(v8, sv)
     ref_o, ref_l = c_oracle.na_forward(to_np(qd), to_np(kd), to_np(vd), *args, None)
     check_out("out", True, to_np(out_f), ref_o, vd)
