@@ -120,3 +120,88 @@ def assert_routes_agree(tag, a, b, shape, dilation, kv_tile):
         assert torch.equal(a, b), "the two routes differ: " + tag
     else:
         assert_close("routes " + tag, to_np(a), to_np(b), atol=4e-3, rtol=8e-3)
+
+
+def _dim_windows(X, k, s, d, causal):
+    """Per token coordinate x of one dimension: (start, end) of its window and its dilation group,
+    in token coordinates: x attends y iff y % d == x % d and start[x] <= y // d < end[x]."""
+    start = np.empty(X, dtype=np.int64)
+    end = np.empty(X, dtype=np.int64)
+    for g in range(d):
+        L = O.fix_dilation_extent(X, d, g)
+        i = np.arange(L)
+        st = O.window_start(i, k, s, L, causal)
+        start[g::d] = st
+        end[g::d] = O.window_end(i, st, k, L, causal)
+    return start, end
+
+
+def sampled_backward_check(q, k, v, d_out, out, lse, dq, dk, dv, kernel, stride, dilation, causal, n_samples, seed,
+                           atol, rtol, scale=None, tag=""):
+    """Checks gradients at a stratified sample of positions against a float64 evaluation of the
+    backward formulas (reference fna_reference_backward.hpp:60-380): dq at sampled queries, dk and dv
+    at sampled keys (all heads of each).  The softmax normalisers (`lse`) and `out` (for
+    delta = rowsum(dO * O)) are the forward's results, which the forward tests check against the
+    oracle on their own; everything else is recomputed from q, k, v, d_out.  One batch entry at a
+    time; only the rows a sample needs leave the device."""
+    B = q.shape[0]
+    n = q.dim() - 3
+    shape = tuple(q.shape[1 : 1 + n])
+    N = int(np.prod(shape))
+    H, Hkv, D = q.shape[-2], k.shape[-2], q.shape[-1]
+    r = H // Hkv
+    kernel, stride, dilation, causal = (tuplify(x, n) for x in (kernel, stride, dilation, causal))
+    scale = float(scale) if scale is not None else float(D) ** -0.5
+    wins = [_dim_windows(X, kk, s, d, c) for X, kk, s, d, c in zip(shape, kernel, stride, dilation, causal)]
+    rng = np.random.default_rng(seed)
+    dev = q.device
+
+    def rows(t, b, tok):  # [len(tok), heads, D] float64
+        return t[b].reshape(N, t.shape[-2], -1)[torch.as_tensor(tok, device=dev)].double().cpu().numpy()
+
+    def keys_of(coord):  # tokens attended by the query at `coord`
+        per = []
+        for a in range(n):
+            st, en = wins[a]
+            d = dilation[a]
+            per.append(np.arange(st[coord[a]], en[coord[a]]) * d + coord[a] % d)
+        return np.ravel_multi_index(tuple(m.ravel() for m in np.meshgrid(*per, indexing="ij")), shape)
+
+    def queries_of(coord):  # tokens of the queries that attend the key at `coord`
+        per = []
+        for a in range(n):
+            st, en = wins[a]
+            d = dilation[a]
+            x = np.arange(coord[a] % d, shape[a], d)
+            j = coord[a] // d
+            per.append(x[(st[x] <= j) & (j < en[x])])
+        return np.ravel_multi_index(tuple(m.ravel() for m in np.meshgrid(*per, indexing="ij")), shape)
+
+    per_batch = -(-n_samples // B)
+    for b in range(B):
+        toks = stratified_tokens(shape, kernel, stride, dilation, causal, per_batch, rng)
+        lse_b = lse[b].reshape(N, H)
+        for tok in toks:
+            coord = np.unravel_index(int(tok), shape)
+            # ---- dq of this query ----------------------------------------------------------------
+            ks = keys_of(coord)
+            qq, dd, oo = (rows(t, b, [tok])[0] for t in (q, d_out, out))          # [H, D]
+            ll = lse_b[int(tok)].double().cpu().numpy()                           # [H]
+            kk_, vv_ = rows(k, b, ks), rows(v, b, ks)                             # [W, Hkv, D]
+            kk_h, vv_h = np.repeat(kk_, r, axis=1), np.repeat(vv_, r, axis=1)     # [W, H, D]
+            p = np.exp(scale * np.einsum("hd,whd->wh", qq, kk_h) - ll[None, :])
+            ds = p * (np.einsum("hd,whd->wh", dd, vv_h) - np.sum(dd * oo, axis=-1)[None, :])
+            ref_dq = scale * np.einsum("wh,whd->hd", ds, kk_h)
+            assert_close(f"sampled dq {tag} batch {b} token {coord}", rows(dq, b, [tok])[0], ref_dq, atol, rtol)
+            # ---- dk, dv of the key at the same position --------------------------------------------
+            qs = queries_of(coord)
+            kx, vx = (rows(t, b, [tok])[0] for t in (k, v))                       # [Hkv, D]
+            kx_h, vx_h = np.repeat(kx, r, axis=0), np.repeat(vx, r, axis=0)       # [H, D]
+            qa, da, oa = rows(q, b, qs), rows(d_out, b, qs), rows(out, b, qs)     # [Wq, H, D]
+            la = lse_b[torch.as_tensor(qs, device=dev)].double().cpu().numpy()    # [Wq, H]
+            p = np.exp(scale * np.einsum("whd,hd->wh", qa, kx_h) - la)
+            ds = p * (np.einsum("whd,hd->wh", da, vx_h) - np.sum(da * oa, axis=-1))
+            ref_dv = np.einsum("wh,whd->hd", p, da).reshape(Hkv, r, D).sum(axis=1)
+            ref_dk = scale * np.einsum("wh,whd->hd", ds, qa).reshape(Hkv, r, D).sum(axis=1)
+            assert_close(f"sampled dk {tag} batch {b} token {coord}", rows(dk, b, [tok])[0], ref_dk, atol, rtol)
+            assert_close(f"sampled dv {tag} batch {b} token {coord}", rows(dv, b, [tok])[0], ref_dv, atol, rtol)

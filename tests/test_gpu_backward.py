@@ -266,8 +266,8 @@ def _pairs(B, H, shape, k):
 def test_reference_problem_lists_backward(na_dim):
     # the hand-picked problems of the reference's test-suite (tests/problems.py), forward + backward
     # as tests/test_blackwell_fna.py runs them, each non-causal and causal along its first
-    # dimension; the largest ones (more than 6e7 query-key pairs for the float64 oracle) are
-    # left to the sampled checks of tests/test_gpu_configs.py
+    # dimension; the largest ones (more than 6e7 query-key pairs for the float64 oracle) run in
+    # test_large_reference_problems_backward_sampled below
     from tests import problems
 
     cases = {1: problems.NA_1D, 2: problems.NA_2D, 3: problems.NA_3D}[na_dim]
@@ -280,3 +280,38 @@ def test_reference_problem_lists_backward(na_dim):
             run_backward(B, H, Hkv, D, shape, k, s, d, causal, dtype, seed=100 + i)
             ran += 1
     assert ran >= 16
+
+
+def _large_backward_cases():
+    from tests import problems
+
+    cases = []
+    for na_dim, lst in ((1, problems.NA_1D), (2, problems.NA_2D), (3, problems.NA_3D)):
+        cases += [(na_dim, i, c) for i, c in enumerate(lst) if _pairs(c[0], c[1], c[4], c[5]) > 6e7]
+    # the long 1-D problems of the reference's profiler tests (tests/problems.py NA_1D_LONG): both ends of the strides
+    cases += [(1, 100 + i, c) for i, c in enumerate(problems.NA_1D_LONG) if c[6] in ((2048,), (1,))]
+    return cases
+
+
+@pytest.mark.parametrize("na_dim,idx,case", _large_backward_cases())
+def test_large_reference_problems_backward_sampled(na_dim, idx, case):
+    # the reference problems too large for the whole-tensor float64 oracle: gradients at a stratified
+    # sample of positions (corners, borders, stride-group and causal boundaries, random ones) against
+    # the backward formulas in float64, non-causal and causal along the first dimension
+    from tests.gpu_utils import sampled_backward_check
+
+    B, H, Hkv, D, shape, k, s, d = case
+    dtype = torch.bfloat16 if idx % 2 == 0 else torch.float16
+    for causal in ((False,) * na_dim, (True,) + (False,) * (na_dim - 1)):
+        q, kk, v = make_qkv(B, shape, H, Hkv, D, dtype, seed=300 + idx)
+        gen = torch.Generator().manual_seed(1300 + idx)
+        d_out = torch.randn(q.shape, generator=gen).to(dtype).cuda()
+        for t in (q, kk, v):
+            t.requires_grad_(True)
+        out, lse = NA[na_dim](q, kk, v, k, s, d, causal, return_lse=True)
+        out.backward(d_out)
+        torch.cuda.synchronize()
+        tag = f"{shape} k={k} s={s} d={d} c={causal} H={H}/{Hkv} D={D} {dtype}"
+        sampled_backward_check(q.detach(), kk.detach(), v.detach(), d_out, out.detach(), lse.detach(), q.grad, kk.grad,
+                               v.grad, k, s, d, causal, n_samples=48, seed=idx, atol=TOL[dtype], rtol=TOL[dtype],
+                               tag=tag)

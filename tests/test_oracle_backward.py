@@ -120,3 +120,38 @@ def test_dense_attention_backward_causal_cross_lengths():
     out.backward(torch.tensor(do))
     for g, t in zip(got, (tq, tk, tv)):
         np.testing.assert_allclose(g, t.grad.numpy(), rtol=1e-9, atol=1e-11)
+
+
+@pytest.mark.parametrize("case", [
+    # shape, kernel, stride, dilation, causal, H, Hkv
+    ((37,), (7,), (2,), (3,), (False,), 2, 1),
+    ((9, 14), (3, 5), (1, 2), (2, 1), (True, False), 4, 2),
+    ((5, 6, 9), (2, 3, 4), (1, 2, 1), (1, 1, 2), (False, True, False), 2, 2),
+])
+def test_sampled_backward_checker_agrees_with_the_whole_tensor_oracle(case):
+    # The GPU tests of the largest problems check gradients position by position with
+    # gpu_utils.sampled_backward_check; here that checker is held against the whole-tensor float64
+    # oracle on small problems (every dilation group, stride groups, causal dims, GQA): exact
+    # gradients must pass at 1e-9, and a gradient with one perturbed row must fail.
+    from tests.gpu_utils import sampled_backward_check
+
+    shape, k, s, d, causal, H, Hkv = case
+    D, B = 8, 2
+    rng = np.random.default_rng(5)
+    q = rng.standard_normal((B, *shape, H, D)).astype(np.float32)
+    kk = rng.standard_normal((B, *shape, Hkv, D)).astype(np.float32)
+    v = rng.standard_normal((B, *shape, Hkv, D)).astype(np.float32)
+    do = rng.standard_normal(q.shape).astype(np.float32)
+    out, lse = O.na_forward(q, kk, v, k, s, d, causal)
+    dq, dk, dv = O.na_backward(q, kk, v, do, k, s, d, causal)
+    t = lambda x: torch.from_numpy(np.ascontiguousarray(x, dtype=np.float64))
+    n_tok = int(np.prod(shape))
+    args = (t(q), t(kk), t(v), t(do), t(out), t(lse), t(dq), t(dk), t(dv), k, s, d, causal)
+    sampled_backward_check(*args, n_samples=2 * n_tok, seed=1, atol=1e-9, rtol=1e-9)
+    for which in (6, 7, 8):
+        bad = list(args)
+        g = args[which].clone()
+        g.view(B, n_tok, -1)[1, n_tok // 2] += 1e-3   # the checker samples 2 * n_tok positions: every one is hit
+        bad[which] = g
+        with pytest.raises(AssertionError):
+            sampled_backward_check(*bad, n_samples=4 * n_tok, seed=1, atol=1e-9, rtol=1e-9)
