@@ -48,6 +48,8 @@ WORKLOADS = {
 # Published forward runtimes of the reference's Blackwell FNA kernel on a B200 for those shapes
 # (kernel only / with token permute; docs/sample-outputs/profiler-*-blackwell-fna-b200.txt): other
 # hardware, context only, never a baseline for `vs_baseline`.
+SUB_MILLISECOND_WORKLOADS = ("c2", "c2d", "c3", "c5")
+
 REFERENCE_B200_MS = {
     "hunyuan_na": (42.243, 47.353),
     "hunyuan_gna": (13.010, 18.538),
@@ -389,16 +391,27 @@ def bench_backward(args, q, k, v, kernel, stride, dilation, causal, dt_name):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=None,
+                    help="timed steps (default 20; 300 for the workloads whose step takes less than a millisecond)")
+    ap.add_argument("--warmup", type=int, default=None, help="untimed steps before them (default 5; 100 for those)")
     ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS))
     ap.add_argument("--q-tile", type=str, default=None, help="comma separated, e.g. 2,8,8")
     ap.add_argument("--kv-tile", type=str, default=None)
     ap.add_argument("--backward", action="store_true",
                     help="measure the backward pass (forward + backward step, backward kernels) instead of the forward metric")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--step-only", action="store_true",
+                    help="skip the side measurements (kernel through the C ABI alone, token-permuted route): "
+                         "a profile of such a run holds the step's launches only")
     ap.add_argument("--no-mfma-probe", action="store_true")
     args = ap.parse_args()
+    # a step of the small workloads lasts 30-200 us: twenty of them end before the device's clocks have
+    # settled (c3 reads 0.19-0.21 ms over 20 steps and 0.162 ms sustained), so they get longer loops
+    short = args.workload in SUB_MILLISECOND_WORKLOADS and not args.backward
+    if args.steps is None:
+        args.steps = 300 if short else 20
+    if args.warmup is None:
+        args.warmup = 100 if short else 5
     if args.gpus != 1:
         print("bench.py: this build measures one GPU; --gpus above 1 is not supported (no multi-GPU path).",
               file=sys.stderr)
@@ -529,12 +542,25 @@ def main():
         # the step is this one launch when the one-launch route applies: its duration is then the
         # event time of the timed steps themselves; otherwise the kernel is timed on its own
         kernel_ms = step_events_ms if fused else timed(kern, args.steps)
-        kernel_alone_ms = timed(kern, args.steps)
-        kernel_permuted_ms = timed(kern_permuted, args.steps)
-        op, lp = kern_permuted()
-        perm_ms = timed(lambda: token_permute_operation(tp_in, q_tile, dilation), args.steps)
-        unperm_ms = timed(lambda: token_unpermute_operation(op, qkv_shape, q_tile, dilation), args.steps)
-    q_bytes = qp.numel() * qp.element_size()
+        extras = {}
+        if not args.step_only:
+            kernel_alone_ms = timed(kern, args.steps)
+            kernel_permuted_ms = timed(kern_permuted, args.steps)
+            op, lp = kern_permuted()
+            perm_ms = timed(lambda: token_permute_operation(tp_in, q_tile, dilation), args.steps)
+            unperm_ms = timed(lambda: token_unpermute_operation(op, qkv_shape, q_tile, dilation), args.steps)
+            q_bytes = qp.numel() * qp.element_size()
+            extras = {
+                "kernel_direct_call_ms": kernel_alone_ms,
+                "kernel_on_permuted_operands_ms": kernel_permuted_ms,
+                "e2e_permuted_route_ms": 3 * perm_ms + kernel_permuted_ms + unperm_ms,
+                "token_permute": {
+                    "permute_q_ms": perm_ms,
+                    "unpermute_o_ms": unperm_ms,
+                    "permute_GBps": 2 * q_bytes / (perm_ms * 1e-3) / 1e9,
+                    "unpermute_GBps": 2 * op.numel() * op.element_size() / (unperm_ms * 1e-3) / 1e9,
+                },
+            }
     achieved = flops / (kernel_ms * 1e-3) / 1e12
     peak = PEAK_TFLOPS[dt_name]
     dense_flops = 4.0 * B * H * D * float(q.numel() // (B * H * D)) ** 2
@@ -567,15 +593,7 @@ def main():
         "kernel_ms": kernel_ms,
         "kernel_ms_source": ("HIP events around the timed steps (one launch per step)" if fused else
                              "HIP events around kernel-only launches"),
-        "kernel_direct_call_ms": kernel_alone_ms,
-        "kernel_on_permuted_operands_ms": kernel_permuted_ms,
-        "e2e_permuted_route_ms": 3 * perm_ms + kernel_permuted_ms + unperm_ms,
-        "token_permute": {
-            "permute_q_ms": perm_ms,
-            "unpermute_o_ms": unperm_ms,
-            "permute_GBps": 2 * q_bytes / (perm_ms * 1e-3) / 1e9,
-            "unpermute_GBps": 2 * op.numel() * op.element_size() / (unperm_ms * 1e-3) / 1e9,
-        },
+        **extras,
         "roofline": {
             "kernel": "fna_fwd_fp8_kernel" if quantised else "fna_fwd_kernel",
             "bound": "mfma",
