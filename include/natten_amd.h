@@ -46,7 +46,7 @@ extern "C" {
 #define NATTEN_AMD_F16 0
 #define NATTEN_AMD_BF16 1
 #define NATTEN_AMD_F8E4M3 2 /* OCP e4m3fn operands, bf16 output */
-#define NATTEN_AMD_F32 3    /* merge payloads only */
+#define NATTEN_AMD_F32 3    /* float32 operands and output (natten_amd_fna_forward), merge payloads */
 #define NATTEN_AMD_F8E5M2 4 /* OCP e5m2 operands, bf16 output */
 
 /* ABI version; bumped whenever a signature changes. */
@@ -81,6 +81,11 @@ const char* natten_amd_last_error(void);
  * widen them to bf16 while permuting (natten_amd_token_permute_widen, exact) and call this
  * function with dtype BF16 and the scales.
  *
+ * float32 operands (dtype F32; the reference's tests run float32 at atol 1e-4,
+ * tests/test_fna.py:107-131): tiles of 128 x 64 tokens, head_dim 32, 64 or 128, no scales; products,
+ * sums and softmax in float32 (P not rounded), output float32.  This entry point only (no one-launch
+ * form, no backward).
+ *
  * run_persistent (the reference's `run_persistent` argument, blackwell_fna.h:52, scheduler
  * csrc/include/natten/cuda/fmha_blackwell/kernel/fmha_tile_scheduler.hpp:146-149): non-zero
  * launches as many workgroups as the device keeps resident, which take Q tiles from per-XCD work
@@ -89,7 +94,7 @@ const char* natten_amd_last_error(void);
  * at least natten_amd_fna_forward_workspace_bytes() bytes, cleared by the launch itself (by a
  * kernel, so the call may be captured in a graph) and free for reuse once the work queued on
  * `stream` by this call has run.  Two calls must not use one workspace concurrently.  Tile
- * pairs other than 128 x 64 tokens ignore the flag.  run_persistent == 0:
+ * pairs other than 128 x 64 tokens and float32 operands ignore the flag.  run_persistent == 0:
  * workspace may be NULL.
  */
 uint64_t natten_amd_fna_forward_workspace_bytes(void);

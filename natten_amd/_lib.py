@@ -212,7 +212,7 @@ def fna_forward(
     per-XCD queues kept in a small workspace) instead of a workgroup per Q tile; same results."""
     L = lib()
     _require_gpu(q, k, v)
-    if q.dtype not in (torch.float16, torch.bfloat16) + FP8_DTYPES:
+    if q.dtype not in (torch.float16, torch.bfloat16, torch.float32) + FP8_DTYPES:
         raise NotImplementedError(f"natten_amd fna_forward does not support {q.dtype}.")
     na_dim = len(kernel_size)
     scales = _scale_ptrs(q, k, q_scale, k_scale, v_scale)

@@ -14,6 +14,7 @@
 
 #include "fna_bwd.hpp"
 #include "fna_fwd.hpp"
+#include "fna_fwd_f32.hpp"
 #include "fna_fwd_fp8.hpp"
 #include "merge.hpp"
 #include "mfma_probe.hpp"
@@ -154,6 +155,25 @@ int dispatch_dtype(const FnaParams& p, int dtype, int head_dim, int qt, int kvt,
       return e5m2 ? launch_fna_fp8<true, 128>(p, stream, queues) : launch_fna_fp8<false, 128>(p, stream, queues);
     return e5m2 ? launch_fna_fp8<true, 64>(p, stream, queues) : launch_fna_fp8<false, 64>(p, stream, queues);
   }
+  if (dtype == NATTEN_AMD_F32) {
+    // float32 operands and output: one plain kernel configuration on token-permuted sequences
+    if (qt != 128 || kvt != 64)
+      return fail("fna_forward: float32 operands need a Q tile of 128 and a KV tile of 64 tokens, got %d and %d", qt, kvt);
+    if (p.fused || p.cu_q != nullptr) return fail("fna_forward: float32 operands run on token-permuted sequences only");
+    if (p.seqlen_kv % kvt != 0)
+      return fail("fna_forward: seqlen_kv (%d) must be a multiple of the KV tile (%d tokens)", p.seqlen_kv, kvt);
+    if (p.q_scale || p.k_scale || p.v_scale) return fail("fna_forward: float32 operands take no dequantisation scales");
+    if ((p.seqlen_q + qt - 1) / qt != p.num_q_tiles) return fail("fna_forward: internal tile count mismatch");
+    const long long wgs = (long long)p.num_q_tiles * p.heads_q * p.batch;
+    if (wgs > 0x7fffffffLL) return fail("fna_forward: problem needs more than 2^31 workgroups");
+    switch (head_dim) {
+      case 32: hipLaunchKernelGGL((fna_fwd_f32_kernel<32>), dim3((unsigned)wgs), dim3(256), 0, stream, p); break;
+      case 64: hipLaunchKernelGGL((fna_fwd_f32_kernel<64>), dim3((unsigned)wgs), dim3(256), 0, stream, p); break;
+      case 128: hipLaunchKernelGGL((fna_fwd_f32_kernel<128>), dim3((unsigned)wgs), dim3(256), 0, stream, p); break;
+      default: return fail("fna_forward: unsupported head_dim %d", head_dim);
+    }
+    return check_launch("fna_forward (float32)");
+  }
   return fail("fna_forward: unsupported dtype code %d", dtype);
 }
 
@@ -249,6 +269,12 @@ int natten_amd_window(int query, int kernel_size, int stride, int extent, int is
 int natten_amd_fna_supported_tiles(int dtype, int head_dim, int32_t* q_sizes, int32_t* kv_sizes, int capacity) {
   if (dtype == NATTEN_AMD_F8E4M3 || dtype == NATTEN_AMD_F8E5M2) {
     if (head_dim != 64 && head_dim != 128) return 0;
+    if (capacity > 0 && q_sizes) q_sizes[0] = 128;
+    if (capacity > 0 && kv_sizes) kv_sizes[0] = 64;
+    return 1;
+  }
+  if (dtype == NATTEN_AMD_F32) {
+    if (head_dim != 32 && head_dim != 64 && head_dim != 128) return 0;
     if (capacity > 0 && q_sizes) q_sizes[0] = 128;
     if (capacity > 0 && kv_sizes) kv_sizes[0] = 64;
     return 1;

@@ -19,6 +19,8 @@ from .tile_config import check_fna_backward_config, check_fna_forward_config, pa
 from .token_permute import token_permute_operation, token_unpermute_operation
 
 SUPPORTED_DTYPES = (torch.float16, torch.bfloat16, torch.float8_e4m3fn, torch.float8_e5m2)
+# neighborhood attention also takes float32 (forward only, token-permuted route, a kernel of its own)
+FNA_DTYPES = SUPPORTED_DTYPES + (torch.float32,)
 FP8_DTYPES = _lib.FP8_DTYPES
 
 
@@ -63,8 +65,8 @@ def can_run_amd_fna(query: Tensor, key: Tensor, value: Tensor, raise_error: bool
         return no("natten_amd runs on MI355X device tensors only; got a tensor on " + str(query.device) + ".")
     if not _lib.has_lib():
         return no("natten_amd native library is not built (python -m natten_amd.build).", ImportError)
-    if query.dtype not in SUPPORTED_DTYPES:
-        return no(f"natten_amd FNA supports {SUPPORTED_DTYPES}, got {query.dtype}.")
+    if query.dtype not in FNA_DTYPES:
+        return no(f"natten_amd FNA supports {FNA_DTYPES}, got {query.dtype}.")
     if query.shape[-1] != value.shape[-1]:
         return no("natten_amd FNA does not support different head dims for QK and V.", ValueError)
     if query.shape[-1] > 128 or query.shape[-1] % 8 != 0:
@@ -73,6 +75,8 @@ def can_run_amd_fna(query: Tensor, key: Tensor, value: Tensor, raise_error: bool
         return no(f"natten_amd FNA needs head dims that are multiples of 16 for 8-bit floats, got {query.shape[-1]}.")
     if is_fp8(query.dtype) and torch.is_grad_enabled() and (query.requires_grad or key.requires_grad or value.requires_grad):
         return no("natten_amd has no backward pass for 8-bit float operands.")
+    if query.dtype == torch.float32 and torch.is_grad_enabled() and (query.requires_grad or key.requires_grad or value.requires_grad):
+        return no("natten_amd has no backward pass for float32 operands (forward only).")
     return True
 
 
@@ -160,6 +164,8 @@ def amd_fna_generic(
         query, key, value = (_pad_head_dim(t, d_pad) for t in (query, key, value))
 
     in_dtype = query.dtype
+    if in_dtype == torch.float32 and not (q_scale is None and k_scale is None and v_scale is None):
+        raise ValueError("natten_amd: dequantisation scales belong to 8- and 16-bit operands; float32 operands take none.")
     fp8_ok = (
         is_fp8(in_dtype) and d_pad in (64, 128)
         and _prod(q_tile_shape) == 128 and _prod(kv_tile_shape) == 64
@@ -171,7 +177,7 @@ def amd_fna_generic(
         )
     use_fp8 = fp8_ok and fp8_matmul is not False
     widen = is_fp8(in_dtype) and not use_fp8
-    fusable = (not widen) and _lib.fused_layout_supported(query.shape[1 : 1 + na_dim], dilation, kv_tile_shape,
+    fusable = (not widen) and in_dtype != torch.float32 and _lib.fused_layout_supported(query.shape[1 : 1 + na_dim], dilation, kv_tile_shape,
                                                           row_bytes=key.shape[-2] * d_pad * 2,
                                                           q_tile_shape=q_tile_shape, dtype=in_dtype)
     if fused and not fusable:

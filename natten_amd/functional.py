@@ -130,8 +130,9 @@ def neighborhood_attention_generic(
     attn_kwargs = dict(attention_kwargs or {})
     attn_kwargs.pop("torch_compile", None)
 
-    if is_self_attention(query, kernel_size=kernel_size, is_causal=is_causal,
-                         has_additional_attention=has_additional_attention):
+    # (float32 operands stay with the neighborhood kernel, which has a float32 form; dense attention has none)
+    if query.dtype != torch.float32 and is_self_attention(query, kernel_size=kernel_size, is_causal=is_causal,
+                                                          has_additional_attention=has_additional_attention):
         # a window covering the whole input is plain attention over the flattened tokens
         query_shape = query.shape
         q = query.flatten(1, na_dim)
