@@ -26,7 +26,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 # MI355X dense MFMA peak of the instruction the path multiplies with
-PEAK_TFLOPS = {"bf16": 2500.0, "fp16": 2500.0, "e4m3": 5000.0}
+PEAK_TFLOPS = {"bf16": 2500.0, "fp16": 2500.0, "e4m3": 5000.0, "fp32": 157.3}
 
 WORKLOADS = {
     # name: (B, H, layout, D, kernel, stride, dilation, causal, dtype, std)
@@ -34,6 +34,8 @@ WORKLOADS = {
     "c3": (1, 16, (128, 128), 128, (32, 32), (16, 16), (1, 1), (False, False), "fp16", 0.5),
     "c2": (2, 8, (64, 64), 64, (13, 13), (1, 1), (1, 1), (False, False), "bf16", 1.0),
     "c2d": (2, 8, (64, 64), 64, (13, 13), (1, 1), (2, 2), (False, False), "bf16", 1.0),
+    # the configuration the reference runs on the CPU, at its stated type (the float32 kernel, token-permuted route)
+    "c1": (1, 2, (256,), 32, (7,), (1,), (1,), (False,), "fp32", 1.0),
     # e4m3 operands with per-head absmax scales, bf16 output; multiplied by the 8-bit matrix instruction
     "c5": (1, 16, (16, 64, 64), 128, (8, 16, 16), (4, 8, 8), (1, 2, 2), (False, False, False), "e4m3", 1.0),
     # the shapes the reference publishes runtimes for (docs/profiler.md:853-876, :925-951, :654-755; fp16, batch 1)
@@ -48,7 +50,7 @@ WORKLOADS = {
 # Published forward runtimes of the reference's Blackwell FNA kernel on a B200 for those shapes
 # (kernel only / with token permute; docs/sample-outputs/profiler-*-blackwell-fna-b200.txt): other
 # hardware, context only, never a baseline for `vs_baseline`.
-SUB_MILLISECOND_WORKLOADS = ("c2", "c2d", "c3", "c5")
+SUB_MILLISECOND_WORKLOADS = ("c1", "c2", "c2d", "c3", "c5")
 
 REFERENCE_B200_MS = {
     "hunyuan_na": (42.243, 47.353),
@@ -113,6 +115,7 @@ def measured_traffic(workload, which, q_tile, kv_tile):
 WORKLOAD_NAMES = {
     "c4": "na3d bf16 B=1 H=24 30x48x80 D=128 k=(18,24,24) s=(1,8,8) causal=(T,F,F) +LSE",
     "c3": "na2d fp16 B=1 H=16 128x128 D=128 k=(32,32) s=(16,16)",
+    "c1": "na1d fp32 B=1 H=2 L=256 D=32 k=7",
     "c2": "na2d bf16 B=2 H=8 64x64 D=64 k=(13,13)",
     "c2d": "na2d bf16 B=2 H=8 64x64 D=64 k=(13,13) d=(2,2)",
     "c5": "na3d e4m3 (per-head scales, bf16 out) B=1 H=16 16x64x64 D=128 k=(8,16,16) s=(4,8,8) d=(1,2,2)",
@@ -207,7 +210,7 @@ def cpu_baseline(workload, q, k, v, kernel, stride, dilation, causal, dt_name, s
     n = q.dim() - 3
     layout = tuple(int(x) for x in q.shape[1 : 1 + n])
     N = int(np.prod(layout))
-    cpu_dtype = {"bf16": torch.bfloat16, "fp16": torch.float16, "e4m3": torch.bfloat16}[dt_name]
+    cpu_dtype = {"bf16": torch.bfloat16, "fp16": torch.float16, "e4m3": torch.bfloat16, "fp32": torch.float32}[dt_name]
     info = {"unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
             "call": "torch.nn.attention.flex_attention + create_block_mask(BLOCK_SIZE=(64, 64), device='cpu') on "
                     "[B, H, N, D] CPU tensors, return_lse=True, FORCE_USE_FLEX_ATTENTION: the call of the reference's "
@@ -427,7 +430,7 @@ def main():
     dev = torch.device("cuda:0")
     B, H, layout, D, kernel, stride, dilation, causal, dt_name, std = WORKLOADS[args.workload]
     quantised = dt_name == "e4m3"
-    dtype = {"bf16": torch.bfloat16, "fp16": torch.float16, "e4m3": torch.bfloat16}[dt_name]
+    dtype = {"bf16": torch.bfloat16, "fp16": torch.float16, "e4m3": torch.bfloat16, "fp32": torch.float32}[dt_name]
     n = len(layout)
     gen = torch.Generator().manual_seed(0)
     q, k, v = ((torch.randn((B, *layout, H, D), generator=gen) * std).to(dev) for _ in range(3))
@@ -504,8 +507,9 @@ def main():
             tp_in = q
         scale = D**-0.5
 
-        fused = _lib.fused_layout_supported(layout, dilation, kv_tile, q_tile_shape=q_tile,
-                                            dtype=None if quantised else dtype)
+        # (float32 operands have no one-launch form: their step is permute + kernel + unpermute)
+        fused = dtype != torch.float32 and _lib.fused_layout_supported(layout, dilation, kv_tile, q_tile_shape=q_tile,
+                                                                       dtype=None if quantised else dtype)
 
         from natten_amd.functional import work_queue_default
 
@@ -595,7 +599,8 @@ def main():
                              "HIP events around kernel-only launches"),
         **extras,
         "roofline": {
-            "kernel": "fna_fwd_fp8_kernel" if quantised else "fna_fwd_kernel",
+            "kernel": ("fna_fwd_fp8_kernel" if quantised else
+                       "fna_fwd_f32_kernel" if dtype == torch.float32 else "fna_fwd_kernel"),
             "bound": "mfma",
             "achieved": achieved,
             "peak": peak,
