@@ -26,6 +26,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 # MI355X dense MFMA peak of the instruction the path multiplies with
+HBM_PEAK_GBPS = 8000.0
 PEAK_TFLOPS = {"bf16": 2500.0, "fp16": 2500.0, "e4m3": 5000.0, "fp32": 157.3}
 
 WORKLOADS = {
@@ -569,6 +570,9 @@ def main():
     peak = PEAK_TFLOPS[dt_name]
     dense_flops = 4.0 * B * H * D * float(q.numel() // (B * H * D)) ** 2
 
+    # bytes of Q, K, V read and O, LSE written once
+    alg_bytes = (4 * q.numel() * (1 if quantised else q.element_size()) + (q.numel() if quantised else 0)
+                 + q.numel() // D * 4)
     which = "forward_fp8" if quantised else "forward"
     traffic = measured_traffic(args.workload, which, q_tile, kv_tile) if fused else None
     result = {
@@ -609,10 +613,15 @@ def main():
             "traffic": traffic["bytes"] if traffic else None,
             "traffic_source": traffic["source"] if traffic else None,
             "kernel_digest": kernel_digest(which),
-            "algorithmic_bytes": (4 * q.numel() * (1 if quantised else q.element_size())
-                                  + (q.numel() if quantised else 0) + lse.numel() * 4),
+            "algorithmic_bytes": alg_bytes,
         },
     }
+    if flops / alg_bytes < peak * 1e12 / (HBM_PEAK_GBPS * 1e9):
+        # fewer FLOP per algorithmic byte than the chip's ridge point: memory (here mostly launch latency) bounds
+        # the kernel, and the figure to read is bytes per second (c1, c2)
+        gbps = alg_bytes / (kernel_ms * 1e-3) / 1e9
+        result["roofline"].update({"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                                   "frac": gbps / HBM_PEAK_GBPS, "mfma_frac": achieved / peak})
     if not args.no_mfma_probe:
         # context for roofline.frac: what the matrix cores sustain on random operands under the
         # chip's power limit (the published peak assumes the maximum clock)
