@@ -284,9 +284,12 @@ struct FnaSmem {
 // RAGGED: seqlen_kv is not a multiple of KVT (dense attention on unpadded sequences); the tile
 // copies then clamp their rows and are issued at the top of an iteration instead of one per slot.
 // The work of one workgroup on one Q tile; `pid` is the position of that tile in the launch order
-// (what blockIdx.x is when every Q tile has a workgroup of its own).
-template <typename T, int D, int NWAVES, int MQ, bool RAGGED, int KVT>
-static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const int pid) {
+// (what blockIdx.x is when every Q tile has a workgroup of its own).  `before_stores()` is called
+// once, after the last KV tile and before the results are stored: nothing of this wave is in flight
+// at that point (the work-queue launch fetches its next position there, so that the wait for the
+// fetch does not include the stores); a call that returns early does not make it.
+template <typename T, int D, int NWAVES, int MQ, bool RAGGED, int KVT, typename Hook>
+static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const int pid, Hook&& before_stores) {
   constexpr int NT = NWAVES * 64;
   constexpr int QT = NWAVES * MQ * 32;
   constexpr int KSTEPS = D / 16;
@@ -1079,6 +1082,7 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
     if (j + 1 < total_tiles) iteration(Stage1{}, std::true_type{}, std::true_type{}, j + 1);
   }
   wait_vmcnt<0>();  // the last iterations' copies into the unused stage must land before the LDS is released
+  before_stores();
 
   // ---- epilogue: O = acc / rowsum, LSE = ln(rowsum) + scale * rowmax -------------------------
   T* obase = reinterpret_cast<T*>(p.o) + q_row_base * q_row_stride + int64_t(head) * D;
@@ -1110,7 +1114,7 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
 template <typename T, int D, int NWAVES, int MQ, bool RAGGED, int KVT>
 __global__ void __launch_bounds__(NWAVES * 64) __attribute__((amdgpu_waves_per_eu(MQ == 1 ? 2 : 1, MQ == 1 ? 2 : 1)))
 fna_fwd_kernel(const FnaParams p) {
-  fna_fwd_tile<T, D, NWAVES, MQ, RAGGED, KVT>(p, int(blockIdx.x));
+  fna_fwd_tile<T, D, NWAVES, MQ, RAGGED, KVT>(p, int(blockIdx.x), []() {});
 }
 
 // Work-queue launch: as many workgroups as the chip keeps resident, each taking Q tiles until
@@ -1145,10 +1149,13 @@ static __device__ __forceinline__ const FnaParams& fna_params_for_this_tile(FnaK
 #pragma clang diagnostic pop
 }
 
-// The loop of a resident workgroup: `tile(pid)` is run for every launch position the workgroup
-// pulls, first from the queue of its own XCD, then from the others'.  Thread 0 fetches the position
-// after the current one while the other waves start on the current tile.  All queue state lives in
-// LDS: nothing of it occupies a register while a tile is worked on.
+// The loop of a resident workgroup: `tile(pid, fetch)` is run for every launch position the workgroup
+// pulls, first from the queue of its own XCD, then from the others'.  `fetch` pulls the position after
+// the current one; the tile calls it between its last KV tile and its stores, where the wave has
+// nothing in flight, so that the wait for the counter's old value is a wait for that alone (issued
+// after the stores it would also wait for their completion); a tile that returns without calling it
+// has it called here.  All queue state lives in LDS: nothing of it occupies a register while a tile
+// is worked on.
 template <typename Tile>
 static __device__ __forceinline__ void fna_queue_loop(uint32_t* __restrict__ queues, const int per_xcd, Tile&& tile) {
   __shared__ int s_pos[2];   // s_pos[i & 1]: position of the workgroup's i-th tile (-1: none is left)
@@ -1177,8 +1184,13 @@ static __device__ __forceinline__ void fna_queue_loop(uint32_t* __restrict__ que
     __syncthreads();
     const int pid = __builtin_amdgcn_readfirstlane(s_pos[i]);
     if (pid < 0) break;
-    if (threadIdx.x == 0) s_pos[i ^ 1] = take();
-    tile(pid);
+    bool fetched = false;
+    auto fetch = [&]() __attribute__((always_inline)) {
+      if (threadIdx.x == 0) s_pos[i ^ 1] = take();
+      fetched = true;
+    };
+    tile(pid, fetch);
+    if (!fetched) fetch();
   }
 }
 
@@ -1186,8 +1198,8 @@ template <typename T, int D, int NWAVES, int MQ, bool RAGGED, int KVT>
 __global__ void __launch_bounds__(NWAVES * 64) __attribute__((amdgpu_waves_per_eu(MQ == 1 ? 2 : 1, MQ == 1 ? 2 : 1)))
 fna_fwd_queue_kernel(const FnaParams p, uint32_t* __restrict__ queues, const int per_xcd) {
   FnaKernargPtr args = fna_kernarg_params();
-  fna_queue_loop(queues, per_xcd, [&](int pid) __attribute__((always_inline)) {
-    fna_fwd_tile<T, D, NWAVES, MQ, RAGGED, KVT>(fna_params_for_this_tile(args), pid);
+  fna_queue_loop(queues, per_xcd, [&](int pid, auto& fetch) __attribute__((always_inline)) {
+    fna_fwd_tile<T, D, NWAVES, MQ, RAGGED, KVT>(fna_params_for_this_tile(args), pid, fetch);
   });
   (void)p;
 }

@@ -35,8 +35,8 @@ constexpr float kFp8LazyRescaleLog2 = 2.0f; // so that 2^6 * 2^2 = 256 stays bel
 // LDS tile: 64 rows of D bytes, 16-byte chunks XOR-swizzled by (row / rows-per-256-bytes); the
 // rows of a V tile are stored in the order the P fragment holds its keys (see v_key_of_lds_row).
 // `pid`: the launch position (the workgroup id of a launch with one workgroup per Q tile).
-template <bool E5M2, int D, int NWAVES>
-static __device__ __forceinline__ void fna_fwd_fp8_tile(const FnaParams& p, const uint32_t pid) {
+template <bool E5M2, int D, int NWAVES, typename Hook>
+static __device__ __forceinline__ void fna_fwd_fp8_tile(const FnaParams& p, const uint32_t pid, Hook&& before_stores) {
   constexpr int KVT = 64;
   constexpr int NT = NWAVES * 64;
   constexpr int QT = NWAVES * 32;
@@ -545,6 +545,7 @@ static __device__ __forceinline__ void fna_fwd_fp8_tile(const FnaParams& p, cons
     if (j + 1 < total_tiles) iteration(Stage1{}, j + 1);
   }
   wait_vmcnt<0>();  // copies into the unused stage must land before the LDS is released
+  before_stores();  // (see fna_fwd_tile)
 
   // ---- epilogue: O = acc / rowsum (bf16), LSE = ln(rowsum) + scale * rowmax - ln(2^6) ----------
   __bf16* obase = reinterpret_cast<__bf16*>(p.o) + q_row_base * q_row_stride + int64_t(head) * D;
@@ -575,7 +576,7 @@ static __device__ __forceinline__ void fna_fwd_fp8_tile(const FnaParams& p, cons
 template <bool E5M2, int D, int NWAVES>
 __global__ void __launch_bounds__(NWAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 fna_fwd_fp8_kernel(const FnaParams p) {
-  fna_fwd_fp8_tile<E5M2, D, NWAVES>(p, blockIdx.x);
+  fna_fwd_fp8_tile<E5M2, D, NWAVES>(p, blockIdx.x, []() {});
 }
 
 // Work-queue form (see fna_fwd_queue_kernel).
@@ -583,8 +584,8 @@ template <bool E5M2, int D, int NWAVES>
 __global__ void __launch_bounds__(NWAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 fna_fwd_fp8_queue_kernel(const FnaParams p, uint32_t* __restrict__ queues, const int per_xcd) {
   FnaKernargPtr args = fna_kernarg_params();
-  fna_queue_loop(queues, per_xcd, [&](int pid) __attribute__((always_inline)) {
-    fna_fwd_fp8_tile<E5M2, D, NWAVES>(fna_params_for_this_tile(args), uint32_t(pid));
+  fna_queue_loop(queues, per_xcd, [&](int pid, auto& fetch) __attribute__((always_inline)) {
+    fna_fwd_fp8_tile<E5M2, D, NWAVES>(fna_params_for_this_tile(args), uint32_t(pid), fetch);
   });
   (void)p;
 }
