@@ -91,9 +91,13 @@ const char* natten_amd_last_error(void);
  * launches as many workgroups as the device keeps resident, which take Q tiles from per-XCD work
  * queues until none is left, instead of one workgroup per Q tile; results are bit-identical.
  * The queues are counters in `workspace`: device memory owned by the caller, 64-byte aligned,
- * at least natten_amd_fna_forward_workspace_bytes() bytes, cleared by the launch itself (by a
- * kernel, so the call may be captured in a graph) and free for reuse once the work queued on
- * `stream` by this call has run.  Two calls must not use one workspace concurrently.  Tile
+ * at least natten_amd_fna_forward_workspace_bytes() bytes, free for reuse once the work queued on
+ * `stream` by this call has run.  run_persistent == 1: the launch clears them first (by a kernel,
+ * so the call may be captured in a graph): any memory will do.  run_persistent == 2: the caller
+ * vouches that they are zero, which is how every work-queue launch leaves them (its last workgroup
+ * resets them): a workspace zeroed once and then only handed to these launches, one at a time,
+ * needs no clearing again, and the call is a single kernel launch.  Two calls must not use one
+ * workspace concurrently.  Tile
  * pairs other than 128 x 64 tokens and float32 operands ignore the flag.  run_persistent == 0:
  * workspace may be NULL.
  */

@@ -19,7 +19,7 @@ from torch import Tensor
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libnatten_amd.so")
 
-ABI_VERSION = 9
+ABI_VERSION = 10
 
 DTYPE_CODES = {
     torch.float16: 0,
@@ -231,15 +231,27 @@ def fna_forward(
     return out, lse
 
 
+_QUEUE_WORKSPACES = {}
+
+
 def _queue_workspace(like: Tensor, run_persistent: bool):
     """(flag, pointer, bytes) of the work-queue launch's workspace, allocated by the caller side as
     the reference's wrappers allocate theirs (src/natten/_libnatten/torch_wrappers.py:688-693)."""
     if not run_persistent:
         return 0, None, 0
     nbytes = int(lib().natten_amd_fna_forward_workspace_bytes())
-    # the launch clears it; torch's allocator hands the block out again only to later work of this stream
-    ws = torch.empty(nbytes, dtype=torch.uint8, device=like.device)
-    return 1, ws.data_ptr(), nbytes
+    stream = torch.cuda.current_stream(like.device)
+    if torch.cuda.is_current_stream_capturing():
+        # memory allocated under capture belongs to the graph: a block of its own, cleared by the launch
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=like.device)
+        return 1, ws.data_ptr(), nbytes
+    # One block per (device, stream), zeroed once: every work-queue launch leaves its counters at zero,
+    # and launches of one stream run one after the other, so the block is never cleared again.
+    key = (like.device.index, stream.cuda_stream)
+    ws = _QUEUE_WORKSPACES.get(key)
+    if ws is None:
+        ws = _QUEUE_WORKSPACES[key] = torch.zeros(nbytes, dtype=torch.uint8, device=like.device)
+    return 2, ws.data_ptr(), nbytes
 
 
 def _tile_span_fits(token_layout, dilation, tile_shape, row_bytes: int) -> bool:

@@ -1127,6 +1127,7 @@ fna_fwd_kernel(const FnaParams p) {
 // `8 * per_xcd + 8` counter increments in total, whatever the other workgroups do.
 constexpr int kQueueStride = 16;  // uint32 counters per 64-byte line
 constexpr int kQueueWords = kNumXcd * kQueueStride;
+constexpr int kQueueDoneWord = 1;  // workgroups that have left the loop (in the first queue's line)
 
 // The launch parameters of a work-queue kernel, read anew for every tile.  Left to itself the compiler
 // hoists the set-up's reads of launch parameters (and what it derives from them) out of the loop
@@ -1191,6 +1192,16 @@ static __device__ __forceinline__ void fna_queue_loop(uint32_t* __restrict__ que
     };
     tile(pid, fetch);
     if (!fetched) fetch();
+  }
+  // The last workgroup to leave puts the counters back to zero, so that the next launch finds them
+  // as it needs them.  (Every other workgroup has seen all queues empty by then: its counter
+  // increments, whose old values it waited for, are complete.)
+  if (threadIdx.x == 0) {
+    const uint32_t left = atomicAdd(&queues[kQueueDoneWord], 1u);
+    if (left == gridDim.x - 1) {
+      for (int x = 0; x < kNumXcd; ++x) __hip_atomic_store(&queues[x * kQueueStride], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(&queues[kQueueDoneWord], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
   }
 }
 

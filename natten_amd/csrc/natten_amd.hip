@@ -74,19 +74,26 @@ int resident_workgroups() {
   return cached[dev];
 }
 
-// `queues` != nullptr: work-queue launch (kQueueWords zero-initialised counters are cleared and used).
+// The counters of a work-queue launch (null: one workgroup per Q tile).  Every work-queue kernel
+// leaves the counters at zero when its last workgroup ends; `clear_first` clears them by a kernel
+// before the launch, for memory whose contents are not known.
+struct WorkQueue {
+  uint32_t* counters = nullptr;
+  bool clear_first = true;
+};
+
 template <typename T, int D, int NWAVES, int MQ, bool RAGGED, int KVT>
-int launch_fna(const FnaParams& p, hipStream_t stream, uint32_t* queues = nullptr) {
+int launch_fna(const FnaParams& p, hipStream_t stream, WorkQueue queues = {}) {
   constexpr int QT = NWAVES * MQ * 32;
   if (!fna_tiles_are_powers_of_two(p)) return fail("fna_forward: tile extents must be powers of two");
   if ((p.seqlen_q + QT - 1) / QT != p.num_q_tiles) return fail("fna_forward: internal tile count mismatch");
   const long long wgs = (long long)((p.total_groups + kNumXcd - 1) / kNumXcd) * kNumXcd * p.wg_group;
   if (wgs > 0x7fffffffLL) return fail("fna_forward: problem needs more than 2^31 workgroups");
-  if (queues != nullptr) {
+  if (queues.counters != nullptr) {
     const long long resident = resident_workgroups();
-    hipLaunchKernelGGL(fna_queue_clear_kernel, dim3(1), dim3(kQueueWords), 0, stream, queues);
+    if (queues.clear_first) hipLaunchKernelGGL(fna_queue_clear_kernel, dim3(1), dim3(kQueueWords), 0, stream, queues.counters);
     hipLaunchKernelGGL((fna_fwd_queue_kernel<T, D, NWAVES, MQ, RAGGED, KVT>), dim3((unsigned)(wgs < resident ? wgs : resident)),
-                       dim3(NWAVES * 64), 0, stream, p, queues, int(wgs / kNumXcd));
+                       dim3(NWAVES * 64), 0, stream, p, queues.counters, int(wgs / kNumXcd));
     return check_launch("fna_forward (work queue)");
   }
   hipLaunchKernelGGL((fna_fwd_kernel<T, D, NWAVES, MQ, RAGGED, KVT>), dim3((unsigned)wgs), dim3(NWAVES * 64), 0, stream, p);
@@ -94,17 +101,17 @@ int launch_fna(const FnaParams& p, hipStream_t stream, uint32_t* queues = nullpt
 }
 
 template <bool E5M2, int D>
-int launch_fna_fp8(const FnaParams& p, hipStream_t stream, uint32_t* queues) {
+int launch_fna_fp8(const FnaParams& p, hipStream_t stream, WorkQueue queues) {
   constexpr int QT = 128;
   if (!fna_tiles_are_powers_of_two(p)) return fail("fna_forward: tile extents must be powers of two");
   if ((p.seqlen_q + QT - 1) / QT != p.num_q_tiles) return fail("fna_forward: internal tile count mismatch");
   const long long wgs = (long long)((p.total_groups + kNumXcd - 1) / kNumXcd) * kNumXcd * p.wg_group;
   if (wgs > 0x7fffffffLL) return fail("fna_forward: problem needs more than 2^31 workgroups");
-  if (queues != nullptr) {
+  if (queues.counters != nullptr) {
     const long long resident = resident_workgroups();
-    hipLaunchKernelGGL(fna_queue_clear_kernel, dim3(1), dim3(kQueueWords), 0, stream, queues);
+    if (queues.clear_first) hipLaunchKernelGGL(fna_queue_clear_kernel, dim3(1), dim3(kQueueWords), 0, stream, queues.counters);
     hipLaunchKernelGGL((fna_fwd_fp8_queue_kernel<E5M2, D, 4>), dim3((unsigned)(wgs < resident ? wgs : resident)), dim3(256), 0,
-                       stream, p, queues, int(wgs / kNumXcd));
+                       stream, p, queues.counters, int(wgs / kNumXcd));
     return check_launch("fna_forward (work queue)");
   }
   hipLaunchKernelGGL((fna_fwd_fp8_kernel<E5M2, D, 4>), dim3((unsigned)wgs), dim3(256), 0, stream, p);
@@ -112,7 +119,7 @@ int launch_fna_fp8(const FnaParams& p, hipStream_t stream, uint32_t* queues) {
 }
 
 template <typename T, int D>
-int dispatch_tiles(const FnaParams& p, int qt, int kvt, hipStream_t stream, uint32_t* queues) {
+int dispatch_tiles(const FnaParams& p, int qt, int kvt, hipStream_t stream, WorkQueue queues) {
   if (p.seqlen_kv % kvt != 0 || p.cu_q != nullptr || p.edge == 2) {
     // key sequences that end inside a tile: dense attention on unpadded or packed sequences only
     if (qt == 128 && kvt == 64) return launch_fna<T, D, 4, 1, true, 64>(p, stream);
@@ -126,7 +133,7 @@ int dispatch_tiles(const FnaParams& p, int qt, int kvt, hipStream_t stream, uint
 }
 
 template <typename T>
-int dispatch_head_dim(const FnaParams& p, int head_dim, int qt, int kvt, hipStream_t stream, uint32_t* queues) {
+int dispatch_head_dim(const FnaParams& p, int head_dim, int qt, int kvt, hipStream_t stream, WorkQueue queues) {
   switch (head_dim) {
     case 32: return dispatch_tiles<T, 32>(p, qt, kvt, stream, queues);
     case 64: return dispatch_tiles<T, 64>(p, qt, kvt, stream, queues);
@@ -136,7 +143,7 @@ int dispatch_head_dim(const FnaParams& p, int head_dim, int qt, int kvt, hipStre
 }
 
 int dispatch_dtype(const FnaParams& p, int dtype, int head_dim, int qt, int kvt, hipStream_t stream,
-                   uint32_t* queues = nullptr) {
+                   WorkQueue queues = {}) {
   switch (dtype) {
     case NATTEN_AMD_F16: return dispatch_head_dim<_Float16>(p, head_dim, qt, kvt, stream, queues);
     case NATTEN_AMD_BF16: return dispatch_head_dim<__bf16>(p, head_dim, qt, kvt, stream, queues);
@@ -236,20 +243,22 @@ int fill_fna_params(const char* what, FnaParams& p, int na_dim, const int* q_sha
 
 // The queue counters of a work-queue launch inside the caller's workspace (nullptr: launch a
 // workgroup per Q tile).  rc != 0 on a workspace that cannot hold them.
-int queue_workspace(const char* what, int run_persistent, void* workspace, uint64_t workspace_bytes, uint32_t** queues) {
-  *queues = nullptr;
+int queue_workspace(const char* what, int run_persistent, void* workspace, uint64_t workspace_bytes, WorkQueue* queues) {
+  *queues = WorkQueue{};
   if (!run_persistent) return 0;
+  if (run_persistent != 1 && run_persistent != 2) return fail("%s: run_persistent must be 0, 1 or 2, got %d", what, run_persistent);
   if (!workspace || workspace_bytes < uint64_t(kQueueWords) * 4 || (reinterpret_cast<uintptr_t>(workspace) & 63))
     return fail("%s: run_persistent needs a 64-byte aligned device workspace of at least %d bytes (got %p, %llu bytes)", what,
                 kQueueWords * 4, workspace, (unsigned long long)workspace_bytes);
-  *queues = static_cast<uint32_t*>(workspace);
+  queues->counters = static_cast<uint32_t*>(workspace);
+  queues->clear_first = run_persistent == 1;  // 2: the caller vouches for zeros (what every launch leaves behind)
   return 0;
 }
 }  // namespace
 
 extern "C" {
 
-int natten_amd_abi_version(void) { return 9; }
+int natten_amd_abi_version(void) { return 10; }
 
 uint64_t natten_amd_fna_forward_workspace_bytes(void) { return uint64_t(kQueueWords) * 4; }
 
@@ -297,7 +306,7 @@ int natten_amd_fna_forward(const void* q, const void* k, const void* v, void* ou
                            int run_persistent, void* workspace, uint64_t workspace_bytes, void* stream) {
   g_error[0] = 0;
   if (na_dim < 1 || na_dim > 3) return fail("fna_forward: na_dim must be 1, 2 or 3, got %d", na_dim);
-  uint32_t* queues;
+  WorkQueue queues;
   if (int rc = queue_workspace("fna_forward", run_persistent, workspace, workspace_bytes, &queues)) return rc;
   if (int rc = check_common("fna_forward", q, k, v, out, lse, batch, seqlen_q, seqlen_kv, heads_q, heads_kv, head_dim))
     return rc;
@@ -343,7 +352,7 @@ int fna_forward_fused_impl(const void* q, const void* k, const void* v, void* ou
                            const int32_t* kernel_size, const int32_t* stride, const int32_t* dilation,
                            const int32_t* is_causal, const int32_t* q_tile_shape, const int32_t* kv_tile_shape,
                            float scale, const float* q_scale, const float* k_scale, const float* v_scale,
-                           int anchor_kv_tiles, uint32_t* queues, void* stream) {
+                           int anchor_kv_tiles, WorkQueue queues, void* stream) {
   if (!qkv_shape || !kernel_size || !stride || !dilation || !is_causal || !q_tile_shape || !kv_tile_shape)
     return fail("fna_forward_fused: null shape argument");
   int qs[3] = {1, 1, 1}, ks[3] = {1, 1, 1};
@@ -425,7 +434,7 @@ int natten_amd_fna_forward_fused(const void* q, const void* k, const void* v, vo
                                  void* workspace, uint64_t workspace_bytes, void* stream) {
   g_error[0] = 0;
   if (na_dim < 1 || na_dim > 3) return fail("fna_forward_fused: na_dim must be 1, 2 or 3, got %d", na_dim);
-  uint32_t* queues;
+  WorkQueue queues;
   if (int rc = queue_workspace("fna_forward_fused", run_persistent, workspace, workspace_bytes, &queues)) return rc;
   return fna_forward_fused_impl(q, k, v, out, lse, dtype, na_dim, batch, heads_q, heads_kv, head_dim, qkv_shape,
                                 kernel_size, stride, dilation, is_causal, q_tile_shape, kv_tile_shape, scale, q_scale,
@@ -489,8 +498,9 @@ int natten_amd_fna_forward_fused_static(const void* q, const void* k, const void
   if (batch < 1 || heads_q < 1 || q_tiles * batch * heads_q > (1LL << 31) - 4096)
     return fail("%s: %lld Q tiles x %d x %d exceed the 2^31 positions the static queues can count", what, q_tiles, batch,
                 heads_q);
-  uint32_t* queues = static_scratch(what);
-  if (queues == nullptr) return 1;
+  WorkQueue queues;  // (cleared by a kernel before every launch: the array is shared by all callers on this GPU)
+  queues.counters = static_scratch(what);
+  if (queues.counters == nullptr) return 1;
   return fna_forward_fused_impl(q, k, v, out, lse, dtype, na_dim, batch, heads_q, heads_kv, head_dim, qkv_shape,
                                 kernel_size, stride, dilation, is_causal, q_tile_shape, kv_tile_shape, scale, q_scale,
                                 k_scale, v_scale, /*anchor_kv_tiles=*/1, queues, stream);

@@ -189,16 +189,16 @@ def neighborhood_attention_generic(
 def _use_work_queue(run_persistent_kernel: Optional[bool], is_causal, num_q_tiles: int = 1 << 30,
                     kv_tiles_per_q_tile: int = 1 << 10) -> bool:
     """`run_persistent_kernel` as given, or the measured default.  The work-queue launch (resident
-    workgroups pull Q tiles from per-XCD queues) is 1-7 % faster than a workgroup per Q tile on
-    the large non-causal shapes measured, 2-3.5 % slower when dimension 0 is causal (Q tiles of
-    very different lengths), and no gain on 2 048 Q tiles x 16 KV tiles or less, where its second
-    launch (the one that clears the queues) costs what the queue gains: those cases launch a
-    workgroup per tile.  `num_q_tiles`: Q tiles over all batch entries, dilation groups and heads;
-    `kv_tiles_per_q_tile`: KV tiles a Q tile visits (an estimate).  Results are bit-identical
-    either way."""
+    workgroups pull Q tiles from per-XCD queues; a workgroup fetches its next position between its last
+    KV tile and its stores) saves the 3-4 us a CU slot stands empty between two workgroups of a
+    one-workgroup-per-tile launch: 2.5-10 % on the large shapes measured, causal or not; on 2 048 Q
+    tiles x 16 KV tiles (c3) the two are within 2 % of each other either way, and below that the queue's
+    bookkeeping costs more than it saves.  `num_q_tiles`: Q tiles over all batch entries, dilation
+    groups and heads; `kv_tiles_per_q_tile`: KV tiles a Q tile visits (an estimate).  Results are
+    bit-identical either way."""
     if run_persistent_kernel is not None:
         return bool(run_persistent_kernel)
-    return (not bool(is_causal[0])) and num_q_tiles >= 2048 and num_q_tiles * kv_tiles_per_q_tile >= 65536
+    return num_q_tiles >= 2048 and num_q_tiles * kv_tiles_per_q_tile >= 65536
 
 
 def work_queue_default(batch: int, heads: int, token_layout, kernel_size, stride, dilation, is_causal, q_tile_shape,

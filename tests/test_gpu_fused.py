@@ -174,6 +174,11 @@ def test_work_queue_launch_equals_one_workgroup_per_tile(case, dtype):
     ref_o, ref_l = oracle_full(q, kk, v, k, s, d, causal)
     assert_close("out", to_np(got[0]), ref_o)
     assert_close("lse", to_np(got[1]), ref_l)
+    # the wrapper zeroes its counter block once per (device, stream); every launch must leave it zeroed
+    from natten_amd import _lib
+
+    torch.cuda.synchronize()
+    assert _lib._QUEUE_WORKSPACES and all(int(w.sum()) == 0 for w in _lib._QUEUE_WORKSPACES.values())
 
 
 def test_work_queue_launch_many_more_tiles_than_workgroups():
