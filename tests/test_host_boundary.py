@@ -205,6 +205,12 @@ def test_work_queue_launch_needs_a_workspace():
             args[-4], args[-3], args[-2] = 1, ws, nbytes
             assert getattr(L, name)(*args) != 0
             assert b"workspace" in L.natten_amd_last_error(), L.natten_amd_last_error()
+            args[-4] = 2  # "the workspace is already zero" needs a workspace just the same
+            assert getattr(L, name)(*args) != 0
+            assert b"workspace" in L.natten_amd_last_error(), L.natten_amd_last_error()
+        args[-4], args[-3], args[-2] = 3, 4096, need
+        assert getattr(L, name)(*args) != 0
+        assert b"run_persistent must be 0, 1 or 2" in L.natten_amd_last_error(), L.natten_amd_last_error()
 
 
 def test_kernel_window_arithmetic_equals_oracle():
