@@ -603,8 +603,9 @@ def main():
                              "HIP events around kernel-only launches"),
         **extras,
         "roofline": {
-            "kernel": ("fna_fwd_fp8_kernel" if quantised else
-                       "fna_fwd_f32_kernel" if dtype == torch.float32 else "fna_fwd_kernel"),
+            "kernel": ("fna_fwd_f32_kernel" if dtype == torch.float32 else
+                       ("fna_fwd_fp8" if quantised else "fna_fwd") +
+                       ("_queue_kernel" if kscales["run_persistent"] else "_kernel")),
             "bound": "mfma",
             "achieved": achieved,
             "peak": peak,
