@@ -131,3 +131,18 @@ def test_traffic_is_only_reported_for_the_current_kernel_sources(tmp_path, monke
     assert bench.measured_traffic("c4", "forward", (2, 8, 8), (1, 8, 8))["bytes"] == 1.5e10
     assert bench.measured_traffic("c4", "forward", (4, 8, 8), (1, 8, 8)) is None
     assert bench.measured_traffic("c3", "forward", (8, 16), (8, 8)) is None  # measured on other sources
+
+
+def test_work_queue_default_by_problem_size():
+    # the launch kind the ops pick when `run_persistent_kernel` is None: the work queue from 2 048 Q
+    # tiles x 32 KV tiles up (every large benchmark shape, causal or not), one workgroup per Q tile below
+    import bench
+    from natten_amd.functional import _use_work_queue, work_queue_default
+    from natten_amd.tile_config import choose_tile_shapes
+
+    expect = {"c1": False, "c2": False, "c2d": False, "c3": False, "c4": True, "c5": True, "hunyuan_na": True,
+              "hunyuan_gna": True, "flux_na": True, "flux_gna": True, "odd3d": True}
+    for w, (B, H, layout, D, k, s, d, c, _, _) in bench.WORKLOADS.items():
+        qt, kt = choose_tile_shapes(layout, k, s, d, c, 128, 64, anchored=True)
+        assert work_queue_default(B, H, layout, k, s, d, c, qt, kt) == expect[w], w
+    assert _use_work_queue(True, (True,), 1, 1) and not _use_work_queue(False, (False,), 1 << 20, 1 << 10)
