@@ -83,3 +83,6 @@ def test_fp32_limits_are_reported():
         na1d(qg, k, v, 7)
     with pytest.raises((NotImplementedError, ValueError)):  # no dequantisation scales for float32
         na1d(q, k, v, 7, q_scale=2.0)
+    extra = torch.randn((1, 16, 2, 32), device="cuda")
+    with pytest.raises(NotImplementedError):             # dense attention (the additional keys' path) has no float32 form
+        na1d(q, k, v, 7, additional_keys=extra, additional_values=extra)

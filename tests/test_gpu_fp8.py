@@ -216,6 +216,34 @@ def test_fp8_matmul_fused_equals_permuted(dtype, D):
     assert_close("lse, anchored tiles", to_np(lse_a), ref_l)
 
 
+@pytest.mark.parametrize("shape,kernel,stride,dilation,causal", [
+    ((5, 18, 30), (3, 7, 9), (1, 2, 3), (1, 2, 1), (True, False, False)),   # extents no tile shape divides
+    ((37, 50), (9, 12), (2, 4), (1, 3), (False, True)),                      # uneven dilation groups
+    ((333,), (65,), (8,), (2,), (False,)),
+])
+def test_fp8_odd_extents_work_queue_equals_per_tile(shape, kernel, stride, dilation, causal):
+    # whatever route the driver picks for extents the tiles do not divide, the 8-bit kernel's
+    # work-queue launch gives the bits of the one-workgroup-per-tile launch, and both match the oracle
+    from natten_amd.fna import amd_fna_generic
+
+    gen = torch.Generator().manual_seed(21)
+    H, Hkv, D = 4, 2, 128
+    q = torch.randn((2, *shape, H, D), generator=gen).cuda()
+    k = torch.randn((2, *shape, Hkv, D), generator=gen).cuda()
+    v = torch.randn((2, *shape, Hkv, D), generator=gen).cuda()
+    (q8, sq), (k8, sk), (v8, sv) = (quantise_per_head(t, torch.float8_e4m3fn) for t in (q, k, v))
+    kw = dict(return_lse=True, q_scale=sq, k_scale=sk, v_scale=sv, out_dtype=torch.bfloat16, fp8_matmul=True)
+    with torch.no_grad():
+        out_t, lse_t = amd_fna_generic(q8, k8, v8, kernel, stride, dilation, causal, run_persistent_kernel=False, **kw)
+        for _ in range(2):
+            out_q, lse_q = amd_fna_generic(q8, k8, v8, kernel, stride, dilation, causal, run_persistent_kernel=True, **kw)
+            assert torch.equal(out_q, out_t) and torch.equal(lse_q, lse_t)
+    qd, kd, vd = dequantise(q8, sq), dequantise(k8, sk), dequantise(v8, sv)
+    ref_o, ref_l = c_oracle.na_forward(to_np(qd), to_np(kd), to_np(vd), kernel, stride, dilation, causal, None)
+    check_out("out", True, to_np(out_q), ref_o, vd)
+    assert_close("lse", to_np(lse_q), ref_l)
+
+
 def test_fp8_matmul_rejects_unsupported_shapes():
     from natten_amd.fna import amd_fna_generic
 
