@@ -110,16 +110,18 @@ fna_bwd_kernel(const FnaBwdParams p) {
   // transpose reads (the accumulations) alike.
   // Stages: tiles are copied NS - 1 ahead.  Two stages at head dim 128 keep a workgroup under
   // half of the CU's LDS, so that two workgroups (two waves per SIMD) share a CU.
-  // The paired role keeps a tile for two steps (the dS waves run one tile behind): three stages
-  // with copies one tile ahead.
+  // The paired role copies two tiles ahead, at any point of a step: Y2 (dO) is read in its own
+  // step only and has three stages; Y1 (Q) and the tables are read for two steps (the dS waves
+  // run one tile behind) and have four.
   constexpr int NS = (D == 128 && !PAIR) ? 2 : 3;
+  constexpr int NS1 = PAIR ? 4 : NS;  // stages of Y1 and of the tables
   static_assert(!PAIR || D == 128, "the paired role is for head dim 128 (smaller ones fit the combined role)");
-  __shared__ __attribute__((aligned(1024))) char sY1[NS * TILE_BYTES];
+  __shared__ __attribute__((aligned(1024))) char sY1[NS1 * TILE_BYTES];
   __shared__ __attribute__((aligned(1024))) char sY2[NS * TILE_BYTES];
-  __shared__ __attribute__((aligned(16))) uint32_t sTabA[NS * BT];
-  __shared__ __attribute__((aligned(16))) uint32_t sTabB[NS * BT];
-  __shared__ __attribute__((aligned(16))) float sLse[NS * BT];
-  __shared__ __attribute__((aligned(16))) float sDelta[NS * BT];
+  __shared__ __attribute__((aligned(16))) uint32_t sTabA[NS1 * BT];
+  __shared__ __attribute__((aligned(16))) uint32_t sTabB[NS1 * BT];
+  __shared__ __attribute__((aligned(16))) float sLse[NS1 * BT];
+  __shared__ __attribute__((aligned(16))) float sDelta[NS1 * BT];
   __shared__ __attribute__((aligned(16))) float sSpare[BT];
   // paired role: probabilities from the P waves to the dS waves, fp16, [tile parity][row block]
   // [sub-block][half of the 16 values][lane] x 16 bytes
@@ -474,7 +476,7 @@ fna_bwd_kernel(const FnaBwdParams p) {
     }
   };
   // the asynchronous copies of a streamed tile (and of its LSE / delta values) into a stage
-  auto issue_copies = [&](const Tile& t, int stage) {
+  auto issue_copies = [&](const Tile& t, int stage, int stage2) {
     const int64_t row = p.fused ? batch_row0 + t.row0 : seq_row_b + t.row0;
     if constexpr (KV_STATIONARY) {
       // LSE / delta of the tile's 64 queries: one asynchronous 4-byte-per-lane copy each
@@ -489,16 +491,16 @@ fna_bwd_kernel(const FnaBwdParams p) {
     const int64_t elem = row * b_stride + int64_t(t.head_b) * D;
     const uint64_t y1 = uniform64(y1_all + elem), y2 = uniform64(y2_all + elem);
     const uint32_t dst = uint32_t(__builtin_amdgcn_readfirstlane(stage * TILE_BYTES + wave * 1024));
+    const uint32_t dst2 = uint32_t(__builtin_amdgcn_readfirstlane(stage2 * TILE_BYTES + wave * 1024));
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
-      const uint32_t d = dst + uint32_t(i * NT * 16);
-      async_copy16_uniform(y1, off_u[i], lds_y1 + d);
-      async_copy16_uniform(y2, off_u[i], lds_y2 + d);
+      async_copy16_uniform(y1, off_u[i], lds_y1 + dst + uint32_t(i * NT * 16));
+      async_copy16_uniform(y2, off_u[i], lds_y2 + dst2 + uint32_t(i * NT * 16));
     }
   };
   auto issue = [&](const Tile& t, int stage, bool masked) {
     build_tables(t, stage, masked);
-    issue_copies(t, stage);
+    issue_copies(t, stage, stage);
   };
 
   // lane-constant LDS read offsets (same fragment layouts as the forward kernel)
@@ -537,11 +539,17 @@ fna_bwd_kernel(const FnaBwdParams p) {
   constexpr int NC = 2 * DB * W;                           // accumulation slots per sub-block
   constexpr int G = N1 + 2 * NC;
   constexpr int PF = 2;                                    // fragments read ahead
-  auto tile_body = [&](auto masked_tag, int stage, uint32_t addc, uint32_t subc, int exch, auto&& after_slot) __attribute__((always_inline)) {
+  // P waves of the paired role: the products of both sub-blocks first, then the accumulations of
+  // both, and the probabilities of a sub-block two per slot between the matrix instructions that
+  // follow its products (sub-block 0: the products of sub-block 1; sub-block 1: the accumulations
+  // of sub-block 0), so that the wave's vector work runs while the matrix pipe does.
+  constexpr bool SPREAD = PAIR;
+  static_assert(!SPREAD || (NP == 8 && NC == 8), "two of a sub-block's 16 probabilities per slot");
+  auto tile_body = [&](auto masked_tag, int stage, int stage2, uint32_t addc, uint32_t subc, int exch, auto&& after_slot) __attribute__((always_inline)) {
     constexpr bool MASKED = decltype(masked_tag)::value;
     (void)exch;  // paired role: which of the two probability buffers this tile writes
     const char* y1 = sY1 + stage * TILE_BYTES;
-    const char* y2 = sY2 + stage * TILE_BYTES;
+    const char* y2 = sY2 + stage2 * TILE_BYTES;  // (stage2 differs from stage in the paired role only)
 
     // slot x of the tile: a product slot (sub-block, index i < NP) or an accumulation slot (i < NC)
     struct Slot {
@@ -549,8 +557,14 @@ fna_bwd_kernel(const FnaBwdParams p) {
       int sb, i;
     };
     auto slot_of = [](int x) constexpr {
-      const int sb = x / (NP + NC), z = x % (NP + NC);
-      return Slot{z < NP, sb, z < NP ? z : z - NP};
+      if constexpr (SPREAD) {
+        const bool prod = x < 2 * NP;
+        const int z = prod ? x : x - 2 * NP, n = prod ? NP : NC;
+        return Slot{prod, z / n, z % n};
+      } else {
+        const int sb = x / (NP + NC), z = x % (NP + NC);
+        return Slot{z < NP, sb, z < NP ? z : z - NP};
+      }
     };
     auto frag = [&](auto x_tag) {
       constexpr Slot sl = slot_of(decltype(x_tag)::value);
@@ -657,12 +671,18 @@ fna_bwd_kernel(const FnaBwdParams p) {
         if constexpr (which == 0) S[sb] = M::run(fr[x], x1f[ks], ks == 0 ? zero : S[sb]);
         else dP[sb] = M::run(fr[x], x2f[ks], ks == 0 ? zero : dP[sb]);
         // all probabilities of the sub-block once its products are complete
-        if constexpr (sl.i == NP - 1) for_range<0, 16>([&](auto r_tag) { elem(std::integral_constant<int, sb>{}, r_tag); });
+        if constexpr (!SPREAD && sl.i == NP - 1) for_range<0, 16>([&](auto r_tag) { elem(std::integral_constant<int, sb>{}, r_tag); });
       } else {
         constexpr int h = sl.i / (DB * W), db = (sl.i / W) % DB;
         constexpr bool to_acc1 = HAS_DS && (sl.i % W == 0);
         if constexpr (to_acc1) acc1[db] = M::run(fr[x], dsf[sb][h], acc1[db]);
         else acc2[db] = M::run(fr[x], pf[sb][h], acc2[db]);
+      }
+      if constexpr (SPREAD && x >= NP && x < 2 * NP + NC) {
+        // two probabilities per slot, between the matrix instructions of the other sub-block
+        constexpr int esb = x < 2 * NP ? 0 : 1, r0 = 2 * (x < 2 * NP ? x - NP : x - 2 * NP);
+        elem(std::integral_constant<int, esb>{}, std::integral_constant<int, r0>{});
+        elem(std::integral_constant<int, esb>{}, std::integral_constant<int, r0 + 1>{});
       }
       after_slot(x_tag);
       __builtin_amdgcn_sched_barrier(0);
@@ -696,34 +716,37 @@ fna_bwd_kernel(const FnaBwdParams p) {
   auto pair_consume = [&](int stage, int exch) __attribute__((always_inline)) {
     const char* y1 = sY1 + stage * TILE_BYTES;
     vec8 dsf[NSB][2];
+    u32x4_t plo[NSB], phi[NSB];
 #pragma unroll
     for (int sb = 0; sb < NSB; ++sb) {
       const char* src = sX + ((((exch * 4 + rw) * NSB + sb) * 2) * 64 + lane) * 16;
-      const u32x4_t lo = *reinterpret_cast<const u32x4_t*>(src);
-      const u32x4_t hi = *reinterpret_cast<const u32x4_t*>(src + 64 * 16);
-#pragma unroll
-      for (int jj = 0; jj < 4; ++jj) {
-        const f32x4_t dl4 = *reinterpret_cast<const f32x4_t*>(&sDelta[stage * BT + sb * 32 + 8 * jj + 4 * g]);
-#pragma unroll
-        for (int i2 = 0; i2 < 2; ++i2) {
-          const int r = 4 * jj + 2 * i2;  // this lane's values r and r + 1 of the sub-block
-          const uint32_t pw = (r < 8) ? lo[r / 2] : hi[r / 2 - 4];
-          const h16x2_t h2 = __builtin_bit_cast(h16x2_t, pw);
-          const float d0 = float(h2[0]) * (held_dp[sb][r] - dl4[2 * i2]);
-          const float d1 = float(h2[1]) * (held_dp[sb][r + 1] - dl4[2 * i2 + 1]);
-          vec2 d2 = {static_cast<T>(d0), static_cast<T>(d1)};
-          dsf[sb][r / 8][r % 8] = d2[0];
-          dsf[sb][r / 8][r % 8 + 1] = d2[1];
-        }
-      }
+      plo[sb] = *reinterpret_cast<const u32x4_t*>(src);
+      phi[sb] = *reinterpret_cast<const u32x4_t*>(src + 64 * 16);
     }
+    // dS values 4 jj + 2 i2 and + 1 of a sub-block (k = 2 jj + i2)
+    f32x4_t dl4;
+    auto ds_pair = [&](auto sb_tag, auto k_tag) {
+      constexpr int sb = decltype(sb_tag)::value, k = decltype(k_tag)::value;
+      constexpr int jj = k / 2, i2 = k % 2, r = 4 * jj + 2 * i2;
+      if constexpr (i2 == 0) dl4 = *reinterpret_cast<const f32x4_t*>(&sDelta[stage * BT + sb * 32 + 8 * jj + 4 * g]);
+      const uint32_t pw = (r < 8) ? plo[sb][r / 2] : phi[sb][r / 2 - 4];
+      const h16x2_t h2 = __builtin_bit_cast(h16x2_t, pw);
+      const float d0 = float(h2[0]) * (held_dp[sb][r] - dl4[2 * i2]);
+      const float d1 = float(h2[1]) * (held_dp[sb][r + 1] - dl4[2 * i2 + 1]);
+      vec2 d2 = {static_cast<T>(d0), static_cast<T>(d1)};
+      dsf[sb][r / 8][r % 8] = d2[0];
+      dsf[sb][r / 8][r % 8 + 1] = d2[1];
+    };
     constexpr int NCB = 2 * DB;  // accumulation slots per sub-block
     constexpr int N = NSB * NCB;
+    static_assert(!PAIR || NCB == 8, "one pair of dS values of sub-block 1 per accumulation slot of sub-block 0");
     vec8 fr[N];
     for_range<0, PF>([&](auto x_tag) {
       constexpr int x = decltype(x_tag)::value;
       fr[x] = tr_frag(y1, x / NCB, (x % NCB) / DB, x % DB);
     });
+    for_range<0, 8>([&](auto k_tag) { ds_pair(std::integral_constant<int, 0>{}, k_tag); });
+    __builtin_amdgcn_sched_barrier(0);
     for_range<0, N>([&](auto x_tag) __attribute__((always_inline)) {
       constexpr int x = decltype(x_tag)::value;
       constexpr int sb = x / NCB, h = (x % NCB) / DB, db = x % DB;
@@ -732,14 +755,17 @@ fna_bwd_kernel(const FnaBwdParams p) {
         fr[y] = tr_frag(y1, y / NCB, (y % NCB) / DB, y % DB);
       }
       acc2[db] = M::run(fr[x], dsf[sb][h], acc2[db]);
+      if constexpr (PAIR && x < NCB) ds_pair(std::integral_constant<int, 1>{}, x_tag);
       __builtin_amdgcn_sched_barrier(0);
     });
   };
+  constexpr int CPT = 2 * PER;  // tile copies per thread and tile
   // One pass of the paired role over n_iter tiles: step `it` has the P waves on tile `it` and the
   // dS waves forming dP of tile `it` after finishing tile it - 1; one more step drains the dS
-  // waves.  The barrier at the top of a step makes tile `it` (copied during step it - 1) and the
-  // probabilities of tile it - 1 visible, and frees the stage of tile it - 2 for the copy of
-  // tile it + 1.
+  // waves.  Tiles are copied two steps ahead: tile it + 2 during step `it`, into the Y2 stage of
+  // tile it - 1 and the Y1 / table stage of tile it - 2, both last read in step it - 1.  The
+  // barrier at the top of a step makes tile `it` and the probabilities of tile it - 1 visible and
+  // separates those last reads from the copies that overwrite them.
   auto run_pass_pair = [&](auto masked_tag, auto ds_wave_tag, int n_iter) __attribute__((always_inline)) {
     constexpr bool MASKED = decltype(masked_tag)::value;
     constexpr bool DS_WAVE = decltype(ds_wave_tag)::value;
@@ -747,30 +773,45 @@ fna_bwd_kernel(const FnaBwdParams p) {
     start_walk(std::integral_constant<bool, !MASKED>{});
     Tile tn = next_tile(std::integral_constant<bool, !MASKED>{}, 1 < n_iter);
     issue(tn, 0, MASKED && !DS_WAVE);  // wave 0, which builds the window tables, is a P wave
-    // The dS waves issue their copies of tile it + 1 right after the barrier (they begin a step
-    // with vector work); the P waves, which begin with matrix work, issue theirs after the
-    // products of the first sub-block, so that the eight waves do not all queue on the CU's
-    // address path while the matrix pipe idles.  (No branch around those copies: past the last
-    // tile the descriptor still names the last one, which is copied again into a stage nobody
-    // reads any more.)
+    if (1 < n_iter) {
+      tn = next_tile(std::integral_constant<bool, !MASKED>{}, 2 < n_iter);
+      issue(tn, 1, MASKED && !DS_WAVE);
+    }
+    // A wave walks to tile it + 2 and issues its share of the copies where it has vector or
+    // scalar work anyway: the dS waves between their two matrix phases, the P waves after the
+    // products of their first sub-block; the eight waves then do not queue on the CU's address
+    // path together while the matrix pipe idles.
+    int s2 = 0;  // it % 3
     for (int it = 0; it <= n_iter; ++it) {
-      wait_vmcnt<0>();
-      __syncthreads();
+      // this thread's copies of tile `it` have landed once only those of tile it + 1 are
+      // outstanding (wave 0 makes one copy less per tile)
       if (it + 1 < n_iter) {
-        tn = next_tile(std::integral_constant<bool, !MASKED>{}, it + 2 < n_iter);
-        build_tables(tn, (it + 1) % NS, MASKED && !DS_WAVE);
+        if (wave != 0) wait_vmcnt<CPT + 1>();
+        else wait_vmcnt<CPT>();
+      } else {
+        wait_vmcnt<0>();
       }
+      __syncthreads();
+      const int s2_ahead = s2 == 0 ? 2 : s2 - 1;  // (it + 2) % 3
+      auto ahead = [&]() __attribute__((always_inline)) {
+        if (it + 2 < n_iter) {
+          tn = next_tile(std::integral_constant<bool, !MASKED>{}, it + 3 < n_iter);
+          build_tables(tn, (it + 2) & 3, MASKED && !DS_WAVE);
+          issue_copies(tn, (it + 2) & 3, s2_ahead);
+        }
+      };
       if constexpr (DS_WAVE) {
-        if (it + 1 < n_iter) issue_copies(tn, (it + 1) % NS);
-        if (it > 0) pair_consume((it - 1) % NS, (it - 1) & 1);
-        if (it < n_iter) pair_produce(it % NS);
+        if (it > 0) pair_consume((it - 1) & 3, (it - 1) & 1);
+        ahead();
+        if (it < n_iter) pair_produce(s2);
       } else {
         if (it < n_iter) {
-          tile_body(masked_tag, it % NS, 0u, 0u, it & 1, [&](auto x_tag) {
-            if constexpr (decltype(x_tag)::value == NP - 1) issue_copies(tn, (it + 1) % NS);
+          tile_body(masked_tag, it & 3, s2, 0u, 0u, it & 1, [&](auto x_tag) __attribute__((always_inline)) {
+            if constexpr (decltype(x_tag)::value == NP - 1) ahead();
           });
         }
       }
+      s2 = s2 == 2 ? 0 : s2 + 1;
     }
     wait_vmcnt<0>();
     __syncthreads();  // stages and probability buffers are free for the next pass
@@ -778,7 +819,6 @@ fna_bwd_kernel(const FnaBwdParams p) {
 
   // ---- pipeline: tile `it` is multiplied while tiles it+1 .. it+NS-1 are in flight ----------------
   // Descriptor queue: d[0] = tile `it`, d[k] = tile it + k.
-  constexpr int CPT = 2 * PER;  // tile copies per thread and tile
   auto run_pass = [&](auto masked_tag, int n_iter) __attribute__((always_inline)) {
     constexpr bool MASKED = decltype(masked_tag)::value;
     if (n_iter <= 0) return;
@@ -835,7 +875,7 @@ fna_bwd_kernel(const FnaBwdParams p) {
           subc |= uint32_t(511 + hi) << (10 * a);
         }
       }
-      tile_body(masked_tag, stage, addc, subc, 0, [](auto) {});
+      tile_body(masked_tag, stage, stage, addc, subc, 0, [](auto) {});
       if constexpr (NEED_ORIGIN) {
 #pragma unroll
         for (int a = 0; a < 3; ++a) {
