@@ -44,6 +44,10 @@ WORKLOADS = {
     "hunyuan_gna": (1, 24, (30, 48, 80), 128, (18, 24, 24), (16, 8, 8), (1, 1, 1), (False, False, False), "fp16", 1.0),
     "flux_na": (1, 24, (256, 256), 128, (80, 80), (1, 1), (1, 1), (False, False), "fp16", 1.0),
     "flux_gna": (1, 24, (256, 256), 128, (80, 80), (16, 16), (1, 1), (False, False), "fp16", 1.0),
+    # its 1-D use case (docs/profiler.md:325-560; one head, 32K tokens, 2K window: sliding, strided, blocked)
+    "na1d_32k": (1, 1, (32768,), 128, (2048,), (1,), (1,), (False,), "fp16", 1.0),
+    "na1d_32k_s256": (1, 1, (32768,), 128, (2048,), (256,), (1,), (False,), "fp16", 1.0),
+    "na1d_32k_blocked": (1, 1, (32768,), 128, (2048,), (2048,), (1,), (False,), "fp16", 1.0),
     # extents that no tile shape divides (and an uneven dilation in time): the one-launch route clamps
     # its gathers; compare `ms_per_step` with `e2e_permuted_route_ms`
     "odd3d": (1, 24, (29, 46, 78), 128, (9, 24, 24), (1, 8, 8), (2, 1, 1), (False, False, False), "bf16", 1.0),
@@ -51,13 +55,17 @@ WORKLOADS = {
 # Published forward runtimes of the reference's Blackwell FNA kernel on a B200 for those shapes
 # (kernel only / with token permute; docs/sample-outputs/profiler-*-blackwell-fna-b200.txt): other
 # hardware, context only, never a baseline for `vs_baseline`.
-SUB_MILLISECOND_WORKLOADS = ("c1", "c2", "c2d", "c3", "c5")
+SUB_MILLISECOND_WORKLOADS = ("c1", "c2", "c2d", "c3", "c5", "na1d_32k", "na1d_32k_s256", "na1d_32k_blocked")
 
 REFERENCE_B200_MS = {
     "hunyuan_na": (42.243, 47.353),
     "hunyuan_gna": (13.010, 18.538),
     "flux_na": (8.692, 10.931),
     "flux_gna": (4.114, 6.389),
+    # (1-D, dilation 1: the reference launches its kernel on the tensors as they are)
+    "na1d_32k": (0.058111, 0.058111),
+    "na1d_32k_s256": (0.037888, 0.037888),
+    "na1d_32k_blocked": (0.038240, 0.038240),
 }
 # Cropped proxies for the CPU baseline where the reference's CPU path (dense N x N mask and scores)
 # does not fit in memory: same kernel / stride / dilation / causal / head dim on a smaller layout
@@ -70,6 +78,9 @@ CPU_PROXY = {
     "flux_na": ((96, 96), 2),
     "flux_gna": ((96, 96), 2),
     "odd3d": ((19, 25, 27), 2),
+    "na1d_32k": ((8192,), 1),
+    "na1d_32k_s256": ((8192,), 1),
+    "na1d_32k_blocked": ((8192,), 1),
 }
 # HBM-side traffic of a launch (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, calibrated on a copy of known
 # size) is read from the profile summaries, which carry one line per measurement:
@@ -125,6 +136,9 @@ WORKLOAD_NAMES = {
     "flux_na": "na2d fp16 B=1 H=24 256x256 D=128 k=(80,80)",
     "flux_gna": "na2d fp16 B=1 H=24 256x256 D=128 k=(80,80) s=(16,16)",
     "odd3d": "na3d bf16 B=1 H=24 29x46x78 D=128 k=(9,24,24) s=(1,8,8) d=(2,1,1)",
+    "na1d_32k": "na1d fp16 B=1 H=1 L=32768 D=128 k=2048",
+    "na1d_32k_s256": "na1d fp16 B=1 H=1 L=32768 D=128 k=2048 s=256",
+    "na1d_32k_blocked": "na1d fp16 B=1 H=1 L=32768 D=128 k=2048 s=2048",
 }
 
 
