@@ -141,8 +141,30 @@ def test_work_queue_default_by_problem_size():
     from natten_amd.tile_config import choose_tile_shapes
 
     expect = {"c1": False, "c2": False, "c2d": False, "c3": False, "c4": True, "c5": True, "hunyuan_na": True,
-              "hunyuan_gna": True, "flux_na": True, "flux_gna": True, "odd3d": True}
+              "hunyuan_gna": True, "flux_na": True, "flux_gna": True, "odd3d": True,
+              "na1d_32k": False, "na1d_32k_s256": False, "na1d_32k_blocked": False}
     for w, (B, H, layout, D, k, s, d, c, _, _) in bench.WORKLOADS.items():
         qt, kt = choose_tile_shapes(layout, k, s, d, c, 128, 64, anchored=True)
         assert work_queue_default(B, H, layout, k, s, d, c, qt, kt) == expect[w], w
     assert _use_work_queue(True, (True,), 1, 1) and not _use_work_queue(False, (False,), 1 << 20, 1 << 10)
+
+
+def test_every_bench_workload_is_named_and_its_cpu_leg_is_bounded():
+    # a workload without a name fails at the end of its run, one whose CPU leg is the full dense
+    # problem runs for minutes without output: both are tables that must follow WORKLOADS
+    import bench
+
+    for w, (B, H, layout, D, k, s, d, c, _, _) in bench.WORKLOADS.items():
+        assert w in bench.WORKLOAD_NAMES, w
+        tokens = 1
+        for x in layout:
+            tokens *= x
+        timed = bench.CPU_PROXY[w][0] if w in bench.CPU_PROXY else layout
+        n = 1
+        for x in timed:
+            n *= x
+        assert n <= 16384, (w, "dense N x N mask and scores of the CPU leg", n)
+        if w in bench.CPU_PROXY:
+            # the proxy keeps the window legal: kernel * dilation fits its layout
+            assert all(kk * dd <= x for kk, dd, x in zip(k, d, timed)), w
+    assert set(bench.REFERENCE_B200_MS) <= set(bench.WORKLOADS)
