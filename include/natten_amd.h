@@ -144,6 +144,28 @@ int natten_amd_fna_forward_fused(const void* q, const void* k, const void* v, vo
                                  void* workspace, uint64_t workspace_bytes, void* stream);
 
 /*
+ * natten_amd_fna_forward_fused for problems with fewer Q tiles than the chip keeps workgroups
+ * resident (few heads, small inputs, long windows): the same operation
+ * (blackwell_na{1,2,3}d_forward, csrc/include/natten/blackwell_fna.h:36-52, with the driver's
+ * permutes folded in) launched with kv_splits (2 .. 8) workgroups per Q tile, each on a
+ * contiguous run of the tile's KV tiles.  out_parts [kv_splits][batch, *qkv_shape, heads_q,
+ * head_dim] and lse_parts [kv_splits][batch, *qkv_shape, heads_q] receive one partial result per
+ * run, normalised over the keys of that run, with their log-sum-exp (zeros and -inf for a query
+ * none of whose keys lie in the run); natten_amd_merge_attentions combines two of them at a time
+ * (src/natten/attn_merge.py:48-105 is the arithmetic), in any order.  fp16 / bf16 operands, Q
+ * tiles of 128 and KV tiles of 64 tokens, no dequantisation scales; other arguments as in
+ * natten_amd_fna_forward_fused.
+ */
+int natten_amd_fna_forward_fused_split(const void* q, const void* k, const void* v, void* out_parts,
+                                       float* lse_parts, int dtype, int na_dim, int batch,
+                                       int heads_q, int heads_kv, int head_dim,
+                                       const int32_t* qkv_shape, const int32_t* kernel_size,
+                                       const int32_t* stride, const int32_t* dilation,
+                                       const int32_t* is_causal, const int32_t* q_tile_shape,
+                                       const int32_t* kv_tile_shape, float scale,
+                                       int anchor_kv_tiles, int kv_splits, void* stream);
+
+/*
  * natten_amd_fna_forward_fused with run_persistent = 1 for callers that cannot allocate device
  * memory (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc):
  * it has no counterpart in the reference.  The queue counters live in a 512-byte array inside

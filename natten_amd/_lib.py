@@ -19,7 +19,7 @@ from torch import Tensor
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libnatten_amd.so")
 
-ABI_VERSION = 10
+ABI_VERSION = 11
 
 DTYPE_CODES = {
     torch.float16: 0,
@@ -55,6 +55,11 @@ _SIGNATURES = {
         ctypes.c_int,
         [ctypes.c_void_p] * 5 + [ctypes.c_int] * 6 + [ctypes.c_void_p] * 7 + [ctypes.c_float] + [ctypes.c_void_p] * 3
         + [ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p],
+    ),
+    "natten_amd_fna_forward_fused_split": (
+        ctypes.c_int,
+        [ctypes.c_void_p] * 5 + [ctypes.c_int] * 6 + [ctypes.c_void_p] * 7 + [ctypes.c_float]
+        + [ctypes.c_int, ctypes.c_int, ctypes.c_void_p],
     ),
     "natten_amd_fna_forward_fused_static": (
         ctypes.c_int,
@@ -311,6 +316,35 @@ def fna_forward_fused(
             _i32(qkv_shape), _i32(kernel_size), _i32(stride), _i32(dilation),
             _i32([1 if c else 0 for c in is_causal]), _i32(q_tile_shape), _i32(kv_tile_shape),
             float(scale), *scales, 1 if anchored_tiles else 0, *_queue_workspace(q, run_persistent), _stream(q),
+        )
+    _check(rc)
+    return out, lse
+
+
+def fna_forward_fused_split(
+    q: Tensor, k: Tensor, v: Tensor,
+    kernel_size, stride, dilation, is_causal, scale: float, q_tile_shape, kv_tile_shape,
+    kv_splits: int, anchored_tiles: bool = True,
+) -> Tuple[Tensor, Tensor]:
+    """fna_forward_fused with the KV tiles of every Q tile dealt to `kv_splits` workgroups: returns
+    the partial results (out_parts [kv_splits, B, *X, H, D], lse_parts float32 [kv_splits, B, *X, H]),
+    each normalised over the keys of its own run of tiles (zeros and -inf where a run holds none of a
+    query's keys); merge_two combines them."""
+    L = lib()
+    _require_gpu(q, k, v)
+    if q.dtype not in (torch.float16, torch.bfloat16):
+        raise NotImplementedError(f"natten_amd fna_forward_fused_split does not support {q.dtype}.")
+    na_dim = len(kernel_size)
+    qkv_shape = [int(x) for x in q.shape[1 : 1 + na_dim]]
+    out = torch.empty((kv_splits, *q.shape), dtype=q.dtype, device=q.device)
+    lse = torch.empty((kv_splits, *q.shape[:-1]), dtype=torch.float32, device=q.device)
+    with torch.cuda.device(q.device):
+        rc = L.natten_amd_fna_forward_fused_split(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
+            DTYPE_CODES[q.dtype], na_dim, q.shape[0], q.shape[-2], k.shape[-2], q.shape[-1],
+            _i32(qkv_shape), _i32(kernel_size), _i32(stride), _i32(dilation),
+            _i32([1 if c else 0 for c in is_causal]), _i32(q_tile_shape), _i32(kv_tile_shape),
+            float(scale), 1 if anchored_tiles else 0, int(kv_splits), _stream(q),
         )
     _check(rc)
     return out, lse

@@ -82,6 +82,12 @@ struct FnaParams {
   int ext_base[3], ext_rem[3];  // qkv_shape / dil and qkv_shape % dil: extent of dilation group g = base + (g < rem)
   NaDiv d_stride[3], d_dil[3], d_q_tiled[3];
   NaDiv d_wg_group, d_groups_per_bh, d_heads_q, d_q_per_kv, d_num_groups;
+  // Split launches only (fna_fwd_split_kernel; 0 otherwise): the KV tiles of every Q tile are dealt
+  // to `kv_splits` workgroups in contiguous runs; workgroup `pid` of the grid works on Q-tile
+  // position pid % split_grid for split pid / split_grid and stores its partial result (normalised
+  // over its own keys, with their LSE) `split` strides into o and lse.
+  int kv_splits, split_grid;
+  int64_t o_split_stride, lse_split_stride;  // elements of the output type / floats
 };
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
@@ -288,8 +294,11 @@ struct FnaSmem {
 // once, after the last KV tile and before the results are stored: nothing of this wave is in flight
 // at that point (the work-queue launch fetches its next position there, so that the wait for the
 // fetch does not include the stores); a call that returns early does not make it.
-template <typename T, int D, int NWAVES, int MQ, bool RAGGED, int KVT, typename Hook>
-static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const int pid, Hook&& before_stores) {
+template <typename T, int D, int NWAVES, int MQ, bool RAGGED, int KVT, bool SPLIT = false, typename Hook>
+static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const int pid_in, Hook&& before_stores) {
+  // split launches: which run of the Q tile's KV tiles this workgroup takes
+  const int split = SPLIT ? pid_in / p.split_grid : 0;
+  const int pid = SPLIT ? pid_in - split * p.split_grid : pid_in;
   constexpr int NT = NWAVES * 64;
   constexpr int QT = NWAVES * MQ * 32;
   constexpr int KSTEPS = D / 16;
@@ -418,7 +427,21 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
       box_n[a] = (en_l - box_org[a] + p.kv_tile[a] - 1) >> p.kv_tile_lg[a];
     }
   }
-  const int total_tiles = box_n[0] * box_n[1] * box_n[2];
+  // The tiles this workgroup visits: all of the box, or run `split` of its kv_splits runs.  A run
+  // that is empty (a box of fewer tiles than splits) still walks one tile, for the sake of one code
+  // path, and stores the result of no keys at all: zeros and an LSE of -inf.
+  const int box_tiles = box_n[0] * box_n[1] * box_n[2];
+  int first_tile = 0, total_tiles = box_tiles;
+  bool empty_split = false;
+  if constexpr (SPLIT) {
+    first_tile = int(int64_t(split) * box_tiles / p.kv_splits);
+    total_tiles = int(int64_t(split + 1) * box_tiles / p.kv_splits) - first_tile;
+    if (total_tiles == 0) {
+      empty_split = true;
+      first_tile = 0;
+      total_tiles = 1;
+    }
+  }
 
   // ---- this wave's share of the Q tile ------------------------------------------------------------
   // Lanes take the tile's tokens in row-major order (dimension 0 slowest), MQ * 32 consecutive
@@ -631,6 +654,12 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
     bool skip;      // no key of the tile is attended by any query of this wave
   };
   int itc[3] = {0, 0, 0};
+  if constexpr (SPLIT) {
+    itc[2] = first_tile % box_n[2];
+    const int rest = first_tile / box_n[2];
+    itc[1] = rest % box_n[1];
+    itc[0] = rest / box_n[1];
+  }
   auto next_tile = [&]() {
     TileInfo t;
     t.full = true;
@@ -1086,9 +1115,14 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
 
   // ---- epilogue: O = acc / rowsum, LSE = ln(rowsum) + scale * rowmax -------------------------
   T* obase = reinterpret_cast<T*>(p.o) + q_row_base * q_row_stride + int64_t(head) * D;
+  float* lse_base = p.lse;
+  if constexpr (SPLIT) {
+    obase += split * p.o_split_stride;
+    lse_base += split * p.lse_split_stride;
+  }
 #pragma unroll
   for (int mb = 0; mb < MQ; ++mb) {
-    const float l = l_run[mb] + __shfl_xor(l_run[mb], 32);
+    const float l = empty_split ? 0.f : l_run[mb] + __shfl_xor(l_run[mb], 32);
     const float inv = (l > 0.f) ? out_scale / l : 0.f;
     const int row = q_row[mb];
     if (row >= 0) {
@@ -1105,7 +1139,7 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
         }
       if (g == 0) {
         const float lse = (l > 0.f) ? (m_run[mb] * 0.6931471805599453f + __logf(l)) : -INFINITY;
-        p.lse[(q_row_base + row) * p.heads_q + head] = lse;
+        lse_base[(q_row_base + row) * p.heads_q + head] = lse;
       }
     }
   }
@@ -1115,6 +1149,17 @@ template <typename T, int D, int NWAVES, int MQ, bool RAGGED, int KVT>
 __global__ void __launch_bounds__(NWAVES * 64) __attribute__((amdgpu_waves_per_eu(MQ == 1 ? 2 : 1, MQ == 1 ? 2 : 1)))
 fna_fwd_kernel(const FnaParams p) {
   fna_fwd_tile<T, D, NWAVES, MQ, RAGGED, KVT>(p, int(blockIdx.x), []() {});
+}
+
+// Split launch: kv_splits workgroups per Q tile, each on a contiguous run of the tile's KV tiles,
+// each storing a partial result; a two-way merge per extra split combines them.  For problems with
+// fewer Q tiles than the chip keeps workgroups resident: a lone workgroup's tile loop is bound by
+// its own instruction issue, not by anything it shares, so two on half the tiles each take about
+// half the time.
+template <typename T, int D, int NWAVES, int MQ, bool RAGGED, int KVT>
+__global__ void __launch_bounds__(NWAVES * 64) __attribute__((amdgpu_waves_per_eu(MQ == 1 ? 2 : 1, MQ == 1 ? 2 : 1)))
+fna_fwd_split_kernel(const FnaParams p) {
+  fna_fwd_tile<T, D, NWAVES, MQ, RAGGED, KVT, true>(p, int(blockIdx.x), []() {});
 }
 
 // Work-queue launch: as many workgroups as the chip keeps resident, each taking Q tiles until
@@ -1236,6 +1281,14 @@ inline void set_wg_layout(FnaParams& p, int tiles_per_wg = 1) {
   const int units = (p.num_q_tiles + tiles_per_wg - 1) / tiles_per_wg;
   p.wg_group = (slab * rows + tiles_per_wg - 1) / tiles_per_wg;
   if (p.wg_group > units) p.wg_group = units;
+  // Few tiles in all (one head, a small input): groups of that size would leave XCDs without work
+  // while others hold several workgroups per CU; smaller groups give every XCD its share.
+  const long long bh = (long long)p.batch * p.heads_q;
+  if (bh * ((units + p.wg_group - 1) / p.wg_group) < kNumXcd) {
+    int want = int((kNumXcd + bh - 1) / bh);  // groups per (batch, head) pair
+    if (want > units) want = units;
+    p.wg_group = (units + want - 1) / want;
+  }
   p.groups_per_bh = (units + p.wg_group - 1) / p.wg_group;
   p.total_groups = p.batch * p.heads_q * p.groups_per_bh;
   // what the kernels' set-up would otherwise divide for (every forward launch comes through here)

@@ -96,6 +96,19 @@ int launch_fna(const FnaParams& p, hipStream_t stream, WorkQueue queues = {}) {
                        dim3(NWAVES * 64), 0, stream, p, queues.counters, int(wgs / kNumXcd));
     return check_launch("fna_forward (work queue)");
   }
+  if (p.kv_splits > 1) {
+    // kv_splits workgroups per Q-tile position, split slowest (positions keep their XCDs: wgs is a multiple of 8)
+    if constexpr (NWAVES == 4 && MQ == 1 && KVT == 64) {
+      if (wgs * p.kv_splits > 0x7fffffffLL) return fail("fna_forward: problem needs more than 2^31 workgroups");
+      FnaParams ps = p;
+      ps.split_grid = int(wgs);
+      hipLaunchKernelGGL((fna_fwd_split_kernel<T, D, NWAVES, MQ, RAGGED, KVT>), dim3((unsigned)(wgs * p.kv_splits)),
+                         dim3(NWAVES * 64), 0, stream, ps);
+      return check_launch("fna_forward (split)");
+    } else {
+      return fail("fna_forward: KV splits exist for Q tiles of 128 and KV tiles of 64 tokens");
+    }
+  }
   hipLaunchKernelGGL((fna_fwd_kernel<T, D, NWAVES, MQ, RAGGED, KVT>), dim3((unsigned)wgs), dim3(NWAVES * 64), 0, stream, p);
   return check_launch("fna_forward");
 }
@@ -148,6 +161,7 @@ int dispatch_dtype(const FnaParams& p, int dtype, int head_dim, int qt, int kvt,
     case NATTEN_AMD_F16: return dispatch_head_dim<_Float16>(p, head_dim, qt, kvt, stream, queues);
     case NATTEN_AMD_BF16: return dispatch_head_dim<__bf16>(p, head_dim, qt, kvt, stream, queues);
   }
+  if (p.kv_splits > 1) return fail("fna_forward: KV splits need fp16 / bf16 operands, got dtype code %d", dtype);
   if (dtype == NATTEN_AMD_F8E4M3 || dtype == NATTEN_AMD_F8E5M2) {
     // 8-bit float operands, bf16 output: one kernel configuration
     if (qt != 128 || kvt != 64)
@@ -258,7 +272,7 @@ int queue_workspace(const char* what, int run_persistent, void* workspace, uint6
 
 extern "C" {
 
-int natten_amd_abi_version(void) { return 10; }
+int natten_amd_abi_version(void) { return 11; }
 
 uint64_t natten_amd_fna_forward_workspace_bytes(void) { return uint64_t(kQueueWords) * 4; }
 
@@ -352,7 +366,7 @@ int fna_forward_fused_impl(const void* q, const void* k, const void* v, void* ou
                            const int32_t* kernel_size, const int32_t* stride, const int32_t* dilation,
                            const int32_t* is_causal, const int32_t* q_tile_shape, const int32_t* kv_tile_shape,
                            float scale, const float* q_scale, const float* k_scale, const float* v_scale,
-                           int anchor_kv_tiles, WorkQueue queues, void* stream) {
+                           int anchor_kv_tiles, WorkQueue queues, void* stream, int kv_splits = 1) {
   if (!qkv_shape || !kernel_size || !stride || !dilation || !is_causal || !q_tile_shape || !kv_tile_shape)
     return fail("fna_forward_fused: null shape argument");
   int qs[3] = {1, 1, 1}, ks[3] = {1, 1, 1};
@@ -420,6 +434,12 @@ int fna_forward_fused_impl(const void* q, const void* k, const void* v, void* ou
   for (int a = 0; a < na_dim; ++a)
     if (qkv_shape[a] / dilation[a] < kv_tile_shape[a]) p.anchor = 0;
   p.tokens = int(tokens);
+  if (kv_splits > 1) {
+    // out and lse hold kv_splits results of the full shape, one after the other
+    p.kv_splits = kv_splits;
+    p.o_split_stride = (int64_t)batch * tokens * heads_q * head_dim;
+    p.lse_split_stride = (int64_t)batch * tokens * heads_q;
+  }
   set_wg_layout(p, 1);
   return dispatch_dtype(p, dtype, head_dim, prod3(p.q_tile), prod3(p.kv_tile), static_cast<hipStream_t>(stream), queues);
 }
@@ -439,6 +459,31 @@ int natten_amd_fna_forward_fused(const void* q, const void* k, const void* v, vo
   return fna_forward_fused_impl(q, k, v, out, lse, dtype, na_dim, batch, heads_q, heads_kv, head_dim, qkv_shape,
                                 kernel_size, stride, dilation, is_causal, q_tile_shape, kv_tile_shape, scale, q_scale,
                                 k_scale, v_scale, anchor_kv_tiles, queues, stream);
+}
+
+int natten_amd_fna_forward_fused_split(const void* q, const void* k, const void* v, void* out_parts, float* lse_parts,
+                                       int dtype, int na_dim, int batch, int heads_q, int heads_kv, int head_dim,
+                                       const int32_t* qkv_shape, const int32_t* kernel_size, const int32_t* stride,
+                                       const int32_t* dilation, const int32_t* is_causal,
+                                       const int32_t* q_tile_shape, const int32_t* kv_tile_shape, float scale,
+                                       int anchor_kv_tiles, int kv_splits, void* stream) {
+  g_error[0] = 0;
+  const char* what = "fna_forward_fused_split";
+  if (na_dim < 1 || na_dim > 3) return fail("%s: na_dim must be 1, 2 or 3, got %d", what, na_dim);
+  if (kv_splits < 2 || kv_splits > 8) return fail("%s: kv_splits must be 2 .. 8, got %d", what, kv_splits);
+  if (dtype != NATTEN_AMD_F16 && dtype != NATTEN_AMD_BF16)
+    return fail("%s: KV splits need fp16 / bf16 operands, got dtype code %d", what, dtype);
+  if (!q_tile_shape || !kv_tile_shape) return fail("%s: null shape argument", what);
+  long long qt = 1, kvt = 1;
+  for (int a = 0; a < na_dim; ++a) {
+    qt *= q_tile_shape[a];
+    kvt *= kv_tile_shape[a];
+  }
+  if (qt != 128 || kvt != 64)
+    return fail("%s: KV splits exist for Q tiles of 128 and KV tiles of 64 tokens, got %lld and %lld", what, qt, kvt);
+  return fna_forward_fused_impl(q, k, v, out_parts, lse_parts, dtype, na_dim, batch, heads_q, heads_kv, head_dim, qkv_shape,
+                                kernel_size, stride, dilation, is_causal, q_tile_shape, kv_tile_shape, scale, nullptr,
+                                nullptr, nullptr, anchor_kv_tiles, WorkQueue{}, stream, kv_splits);
 }
 
 namespace {

@@ -112,8 +112,15 @@ def amd_fna_generic(
     backward_kv_tile_shape=None,
     run_persistent_kernel: Optional[bool] = False,
     anchored_tiles: bool = True,
+    kv_splits: Optional[int] = None,
 ) -> Union[Tensor, Tuple[Tensor, Tensor]]:
-    """`run_persistent_kernel`: work-queue launch of the forward kernel (resident workgroups pull
+    """`kv_splits` (one-launch path, fp16 / bf16, tiles of 128 x 64 tokens): that many workgroups
+    share the KV tiles of every Q tile and their partial results are merged -- for problems with
+    fewer Q tiles than the chip has workgroup slots.  None: `functional.kv_splits_default`, unless
+    `anchored_tiles` is False or a work-queue launch was asked for (both promise the bits of another
+    route); 1: never.  Results differ from the unsplit launch by the rounding of the partial outputs.
+
+    `run_persistent_kernel`: work-queue launch of the forward kernel (resident workgroups pull
     Q tiles from per-XCD queues) instead of a workgroup per Q tile; bit-identical results.  None:
     whichever was measured faster for this kind of problem (`functional.work_queue_default`).
 
@@ -187,15 +194,42 @@ def amd_fna_generic(
             f"dilation * KV tile in every dimension; got {tuple(query.shape[1:1 + na_dim])}, {dilation=}, "
             f"{kv_tile_shape=}, {in_dtype}."
         )
-    if fusable and fused is not False:
-        output, lse = torch_ops.fna_forward_fused(
-            query.contiguous(), key.contiguous(), value.contiguous(), kernel_size, stride, dilation, is_causal,
-            scale, q_tile_shape, kv_tile_shape,
-            q_scale=resolve_scale(q_scale, query.shape[-2], query.device, "q_scale"),
-            k_scale=resolve_scale(k_scale, key.shape[-2], query.device, "k_scale"),
-            v_scale=resolve_scale(v_scale, key.shape[-2], query.device, "v_scale"),
-            run_persistent=bool(run_persistent_kernel), anchored_tiles=bool(anchored_tiles),
+    splittable = (
+        fusable and fused is not False and in_dtype in (torch.float16, torch.bfloat16)
+        and q_scale is None and k_scale is None and v_scale is None
+        and _prod(q_tile_shape) == 128 and _prod(kv_tile_shape) == 64 and not torch_ops._tracing()
+    )
+    if kv_splits is None:
+        from .functional import kv_splits_default
+
+        kv_splits = kv_splits_default(
+            query.shape[0], query.shape[-2], query.shape[1 : 1 + na_dim], kernel_size, stride, dilation, is_causal,
+            q_tile_shape, kv_tile_shape) if (splittable and anchored_tiles and not run_persistent_kernel) else 1
+    if not isinstance(kv_splits, int) or not 1 <= kv_splits <= 8:
+        raise ValueError(f"natten_amd: kv_splits must be an integer from 1 to 8, got {kv_splits!r}.")
+    if kv_splits > 1 and not splittable:
+        raise ValueError(
+            "natten_amd: kv_splits > 1 needs the one-launch path, fp16 / bf16 operands without dequantisation scales "
+            f"and tiles of 128 x 64 tokens (and no graph tracing); got {in_dtype}, {q_tile_shape=}, {kv_tile_shape=}, {fused=}."
         )
+    if fusable and fused is not False:
+        if kv_splits > 1:
+            out_parts, lse_parts = _lib.fna_forward_fused_split(
+                query.contiguous(), key.contiguous(), value.contiguous(), kernel_size, stride, dilation, is_causal,
+                scale, q_tile_shape, kv_tile_shape, kv_splits, anchored_tiles=bool(anchored_tiles),
+            )
+            output, lse = out_parts[0], lse_parts[0]
+            for i in range(1, kv_splits):
+                output, lse = _lib.merge_two(output, lse, out_parts[i], lse_parts[i])
+        else:
+            output, lse = torch_ops.fna_forward_fused(
+                query.contiguous(), key.contiguous(), value.contiguous(), kernel_size, stride, dilation, is_causal,
+                scale, q_tile_shape, kv_tile_shape,
+                q_scale=resolve_scale(q_scale, query.shape[-2], query.device, "q_scale"),
+                k_scale=resolve_scale(k_scale, key.shape[-2], query.device, "k_scale"),
+                v_scale=resolve_scale(v_scale, key.shape[-2], query.device, "v_scale"),
+                run_persistent=bool(run_persistent_kernel), anchored_tiles=bool(anchored_tiles),
+            )
         if d_pad != head_dim:
             output = output[..., :head_dim].contiguous()
         out_dtype = out_dtype or in_dtype
