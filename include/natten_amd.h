@@ -13,6 +13,8 @@
  *                                  csrc/include/natten/blackwell_fna.h:36-52, csrc/natten.cpp:39-160
  *   natten_amd_fna_forward_fused<- the reference driver's permute + kernel + unpermute sequence,
  *                                  src/natten/backends/blackwell_fna.py:99-164, in one launch
+ *   natten_amd_fna_forward_fused_split <- the same forward for small grids: several workgroups per
+ *                                  Q tile, partial results merged by natten_amd_merge_attentions
  *   natten_amd_token_permute    <- token_permute_{1,2,3}d   csrc/include/natten/token_permute.h:34-52
  *   natten_amd_token_permute_widen <- the same, for e4m3 / e5m2 operands (writes bf16)
  *   natten_amd_token_unpermute  <- token_unpermute_{1,2,3}d csrc/include/natten/token_permute.h:54-74
