@@ -14,7 +14,7 @@
  *   natten_amd_fna_forward_fused<- the reference driver's permute + kernel + unpermute sequence,
  *                                  src/natten/backends/blackwell_fna.py:99-164, in one launch
  *   natten_amd_fna_forward_fused_split <- the same forward for small grids: several workgroups per
- *                                  Q tile, partial results merged by natten_amd_merge_attentions
+ *                                  Q tile, partial results merged by natten_amd_merge_attention_parts
  *   natten_amd_token_permute    <- token_permute_{1,2,3}d   csrc/include/natten/token_permute.h:34-52
  *   natten_amd_token_permute_widen <- the same, for e4m3 / e5m2 operands (writes bf16)
  *   natten_amd_token_unpermute  <- token_unpermute_{1,2,3}d csrc/include/natten/token_permute.h:54-74
@@ -34,6 +34,7 @@
  *   natten_amd_compute_delta    <- compute_delta            csrc/include/natten/compute_delta.h:33-36
  *   natten_amd_merge_attentions <- the elementwise merge of src/natten/attn_merge.py:48-105
  *                                  (the reference runs it as framework ops; here it is one kernel)
+ *   natten_amd_merge_attention_parts <- the same merge over any number of partial results at once
  */
 #ifndef NATTEN_AMD_H_
 #define NATTEN_AMD_H_
@@ -153,8 +154,8 @@ int natten_amd_fna_forward_fused(const void* q, const void* k, const void* v, vo
  * contiguous run of the tile's KV tiles.  out_parts [kv_splits][batch, *qkv_shape, heads_q,
  * head_dim] and lse_parts [kv_splits][batch, *qkv_shape, heads_q] receive one partial result per
  * run, normalised over the keys of that run, with their log-sum-exp (zeros and -inf for a query
- * none of whose keys lie in the run); natten_amd_merge_attentions combines two of them at a time
- * (src/natten/attn_merge.py:48-105 is the arithmetic), in any order.  fp16 / bf16 operands, Q
+ * none of whose keys lie in the run); natten_amd_merge_attention_parts combines them
+ * (src/natten/attn_merge.py:48-105 is the arithmetic).  fp16 / bf16 operands, Q
  * tiles of 128 and KV tiles of 64 tokens, no dequantisation scales; other arguments as in
  * natten_amd_fna_forward_fused.
  */
@@ -373,6 +374,18 @@ int natten_amd_token_unpermute(const void* src, void* dst, int elem_bytes, int n
 int natten_amd_merge_attentions(const void* o0, const float* lse0, const void* o1,
                                 const float* lse1, void* out, float* lse_out, int dtype,
                                 int64_t rows, int head_dim, void* stream);
+
+/*
+ * The same merge over num_parts (1 .. 64) partial attentions that lie one after the other:
+ * parts [num_parts][rows, head_dim], lse_parts [num_parts][rows] -- the layout
+ * natten_amd_fna_forward_fused_split writes.  out = sum_i exp(lse_i - lse) parts_i,
+ * lse = log sum_i exp(lse_i), in float32 and rounded once: what src/natten/attn_merge.py:48-105
+ * computes by merging two at a time, without the roundings in between.  A row all of whose parts
+ * hold no key (lse -inf) gives zeros and -inf.
+ */
+int natten_amd_merge_attention_parts(const void* parts, const float* lse_parts, int num_parts,
+                                     void* out, float* lse_out, int dtype, int64_t rows,
+                                     int head_dim, void* stream);
 
 /*
  * Diagnostic without a counterpart in the reference: sustained rate of the bf16 matrix

@@ -19,7 +19,7 @@ from torch import Tensor
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libnatten_amd.so")
 
-ABI_VERSION = 11
+ABI_VERSION = 12
 
 DTYPE_CODES = {
     torch.float16: 0,
@@ -115,6 +115,11 @@ _SIGNATURES = {
     "natten_amd_merge_attentions": (
         ctypes.c_int,
         [ctypes.c_void_p] * 6 + [ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_void_p],
+    ),
+    "natten_amd_merge_attention_parts": (
+        ctypes.c_int,
+        [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int64,
+         ctypes.c_int, ctypes.c_void_p],
     ),
 }
 
@@ -329,7 +334,7 @@ def fna_forward_fused_split(
     """fna_forward_fused with the KV tiles of every Q tile dealt to `kv_splits` workgroups: returns
     the partial results (out_parts [kv_splits, B, *X, H, D], lse_parts float32 [kv_splits, B, *X, H]),
     each normalised over the keys of its own run of tiles (zeros and -inf where a run holds none of a
-    query's keys); merge_two combines them."""
+    query's keys); merge_parts combines them."""
     L = lib()
     _require_gpu(q, k, v)
     if q.dtype not in (torch.float16, torch.bfloat16):
@@ -664,6 +669,28 @@ def merge_two(o0: Tensor, lse0: Tensor, o1: Tensor, lse1: Tensor) -> Tuple[Tenso
         rc = L.natten_amd_merge_attentions(
             o0.data_ptr(), lse0.data_ptr(), o1.data_ptr(), lse1.data_ptr(), out.data_ptr(), lse.data_ptr(),
             DTYPE_CODES[o0.dtype], rows, o0.shape[-1], _stream(o0),
+        )
+    _check(rc)
+    return out, lse
+
+
+def merge_parts(out_parts: Tensor, lse_parts: Tensor) -> Tuple[Tensor, Tensor]:
+    """Merge the partial attentions out_parts [n, ..., D] with float32 LSE lse_parts [n, ...] (the
+    layout fna_forward_fused_split returns) in one launch, float32 arithmetic, one rounding."""
+    L = lib()
+    _require_gpu(out_parts, lse_parts)
+    if out_parts.dtype not in (torch.float16, torch.bfloat16, torch.float32):
+        raise NotImplementedError(f"natten_amd merge does not support {out_parts.dtype}.")
+    if lse_parts.dtype != torch.float32 or lse_parts.shape != out_parts.shape[:-1]:
+        raise ValueError("lse_parts must be float32 of out_parts' shape without the last dimension.")
+    if not (out_parts.is_contiguous() and lse_parts.is_contiguous()):
+        raise ValueError("out_parts and lse_parts must be contiguous.")
+    out = torch.empty(out_parts.shape[1:], dtype=out_parts.dtype, device=out_parts.device)
+    lse = torch.empty(lse_parts.shape[1:], dtype=torch.float32, device=out_parts.device)
+    with torch.cuda.device(out_parts.device):
+        rc = L.natten_amd_merge_attention_parts(
+            out_parts.data_ptr(), lse_parts.data_ptr(), out_parts.shape[0], out.data_ptr(), lse.data_ptr(),
+            DTYPE_CODES[out_parts.dtype], lse.numel(), out_parts.shape[-1], _stream(out_parts),
         )
     _check(rc)
     return out, lse

@@ -61,4 +61,52 @@ __global__ void __launch_bounds__(256) merge_kernel(const T* __restrict__ o0, co
   }
 }
 
+// N-way merge of partial attentions that lie one after the other (`parts[i]` = part 0 + i *
+// part_stride elements, `lses[i]` = lse 0 + i * rows): out = sum_i w_i o_i with
+// w_i = exp(lse_i - lse), lse = log sum_i exp(lse_i), in float32, rounded once.  The same value as
+// the two-way merge applied n - 1 times, without the roundings of its intermediate results.
+// A row whose parts all hold no key (every lse -inf) gives zeros and -inf.
+template <typename T, int VEC>
+__global__ void __launch_bounds__(256) merge_parts_kernel(const T* __restrict__ parts, const float* __restrict__ lses,
+                                                          int num_parts, int64_t part_stride, T* out, float* lse_out,
+                                                          int64_t rows, int head_dim) {
+  typedef T tvec __attribute__((ext_vector_type(VEC)));
+  const int slices = head_dim / VEC;
+  const int64_t total = rows * slices;
+  for (int64_t idx = int64_t(blockIdx.x) * 256 + threadIdx.x; idx < total; idx += int64_t(gridDim.x) * 256) {
+    const int64_t row = idx / slices;
+    const int slice = int(idx - row * slices);
+    float mx = -INFINITY;
+    for (int i = 0; i < num_parts; ++i) mx = fmaxf(mx, lses[i * rows + row]);
+    float acc[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) acc[e] = 0.f;
+    float sum = 0.f;
+    const int64_t at = row * head_dim + int64_t(slice) * VEC;
+    if (mx != -INFINITY) {
+      for (int i = 0; i < num_parts; ++i) {
+        const float w = __expf(lses[i * rows + row] - mx);  // 0 for a part without keys
+        sum += w;
+        if constexpr (VEC == 1) {
+          acc[0] += w * static_cast<float>(parts[i * part_stride + at]);
+        } else {
+          const tvec a = *reinterpret_cast<const tvec*>(parts + i * part_stride + at);
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) acc[e] += w * static_cast<float>(a[e]);
+        }
+      }
+    }
+    const float inv = sum > 0.f ? 1.f / sum : 0.f;
+    if constexpr (VEC == 1) {
+      out[at] = static_cast<T>(acc[0] * inv);
+    } else {
+      tvec r;
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) r[e] = static_cast<T>(acc[e] * inv);
+      *reinterpret_cast<tvec*>(out + at) = r;
+    }
+    if (slice == 0) lse_out[row] = sum > 0.f ? mx + __logf(sum) : -INFINITY;
+  }
+}
+
 }  // namespace natten_amd

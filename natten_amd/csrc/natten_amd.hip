@@ -272,7 +272,7 @@ int queue_workspace(const char* what, int run_persistent, void* workspace, uint6
 
 extern "C" {
 
-int natten_amd_abi_version(void) { return 11; }
+int natten_amd_abi_version(void) { return 12; }
 
 uint64_t natten_amd_fna_forward_workspace_bytes(void) { return uint64_t(kQueueWords) * 4; }
 
@@ -1163,6 +1163,39 @@ int natten_amd_merge_attentions(const void* o0, const float* lse0, const void* o
   }
 #undef NA_MERGE_LAUNCH
   return check_launch("merge_attentions");
+}
+
+int natten_amd_merge_attention_parts(const void* parts, const float* lse_parts, int num_parts, void* out, float* lse_out,
+                                     int dtype, int64_t rows, int head_dim, void* stream) {
+  g_error[0] = 0;
+  if (!parts || !lse_parts || !out || !lse_out) return fail("merge_attention_parts: null pointer argument");
+  if (rows < 1 || head_dim < 1) return fail("merge_attention_parts: rows and head_dim must be positive");
+  if (num_parts < 1 || num_parts > 64) return fail("merge_attention_parts: num_parts must be 1 .. 64, got %d", num_parts);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const uintptr_t align = reinterpret_cast<uintptr_t>(parts) | reinterpret_cast<uintptr_t>(out);
+  const bool wide = head_dim % 8 == 0 && align % (dtype == NATTEN_AMD_F32 ? 32 : 16) == 0;
+  const int64_t total = rows * (wide ? head_dim / 8 : head_dim);
+  int64_t blocks = (total + 255) / 256;
+  if (blocks > 256 * 64) blocks = 256 * 64;
+  const int64_t part_stride = rows * head_dim;
+#define NA_MERGE_LAUNCH(T, VEC)                                                                                      \
+  hipLaunchKernelGGL((merge_parts_kernel<T, VEC>), dim3(unsigned(blocks)), dim3(256), 0, s, static_cast<const T*>(parts), \
+                     lse_parts, num_parts, part_stride, static_cast<T*>(out), lse_out, rows, head_dim)
+  switch (dtype) {
+    case NATTEN_AMD_F16:
+      if (wide) NA_MERGE_LAUNCH(_Float16, 8); else NA_MERGE_LAUNCH(_Float16, 1);
+      break;
+    case NATTEN_AMD_BF16:
+      if (wide) NA_MERGE_LAUNCH(__bf16, 8); else NA_MERGE_LAUNCH(__bf16, 1);
+      break;
+    case NATTEN_AMD_F32:
+      if (wide) NA_MERGE_LAUNCH(float, 8); else NA_MERGE_LAUNCH(float, 1);
+      break;
+    default:
+      return fail("merge_attention_parts: unsupported dtype code %d", dtype);
+  }
+#undef NA_MERGE_LAUNCH
+  return check_launch("merge_attention_parts");
 }
 
 int natten_amd_mfma_probe(const void* operands, float* sink, uint64_t* clocks, int iters, int fma_per_mfma,

@@ -218,9 +218,7 @@ def amd_fna_generic(
                 query.contiguous(), key.contiguous(), value.contiguous(), kernel_size, stride, dilation, is_causal,
                 scale, q_tile_shape, kv_tile_shape, kv_splits, anchored_tiles=bool(anchored_tiles),
             )
-            output, lse = out_parts[0], lse_parts[0]
-            for i in range(1, kv_splits):
-                output, lse = _lib.merge_two(output, lse, out_parts[i], lse_parts[i])
+            output, lse = _lib.merge_parts(out_parts, lse_parts)
         else:
             output, lse = torch_ops.fna_forward_fused(
                 query.contiguous(), key.contiguous(), value.contiguous(), kernel_size, stride, dilation, is_causal,

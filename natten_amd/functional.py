@@ -216,20 +216,23 @@ def work_queue_default(batch: int, heads: int, token_layout, kernel_size, stride
 
 def kv_splits_default(batch: int, heads: int, token_layout, kernel_size, stride, dilation, is_causal, q_tile_shape,
                       kv_tile_shape) -> int:
-    """How many workgroups share the KV tiles of a Q tile when `kv_splits` is None: 2 when the problem
-    has so few Q tiles that, split, they still leave every workgroup a compute unit of its own (256 of
-    them) and every Q tile has at least eight KV tiles; else 1.  Measured (kernel + merge against the
-    unsplit kernel, microseconds): 64 Q tiles of 34 KV tiles 28 + 6 against 46, a 64 x 64 image with
-    2 heads and a 33 x 33 window 33 + 6 against 58; four ways 22 + 3 x 6 and 24 + 3 x 6 (each further
-    split costs a merge launch); 256 Q tiles of 34 KV tiles two ways 46 + 6 against 53 (no gain: the
-    loop only shortens in proportion while a workgroup does not share its SIMDs)."""
+    """How many workgroups share the KV tiles of a Q tile when `kv_splits` is None: 4 or 2 when the
+    problem has so few Q tiles that, split, they still leave every workgroup a compute unit of its
+    own (256 of them) and every split has at least four KV tiles of every Q tile; else 1.  Measured
+    (split kernel + the 6-7 us merge launch against the unsplit kernel, microseconds): 64 Q tiles of
+    34 KV tiles 28 + 6 two ways and 22 + 7 four ways against 46; a 64 x 64 image with 2 heads and a
+    33 x 33 window 33 + 6 and 24 + 7 against 58; 256 Q tiles of 34 KV tiles two ways 46 + 6 against
+    53 (no gain: the loop only shortens in proportion while a workgroup does not share its SIMDs)."""
     tiles, min_visits = batch * heads, 1
     for X, k, d, c, qt, kt in zip(token_layout, kernel_size, dilation, is_causal, q_tile_shape, kv_tile_shape):
         extent = -(-X // d)
         tiles *= -(-extent // qt) * d
         # fewest KV tiles a Q tile meets along this dimension: a whole window, or one key where causal
         min_visits *= max((1 if c else min(extent, k)) // kt, 1)
-    return 2 if (tiles * 2 <= 256 and min_visits >= 8) else 1
+    for splits in (4, 2):
+        if tiles * splits <= 256 and min_visits >= 4 * splits:
+            return splits
+    return 1
 
 
 def _make_na(na_dim: int, name: str):

@@ -59,9 +59,13 @@ def test_partial_results_of_the_split_entry_point():
     assert int(torch.isinf(first).sum()) == 3 * first.shape[-1] and bool(torch.isfinite(first).any(dim=0).all())
     assert bool((parts[:, 0, 0][torch.isinf(first)] == 0).all())
     assert bool(torch.isfinite(parts.float()).all()) and not bool(torch.isnan(lses).any())
-    out, lse = parts[0], lses[0]
+    out, lse = _lib.merge_parts(parts, lses)
+    # the same by two-way merges (more roundings of the intermediate outputs, same LSE)
+    o2, l2 = parts[0], lses[0]
     for i in range(1, 4):
-        out, lse = _lib.merge_two(out, lse, parts[i], lses[i])
+        o2, l2 = _lib.merge_two(o2, l2, parts[i], lses[i])
+    assert_close("merge_parts vs merge_two, out", to_np(out), to_np(o2), atol=2.0 ** -9, rtol=2.0 ** -9)
+    assert_close("merge_parts vs merge_two, lse", to_np(lse), to_np(l2), atol=1e-5, rtol=1e-5)
     ref_o, ref_l = oracle_full(q, k, v, kernel, (1,), (1,), causal)
     assert_close("out", to_np(out), ref_o)
     assert_close("lse", to_np(lse), ref_l)
@@ -70,18 +74,19 @@ def test_partial_results_of_the_split_entry_point():
 
 
 def test_default_splits_a_small_grid_with_long_windows():
-    # one head, 64 Q tiles of 34 KV tiles each: the public op splits two ways by itself
+    # one head, 64 Q tiles of 34 KV tiles each: the public op splits four ways by itself
     shape, kernel = (8192,), (2048,)
     q, k, v = make_qkv(1, shape, 1, 1, 128, torch.float16, seed=9)
     qt, kt = check_fna_forward_config(q, kernel, (1,), (1,), (False,), None, None)
-    assert kv_splits_default(1, 1, shape, kernel, (1,), (1,), (False,), qt, kt) == 2
+    assert kv_splits_default(1, 1, shape, kernel, (1,), (1,), (False,), qt, kt) == 4
+    assert kv_splits_default(1, 2, shape, kernel, (1,), (1,), (False,), qt, kt) == 2
     # (not with 256 Q tiles, not with short or causal windows)
     assert kv_splits_default(1, 1, (32768,), kernel, (1,), (1,), (False,), qt, kt) == 1
     assert kv_splits_default(1, 1, shape, (256,), (1,), (1,), (False,), qt, kt) == 1
     assert kv_splits_default(1, 1, shape, kernel, (1,), (1,), (True,), qt, kt) == 1
     out, lse = na1d(q, k, v, kernel, return_lse=True)
     sampled_check(q, k, v, out, lse, kernel, (1,), (1,), (False,), n_samples=300, seed=1)
-    same_o, same_l = amd_fna_generic(q, k, v, kernel, 1, 1, False, return_lse=True, kv_splits=2)
+    same_o, same_l = amd_fna_generic(q, k, v, kernel, 1, 1, False, return_lse=True, kv_splits=4)
     assert torch.equal(out, same_o) and torch.equal(lse, same_l)
     # gradients flow through the split forward (the backward takes the merged output and LSE)
     qg, kg, vg = (t.clone().requires_grad_(True) for t in (q[:, :2048], k[:, :2048], v[:, :2048]))
@@ -104,3 +109,35 @@ def test_split_limits():
     qt, kt = check_fna_forward_config(q, (128,), (1,), (1,), (False,), None, None)
     with pytest.raises(RuntimeError, match="kv_splits"):
         _lib.fna_forward_fused_split(q, k, v, (128,), (1,), (1,), (False,), 0.125, qt, kt, 1)
+
+
+@pytest.mark.parametrize("n", [1, 2, 3])
+def test_split_random_sweep(n):
+    # 40 random legal problems per rank (drawn like the reference's sweep), 2 .. 8 splits: the merged
+    # result against the oracle, and against the unsplit launch up to the rounding of the partial outputs
+    import numpy as np
+
+    from tests.test_gpu_fna import _random_problem
+
+    rng = np.random.default_rng(77 + n)
+    for case in range(40):
+        B, H, Hkv, D, shape, k, s, d, causal = _random_problem(rng, n)
+        if all(kk == x for kk, x in zip(k, shape)) and not any(causal):
+            continue  # the dense-attention shortcut of the public ops, not this kernel
+        dtype = [torch.bfloat16, torch.float16][case % 2]
+        splits = int(rng.integers(2, 9))
+        q, kk_, v = make_qkv(B, shape, H, Hkv, D, dtype, seed=case)
+        tag = f"{shape} k={k} s={s} d={d} c={causal} H={H}/{Hkv} D={D} {dtype} splits={splits}"
+        print(tag, flush=True)
+        whole_o, whole_l = amd_fna_generic(q, kk_, v, k, s, d, causal, return_lse=True, kv_splits=1)
+        out, lse = amd_fna_generic(q, kk_, v, k, s, d, causal, return_lse=True, kv_splits=splits)
+        cost = B * H * int(np.prod(shape)) * int(np.prod(k))
+        if cost < 3e7:
+            ref_o, ref_l = oracle_full(q, kk_, v, k, s, d, causal)
+            assert_close("out " + tag, to_np(out), ref_o)
+            assert_close("lse " + tag, to_np(lse), ref_l)
+        else:
+            sampled_check(q, kk_, v, out, lse, k, s, d, causal, 300, seed=case + 500, tag=tag)
+        eps = 2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10
+        assert_close("out vs unsplit " + tag, to_np(out), to_np(whole_o), atol=eps, rtol=eps)
+        assert_close("lse vs unsplit " + tag, to_np(lse), to_np(whole_l), atol=1e-5, rtol=1e-5)
