@@ -9,7 +9,9 @@ src/natten/_libnatten/stubs.py:25-31).
 
 from __future__ import annotations
 
+import contextlib
 import ctypes
+import functools
 import os
 from typing import Optional, Sequence, Tuple
 
@@ -162,8 +164,14 @@ def lib():
     return _lib
 
 
+@functools.lru_cache(maxsize=4096)
+def _i32_array(values: Tuple[int, ...]):
+    return (ctypes.c_int32 * len(values))(*values)
+
+
 def _i32(values: Sequence[int]):
-    return (ctypes.c_int32 * len(values))(*[int(v) for v in values])
+    # (the arrays are only ever read, by the library: equal tuples share one)
+    return _i32_array(tuple(int(v) for v in values))
 
 
 def _check(rc: int):
@@ -171,8 +179,25 @@ def _check(rc: int):
         raise RuntimeError(lib().natten_amd_last_error().decode())
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream(t: Tensor) -> int:
+    """Handle of torch's current stream on the tensor's device (the capturing stream under graph capture)."""
+    if _raw_stream is not None and t.device.index is not None:
+        return _raw_stream(t.device.index)
     return torch.cuda.current_stream(t.device).cuda_stream
+
+
+_NO_GUARD = contextlib.nullcontext()
+
+
+def _on_device(t: Tensor):
+    """Context that makes the tensor's device current for the launch; nothing when it already is."""
+    idx = t.device.index
+    if idx is None or idx == torch.cuda.current_device():
+        return _NO_GUARD
+    return torch.cuda.device(idx)
 
 
 def _require_gpu(*tensors: Tensor):
@@ -198,7 +223,7 @@ def supported_tile_sizes(dtype: torch.dtype, head_dim: int):
 def _scale_ptrs(q: Tensor, k: Tensor, q_scale, k_scale, v_scale):
     """Device pointers (or None) of the per-head scale arrays, after checking shape/dtype/device."""
     ptrs = []
-    for name, s, heads in (("q_scale", q_scale, q.shape[2]), ("k_scale", k_scale, k.shape[2]), ("v_scale", v_scale, k.shape[2])):
+    for name, s, heads in (("q_scale", q_scale, q.shape[-2]), ("k_scale", k_scale, k.shape[-2]), ("v_scale", v_scale, k.shape[-2])):
         if s is None:
             ptrs.append(None)
             continue
@@ -229,7 +254,7 @@ def fna_forward(
     # 8-bit float operands are multiplied by the 8-bit matrix instruction; the result is bf16
     out = torch.empty(q.shape, dtype=torch.bfloat16 if q.dtype in FP8_DTYPES else q.dtype, device=q.device)
     lse = torch.empty(q.shape[:-1], dtype=torch.float32, device=q.device)
-    with torch.cuda.device(q.device):
+    with _on_device(q):
         rc = L.natten_amd_fna_forward(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
             DTYPE_CODES[q.dtype], na_dim, q.shape[0], q.shape[1], k.shape[1], q.shape[2], k.shape[2], q.shape[3],
@@ -311,10 +336,10 @@ def fna_forward_fused(
         raise NotImplementedError(f"natten_amd fna_forward_fused does not support {q.dtype}.")
     na_dim = len(kernel_size)
     qkv_shape = [int(x) for x in q.shape[1 : 1 + na_dim]]
-    scales = _scale_ptrs(q.flatten(1, na_dim), k.flatten(1, na_dim), q_scale, k_scale, v_scale)
+    scales = _scale_ptrs(q, k, q_scale, k_scale, v_scale)
     out = torch.empty(q.shape, dtype=torch.bfloat16 if q.dtype in FP8_DTYPES else q.dtype, device=q.device)
     lse = torch.empty(q.shape[:-1], dtype=torch.float32, device=q.device)
-    with torch.cuda.device(q.device):
+    with _on_device(q):
         rc = L.natten_amd_fna_forward_fused(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
             DTYPE_CODES[q.dtype], na_dim, q.shape[0], q.shape[-2], k.shape[-2], q.shape[-1],
@@ -343,7 +368,7 @@ def fna_forward_fused_split(
     qkv_shape = [int(x) for x in q.shape[1 : 1 + na_dim]]
     out = torch.empty((kv_splits, *q.shape), dtype=q.dtype, device=q.device)
     lse = torch.empty((kv_splits, *q.shape[:-1]), dtype=torch.float32, device=q.device)
-    with torch.cuda.device(q.device):
+    with _on_device(q):
         rc = L.natten_amd_fna_forward_fused_split(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
             DTYPE_CODES[q.dtype], na_dim, q.shape[0], q.shape[-2], k.shape[-2], q.shape[-1],
@@ -373,7 +398,7 @@ def fna_forward_fused_static(
         raise ValueError("lse must be a contiguous float32 tensor of q's shape without the last dimension.")
     na_dim = len(kernel_size)
     qkv_shape = [int(x) for x in q.shape[1 : 1 + na_dim]]
-    with torch.cuda.device(q.device):
+    with _on_device(q):
         rc = L.natten_amd_fna_forward_fused_static(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
             DTYPE_CODES[q.dtype], na_dim, q.shape[0], q.shape[-2], k.shape[-2], q.shape[-1],
@@ -396,7 +421,7 @@ def attention_forward(
     scales = _scale_ptrs(q, k, q_scale, k_scale, v_scale)
     out = torch.empty_like(q)
     lse = torch.empty(q.shape[:-1], dtype=torch.float32, device=q.device)
-    with torch.cuda.device(q.device):
+    with _on_device(q):
         rc = L.natten_amd_attention_forward(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(), DTYPE_CODES[q.dtype],
             q.shape[0], q.shape[1], k.shape[1], q.shape[2], k.shape[2], q.shape[3], 1 if is_causal else 0,
@@ -428,7 +453,7 @@ def attention_forward_varlen(
     scales = _scale_ptrs(q, k, q_scale, k_scale, v_scale)
     out = torch.zeros_like(q)
     lse = torch.zeros(q.shape[:-1], dtype=torch.float32, device=q.device)
-    with torch.cuda.device(q.device):
+    with _on_device(q):
         rc = L.natten_amd_attention_forward_varlen(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(), DTYPE_CODES[q.dtype],
             cumulative_seqlen_q.shape[0] - 1, q.shape[1], k.shape[1], int(max_seqlen_q), int(max_seqlen_kv),
@@ -465,7 +490,7 @@ def compute_delta(out: Tensor, d_out: Tensor) -> Tensor:
     if out.dtype not in (torch.float16, torch.bfloat16) or d_out.dtype != out.dtype or d_out.shape != out.shape:
         raise ValueError("compute_delta needs two fp16 / bf16 tensors of the same shape and dtype.")
     delta = torch.empty(out.shape[:-1], dtype=torch.float32, device=out.device)
-    with torch.cuda.device(out.device):
+    with _on_device(out):
         rc = L.natten_amd_compute_delta(out.data_ptr(), d_out.data_ptr(), delta.data_ptr(), DTYPE_CODES[out.dtype],
                                         delta.numel(), out.shape[-1], _stream(out))
     _check(rc)
@@ -487,7 +512,7 @@ def fna_backward(
         raise ValueError("lse and delta must be float32.")
     na_dim = len(kernel_size)
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
-    with torch.cuda.device(q.device):
+    with _on_device(q):
         rc = L.natten_amd_fna_backward(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), d_out.data_ptr(), lse.data_ptr(), delta.data_ptr(),
             dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), DTYPE_CODES[q.dtype], na_dim, q.shape[0], q.shape[1],
@@ -526,7 +551,7 @@ def fna_backward_fused(
     if lse.dtype != torch.float32 or delta.dtype != torch.float32:
         raise ValueError("lse and delta must be float32.")
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
-    with torch.cuda.device(q.device):
+    with _on_device(q):
         rc = L.natten_amd_fna_backward_fused(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), d_out.data_ptr(), lse.data_ptr(), delta.data_ptr(),
             dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), DTYPE_CODES[q.dtype], na_dim, B, H, k.shape[-2], q.shape[-1],
@@ -549,7 +574,7 @@ def attention_backward(
     if q.dtype not in (torch.float16, torch.bfloat16):
         raise NotImplementedError(f"natten_amd attention_backward does not support {q.dtype}.")
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
-    with torch.cuda.device(q.device):
+    with _on_device(q):
         rc = L.natten_amd_attention_backward(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), d_out.data_ptr(), lse.data_ptr(), delta.data_ptr(),
             dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), DTYPE_CODES[q.dtype], q.shape[0], int(seqlen_q),
@@ -580,7 +605,7 @@ def attention_backward_varlen(
     if cu_q.numel() < 2 or q.shape[0] != 1 or k.shape[0] != 1:
         raise ValueError("sequence-packed operands have batch 1 and at least one sequence.")
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
-    with torch.cuda.device(q.device):
+    with _on_device(q):
         rc = L.natten_amd_attention_backward_varlen(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), d_out.data_ptr(), lse.data_ptr(), delta.data_ptr(),
             dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), DTYPE_CODES[q.dtype], cu_q.numel() - 1, q.shape[1], k.shape[1],
@@ -614,14 +639,14 @@ def token_permute(x: Tensor, tile_shape, dilation, flip_tiled_dims: bool, widen:
     out_dtype = torch.bfloat16 if widen else x.dtype
     out = torch.empty((x.shape[0] * groups, seqlen, x.shape[-2], x.shape[-1]), dtype=out_dtype, device=x.device)
     if widen:
-        with torch.cuda.device(x.device):
+        with _on_device(x):
             rc = L.natten_amd_token_permute_widen(
                 x.data_ptr(), out.data_ptr(), DTYPE_CODES[x.dtype], na_dim, x.shape[0], x.shape[-2], x.shape[-1],
                 _i32(layout), _i32(tile_shape), _i32(dilation), 1 if flip_tiled_dims else 0, _stream(x),
             )
         _check(rc)
         return out
-    with torch.cuda.device(x.device):
+    with _on_device(x):
         rc = L.natten_amd_token_permute(
             x.data_ptr(), out.data_ptr(), x.element_size(), na_dim, x.shape[0], x.shape[-2], x.shape[-1],
             _i32(layout), _i32(tile_shape), _i32(dilation), 1 if flip_tiled_dims else 0, _stream(x),
@@ -647,7 +672,7 @@ def token_unpermute(y: Tensor, token_layout, tile_shape, dilation, flip_tiled_di
         )
     batch = y.shape[0] // groups
     out = torch.empty((batch, *token_layout, y.shape[-2], y.shape[-1]), dtype=y.dtype, device=y.device)
-    with torch.cuda.device(y.device):
+    with _on_device(y):
         rc = L.natten_amd_token_unpermute(
             y.data_ptr(), out.data_ptr(), y.element_size(), na_dim, batch, y.shape[-2], y.shape[-1],
             _i32(token_layout), _i32(tile_shape), _i32(dilation), 1 if flip_tiled_dims else 0, _stream(y),
@@ -665,7 +690,7 @@ def merge_two(o0: Tensor, lse0: Tensor, o1: Tensor, lse1: Tensor) -> Tuple[Tenso
     out = torch.empty_like(o0)
     lse = torch.empty_like(lse0)
     rows = lse0.numel()
-    with torch.cuda.device(o0.device):
+    with _on_device(o0):
         rc = L.natten_amd_merge_attentions(
             o0.data_ptr(), lse0.data_ptr(), o1.data_ptr(), lse1.data_ptr(), out.data_ptr(), lse.data_ptr(),
             DTYPE_CODES[o0.dtype], rows, o0.shape[-1], _stream(o0),
@@ -687,7 +712,7 @@ def merge_parts(out_parts: Tensor, lse_parts: Tensor) -> Tuple[Tensor, Tensor]:
         raise ValueError("out_parts and lse_parts must be contiguous.")
     out = torch.empty(out_parts.shape[1:], dtype=out_parts.dtype, device=out_parts.device)
     lse = torch.empty(lse_parts.shape[1:], dtype=torch.float32, device=out_parts.device)
-    with torch.cuda.device(out_parts.device):
+    with _on_device(out_parts):
         rc = L.natten_amd_merge_attention_parts(
             out_parts.data_ptr(), lse_parts.data_ptr(), out_parts.shape[0], out.data_ptr(), lse.data_ptr(),
             DTYPE_CODES[out_parts.dtype], lse.numel(), out_parts.shape[-1], _stream(out_parts),

@@ -113,6 +113,7 @@ def amd_fna_generic(
     run_persistent_kernel: Optional[bool] = False,
     anchored_tiles: bool = True,
     kv_splits: Optional[int] = None,
+    _checked: bool = False,
 ) -> Union[Tensor, Tuple[Tensor, Tensor]]:
     """`kv_splits` (one-launch path, fp16 / bf16, tiles of 128 x 64 tokens): that many workgroups
     share the KV tiles of every Q tile and their partial results are merged -- for problems with
@@ -138,11 +139,12 @@ def amd_fna_generic(
     the reference.  `fp8_matmul` (None: whenever head dim and tiles allow) multiplies them with
     the 8-bit matrix instruction, P rounded to e4m3 as the reference does; False widens them to
     bf16 (exactly) in the token permute and multiplies in bf16, which is slower and more accurate."""
-    na_tensor_checks(query, key, value, must_match_head_dims=True)
-    can_run_amd_fna(query, key, value, raise_error=True)
     na_dim = query.dim() - 3
-    kernel_size, stride, dilation, is_causal = check_all_args(na_dim, kernel_size, stride, dilation, is_causal)
-    check_args_against_input(query, kernel_size, stride, dilation, is_causal)
+    if not _checked:  # (the public ops have made these checks on the same arguments already)
+        na_tensor_checks(query, key, value, must_match_head_dims=True)
+        kernel_size, stride, dilation, is_causal = check_all_args(na_dim, kernel_size, stride, dilation, is_causal)
+        check_args_against_input(query, kernel_size, stride, dilation, is_causal)
+    can_run_amd_fna(query, key, value, raise_error=True)
     q_tile_shape, kv_tile_shape = check_fna_forward_config(
         query, kernel_size, stride, dilation, is_causal, q_tile_shape, kv_tile_shape
     )

@@ -9,6 +9,7 @@ accepted and ignored, except `q_tile_shape` / `kv_tile_shape`, which select the 
 
 from __future__ import annotations
 
+import functools
 from typing import Dict, Optional, Tuple, Union
 
 import torch
@@ -168,7 +169,7 @@ def neighborhood_attention_generic(
         q_scale=q_scale, k_scale=k_scale, v_scale=v_scale,
         out_dtype=work_dtype if has_additional_attention else final_dtype, fp8_matmul=fp8_matmul,
         backward_q_tile_shape=backward_q_tile_shape, backward_kv_tile_shape=backward_kv_tile_shape,
-        run_persistent_kernel=run_persistent_kernel,
+        run_persistent_kernel=run_persistent_kernel, _checked=True,
     )
 
     if has_additional_attention:
@@ -204,6 +205,12 @@ def _use_work_queue(run_persistent_kernel: Optional[bool], is_causal, num_q_tile
 def work_queue_default(batch: int, heads: int, token_layout, kernel_size, stride, dilation, is_causal, q_tile_shape,
                        kv_tile_shape) -> bool:
     """The launch kind the ops pick when `run_persistent_kernel` is None, from the problem's tile counts."""
+    return _work_queue_default(int(batch), int(heads), *(tuple(x) for x in (
+        token_layout, kernel_size, stride, dilation, is_causal, q_tile_shape, kv_tile_shape)))
+
+
+@functools.lru_cache(maxsize=1024)
+def _work_queue_default(batch, heads, token_layout, kernel_size, stride, dilation, is_causal, q_tile_shape, kv_tile_shape):
     tiles, visits = batch * heads, 1
     for X, k, s, d, qt, kt in zip(token_layout, kernel_size, stride, dilation, q_tile_shape, kv_tile_shape):
         extent = -(-X // d)
@@ -223,6 +230,12 @@ def kv_splits_default(batch: int, heads: int, token_layout, kernel_size, stride,
     34 KV tiles 28 + 6 two ways and 22 + 7 four ways against 46; a 64 x 64 image with 2 heads and a
     33 x 33 window 33 + 6 and 24 + 7 against 58; 256 Q tiles of 34 KV tiles two ways 46 + 6 against
     53 (no gain: the loop only shortens in proportion while a workgroup does not share its SIMDs)."""
+    return _kv_splits_default(int(batch), int(heads), *(tuple(x) for x in (
+        token_layout, kernel_size, dilation, is_causal, q_tile_shape, kv_tile_shape)))
+
+
+@functools.lru_cache(maxsize=1024)
+def _kv_splits_default(batch, heads, token_layout, kernel_size, dilation, is_causal, q_tile_shape, kv_tile_shape):
     tiles, min_visits = batch * heads, 1
     for X, k, d, c, qt, kt in zip(token_layout, kernel_size, dilation, is_causal, q_tile_shape, kv_tile_shape):
         extent = -(-X // d)
