@@ -37,6 +37,38 @@ def test_forward_replays_from_a_graph(shape, kernel, causal):
             assert torch.equal(out, ref_out) and torch.equal(lse, ref_lse), f"replay {i} differs from the eager call"
 
 
+def test_split_forward_replays_from_a_graph():
+    # a small grid with long windows: the op splits the KV tiles of every Q tile over several
+    # workgroups and merges the partial results -- two launches and two allocations inside the capture
+    from natten_amd.functional import kv_splits_default
+    from natten_amd.tile_config import check_fna_forward_config
+
+    shape, kernel = (2048,), (1024,)
+    gen = torch.Generator().manual_seed(3)
+    mk = lambda: torch.randn((1, *shape, 2, 128), generator=gen).to(torch.float16).cuda()
+    q, k, v = mk(), mk(), mk()
+    qt, kt = check_fna_forward_config(q, kernel, (1,), (1,), (False,), None, None)
+    assert kv_splits_default(1, 2, shape, kernel, (1,), (1,), (False,), qt, kt) > 1
+    fn = lambda: natten_amd.na1d(q, k, v, kernel, return_lse=True)
+    side = torch.cuda.Stream()
+    with torch.no_grad():
+        with torch.cuda.stream(side):
+            for _ in range(2):
+                fn()
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            out, lse = fn()
+        for i in range(3):
+            for t in (q, k, v):
+                t.copy_(mk())
+            graph.replay()
+            torch.cuda.synchronize()
+            ref_out, ref_lse = fn()
+            torch.cuda.synchronize()
+            assert torch.equal(out, ref_out) and torch.equal(lse, ref_lse), f"replay {i} differs from the eager call"
+
+
 @pytest.mark.parametrize("shape,kernel,causal,head_dim", [
     ((16, 16), (5, 5), (False, True), 64),     # backward on the original tensors, dQ + combined dK/dV role
     ((16, 32), (7, 9), (True, False), 128),    # the same with the paired dK/dV role
