@@ -302,6 +302,7 @@ def bench_backward(args, q, k, v, kernel, stride, dilation, causal, dt_name):
     na = {1: natten_amd.na1d, 2: natten_amd.na2d, 3: natten_amd.na3d}[n]
     q_tile = tuple(int(x) for x in args.q_tile.split(",")) if args.q_tile else None
     kv_tile = tuple(int(x) for x in args.kv_tile.split(",")) if args.kv_tile else None
+    tiles_given = q_tile is not None
     q_tile, kv_tile = check_fna_backward_config(q, kernel, stride, dilation, causal, q_tile, kv_tile)
     gen = torch.Generator().manual_seed(1)
     d_out = torch.randn(q.shape, generator=gen).to(q.dtype).to(q.device)
@@ -309,8 +310,8 @@ def bench_backward(args, q, k, v, kernel, stride, dilation, causal, dt_name):
 
     def step():
         q.grad = k.grad = v.grad = None
-        out = na(q, k, v, kernel, stride, dilation, causal, backward_q_tile_shape=q_tile,
-                 backward_kv_tile_shape=kv_tile)
+        out = na(q, k, v, kernel, stride, dilation, causal, backward_q_tile_shape=q_tile if tiles_given else None,
+                 backward_kv_tile_shape=kv_tile if tiles_given else None)
         out.backward(d_out)
 
     for _ in range(args.warmup):
@@ -338,6 +339,18 @@ def bench_backward(args, q, k, v, kernel, stride, dilation, causal, dt_name):
 
         fused = _lib.backward_fused_layout_supported(layout, dilation, q_tile, kv_tile)
         qd, kd, vd = q.detach(), k.detach(), v.detach()
+        # left to itself the op gives each launch on the original tensors the tile shapes that suit its role
+        kv_role = (None, None)
+        if fused and not tiles_given:
+            from natten_amd.tile_config import choose_backward_role_tile_shapes
+
+            roles = choose_backward_role_tile_shapes(layout, tuple(kernel), tuple(stride), tuple(dilation), tuple(causal))
+            if roles is not None and all(_lib.backward_fused_layout_supported(layout, dilation, a, b) for a, b in roles):
+                (q_tile_dq, kv_tile_dq), kv_role = roles
+            else:
+                q_tile_dq, kv_tile_dq = q_tile, kv_tile
+        else:
+            q_tile_dq, kv_tile_dq = q_tile, kv_tile
 
         def kern_permuted():
             return _lib.fna_backward(qp, kp, vp, dop, lp, dp, kernel, stride, dilation, causal, D**-0.5, q_shape,
@@ -347,7 +360,7 @@ def bench_backward(args, q, k, v, kernel, stride, dilation, causal, dt_name):
             # the launches the step above makes
             if fused:
                 return _lib.fna_backward_fused(qd, kd, vd, d_out, lse, delta, kernel, stride, dilation, causal,
-                                               D**-0.5, q_tile, kv_tile)
+                                               D**-0.5, q_tile_dq, kv_tile_dq, *kv_role)
             return kern_permuted()
 
         def timed(fn):
@@ -363,10 +376,11 @@ def bench_backward(args, q, k, v, kernel, stride, dilation, causal, dt_name):
             torch.cuda.synchronize()
             return e0.elapsed_time(e1) / args.steps
 
-        kernel_ms = timed(kern)
-        kernel_permuted_ms = timed(kern_permuted)
+        # (--step-only: the step's launches alone, for profiles; the rate then counts the whole step's time)
+        kernel_ms = None if args.step_only else timed(kern)
+        kernel_permuted_ms = None if args.step_only else timed(kern_permuted)
     fwd_flops = 4.0 * B * H * D * count_attended(layout, kernel, stride, dilation, causal)
-    achieved = 2.5 * fwd_flops / (kernel_ms * 1e-3) / 1e12
+    achieved = 2.5 * fwd_flops / ((kernel_ms if kernel_ms is not None else ms_per_step) * 1e-3) / 1e12
     peak = PEAK_TFLOPS[dt_name]
     print(json.dumps({
         "metric": "FNA fwd+bwd ms per step and effective TFLOP/s of the backward kernels, 1 GPU",
@@ -383,8 +397,10 @@ def bench_backward(args, q, k, v, kernel, stride, dilation, causal, dt_name):
         "data": "synthetic",
         "config": {
             "workload": WORKLOAD_NAMES[args.workload] + ", forward + backward",
-            "backward_q_tile_shape": list(q_tile),
-            "backward_kv_tile_shape": list(kv_tile),
+            "backward_q_tile_shape": list(q_tile_dq),
+            "backward_kv_tile_shape": list(kv_tile_dq),
+            "dk_dv_launch_tile_shapes": [list(t) for t in kv_role] if kv_role[0] is not None else None,
+            "permuted_route_tile_shapes": [list(q_tile), list(kv_tile)],
             "path": ("forward (one launch) + delta + dQ kernel + dK/dV kernel on the original tensors" if fused else
                      "forward + delta + token permutes + dQ and dK/dV kernels + unpermutes"),
         },
@@ -398,7 +414,7 @@ def bench_backward(args, q, k, v, kernel, stride, dilation, causal, dt_name):
             "peak": peak,
             "unit": "TFLOP/s",
             "frac": achieved / peak,
-            "traffic": (measured_traffic(args.workload, "backward", q_tile, kv_tile) or {}).get("bytes"),
+            "traffic": (measured_traffic(args.workload, "backward", q_tile_dq, kv_tile_dq) or {}).get("bytes"),
             "kernel_digest": kernel_digest("backward"),
             "algorithmic_flop": 2.5 * fwd_flops,
         },

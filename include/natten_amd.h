@@ -289,6 +289,12 @@ int natten_amd_fna_backward(const void* q, const void* k, const void* v, const v
  * backward driver (src/natten/backends/blackwell_fna.py:205-297); results are bit-identical to
  * them.  Every extent must be a multiple of dilation x tile for both tile shapes (an error
  * otherwise: use natten_amd_fna_backward on permuted operands).
+ *
+ * roles: 3 makes both launches; 1 only the one that writes dq, 2 only the one that writes dk and
+ * dv (the other results are left untouched).  With no permuted layout to share, the two launches
+ * need not use the same tile shapes: the dq launch streams half KV tiles past a Q tile, the
+ * dk / dv launch half Q tiles past a KV tile, and the shapes that visit the fewest tiles differ
+ * (a caller makes one call per role, each with that role's shapes).
  */
 int natten_amd_fna_backward_fused(const void* q, const void* k, const void* v, const void* d_out,
                                   const float* lse, const float* delta, void* dq, void* dk,
@@ -297,7 +303,7 @@ int natten_amd_fna_backward_fused(const void* q, const void* k, const void* v, c
                                   const int32_t* kernel_size, const int32_t* stride,
                                   const int32_t* dilation, const int32_t* is_causal,
                                   const int32_t* q_tile_shape, const int32_t* kv_tile_shape,
-                                  float scale, void* stream);
+                                  float scale, int roles, void* stream);
 
 /*
  * Dense attention backward (optional top-left causal mask).  Operands as above (lse and delta

@@ -21,7 +21,7 @@ from torch import Tensor
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libnatten_amd.so")
 
-ABI_VERSION = 12
+ABI_VERSION = 13
 
 DTYPE_CODES = {
     torch.float16: 0,
@@ -87,7 +87,8 @@ _SIGNATURES = {
     ),
     "natten_amd_fna_backward_fused": (
         ctypes.c_int,
-        [ctypes.c_void_p] * 9 + [ctypes.c_int] * 6 + [ctypes.c_void_p] * 7 + [ctypes.c_float, ctypes.c_void_p],
+        [ctypes.c_void_p] * 9 + [ctypes.c_int] * 6 + [ctypes.c_void_p] * 7
+        + [ctypes.c_float, ctypes.c_int, ctypes.c_void_p],
     ),
     "natten_amd_attention_backward": (
         ctypes.c_int,
@@ -537,9 +538,11 @@ def backward_fused_layout_supported(token_layout, dilation, q_tile_shape, kv_til
 
 def fna_backward_fused(
     q: Tensor, k: Tensor, v: Tensor, d_out: Tensor, lse: Tensor, delta: Tensor, kernel_size, stride, dilation,
-    is_causal, scale: float, q_tile_shape, kv_tile_shape,
+    is_causal, scale: float, q_tile_shape, kv_tile_shape, kv_role_q_tile_shape=None, kv_role_kv_tile_shape=None,
 ) -> Tuple[Tensor, Tensor, Tensor]:
-    """Backward on the original tensors [B, *X, H, D] (lse, delta [B, *X, H]) -> (dq, dk, dv)."""
+    """Backward on the original tensors [B, *X, H, D] (lse, delta [B, *X, H]) -> (dq, dk, dv).
+    kv_role_*_tile_shape: tile shapes of the launch that forms dk and dv, when they differ from those
+    of the dq launch (q_tile_shape, kv_tile_shape)."""
     L = lib()
     na_dim = len(kernel_size)
     B, H = q.shape[0], q.shape[-2]
@@ -550,15 +553,22 @@ def fna_backward_fused(
         raise NotImplementedError(f"natten_amd fna_backward_fused does not support {q.dtype}.")
     if lse.dtype != torch.float32 or delta.dtype != torch.float32:
         raise ValueError("lse and delta must be float32.")
+    if (kv_role_q_tile_shape is None) != (kv_role_kv_tile_shape is None):
+        raise ValueError("kv_role_q_tile_shape and kv_role_kv_tile_shape must be given together.")
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    same = kv_role_q_tile_shape is None or (
+        tuple(kv_role_q_tile_shape) == tuple(q_tile_shape) and tuple(kv_role_kv_tile_shape) == tuple(kv_tile_shape))
+    launches = [(3, q_tile_shape, kv_tile_shape)] if same else [
+        (1, q_tile_shape, kv_tile_shape), (2, kv_role_q_tile_shape, kv_role_kv_tile_shape)]
     with _on_device(q):
-        rc = L.natten_amd_fna_backward_fused(
-            q.data_ptr(), k.data_ptr(), v.data_ptr(), d_out.data_ptr(), lse.data_ptr(), delta.data_ptr(),
-            dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), DTYPE_CODES[q.dtype], na_dim, B, H, k.shape[-2], q.shape[-1],
-            _i32(q.shape[1 : 1 + na_dim]), _i32(kernel_size), _i32(stride), _i32(dilation),
-            _i32([1 if c else 0 for c in is_causal]), _i32(q_tile_shape), _i32(kv_tile_shape), float(scale), _stream(q),
-        )
-    _check(rc)
+        for roles, qt, kt in launches:
+            rc = L.natten_amd_fna_backward_fused(
+                q.data_ptr(), k.data_ptr(), v.data_ptr(), d_out.data_ptr(), lse.data_ptr(), delta.data_ptr(),
+                dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), DTYPE_CODES[q.dtype], na_dim, B, H, k.shape[-2],
+                q.shape[-1], _i32(q.shape[1 : 1 + na_dim]), _i32(kernel_size), _i32(stride), _i32(dilation),
+                _i32([1 if c else 0 for c in is_causal]), _i32(qt), _i32(kt), float(scale), roles, _stream(q),
+            )
+            _check(rc)
     return dq, dk, dv
 
 

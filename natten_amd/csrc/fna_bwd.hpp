@@ -74,6 +74,8 @@ struct FnaBwdParams {
   // the (batch, head, tile) space.  > 0: runs of this many consecutive tiles are dealt round-robin
   // to the XCDs (the grid is then a whole number of rounds of 8 runs).
   int kv_wg_run;
+  // Host side only: which launches a call makes (bit 0: the dQ role, bit 1: the dK / dV role; 0 = both).
+  int roles;
 };
 
 enum BwdRole : int { kBwdDQ = 0, kBwdDKV = 1, kBwdPair = 2 };

@@ -272,7 +272,7 @@ int queue_workspace(const char* what, int run_persistent, void* workspace, uint6
 
 extern "C" {
 
-int natten_amd_abi_version(void) { return 12; }
+int natten_amd_abi_version(void) { return 13; }
 
 uint64_t natten_amd_fna_forward_workspace_bytes(void) { return uint64_t(kQueueWords) * 4; }
 
@@ -681,8 +681,12 @@ static int launch_bwd(const FnaBwdParams& params, hipStream_t stream) {
     wg_kv = (runs + kNumXcd - 1) / kNumXcd * kNumXcd * run;
   }
   if (wg_q > 0x7fffffffLL || wg_kv > 0x7fffffffLL) return fail("fna_backward: problem needs more than 2^31 workgroups");
-  hipLaunchKernelGGL((fna_bwd_kernel<T, D, kBwdDQ, VARLEN>), dim3((unsigned)wg_q), dim3(256), 0, stream, p);
-  if (int rc = check_launch("fna_backward (dQ)")) return rc;
+  const int roles = p.roles ? p.roles : 3;
+  if (roles & 1) {
+    hipLaunchKernelGGL((fna_bwd_kernel<T, D, kBwdDQ, VARLEN>), dim3((unsigned)wg_q), dim3(256), 0, stream, p);
+    if (int rc = check_launch("fna_backward (dQ)")) return rc;
+  }
+  if (!(roles & 2)) return 0;
   if constexpr (D == 128) {
     // dK and dV by wave pairs (eight waves per workgroup): one wave's registers cannot hold the
     // accumulators, fragments and products of both
@@ -800,11 +804,12 @@ int natten_amd_fna_backward_fused(const void* q, const void* k, const void* v, c
                                   int heads_q, int heads_kv, int head_dim, const int32_t* qkv_shape,
                                   const int32_t* kernel_size, const int32_t* stride, const int32_t* dilation,
                                   const int32_t* is_causal, const int32_t* q_tile_shape, const int32_t* kv_tile_shape,
-                                  float scale, void* stream) {
+                                  float scale, int roles, void* stream) {
   g_error[0] = 0;
   const char* what = "fna_backward_fused";
   if (int rc = check_bwd_pointers(what, q, k, v, d_out, lse, delta, dq, dk, dv)) return rc;
   if (na_dim < 1 || na_dim > 3) return fail("%s: na_dim must be 1, 2 or 3, got %d", what, na_dim);
+  if (roles < 1 || roles > 3) return fail("%s: roles must be 1 (dq), 2 (dk and dv) or 3 (all), got %d", what, roles);
   if (!qkv_shape || !kernel_size || !stride || !dilation || !is_causal || !q_tile_shape || !kv_tile_shape)
     return fail("%s: null shape argument", what);
   // per-group layouts: without padding, which needs every extent to be a multiple of dilation x tile
@@ -875,6 +880,7 @@ int natten_amd_fna_backward_fused(const void* q, const void* k, const void* v, c
   p.scale = scale;
   p.fused = 1;
   p.tokens = int(tokens);
+  p.roles = roles;
   return dispatch_bwd(p, dtype, head_dim, static_cast<hipStream_t>(stream));
 }
 

@@ -164,6 +164,7 @@ def amd_fna_generic(
         output, lse = AmdFnaFunction.apply(
             query, key, value, kernel_size, stride, dilation, is_causal, scale, q_tile_shape, kv_tile_shape,
             bwd_q_tile, bwd_kv_tile, fused, bool(run_persistent_kernel), bool(anchored_tiles),
+            backward_q_tile_shape is not None,
         )
         if out_dtype is not None and output.dtype != out_dtype:
             output = output.to(out_dtype)
@@ -278,7 +279,8 @@ class AmdFnaFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, query, key, value, kernel_size, stride, dilation, is_causal, scale, q_tile_shape, kv_tile_shape,
-                bwd_q_tile_shape, bwd_kv_tile_shape, fused, run_persistent_kernel=False, anchored_tiles=True):
+                bwd_q_tile_shape, bwd_kv_tile_shape, fused, run_persistent_kernel=False, anchored_tiles=True,
+                bwd_tiles_given=True):
         with torch.no_grad():
             output, lse = amd_fna_generic(
                 query, key, value, kernel_size, stride, dilation, is_causal, scale, q_tile_shape, kv_tile_shape,
@@ -288,6 +290,9 @@ class AmdFnaFunction(torch.autograd.Function):
         ctx.save_for_backward(query, key, value, output, lse)
         ctx.na_args = (kernel_size, stride, dilation, is_causal, scale, bwd_q_tile_shape, bwd_kv_tile_shape)
         ctx.fused = fused
+        # the backward may pick tile shapes per launch when the caller fixed none and asked for no
+        # other route's bits (anchored_tiles=False promises those of the permuted route)
+        ctx.role_tiles = bool(anchored_tiles) and not bwd_tiles_given
         ctx.mark_non_differentiable(lse)
         return output, lse
 
@@ -306,14 +311,28 @@ class AmdFnaFunction(torch.autograd.Function):
         fusable = _lib.backward_fused_layout_supported(query.shape[1 : 1 + na_dim], dilation, q_tile, kv_tile,
                                                        row_bytes=query.shape[-2] * query.shape[-1] * 2)
         if fusable and ctx.fused is not False:
-            # the kernels gather and scatter their tiles themselves: no permuted copies
+            # the kernels gather and scatter their tiles themselves: no permuted copies; each launch
+            # with the tile shapes that visit the fewest tiles for its role
+            kv_role = (None, None)
+            if ctx.role_tiles:
+                from .tile_config import choose_backward_role_tile_shapes
+
+                roles = choose_backward_role_tile_shapes(
+                    tuple(int(x) for x in query.shape[1 : 1 + na_dim]), tuple(kernel_size), tuple(stride),
+                    tuple(dilation), tuple(is_causal))
+                row_bytes = query.shape[-2] * query.shape[-1] * 2
+                if roles is not None and all(
+                    _lib.backward_fused_layout_supported(query.shape[1 : 1 + na_dim], dilation, qt, kt, row_bytes=row_bytes)
+                    for qt, kt in roles
+                ):
+                    (q_tile, kv_tile), kv_role = roles
             dq, dk, dv = torch_ops.fna_backward_fused(
                 query, key, value, d_output, lse.contiguous(), delta, kernel_size, stride, dilation, is_causal, scale,
-                q_tile, kv_tile,
+                q_tile, kv_tile, *kv_role,
             )
             if d_pad != head_dim:
                 dq, dk, dv = (t[..., :head_dim].contiguous() for t in (dq, dk, dv))
-            return (dq, dk, dv) + (None,) * 12
+            return (dq, dk, dv) + (None,) * 13
 
         def perm(x, tile):
             return token_permute_operation(x.contiguous(), tile, dilation, flip_tiled_dims=True)
@@ -333,4 +352,4 @@ class AmdFnaFunction(torch.autograd.Function):
         dv = token_unpermute_operation(dv_perm, qkv_shape, kv_tile, dilation, flip_tiled_dims=True)
         if d_pad != head_dim:
             dq, dk, dv = (t[..., :head_dim].contiguous() for t in (dq, dk, dv))
-        return (dq, dk, dv) + (None,) * 12
+        return (dq, dk, dv) + (None,) * 13

@@ -164,6 +164,50 @@ def check_fna_backward_config(
     return q_tile_shape, kv_tile_shape
 
 
+def _half_tile(tile: DimensionType) -> DimensionType:
+    """The half tile the other role streams: the last extent above 1, halved."""
+    t = list(tile)
+    t[max(i for i, x in enumerate(t) if x > 1)] //= 2
+    return tuple(t)
+
+
+@functools.lru_cache(maxsize=1024)
+def choose_backward_role_tile_shapes(
+    token_layout: DimensionType, kernel_size: DimensionType, stride: DimensionType, dilation: DimensionType,
+    is_causal: Tuple[bool, ...],
+) -> Optional[Tuple[Tuple[DimensionType, DimensionType], Tuple[DimensionType, DimensionType]]]:
+    """Tile shapes per launch of the backward on the original tensors, where no permuted layout ties
+    the two launches together: ((q_tile, kv_tile) of the dq launch, (q_tile, kv_tile) of the dk / dv
+    launch).  The dq launch streams half KV tiles past every Q tile, the dk / dv launch half Q tiles
+    past every KV tile; each gets the shapes that visit the fewest (query, key) pairs, counted like
+    choose_tile_shapes does (partially masked pairs weigh more).  Only shapes that divide every
+    extent (times the dilation) qualify; None when there are none."""
+    n = len(token_layout)
+    shapes = [t for t in _factorisations(BACKWARD_TILE_SIZE, n)
+              if all(x % (d * e) == 0 for x, d, e in zip(token_layout, dilation, t))]
+    if not shapes:
+        return None
+    ext = tuple(x // d for x, d in zip(token_layout, dilation))
+
+    def cost(q_ext: DimensionType, kv_ext: DimensionType) -> float:
+        visited = full = 1
+        for a in range(n):
+            v, f = _dim_cost(ext[a], kernel_size[a], stride[a], is_causal[a], q_ext[a], kv_ext[a])
+            visited *= v
+            full *= f
+        return visited + 0.3 * (visited - full)
+
+    best = []
+    for role in (0, 1):
+        keyed = []
+        for qt in shapes:
+            for kt in shapes:
+                c = cost(qt, _half_tile(kt)) if role == 0 else cost(_half_tile(qt), kt)
+                keyed.append(((c, tuple(-x for x in reversed(qt)), tuple(-x for x in reversed(kt))), (qt, kt)))
+        best.append(min(keyed)[1])
+    return best[0], best[1]
+
+
 def get_all_backward_tile_shapes(na_dim: int) -> List[Tuple[DimensionType, DimensionType]]:
     """Every legal (backward_q_tile_shape, backward_kv_tile_shape) of power-of-two extents."""
     shapes = _factorisations(BACKWARD_TILE_SIZE, na_dim)

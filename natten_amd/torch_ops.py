@@ -119,14 +119,16 @@ def _(q, k, v, d_out, lse, delta, kernel_size, stride, dilation, is_causal, scal
 def _fna_backward_fused_op(
     q: Tensor, k: Tensor, v: Tensor, d_out: Tensor, lse: Tensor, delta: Tensor, kernel_size: List[int],
     stride: List[int], dilation: List[int], is_causal: List[bool], scale: float, q_tile_shape: List[int],
-    kv_tile_shape: List[int],
+    kv_tile_shape: List[int], kv_role_q_tile_shape: Optional[List[int]] = None,
+    kv_role_kv_tile_shape: Optional[List[int]] = None,
 ) -> Tuple[Tensor, Tensor, Tensor]:
     return _lib.fna_backward_fused(q, k, v, d_out, lse, delta, kernel_size, stride, dilation, is_causal, scale,
-                                   q_tile_shape, kv_tile_shape)
+                                   q_tile_shape, kv_tile_shape, kv_role_q_tile_shape, kv_role_kv_tile_shape)
 
 
 @_fna_backward_fused_op.register_fake
-def _(q, k, v, d_out, lse, delta, kernel_size, stride, dilation, is_causal, scale, q_tile_shape, kv_tile_shape):
+def _(q, k, v, d_out, lse, delta, kernel_size, stride, dilation, is_causal, scale, q_tile_shape, kv_tile_shape,
+      kv_role_q_tile_shape=None, kv_role_kv_tile_shape=None):
     return torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
 
 
@@ -269,13 +271,15 @@ def fna_backward(q, k, v, d_out, lse, delta, kernel_size, stride, dilation, is_c
 
 
 def fna_backward_fused(q, k, v, d_out, lse, delta, kernel_size, stride, dilation, is_causal, scale, q_tile_shape,
-                       kv_tile_shape):
+                       kv_tile_shape, kv_role_q_tile_shape=None, kv_role_kv_tile_shape=None):
     if _tracing():
         return _fna_backward_fused_op(q, k, v, d_out, lse, delta, _ints(kernel_size), _ints(stride), _ints(dilation),
                                       [bool(c) for c in is_causal], float(scale), _ints(q_tile_shape),
-                                      _ints(kv_tile_shape))
+                                      _ints(kv_tile_shape),
+                                      None if kv_role_q_tile_shape is None else _ints(kv_role_q_tile_shape),
+                                      None if kv_role_kv_tile_shape is None else _ints(kv_role_kv_tile_shape))
     return _lib.fna_backward_fused(q, k, v, d_out, lse, delta, kernel_size, stride, dilation, is_causal, scale,
-                                   q_tile_shape, kv_tile_shape)
+                                   q_tile_shape, kv_tile_shape, kv_role_q_tile_shape, kv_role_kv_tile_shape)
 
 
 def attention_backward(q, k, v, d_out, lse, delta, seqlen_q, seqlen_kv, is_causal, scale):

@@ -168,3 +168,27 @@ def test_every_bench_workload_is_named_and_its_cpu_leg_is_bounded():
             # the proxy keeps the window legal: kernel * dilation fits its layout
             assert all(kk * dd <= x for kk, dd, x in zip(k, d, timed)), w
     assert set(bench.REFERENCE_B200_MS) <= set(bench.WORKLOADS)
+
+
+def test_backward_tile_shapes_per_launch():
+    # on the original tensors each backward launch gets the shapes that visit the fewest tiles for its
+    # role: the dq launch streams half KV tiles, the dk / dv launch half Q tiles
+    from natten_amd.tile_config import _half_tile, choose_backward_role_tile_shapes
+
+    assert _half_tile((2, 8, 8)) == (2, 8, 4) and _half_tile((1, 8, 16)) == (1, 8, 8) and _half_tile((128, 1)) == (64, 1)
+    # c4: a causal dimension 0 with one-frame half tiles on the streamed side
+    dq, kv = choose_backward_role_tile_shapes((30, 48, 80), (18, 24, 24), (1, 8, 8), (1, 1, 1), (True, False, False))
+    assert dq == ((2, 8, 8), (1, 8, 16)) and kv == ((1, 8, 16), (2, 8, 8))
+    # shapes must divide every extent (times the dilation): none does here
+    assert choose_backward_role_tile_shapes((29, 46, 78), (9, 24, 24), (1, 8, 8), (2, 1, 1), (False,) * 3) is None
+    # 1-D: one factorisation, the same for both launches
+    assert choose_backward_role_tile_shapes((4096,), (512,), (1,), (1,), (True,)) == (((128,), (128,)),) * 2
+    # whatever is chosen holds 128 tokens and divides the extents
+    for layout, k, s, d, c in [((64, 64), (13, 13), (1, 1), (2, 2), (False, False)),
+                               ((256, 256), (80, 80), (16, 16), (1, 1), (False, True))]:
+        for qt, kt in choose_backward_role_tile_shapes(layout, k, s, d, c):
+            for t in (qt, kt):
+                p = 1
+                for x in t:
+                    p *= x
+                assert p == 128 and all(X % (dd * x) == 0 for X, dd, x in zip(layout, d, t))

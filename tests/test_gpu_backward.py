@@ -315,3 +315,29 @@ def test_large_reference_problems_backward_sampled(na_dim, idx, case):
         sampled_backward_check(q.detach(), kk.detach(), v.detach(), d_out, out.detach(), lse.detach(), q.grad, kk.grad,
                                v.grad, k, s, d, causal, n_samples=48, seed=idx, atol=TOL[dtype], rtol=TOL[dtype],
                                tag=tag)
+
+
+def test_backward_tile_shapes_per_launch_match_oracle_and_common_tiles():
+    # on the original tensors the dq launch and the dk / dv launch take tile shapes of their own by
+    # default; the gradients meet the oracle like those of any other tile shapes, and each launch
+    # alone (C ABI `roles`) writes only its own results
+    from natten_amd import _lib
+    from natten_amd.tile_config import choose_backward_role_tile_shapes
+
+    B, H, Hkv, D, shape, k, s, d, causal = 1, 4, 2, 128, (12, 16, 32), (7, 8, 8), (1, 8, 8), (1, 1, 1), (True, False, False)
+    roles = choose_backward_role_tile_shapes(shape, k, s, d, causal)
+    assert roles is not None and roles[0] != roles[1]
+    run_backward(B, H, Hkv, D, shape, k, s, d, causal, torch.bfloat16, seed=21)   # default: per-launch shapes
+    run_backward(B, H, Hkv, D, shape, k, s, d, causal, torch.float16, bq=roles[0][0], bkv=roles[0][1], seed=22)
+    # the two launches one at a time
+    q, kk, v = make_qkv(B, shape, H, Hkv, D, torch.bfloat16, seed=23)
+    gen = torch.Generator().manual_seed(24)
+    d_out = torch.randn(q.shape, generator=gen).to(torch.bfloat16).cuda()
+    with torch.no_grad():
+        out, lse = NA[3](q, kk, v, k, s, d, causal, return_lse=True)
+        delta = _lib.compute_delta(out, d_out)
+        both = _lib.fna_backward_fused(q, kk, v, d_out, lse, delta, k, s, d, causal, D ** -0.5, *roles[0], *roles[1])
+        only_dq = _lib.fna_backward_fused(q, kk, v, d_out, lse, delta, k, s, d, causal, D ** -0.5, *roles[0])
+        only_kv = _lib.fna_backward_fused(q, kk, v, d_out, lse, delta, k, s, d, causal, D ** -0.5, *roles[1])
+    assert torch.equal(both[0], only_dq[0])                                   # dq: the dq launch's shapes
+    assert torch.equal(both[1], only_kv[1]) and torch.equal(both[2], only_kv[2])  # dk, dv: the other launch's

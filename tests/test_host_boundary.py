@@ -164,9 +164,16 @@ def test_backward_entry_point_rejects_tiles_beyond_32_bit_offsets():
     rc = L.natten_amd_fna_backward_fused(
         ptr, ptr, ptr, ptr, ptr, ptr, ptr, ptr, ptr, _lib.DTYPE_CODES[__import__("torch").bfloat16], 3, 1, 24, 24, 128,
         i32((128, 512, 512)), i32((3, 3, 3)), i32((1, 1, 1)), i32((1, 1, 1)), i32((0, 0, 0)), i32((128, 1, 1)),
-        i32((2, 8, 8)), C.c_float(0.1), None,
+        i32((2, 8, 8)), C.c_float(0.1), 3, None,
     )
     assert rc != 0 and b"2^31 bytes" in L.natten_amd_last_error()
+    # `roles` names the launches to make: 1 (dq), 2 (dk and dv) or 3
+    rc = L.natten_amd_fna_backward_fused(
+        ptr, ptr, ptr, ptr, ptr, ptr, ptr, ptr, ptr, _lib.DTYPE_CODES[__import__("torch").bfloat16], 3, 1, 24, 24, 128,
+        i32((16, 16, 16)), i32((3, 3, 3)), i32((1, 1, 1)), i32((1, 1, 1)), i32((0, 0, 0)), i32((2, 8, 8)),
+        i32((2, 8, 8)), C.c_float(0.1), 0, None,
+    )
+    assert rc != 0 and b"roles" in L.natten_amd_last_error()
 
 
 def test_every_entry_point_rejects_null_arguments_before_touching_a_device():
