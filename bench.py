@@ -438,6 +438,8 @@ def main():
                     help="skip the side measurements (kernel through the C ABI alone, token-permuted route): "
                          "a profile of such a run holds the step's launches only")
     ap.add_argument("--no-mfma-probe", action="store_true")
+    ap.add_argument("--no-dense", action="store_true",
+                    help="skip the dense self-attention run of the same tensors (measured speed-up against the FLOP ratio)")
     args = ap.parse_args()
     # a step of the small workloads lasts 30-200 us: twenty of them end before the device's clocks have
     # settled (c3 reads 0.19-0.21 ms over 20 steps and 0.162 ms sustained), so they get longer loops
@@ -598,6 +600,10 @@ def main():
             }
     achieved = flops / (kernel_ms * 1e-3) / 1e12
     peak = PEAK_TFLOPS[dt_name]
+    from natten_amd.tile_config import visited_pairs
+
+    attended = B * H * count_attended(layout, kernel, stride, dilation, causal)
+    visited = B * H * visited_pairs(layout, kernel, stride, dilation, causal, q_tile, kv_tile, anchored=bool(fused))
     dense_flops = 4.0 * B * H * D * float(q.numel() // (B * H * D)) ** 2
 
     # bytes of Q, K, V read and O, LSE written once
@@ -628,6 +634,11 @@ def main():
         },
         "na_flop_per_step": flops,
         "dense_over_na_flop": dense_flops / flops,
+        # (query, key) pairs the kernel multiplies (whole tiles of the KV box of every Q tile, padding
+        # included) against the pairs the neighborhood holds: the geometric waste of the tiling
+        "visited_pairs": visited,
+        "attended_pairs": attended,
+        "visited_over_attended": visited / attended,
         "kernel_ms": kernel_ms,
         "kernel_ms_source": ("HIP events around the timed steps (one launch per step)" if fused else
                              "HIP events around kernel-only launches"),
@@ -653,6 +664,28 @@ def main():
         gbps = alg_bytes / (kernel_ms * 1e-3) / 1e9
         result["roofline"].update({"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                                    "frac": gbps / HBM_PEAK_GBPS, "mfma_frac": achieved / peak})
+    if not args.no_dense and not args.step_only and dtype != torch.float32:
+        # The other half of the comparison the reference publishes per shape (docs/profiler.md:837-876:
+        # measured speed-up over self attention beside the FLOP-wise upper bound): dense attention over the
+        # same tokens, flattened to one sequence, through this library's own dense kernel.
+        N = q.numel() // (B * H * D)
+        flat = lambda t: t.reshape(B, N, H, D)
+        with torch.no_grad():
+            if quantised:
+                dense = lambda: natten_amd.attention(flat(q8), flat(k8), flat(v8), **scales)
+            else:
+                dense = lambda: natten_amd.attention(flat(q), flat(k), flat(v))
+            dense_iters = max(2, min(args.steps, int(0.5 / max(kernel_ms * 1e-3 * dense_flops / flops, 1e-6))))
+            dense_ms = timed(dense, dense_iters)
+        result["dense_self_attention"] = {
+            "call": "natten_amd.attention on the same tensors as one sequence of %d tokens" % N,
+            "dense_ms": dense_ms,
+            "dense_TFLOPs": dense_flops / (dense_ms * 1e-3) / 1e12,
+            "timed_calls": dense_iters,
+            "measured_speedup_vs_dense": dense_ms / kernel_ms,
+            "flop_wise_upper_bound": dense_flops / flops,
+            "fraction_of_bound": (dense_ms / kernel_ms) / (dense_flops / flops),
+        }
     if not args.no_mfma_probe:
         # context for roofline.frac: what the matrix cores sustain on random operands under the
         # chip's power limit (the published peak assumes the maximum clock)

@@ -122,11 +122,19 @@ int natten_amd_fna_forward(const void* q, const void* k, const void* v, void* ou
  * heads_q].  The kernel gathers the rows of each tile from the input and scatters its results,
  * so the three token permutes and two unpermutes around natten_amd_fna_forward (what the
  * reference's driver runs as separate operations, src/natten/backends/blackwell_fna.py:99-164)
- * disappear; results are bit-identical to the permuted path with the same tile shapes.
- * Requires qkv_shape[a] to be a multiple of dilation[a] * kv_tile_shape[a] in every dimension
- * (no KV tile may reach past the input); returns an error otherwise, and the caller uses the
- * permuted path.  dtype, tiles, head_dim, scales, run_persistent and workspace as in
- * natten_amd_fna_forward.
+ * disappear.  Which extents are taken:
+ *   - every qkv_shape[a] a multiple of dilation[a] * kv_tile_shape[a] (no KV tile reaches past
+ *     its dilation group): every dtype but float32 and every tile pair; with anchor_kv_tiles == 0
+ *     the results are bit-identical to the permuted path with the same tile shapes;
+ *   - any other extent with fp16 / bf16 operands: a tile that would reach past its dilation group
+ *     is gathered from one tile extent before the group's end and its leading keys, which the tile
+ *     before it delivered, are masked (sums then run in another order than on the permuted path);
+ *     when some dilation group is narrower than the KV tile in a dimension, only tiles of 128 x 64
+ *     tokens are taken (the instance that clamps its gathers);
+ *   - 8-bit float operands take multiples only.
+ * Anything else returns an error that says which rule was missed, and the caller uses the
+ * permuted path.  A KV tile must span less than 2^31 bytes of the input.  dtype, tiles, head_dim,
+ * scales, run_persistent and workspace as in natten_amd_fna_forward.
  *
  * anchor_kv_tiles != 0: the KV tiles of a Q tile are laid out from the first key of its window
  * box (per dimension) instead of from multiples of the KV tile extent -- there is no permuted
@@ -180,7 +188,9 @@ int natten_amd_fna_forward_fused_split(const void* q, const void* k, const void*
  * natten_amd_fna_forward_fused with anchor_kv_tiles = 1.  Every call on a GPU shares that GPU's array (the launch clears
  * it first, with a kernel): calls that overlap in time on one GPU -- on different streams or
  * from different threads -- race on the queues and must not be made; calls queued on one
- * stream are fine.
+ * stream are fine.  The first call on a device looks the array's address up
+ * (hipGetSymbolAddress, once per device): make one call on the device eagerly before the entry
+ * point is used on a stream that is capturing a graph.
  */
 int natten_amd_fna_forward_fused_static(const void* q, const void* k, const void* v, void* out,
                                         float* lse, int dtype, int na_dim, int batch, int heads_q,
@@ -200,6 +210,29 @@ int natten_amd_fna_forward_fused_static(const void* q, const void* k, const void
  */
 int natten_amd_window(int query, int kernel_size, int stride, int extent, int is_causal,
                       int32_t* start, int32_t* end);
+
+/*
+ * Host arithmetic only: the keys of a 64-key KV tile (numbered with dimension 0 fastest, extents
+ * kv_tile_shape[0..2], powers of two) whose in-tile coordinates lie in [lo[a], hi[a]) along every
+ * dimension, one bit per key -- the element mask the forward kernels apply to a partially attended
+ * tile (csrc/include/natten/cuda/fna_blackwell/collective/fna_fusion.hpp:384-436 tests the same
+ * condition coordinate by coordinate), built from the same per-dimension rows the kernels keep in
+ * LDS, so that tests can pin it against a brute-force decode.
+ */
+int natten_amd_tile_key_mask(const int32_t* kv_tile_shape, const int32_t* lo, const int32_t* hi,
+                             uint64_t* mask);
+
+/*
+ * Host arithmetic only: *result = 1 when natten_amd_fna_forward_fused would run this problem with
+ * the kernel instance that holds no mask code (every KV tile a Q tile visits is attended in full
+ * by all of its queries), the launch-level predicate of
+ * csrc/include/natten/cuda/fna_blackwell/collective/fna_fusion.hpp:503-593 (fully_block_sparse).
+ */
+int natten_amd_fna_fully_block_sparse(int na_dim, const int32_t* qkv_shape,
+                                      const int32_t* kernel_size, const int32_t* stride,
+                                      const int32_t* dilation, const int32_t* is_causal,
+                                      const int32_t* q_tile_shape, const int32_t* kv_tile_shape,
+                                      int anchor_kv_tiles, int32_t* result);
 
 /*
  * Supported tile sizes (tokens per tile).  Writes up to `capacity` pairs

@@ -19,9 +19,10 @@ import torch
 from torch import Tensor
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libnatten_amd.so")
+# NATTEN_AMD_LIBRARY: another build of the library (the timing-only ones of natten_amd.build --ablate)
+LIB_PATH = os.environ.get("NATTEN_AMD_LIBRARY") or os.path.join(_HERE, "libnatten_amd.so")
 
-ABI_VERSION = 13
+ABI_VERSION = 14
 
 DTYPE_CODES = {
     torch.float16: 0,
@@ -39,6 +40,8 @@ _SIGNATURES = {
     "natten_amd_abi_version": (ctypes.c_int, []),
     "natten_amd_last_error": (ctypes.c_char_p, []),
     "natten_amd_window": (ctypes.c_int, [ctypes.c_int] * 5 + [ctypes.c_void_p] * 2),
+    "natten_amd_tile_key_mask": (ctypes.c_int, [ctypes.c_void_p] * 4),
+    "natten_amd_fna_fully_block_sparse": (ctypes.c_int, [ctypes.c_int] + [ctypes.c_void_p] * 7 + [ctypes.c_int, ctypes.c_void_p]),
     "natten_amd_fna_supported_tiles": (
         ctypes.c_int,
         [ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int],
@@ -272,22 +275,24 @@ _QUEUE_WORKSPACES = {}
 
 def _queue_workspace(like: Tensor, run_persistent: bool):
     """(flag, pointer, bytes) of the work-queue launch's workspace, allocated by the caller side as
-    the reference's wrappers allocate theirs (src/natten/_libnatten/torch_wrappers.py:688-693)."""
+    the reference's wrappers allocate theirs (src/natten/_libnatten/torch_wrappers.py:688-693).
+    Always `run_persistent = 1`: the launch clears the counters itself (one small kernel ahead of
+    the work-queue kernel), so nothing rests on what an earlier launch left in the block.  The C
+    interface's `run_persistent = 2`, which skips that kernel for a caller who vouches for zeros,
+    is not used from Python."""
     if not run_persistent:
         return 0, None, 0
     nbytes = int(lib().natten_amd_fna_forward_workspace_bytes())
-    stream = torch.cuda.current_stream(like.device)
     if torch.cuda.is_current_stream_capturing():
-        # memory allocated under capture belongs to the graph: a block of its own, cleared by the launch
+        # memory allocated under capture belongs to the graph: a block of its own
         ws = torch.empty(nbytes, dtype=torch.uint8, device=like.device)
         return 1, ws.data_ptr(), nbytes
-    # One block per (device, stream), zeroed once: every work-queue launch leaves its counters at zero,
-    # and launches of one stream run one after the other, so the block is never cleared again.
-    key = (like.device.index, stream.cuda_stream)
+    # one block per (device, stream): launches of one stream run one after the other
+    key = (like.device.index, torch.cuda.current_stream(like.device).cuda_stream)
     ws = _QUEUE_WORKSPACES.get(key)
     if ws is None:
-        ws = _QUEUE_WORKSPACES[key] = torch.zeros(nbytes, dtype=torch.uint8, device=like.device)
-    return 2, ws.data_ptr(), nbytes
+        ws = _QUEUE_WORKSPACES[key] = torch.empty(nbytes, dtype=torch.uint8, device=like.device)
+    return 1, ws.data_ptr(), nbytes
 
 
 def _tile_span_fits(token_layout, dilation, tile_shape, row_bytes: int) -> bool:
@@ -472,6 +477,28 @@ def window(query: int, kernel_size: int, stride: int, extent: int, is_causal: bo
     _check(lib().natten_amd_window(int(query), int(kernel_size), int(stride), int(extent), int(bool(is_causal)),
                                    ctypes.addressof(st), ctypes.addressof(en)))
     return st.value, en.value
+
+
+def tile_key_mask(kv_tile_shape, lo, hi) -> int:
+    """Bit i set = key i of a 64-key KV tile (dimension 0 fastest) has in-tile coordinates inside
+    [lo, hi) along every dimension (host arithmetic only, the rows of the kernels' element mask)."""
+    pad = lambda x, fill: list(x) + [fill] * (3 - len(x))
+    m = ctypes.c_uint64()
+    _check(lib().natten_amd_tile_key_mask(_i32(pad(kv_tile_shape, 1)), _i32(pad(lo, 0)), _i32(pad(hi, 1)),
+                                          ctypes.addressof(m)))
+    return m.value
+
+
+def fully_block_sparse(qkv_shape, kernel_size, stride, dilation, is_causal, q_tile_shape, kv_tile_shape,
+                       anchored_tiles: bool = True) -> bool:
+    """Whether the one-launch forward runs this problem with the instance that holds no mask code
+    (host arithmetic only)."""
+    r = ctypes.c_int32()
+    _check(lib().natten_amd_fna_fully_block_sparse(
+        len(qkv_shape), _i32(qkv_shape), _i32(kernel_size), _i32(stride), _i32(dilation),
+        _i32([1 if c else 0 for c in is_causal]), _i32(q_tile_shape), _i32(kv_tile_shape), 1 if anchored_tiles else 0,
+        ctypes.addressof(r)))
+    return bool(r.value)
 
 
 def query_range(key_first: int, key_last: int, kernel_size: int, stride: int, extent: int, num_queries: int,

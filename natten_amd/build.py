@@ -1,4 +1,9 @@
-"""Builds libnatten_amd.so in-tree with hipcc for gfx950:  python -m natten_amd.build"""
+"""Builds libnatten_amd.so in-tree with hipcc for gfx950:  python -m natten_amd.build
+
+  python -m natten_amd.build --ablate N --output PATH
+builds a timing-only library instead (NATTEN_AMD_ABLATE = N leaves parts of the forward kernel's
+tile loop out, see csrc/fna_fwd.hpp; its results are wrong by design).  NATTEN_AMD_LIBRARY=PATH makes
+the package load such a library in place of the shipped one."""
 
 from __future__ import annotations
 
@@ -24,17 +29,26 @@ HIPCC_FLAGS = [
 ]
 
 
-def build(verbose: bool = False) -> str:
+def build(verbose: bool = False, ablate: int = 0, output: str = OUTPUT) -> str:
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    cmd = [hipcc, *HIPCC_FLAGS, *SOURCES, "-o", OUTPUT]
+    if ablate and os.path.abspath(output) == OUTPUT:
+        raise ValueError("a timing-only build must not replace the shipped library: give --output")
+    defines = [f"-DNATTEN_AMD_ABLATE={int(ablate)}"] if ablate else []
+    cmd = [hipcc, *HIPCC_FLAGS, *defines, *SOURCES, "-o", output]
     if verbose:
         print(" ".join(cmd), flush=True)
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)
     if proc.returncode != 0:
         sys.stderr.write(proc.stdout + proc.stderr)
         raise RuntimeError("hipcc failed building libnatten_amd.so")
-    return OUTPUT
+    return output
 
 
 if __name__ == "__main__":
-    print(build(verbose=True))
+    import argparse
+
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--ablate", type=int, default=0, help="NATTEN_AMD_ABLATE mask of a timing-only build")
+    ap.add_argument("--output", default=OUTPUT)
+    a = ap.parse_args()
+    print(build(verbose=True, ablate=a.ablate, output=a.output))

@@ -25,6 +25,7 @@
 #include <utility>
 
 #include "na_math.hpp"
+#include "work_queue.hpp"
 
 namespace natten_amd {
 
@@ -76,7 +77,7 @@ struct FnaParams {
   const int32_t* cu_q;   // [batch + 1]
   const int32_t* cu_kv;  // [batch + 1]
   int total_q, total_kv;  // rows of the packed operands: offsets that do not fit them are not followed
-  // Derived by finish_fna_params(): what the per-workgroup set-up would otherwise divide for.
+  // Derived by set_wg_layout(): what the per-workgroup set-up would otherwise divide for.
   // Tile extents are powers of two (log2 below); the other divisors get multiply-shift pairs.
   int q_tile_lg[3], kv_tile_lg[3];
   int ext_base[3], ext_rem[3];  // qkv_shape / dil and qkv_shape % dil: extent of dilation group g = base + (g < rem)
@@ -103,7 +104,21 @@ typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 #define NA_LDS __attribute__((address_space(3)))
 #define NA_GLOBAL __attribute__((address_space(1)))
 
-constexpr int kNumXcd = 8;
+// Timing-only builds.  NATTEN_AMD_ABLATE (0 in the shipped library) is a mask of parts of the tile
+// loop to leave out, to time what each costs on a given machine; every non-zero value computes
+// wrong results.  `python -m natten_amd.build --ablate N --output PATH` builds such a library.
+#ifndef NATTEN_AMD_ABLATE
+#define NATTEN_AMD_ABLATE 0
+#endif
+constexpr int kAblate = NATTEN_AMD_ABLATE;
+enum {
+  kAblateMask = 1,      // every tile is taken as fully attended: no element masks
+  kAblateCopies = 2,    // no global -> LDS tile copies inside the loop (tiles 0 and 1 are read over and over)
+  kAblateSoftmax = 4,   // no exponentials, row sums or conversions: P stays what it was before the loop
+  kAblateMax = 8,       // no row maxima, no rescaling
+  kAblateBarrier = 16,  // no workgroup barrier per KV tile
+  kAblateLdsReads = 32, // matrix operands are read from LDS once per iteration instead of once per instruction
+};
 
 template <typename T>
 struct Mma;
@@ -294,7 +309,10 @@ struct FnaSmem {
 // once, after the last KV tile and before the results are stored: nothing of this wave is in flight
 // at that point (the work-queue launch fetches its next position there, so that the wait for the
 // fetch does not include the stores); a call that returns early does not make it.
-template <typename T, int D, int NWAVES, int MQ, bool RAGGED, int KVT, bool SPLIT = false, typename Hook>
+// NOMASK: the launch is fully block-sparse (the host has checked that every KV tile a Q tile visits is
+// attended in full by every query of that Q tile: reference fna_fusion.hpp:503-593); the instance then
+// holds no mask code, tables or per-wave windows at all.
+template <typename T, int D, int NWAVES, int MQ, bool RAGGED, int KVT, bool SPLIT = false, bool NOMASK = false, typename Hook>
 static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const int pid_in, Hook&& before_stores) {
   // split launches: which run of the Q tile's KV tiles this workgroup takes
   const int split = SPLIT ? pid_in / p.split_grid : 0;
@@ -322,11 +340,17 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
   __shared__ __attribute__((aligned(1024))) char sV0[TILE_BYTES];
   __shared__ __attribute__((aligned(1024))) char sK1[TILE_BYTES];
   __shared__ __attribute__((aligned(1024))) char sV1[TILE_BYTES];
-  __shared__ __attribute__((aligned(16))) uint32_t sTab[KVT];
-  // Per-dimension geometry the element mask of a PARTIAL tile needs (twelve words per dimension, see
-  // kGeo* below).  Kept in LDS and read where a masked tile is met: in scalar registers for the
-  // whole loop these thirty-odd values would push the loop's own scalars out to spill lanes.
-  __shared__ __attribute__((aligned(16))) int sGeo[3][12];
+  // What the element mask of a PARTIAL tile needs (absent from NOMASK instances), kept in LDS and read
+  // where such a tile is met -- in registers for the whole loop these values would push the loop's own
+  // out to spill lanes:
+  //   sKeys[a][x]  the keys of a tile whose coordinate along dimension a is >= x, one bit per key
+  //   sWin[row]    window of the Q tile's query `row` (row-major): start and end per dimension
+  //   sGeo[a]      KV tile extent, its log2, and the box origin along dimension a
+  constexpr int MASK_ROWS = NOMASK ? 1 : KVT + 1;
+  __shared__ __attribute__((aligned(16))) uint64_t sKeys[NOMASK ? 1 : 3][MASK_ROWS];
+  __shared__ __attribute__((aligned(16))) int sWin[NOMASK ? 1 : NWAVES * MQ * 32][8];
+  __shared__ __attribute__((aligned(16))) int sGeo[3][4];
+  static_assert(NOMASK || KVT == 64, "the element mask holds one bit per key of a 64-key tile");
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -452,7 +476,7 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
   // dimension: a KV tile outside the union is skipped by this wave, one inside the
   // intersection needs no mask.
   int wave_lo[3], wave_hi[3], wave_full_lo[3], wave_full_hi[3];
-  {
+  if constexpr (!NOMASK) {
     const int i0 = wave * (MQ * 32), i1 = i0 + MQ * 32 - 1;
     const int lg2 = p.q_tile_lg[2], lg12 = p.q_tile_lg[1] + p.q_tile_lg[2];
     int f[3], l[3];
@@ -486,29 +510,20 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
     }
   }
 
-  enum { kGeoQFirst, kGeoKernel, kGeoStride, kGeoExtent, kGeoDivMul, kGeoDivShift, kGeoCausal, kGeoQMask, kGeoQLog2,
-         kGeoKvTile, kGeoKvLog2, kGeoBoxOrg };
-  if (tid < 3) {
-    const int a = tid;
-    sGeo[a][kGeoQFirst] = q_first[a];
-    sGeo[a][kGeoKernel] = ksz[a];
-    sGeo[a][kGeoStride] = p.stride[a];
-    sGeo[a][kGeoExtent] = extent[a];
-    sGeo[a][kGeoDivMul] = int(p.d_stride[a].mul);
-    sGeo[a][kGeoDivShift] = int(p.d_stride[a].shift);
-    sGeo[a][kGeoCausal] = p.causal[a];
-    sGeo[a][kGeoQMask] = p.q_tile[a] - 1;
-    sGeo[a][kGeoQLog2] = p.q_tile_lg[a];
-    sGeo[a][kGeoKvTile] = p.kv_tile[a];
-    sGeo[a][kGeoKvLog2] = p.kv_tile_lg[a];
-    sGeo[a][kGeoBoxOrg] = box_org[a];
-  }
-  // in-tile coordinates of every KV position, packed in 10-bit fields
-  for (int i = tid; i < KVT; i += NT) {
-    const int t0 = i & (p.kv_tile[0] - 1);
-    const int r1 = i >> p.kv_tile_lg[0];
-    const int t1 = r1 & (p.kv_tile[1] - 1);
-    sTab[i] = uint32_t(t0) | (uint32_t(t1) << 10) | (uint32_t(r1 >> p.kv_tile_lg[1]) << 20);
+  enum { kGeoKvTile, kGeoKvLog2, kGeoBoxOrg };
+  if constexpr (!NOMASK) {
+    if (tid < 3) {
+      sGeo[tid][kGeoKvTile] = p.kv_tile[tid];
+      sGeo[tid][kGeoKvLog2] = p.kv_tile_lg[tid];
+      sGeo[tid][kGeoBoxOrg] = box_org[tid];
+    }
+    // one row per thread and dimension: keys are numbered with dimension 0 fastest
+    int lg_stride = 0;
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+      if (tid <= p.kv_tile[a]) sKeys[a][tid] = na_keys_at_or_after(tid, lg_stride, p.kv_tile_lg[a]);
+      lg_stride += p.kv_tile_lg[a];
+    }
   }
 
   const int64_t q_row_stride = int64_t(p.heads_q) * D;
@@ -668,8 +683,10 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
     for (int a = 0; a < 3; ++a) {
       const int org = box_org[a] + (itc[a] << p.kv_tile_lg[a]);
       const int end = org + p.kv_tile[a];
-      t.full = t.full && (org >= wave_full_lo[a]) && (end <= wave_full_hi[a]);  // never when end > extent
-      t.skip = t.skip || (end <= wave_lo[a]) || (org >= wave_hi[a]);
+      if constexpr (!NOMASK) {
+        t.full = t.full && (org >= wave_full_lo[a]) && (end <= wave_full_hi[a]);  // never when end > extent
+        t.skip = t.skip || (end <= wave_lo[a]) || (org >= wave_hi[a]);
+      }
       // a tile that would reach past the group is moved back to end at the group's last position
       t.origin[a] = (p.edge == 1 || p.anchor) ? na_min(org, extent[a] - p.kv_tile[a]) : org;
     }
@@ -683,6 +700,10 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
         itc[1] = 0;
         ++itc[0];
       }
+    }
+    if constexpr (NOMASK || (kAblate & kAblateMask) != 0) {
+      t.full = true;
+      t.skip = false;
     }
     return t;
   };
@@ -728,6 +749,16 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
         valid = valid && (c < extent[a]);
         row += c * tok_step[a];
         row_c += na_min(c, extent[a] - 1) * tok_step[a];
+      }
+      if constexpr (!NOMASK) {
+        // this query's window (padding queries: that of the last real one), for the element masks
+        if (g == 0) {
+          const int qc = na_min(c, extent[a] - 1);
+          const bool cs = p.causal[a] != 0;
+          const int ws = na_window_start(qc, ksz[a], p.stride[a], p.d_stride[a], extent[a], cs);
+          sWin[(wave * MQ + mb) * 32 + l32][2 * a] = ws;
+          sWin[(wave * MQ + mb) * 32 + l32][2 * a + 1] = na_window_end(qc, ws, ksz[a], extent[a], cs);
+        }
       }
     }
     q_row[mb] = valid ? row : -1;
@@ -805,12 +836,28 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
   vec8 pf[MQ][NSB][2];
   f32x16_t c_init[MQ];          // -(running maximum), 0 while it is -inf: accumulator input of S = K Q^T
   float psum[MQ][2];
+  if constexpr ((kAblate & kAblateSoftmax) != 0) {
+    // probability-like operands (values in (0, 1]) in place of the ones the loop would form
+#pragma unroll
+    for (int mb = 0; mb < MQ; ++mb)
+#pragma unroll
+      for (int sb = 0; sb < NSB; ++sb)
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            pf[mb][sb][h][e] = static_cast<T>(fast_exp2(-fabsf(float(qf[mb][(sb * 2 + h) % KSTEPS][e]))));
+  }
 
   // Element e of the current tile's probabilities: row block e % MQ, logit v = e / MQ of the lane
   // (sub-block v / 16, register v % 16): exp2(c*s - c*m), summed in float; every second
   // element of a row block rounds its pair to T.
   float held[MQ];
   auto exp_elem = [&](const f32x16_t (&S_cur)[MQ][NSB], int e) {
+    if constexpr ((kAblate & kAblateSoftmax) != 0) {
+      asm volatile("" ::"v"(S_cur[e % MQ][(e / MQ) / 16][(e / MQ) % 16]));  // the logits stay in use
+      return;
+    }
     const int mb = e % MQ, v = e / MQ;
     const int sb = v / 16, r = v % 16;
     float x = fast_exp2(S_cur[mb][sb][r]);
@@ -836,46 +883,45 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
     return x < 0 ? 0 : (n > N_ELEMS ? N_ELEMS : n);
   };
 
-  // element mask of a PARTIAL tile for row block mb: the lane's query coordinates and window are
-  // worked out here, from the geometry in LDS (a masked tile is the exception)
+  // Element mask of a PARTIAL tile for row block mb.  Per dimension the lane's window, relative to the
+  // tile origin and clamped to the tile, selects two rows of sKeys (keys at or after its start, keys at
+  // or after its end); the AND over the dimensions has one bit per key of the tile.  A tile moved back
+  // from the group's edge starts before its place in the tiling (the box origin plus a multiple of the
+  // tile extent): the keys up to there (`lead`) belong to the tile before it.
   auto apply_mask = [&](f32x16_t (&S)[NSB], int mb, const int (&origin)[3]) __attribute__((always_inline)) {
-    uint32_t addc = 0, subc = 0;
-    int r = (wave * MQ + mb) * 32 + l32;  // row-major index of the query inside the Q tile
-#pragma unroll
-    for (int a = 2; a >= 0; --a) {
+    if constexpr (!NOMASK) {
       typedef int i32x4 __attribute__((ext_vector_type(4)));
-      const i32x4 g0 = *reinterpret_cast<const i32x4*>(&sGeo[a][0]);
-      const i32x4 g1 = *reinterpret_cast<const i32x4*>(&sGeo[a][4]);
-      const i32x4 g2 = *reinterpret_cast<const i32x4*>(&sGeo[a][8]);
-      const int qc = g0[kGeoQFirst] + (r & g1[kGeoQMask - 4]);
-      r >>= g2[kGeoQLog2 - 8];
-      const int kt = g2[kGeoKvTile - 8], kt_lg = g2[kGeoKvLog2 - 8];
-      const bool causal = g1[kGeoCausal - 4] != 0;
-      const NaDiv sd = {uint32_t(g1[kGeoDivMul - 4]), uint32_t(g1[kGeoDivShift - 4])};
-      const int ws = na_window_start(qc, g0[kGeoKernel], g0[kGeoStride], sd, g0[kGeoExtent], causal);
-      const int we = na_window_end(qc, ws, g0[kGeoKernel], g0[kGeoExtent], causal);
-      // window of this lane's query relative to the tile origin, clamped to the tile.  A tile
-      // moved back from the group's edge starts before its place in the tiling (the box origin
-      // plus a multiple of the tile extent): the keys up to there belong to the tile before it
-      const int from_box = origin[a] - g2[kGeoBoxOrg - 8];
-      const int lead = (((from_box + kt - 1) >> kt_lg) << kt_lg) - from_box;
-      const int lo = na_min(na_max(ws - origin[a], lead), kt);
-      const int hi = na_min(na_max(we - origin[a], 0), kt);
-      addc |= uint32_t(512 - lo) << (10 * a);
-      subc |= uint32_t(511 + hi) << (10 * a);
-    }
+      typedef int i32x2 __attribute__((ext_vector_type(2)));
+      const int row = (wave * MQ + mb) * 32 + l32;
+      const i32x4 w01 = *reinterpret_cast<const i32x4*>(&sWin[row][0]);
+      const i32x2 w2 = *reinterpret_cast<const i32x2*>(&sWin[row][4]);
+      const int ws[3] = {w01[0], w01[2], w2[0]}, we[3] = {w01[1], w01[3], w2[1]};
+      uint64_t keys = ~uint64_t(0);
 #pragma unroll
-    for (int sb = 0; sb < NSB; ++sb)
+      for (int a = 0; a < 3; ++a) {
+        const i32x4 geo = *reinterpret_cast<const i32x4*>(&sGeo[a][0]);
+        const int kt = geo[kGeoKvTile], kt_lg = geo[kGeoKvLog2];
+        const int from_box = origin[a] - geo[kGeoBoxOrg];
+        const int lead = (((from_box + kt - 1) >> kt_lg) << kt_lg) - from_box;
+        const int lo = na_min(na_max(ws[a] - origin[a], lead), kt);
+        const int hi = na_min(na_max(we[a] - origin[a], 0), kt);
+        keys &= sKeys[a][lo] & ~sKeys[a][hi];
+      }
+      // the lane's logit r of sub-block sb belongs to key 32 sb + 8 (r / 4) + 4 g + r % 4
+      keys >>= 4 * g;
 #pragma unroll
-      for (int jj = 0; jj < 4; ++jj) {
-        const u32x4_t tc4 = *reinterpret_cast<const u32x4_t*>(&sTab[sb * 32 + 8 * jj + 4 * g]);
+      for (int sb = 0; sb < NSB; ++sb) {
+        const uint32_t half = uint32_t(keys >> (32 * sb));
+        // two instructions per logit (sign-extended bit, bitwise select) and no condition codes
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const uint32_t tp = tc4[i];
-          const uint32_t ok = (tp + addc) & (subc - tp) & kGuardBits;
-          S[sb][4 * jj + i] = (ok == kGuardBits) ? S[sb][4 * jj + i] : -INFINITY;
+        for (int r = 0; r < 16; ++r) {
+          const uint32_t keep = uint32_t(__builtin_amdgcn_sbfe(int(half), 8 * (r / 4) + r % 4, 1));  // 0 or ~0
+          const float logit = S[sb][r];  // (a copy: a bit cast of the vector element itself reads element 0)
+          const uint32_t bits = __builtin_bit_cast(uint32_t, logit);
+          S[sb][r] = __builtin_bit_cast(float, (bits & keep) | (~keep & 0xff800000u));
         }
       }
+    }
   };
 
   // adopts the maximum `mx` of the lane's half row of the coming tile (relative to the running
@@ -977,14 +1023,15 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
     char* sV_nxt = st ? sV0 : sV1;  // held V(j-1): free, receives V(j+1)
 
     wait_vmcnt<0>();   // this thread's copies of K(j+1) and V(j) have landed
-    __syncthreads();   // ... and everyone's; everyone is done reading K(j) and V(j-1)
+    if constexpr ((kAblate & kAblateBarrier) == 0)
+      __syncthreads();   // ... and everyone's; everyone is done reading K(j) and V(j-1)
     const TileInfo t2 = next_tile();
     // Past the end of the box the spread copies re-read the current tile into the free stage
     // (never used), which keeps the slots below free of control flow.
     // (the spread copies only exist without RAGGED, where a tile's origin is not looked at)
     const TileCopy ck = make_copy(kbase, sK_cur, (j + 2 < total_tiles) ? t2.row0 : cur.row0, cur.origin);
     const TileCopy cv = make_copy(vbase, sV_nxt, (j + 1 < total_tiles) ? nxt.row0 : cur.row0, cur.origin);
-    if constexpr (!SPREAD) {
+    if constexpr (!SPREAD && (kAblate & kAblateCopies) == 0) {
       if (j + 2 < total_tiles) issue_tile_load(kbase, ld_koff, sK_cur, t2.row0, t2.origin, KLayout{});
       if (j + 1 < total_tiles) issue_tile_load(vbase, ld_voff, sV_nxt, nxt.row0, nxt.origin, VLayout{});
     }
@@ -1000,7 +1047,10 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
     auto g1_slot = [&](auto s_tag) __attribute__((always_inline)) {
       constexpr int s = decltype(s_tag)::value;
       if constexpr (NXT) {
-        if constexpr (s + PF_K < N_QK) kf[s + PF_K] = k_frag(sK_nxt, s + PF_K);
+        if constexpr (s + PF_K < N_QK) {
+          if constexpr ((kAblate & kAblateLdsReads) == 0 || s + PF_K < 4) kf[s + PF_K] = k_frag(sK_nxt, s + PF_K);
+          else kf[s + PF_K] = kf[(s + PF_K) % 4];
+        }
 #pragma unroll
         for (int mb = 0; mb < MQ; ++mb) {
           if constexpr (s % KSTEPS == 0) {
@@ -1020,7 +1070,7 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
           pin(psum[mb][1]);
         }
       }
-      if constexpr (SPREAD) {
+      if constexpr (SPREAD && (kAblate & kAblateCopies) == 0) {
         // 2 * PER copies spread over the first half of the slots, K first
         constexpr int c_lo = (s * 2 * PER * 2) / N_QK, c_hi = ((s + 1) * 2 * PER * 2) / N_QK;
         for_range<c_lo, c_hi - c_lo>([&](auto c_tag) {
@@ -1054,7 +1104,10 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
       static_assert(elems_done(N_QK + (t / DB) * DB - 1) >= MQ * 8 * (t / DB + 1), "exponentials scheduled too late");
       constexpr int x_lo = elems_done(N_QK + t - 1), x_hi = elems_done(N_QK + t);
       if constexpr (CUR) {
-        if constexpr (t + PF_V < N_PV) vf[t + PF_V] = v_frag(sV_cur, t + PF_V);
+        if constexpr (t + PF_V < N_PV) {
+          if constexpr ((kAblate & kAblateLdsReads) == 0 || t + PF_V < 4) vf[t + PF_V] = v_frag(sV_cur, t + PF_V);
+          else vf[t + PF_V] = vf[(t + PF_V) % 4];
+        }
 #pragma unroll
         for (int mb = 0; mb < MQ; ++mb)
           acc[mb][t % DB] = M::run(vf[t], pf[mb][t / (2 * DB)][(t / DB) % 2], acc[mb][t % DB]);
@@ -1068,7 +1121,7 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
           }
         }
       }
-      if constexpr (NXT && t >= N_PV / 2) {
+      if constexpr (NXT && t >= N_PV / 2 && (kAblate & kAblateMax) == 0) {
         // row maxima of the coming tile (as if unmasked), MQ * NSB * 16 values over N_PV / 2 slots
         constexpr int t3 = t - N_PV / 2;
         constexpr int NV = MQ * NSB * 16;
@@ -1094,7 +1147,7 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
       for (int mb = 0; mb < MQ; ++mb) l_run[mb] += psum[mb][0] + psum[mb][1];
     }
 
-    if (NXT && j + 1 < total_tiles) {
+    if ((kAblate & kAblateMax) == 0 && NXT && j + 1 < total_tiles) {
       float mxs[MQ];
 #pragma unroll
       for (int mb = 0; mb < MQ; ++mb) mxs[mb] = fmaxf(mx[mb][0], mx[mb][1]);
@@ -1145,10 +1198,10 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
   }
 }
 
-template <typename T, int D, int NWAVES, int MQ, bool RAGGED, int KVT>
+template <typename T, int D, int NWAVES, int MQ, bool RAGGED, int KVT, bool NOMASK = false>
 __global__ void __launch_bounds__(NWAVES * 64) __attribute__((amdgpu_waves_per_eu(MQ == 1 ? 2 : 1, MQ == 1 ? 2 : 1)))
 fna_fwd_kernel(const FnaParams p) {
-  fna_fwd_tile<T, D, NWAVES, MQ, RAGGED, KVT>(p, int(blockIdx.x), []() {});
+  fna_fwd_tile<T, D, NWAVES, MQ, RAGGED, KVT, false, NOMASK>(p, int(blockIdx.x), []() {});
 }
 
 // Split launch: kv_splits workgroups per Q tile, each on a contiguous run of the tile's KV tiles,
@@ -1165,14 +1218,10 @@ fna_fwd_split_kernel(const FnaParams p) {
 // Work-queue launch: as many workgroups as the chip keeps resident, each taking Q tiles until
 // none is left.  Workgroup i runs on XCD i % 8 (the dispatcher deals workgroups to XCDs in turn),
 // and launch position `local * 8 + x` is what the one-tile-per-workgroup launch runs on XCD x:
-// every XCD has a queue of its own (`queues[16 * x]`, one counter per 64-byte line) over its
-// `per_xcd` positions in the same order, so the tiles resident on an XCD share K/V in its L2 as
-// before; a workgroup whose queue has run dry takes from the other XCDs' queues, which evens
-// out the tail.  The counters must be zero at launch.  Every workgroup ends after at most
-// `8 * per_xcd + 8` counter increments in total, whatever the other workgroups do.
-constexpr int kQueueStride = 16;  // uint32 counters per 64-byte line
-constexpr int kQueueWords = kNumXcd * kQueueStride;
-constexpr int kQueueDoneWord = 1;  // workgroups that have left the loop (in the first queue's line)
+// every XCD has a queue of its own over its `per_xcd` positions in the same order, so the tiles
+// resident on an XCD share K/V in its L2 as before; a workgroup whose queue has run dry takes from
+// the other XCDs' queues, which evens out the tail.  The protocol (counter layout, what a ticket
+// means, who resets the counters) is work_queue.hpp's.
 
 // The launch parameters of a work-queue kernel, read anew for every tile.  Left to itself the compiler
 // hoists the set-up's reads of launch parameters (and what it derives from them) out of the loop
@@ -1207,19 +1256,21 @@ static __device__ __forceinline__ void fna_queue_loop(uint32_t* __restrict__ que
   __shared__ int s_pos[2];   // s_pos[i & 1]: position of the workgroup's i-th tile (-1: none is left)
   __shared__ int s_victim;   // queues found empty so far: the home queue first, then the others in turn
   const int home = int(blockIdx.x) % kNumXcd;
-  auto queue_of = [&](int victim) __attribute__((always_inline)) {
-    return &queues[((home + victim) % kNumXcd) * kQueueStride];
-  };
-  // thread 0: the next position (-1: every queue is empty)
+  // thread 0: the next position (-1: every queue is empty).  The wait for the counter's old value is
+  // written out as a wait for everything outstanding rather than left to the compiler's count of
+  // the operations it knows about: the tile copies are issued from assembly statements it does not see.
+  // (Vector memory operations of a wave complete in issue order, so operations it does not count can
+  // only make its counted waits longer, never shorter; a full wait does not depend on that either.)
   auto take = [&]() __attribute__((always_inline)) {
-    int victim = s_victim;
-    uint32_t ticket = atomicAdd(queue_of(victim), 1u);
-    while (ticket >= uint32_t(per_xcd)) {  // that queue is empty for good
-      if (++victim == kNumXcd) break;
-      ticket = atomicAdd(queue_of(victim), 1u);
+    int victim = s_victim, pos = -1;
+    while (victim < kNumXcd) {
+      const uint32_t ticket = atomicAdd(&queues[queue_counter_word(home, victim)], 1u);
+      wait_vmcnt<0>();
+      pos = queue_position(home, victim, ticket, per_xcd);  // an empty queue counts into `victim`
+      if (pos >= 0) break;
     }
     s_victim = victim;
-    return victim == kNumXcd ? -1 : int(ticket) * kNumXcd + (home + victim) % kNumXcd;
+    return pos;
   };
   if (threadIdx.x == 0) {
     s_victim = 0;
@@ -1243,19 +1294,19 @@ static __device__ __forceinline__ void fna_queue_loop(uint32_t* __restrict__ que
   // increments, whose old values it waited for, are complete.)
   if (threadIdx.x == 0) {
     const uint32_t left = atomicAdd(&queues[kQueueDoneWord], 1u);
-    if (left == gridDim.x - 1) {
+    if (queue_last_one_out(left, gridDim.x)) {
       for (int x = 0; x < kNumXcd; ++x) __hip_atomic_store(&queues[x * kQueueStride], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       __hip_atomic_store(&queues[kQueueDoneWord], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
   }
 }
 
-template <typename T, int D, int NWAVES, int MQ, bool RAGGED, int KVT>
+template <typename T, int D, int NWAVES, int MQ, bool RAGGED, int KVT, bool NOMASK = false>
 __global__ void __launch_bounds__(NWAVES * 64) __attribute__((amdgpu_waves_per_eu(MQ == 1 ? 2 : 1, MQ == 1 ? 2 : 1)))
 fna_fwd_queue_kernel(const FnaParams p, uint32_t* __restrict__ queues, const int per_xcd) {
   FnaKernargPtr args = fna_kernarg_params();
   fna_queue_loop(queues, per_xcd, [&](int pid, auto& fetch) __attribute__((always_inline)) {
-    fna_fwd_tile<T, D, NWAVES, MQ, RAGGED, KVT>(fna_params_for_this_tile(args), pid, fetch);
+    fna_fwd_tile<T, D, NWAVES, MQ, RAGGED, KVT, false, NOMASK>(fna_params_for_this_tile(args), pid, fetch);
   });
   (void)p;
 }

@@ -70,6 +70,20 @@ NA_HD int na_window_start(int i, int k, int s, NaDiv s_div, int L, bool causal) 
   return na_max(leader - wl, 0) + ((leader + wr >= L) ? (L - wr - leader - 1) : 0);
 }
 
+// Keys of a 64-key KV tile are numbered with dimension 0 fastest and all tile extents are powers of
+// two, so a key's coordinate along one dimension is a bit field of its number: (i >> lg_stride) &
+// (2^lg_extent - 1).  Bit i of the result is set when that coordinate of key i is >= x
+// (0 <= x <= 2^lg_extent).  The keys with coordinate in [lo, hi) are then
+// na_keys_at_or_after(lo) & ~na_keys_at_or_after(hi), and a multi-dimensional window inside the
+// tile is the AND of its per-dimension masks: what the kernels' element mask tests.
+NA_HD uint64_t na_ones64(int n) { return n >= 64 ? ~uint64_t(0) : ((uint64_t(1) << n) - 1); }
+NA_HD uint64_t na_keys_at_or_after(int x, int lg_stride, int lg_extent) {
+  const int lg_period = lg_stride + lg_extent;  // the pattern repeats every 2^lg_period keys
+  uint64_t m = na_ones64(1 << lg_period) & ~na_ones64(x << lg_stride);
+  for (int s = lg_period; s < 6; ++s) m |= m << (1 << s);
+  return m;
+}
+
 // Number of tokens of dilation group g along a dimension of extent X.
 NA_HD int na_group_extent(int X, int d, int g) { return X / d + 1 - ((g + (d - X % d)) / d); }
 

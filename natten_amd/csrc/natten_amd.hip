@@ -9,6 +9,7 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <atomic>
 #include <mutex>
 #include <type_traits>
 
@@ -62,16 +63,18 @@ constexpr int kNumTileConfigs = sizeof(kTileConfigs) / sizeof(kTileConfigs[0]);
 // Workgroups a work-queue launch starts: two per compute unit (what the kernel's LDS and register
 // use keep resident), a multiple of the XCD count; the device's figure is read once.
 int resident_workgroups() {
-  static int cached[64] = {};
+  static std::atomic<int> cached[64] = {};  // (threads that race here compute the same value)
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 512;
-  if (cached[dev] == 0) {
+  int n = cached[dev].load(std::memory_order_relaxed);
+  if (n == 0) {
     int cus = 0;
     if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1) cus = 256;
-    cached[dev] = (2 * cus / kNumXcd) * kNumXcd;
-    if (cached[dev] < kNumXcd) cached[dev] = kNumXcd;
+    n = (2 * cus / kNumXcd) * kNumXcd;
+    if (n < kNumXcd) n = kNumXcd;
+    cached[dev].store(n, std::memory_order_relaxed);
   }
-  return cached[dev];
+  return n;
 }
 
 // The counters of a work-queue launch (null: one workgroup per Q tile).  Every work-queue kernel
@@ -82,7 +85,7 @@ struct WorkQueue {
   bool clear_first = true;
 };
 
-template <typename T, int D, int NWAVES, int MQ, bool RAGGED, int KVT>
+template <typename T, int D, int NWAVES, int MQ, bool RAGGED, int KVT, bool NOMASK = false>
 int launch_fna(const FnaParams& p, hipStream_t stream, WorkQueue queues = {}) {
   constexpr int QT = NWAVES * MQ * 32;
   if (!fna_tiles_are_powers_of_two(p)) return fail("fna_forward: tile extents must be powers of two");
@@ -92,8 +95,9 @@ int launch_fna(const FnaParams& p, hipStream_t stream, WorkQueue queues = {}) {
   if (queues.counters != nullptr) {
     const long long resident = resident_workgroups();
     if (queues.clear_first) hipLaunchKernelGGL(fna_queue_clear_kernel, dim3(1), dim3(kQueueWords), 0, stream, queues.counters);
-    hipLaunchKernelGGL((fna_fwd_queue_kernel<T, D, NWAVES, MQ, RAGGED, KVT>), dim3((unsigned)(wgs < resident ? wgs : resident)),
-                       dim3(NWAVES * 64), 0, stream, p, queues.counters, int(wgs / kNumXcd));
+    hipLaunchKernelGGL((fna_fwd_queue_kernel<T, D, NWAVES, MQ, RAGGED, KVT, NOMASK>),
+                       dim3((unsigned)(wgs < resident ? wgs : resident)), dim3(NWAVES * 64), 0, stream, p, queues.counters,
+                       int(wgs / kNumXcd));
     return check_launch("fna_forward (work queue)");
   }
   if (p.kv_splits > 1) {
@@ -109,8 +113,38 @@ int launch_fna(const FnaParams& p, hipStream_t stream, WorkQueue queues = {}) {
       return fail("fna_forward: KV splits exist for Q tiles of 128 and KV tiles of 64 tokens");
     }
   }
-  hipLaunchKernelGGL((fna_fwd_kernel<T, D, NWAVES, MQ, RAGGED, KVT>), dim3((unsigned)wgs), dim3(NWAVES * 64), 0, stream, p);
+  hipLaunchKernelGGL((fna_fwd_kernel<T, D, NWAVES, MQ, RAGGED, KVT, NOMASK>), dim3((unsigned)wgs), dim3(NWAVES * 64), 0, stream,
+                     p);
   return check_launch("fna_forward");
+}
+
+// Whether the launch is fully block-sparse: every Q tile is whole (no padding queries), all its
+// queries share one window in every dimension, and the KV tiles laid out for it cover that window
+// exactly, so that every (Q tile, KV tile) pair the kernel visits is attended in full and the
+// instance without any mask code gives the same bits.  The role of the reference's
+// fully_block_sparse (csrc/include/natten/cuda/fna_blackwell/collective/fna_fusion.hpp:503-593),
+// evaluated from the kernel's own window and box arithmetic.  Needs set_wg_layout() to have run.
+bool fully_block_sparse(const FnaParams& p) {
+  if (p.cu_q != nullptr || p.edge != 0 || p.kv_splits > 1) return false;
+  for (int a = 0; a < 3; ++a) {
+    // dilation groups come in at most two extents
+    for (int ext = p.ext_base[a] + (p.ext_rem[a] > 0 ? 1 : 0); ext >= p.ext_base[a]; --ext) {
+      if (ext < 1 || ext % p.q_tile[a] != 0) return false;
+      const bool c = p.causal[a] != 0;
+      for (int qf = 0; qf < ext; qf += p.q_tile[a]) {
+        const int ql = qf + p.q_tile[a] - 1;
+        const int st_f = na_window_start(qf, p.ksize[a], p.stride[a], p.d_stride[a], ext, c);
+        const int st_l = na_window_start(ql, p.ksize[a], p.stride[a], p.d_stride[a], ext, c);
+        const int en_f = na_window_end(qf, st_f, p.ksize[a], ext, c);
+        const int en_l = na_window_end(ql, st_l, p.ksize[a], ext, c);
+        // (start and end are monotone in the query: equal at both ends means equal throughout)
+        if (st_f != st_l || en_f != en_l) return false;
+        const int org = p.anchor ? st_f : ((st_f >> p.kv_tile_lg[a]) << p.kv_tile_lg[a]);
+        if (org != st_f || (en_l - org) % p.kv_tile[a] != 0) return false;
+      }
+    }
+  }
+  return true;
 }
 
 template <bool E5M2, int D>
@@ -139,7 +173,10 @@ int dispatch_tiles(const FnaParams& p, int qt, int kvt, hipStream_t stream, Work
     return fail("fna_forward: seqlen_kv (%d) must be a multiple of the KV tile (%d tokens)", p.seqlen_kv, kvt);
   }
   // the work-queue launch exists for the default tile pair; the others launch a workgroup per Q tile
-  if (qt == 128 && kvt == 64) return launch_fna<T, D, 4, 1, false, 64>(p, stream, queues);
+  if (qt == 128 && kvt == 64) {
+    if (fully_block_sparse(p)) return launch_fna<T, D, 4, 1, false, 64, true>(p, stream, queues);
+    return launch_fna<T, D, 4, 1, false, 64>(p, stream, queues);
+  }
   if (qt == 256 && kvt == 64) return launch_fna<T, D, 8, 1, false, 64>(p, stream);
   if (qt == 64 && kvt == 64) return launch_fna<T, D, 2, 1, false, 64>(p, stream);
   return fail("fna_forward: no kernel for Q tile of %d and KV tile of %d tokens", qt, kvt);
@@ -268,11 +305,16 @@ int queue_workspace(const char* what, int run_persistent, void* workspace, uint6
   queues->clear_first = run_persistent == 1;  // 2: the caller vouches for zeros (what every launch leaves behind)
   return 0;
 }
+
+int fused_geometry(const char* what, FnaParams& p, bool sixteen_bit, int na_dim, int heads_kv, int head_dim,
+                   const int32_t* qkv_shape, const int32_t* kernel_size, const int32_t* stride, const int32_t* dilation,
+                   const int32_t* is_causal, const int32_t* q_tile_shape, const int32_t* kv_tile_shape, int anchor_kv_tiles,
+                   long long* tokens_out);
 }  // namespace
 
 extern "C" {
 
-int natten_amd_abi_version(void) { return 13; }
+int natten_amd_abi_version(void) { return 14; }
 
 uint64_t natten_amd_fna_forward_workspace_bytes(void) { return uint64_t(kQueueWords) * 4; }
 
@@ -286,6 +328,50 @@ int natten_amd_window(int query, int kernel_size, int stride, int extent, int is
   // the arithmetic the kernels' set-up runs: stride division by multiply and shift
   *start = na_window_start(query, kernel_size, stride, na_make_div(stride), extent, is_causal != 0);
   *end = na_window_end(query, *start, kernel_size, extent, is_causal != 0);
+  return 0;
+}
+
+int natten_amd_tile_key_mask(const int32_t* kv_tile_shape, const int32_t* lo, const int32_t* hi, uint64_t* mask) {
+  g_error[0] = 0;
+  if (!kv_tile_shape || !lo || !hi || !mask) return fail("tile_key_mask: null pointer argument");
+  int lg[3], keys = 1;
+  for (int a = 0; a < 3; ++a) {
+    lg[a] = 0;
+    while ((1 << lg[a]) < kv_tile_shape[a]) ++lg[a];
+    if (kv_tile_shape[a] < 1 || (1 << lg[a]) != kv_tile_shape[a])
+      return fail("tile_key_mask: tile extents must be powers of two, got %d", kv_tile_shape[a]);
+    if (lo[a] < 0 || hi[a] < 0 || lo[a] > kv_tile_shape[a] || hi[a] > kv_tile_shape[a])
+      return fail("tile_key_mask: bounds must lie in 0 .. extent along dimension %d", a);
+    keys *= kv_tile_shape[a];
+  }
+  if (keys != 64) return fail("tile_key_mask: the tile must hold 64 keys, got %d", keys);
+  // the rows the kernels keep in LDS and how their element mask combines them
+  uint64_t m = ~uint64_t(0);
+  int lg_stride = 0;
+  for (int a = 0; a < 3; ++a) {
+    m &= na_keys_at_or_after(lo[a], lg_stride, lg[a]) & ~na_keys_at_or_after(hi[a], lg_stride, lg[a]);
+    lg_stride += lg[a];
+  }
+  *mask = m;
+  return 0;
+}
+
+int natten_amd_fna_fully_block_sparse(int na_dim, const int32_t* qkv_shape, const int32_t* kernel_size,
+                                      const int32_t* stride, const int32_t* dilation, const int32_t* is_causal,
+                                      const int32_t* q_tile_shape, const int32_t* kv_tile_shape, int anchor_kv_tiles,
+                                      int32_t* result) {
+  g_error[0] = 0;
+  if (na_dim < 1 || na_dim > 3) return fail("fna_fully_block_sparse: na_dim must be 1, 2 or 3, got %d", na_dim);
+  if (!result) return fail("fna_fully_block_sparse: null pointer argument");
+  FnaParams p;
+  long long tokens = 0;
+  if (int rc = fused_geometry("fna_fully_block_sparse", p, true, na_dim, 1, 32, qkv_shape, kernel_size, stride, dilation,
+                              is_causal, q_tile_shape, kv_tile_shape, anchor_kv_tiles, &tokens))
+    return rc;
+  p.batch = p.num_groups;
+  p.heads_q = p.heads_kv = 1;
+  set_wg_layout(p, 1);
+  *result = fully_block_sparse(p) ? 1 : 0;
   return 0;
 }
 
@@ -360,15 +446,14 @@ int natten_amd_fna_forward(const void* q, const void* k, const void* v, void* ou
 }
 
 namespace {
-// natten_amd_fna_forward_fused after its workspace has been resolved (`queues` == nullptr: a workgroup per Q tile)
-int fna_forward_fused_impl(const void* q, const void* k, const void* v, void* out, float* lse, int dtype, int na_dim,
-                           int batch, int heads_q, int heads_kv, int head_dim, const int32_t* qkv_shape,
-                           const int32_t* kernel_size, const int32_t* stride, const int32_t* dilation,
-                           const int32_t* is_causal, const int32_t* q_tile_shape, const int32_t* kv_tile_shape,
-                           float scale, const float* q_scale, const float* k_scale, const float* v_scale,
-                           int anchor_kv_tiles, WorkQueue queues, void* stream, int kv_splits = 1) {
+// The part of natten_amd_fna_forward_fused that needs no operands: checks the shapes and fills the
+// launch geometry of the one-launch route (`sixteen_bit`: fp16 / bf16 operands, which take any extent).
+int fused_geometry(const char* what, FnaParams& p, bool sixteen_bit, int na_dim, int heads_kv, int head_dim,
+                   const int32_t* qkv_shape, const int32_t* kernel_size, const int32_t* stride, const int32_t* dilation,
+                   const int32_t* is_causal, const int32_t* q_tile_shape, const int32_t* kv_tile_shape, int anchor_kv_tiles,
+                   long long* tokens_out) {
   if (!qkv_shape || !kernel_size || !stride || !dilation || !is_causal || !q_tile_shape || !kv_tile_shape)
-    return fail("fna_forward_fused: null shape argument");
+    return fail("%s: null shape argument", what);
   int qs[3] = {1, 1, 1}, ks[3] = {1, 1, 1};
   long long tokens = 1;
   // Extents that are not multiples of dilation x KV tile: some KV tile would reach past its
@@ -378,7 +463,7 @@ int fna_forward_fused_impl(const void* q, const void* k, const void* v, void* ou
   int edge = 0;
   for (int a = 0; a < na_dim; ++a) {
     if (qkv_shape[a] < 1 || dilation[a] < 1 || q_tile_shape[a] < 1 || kv_tile_shape[a] < 1)
-      return fail("fna_forward_fused: invalid parameter along dimension %d", a);
+      return fail("%s: invalid parameter along dimension %d", what, a);
     // dilation groups may differ in extent by one; the padded per-group layouts cover the largest
     const int ext = na_ceil_div(qkv_shape[a], dilation[a]);
     if (qkv_shape[a] % dilation[a] != 0 || ext % kv_tile_shape[a] != 0) edge = edge > 1 ? edge : 1;
@@ -393,26 +478,52 @@ int fna_forward_fused_impl(const void* q, const void* k, const void* v, void* ou
       qt *= q_tile_shape[a];
       kvt *= kv_tile_shape[a];
     }
-    if (dtype != NATTEN_AMD_F16 && dtype != NATTEN_AMD_BF16)
-      return fail("fna_forward_fused: an input extent that is not a multiple of dilation * KV tile in every dimension "
-                  "needs fp16 / bf16 operands (got dtype code %d); use the token-permuted entry point", dtype);
+    if (!sixteen_bit)
+      return fail("%s: an input extent that is not a multiple of dilation * KV tile in every dimension needs fp16 / bf16 "
+                  "operands; use the token-permuted entry point", what);
     if (edge == 2 && (qt != 128 || kvt != 64))
-      return fail("fna_forward_fused: a dilation group narrower than the KV tile needs tiles of 128 x 64 tokens (got "
-                  "%lld x %lld); use the token-permuted entry point", qt, kvt);
+      return fail("%s: a dilation group narrower than the KV tile needs tiles of 128 x 64 tokens (got %lld x %lld); use "
+                  "the token-permuted entry point", what, qt, kvt);
   }
-  if (tokens > 0x7fffffffLL) return fail("fna_forward_fused: more than 2^31 tokens per batch");
-  if (int rc = check_common("fna_forward_fused", q, k, v, out, lse, batch, prod3(qs), prod3(ks), heads_q, heads_kv,
-                            head_dim))
-    return rc;
-  FnaParams p;
-  if (int rc = fill_fna_params("fna_forward_fused", p, na_dim, qs, ks, qkv_shape, kernel_size, stride, dilation,
-                               is_causal, q_tile_shape, kv_tile_shape))
+  if (tokens > 0x7fffffffLL) return fail("%s: more than 2^31 tokens per batch", what);
+  if (int rc = fill_fna_params(what, p, na_dim, qs, ks, qkv_shape, kernel_size, stride, dilation, is_causal, q_tile_shape,
+                               kv_tile_shape))
     return rc;
   // per-lane byte offsets inside a KV tile are 32-bit
   long long span = 0;
   for (int a = 0; a < 3; ++a) span += (long long)(p.kv_tile[a] - 1) * p.dil[a] * p.tok_stride[a];
   if ((span + 1) * heads_kv * head_dim * 2 + 8192 >= 0x7fffffffLL)  // (16-bit rows; 8-bit ones are shorter)
-    return fail("fna_forward_fused: a KV tile spans more than 2^31 bytes of the input; use the token-permuted entry point");
+    return fail("%s: a KV tile spans more than 2^31 bytes of the input; use the token-permuted entry point", what);
+  p.seqlen_q = prod3(qs);
+  p.seqlen_kv = prod3(ks);
+  p.fused = 1;
+  p.edge = edge;
+  // tiles laid out from the window's first key: needs every dilation group at least a KV tile wide
+  p.anchor = (anchor_kv_tiles != 0 && edge != 2) ? 1 : 0;
+  for (int a = 0; a < na_dim; ++a)
+    if (qkv_shape[a] / dilation[a] < kv_tile_shape[a]) p.anchor = 0;
+  p.tokens = int(tokens);
+  *tokens_out = tokens;
+  return 0;
+}
+
+// natten_amd_fna_forward_fused after its workspace has been resolved (`queues` == nullptr: a workgroup per Q tile)
+int fna_forward_fused_impl(const void* q, const void* k, const void* v, void* out, float* lse, int dtype, int na_dim,
+                           int batch, int heads_q, int heads_kv, int head_dim, const int32_t* qkv_shape,
+                           const int32_t* kernel_size, const int32_t* stride, const int32_t* dilation,
+                           const int32_t* is_causal, const int32_t* q_tile_shape, const int32_t* kv_tile_shape,
+                           float scale, const float* q_scale, const float* k_scale, const float* v_scale,
+                           int anchor_kv_tiles, WorkQueue queues, void* stream, int kv_splits = 1) {
+  FnaParams p;
+  long long tokens = 0;
+  if (heads_kv < 1 || head_dim < 1) return fail("fna_forward_fused: head counts and head_dim must be positive");
+  if (int rc = fused_geometry("fna_forward_fused", p, dtype == NATTEN_AMD_F16 || dtype == NATTEN_AMD_BF16, na_dim, heads_kv,
+                              head_dim, qkv_shape, kernel_size, stride, dilation, is_causal, q_tile_shape, kv_tile_shape,
+                              anchor_kv_tiles, &tokens))
+    return rc;
+  if (int rc = check_common("fna_forward_fused", q, k, v, out, lse, batch, p.seqlen_q, p.seqlen_kv, heads_q, heads_kv,
+                            head_dim))
+    return rc;
   p.q = q;
   p.k = k;
   p.v = v;
@@ -421,19 +532,10 @@ int fna_forward_fused_impl(const void* q, const void* k, const void* v, void* ou
   p.batch = batch * p.num_groups;
   p.heads_q = heads_q;
   p.heads_kv = heads_kv;
-  p.seqlen_q = prod3(qs);
-  p.seqlen_kv = prod3(ks);
   p.scale = scale;
   p.q_scale = q_scale;
   p.k_scale = k_scale;
   p.v_scale = v_scale;
-  p.fused = 1;
-  p.edge = edge;
-  // tiles laid out from the window's first key: needs every dilation group at least a KV tile wide
-  p.anchor = (anchor_kv_tiles != 0 && edge != 2) ? 1 : 0;
-  for (int a = 0; a < na_dim; ++a)
-    if (qkv_shape[a] / dilation[a] < kv_tile_shape[a]) p.anchor = 0;
-  p.tokens = int(tokens);
   if (kv_splits > 1) {
     // out and lse hold kv_splits results of the full shape, one after the other
     p.kv_splits = kv_splits;

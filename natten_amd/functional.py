@@ -128,6 +128,12 @@ def neighborhood_attention_generic(
         raise NotImplementedError(f"Unrecognized backend {backend}; natten_amd provides '{_BACKEND_FNA}'.")
 
     has_additional_attention = additional_keys is not None and additional_values is not None
+    if has_additional_attention and query.dtype == torch.float32:
+        # refused before anything is launched: the additional context goes through dense attention
+        raise NotImplementedError(
+            "natten_amd: float32 operands with additional_keys / additional_values are not supported (dense "
+            "attention, which serves the additional context, has no float32 kernel); use fp16 or bf16 operands."
+        )
     attn_kwargs = dict(attention_kwargs or {})
     attn_kwargs.pop("torch_compile", None)
 
@@ -202,6 +208,7 @@ def _use_work_queue(run_persistent_kernel: Optional[bool], is_causal, num_q_tile
     return num_q_tiles >= 2048 and num_q_tiles * kv_tiles_per_q_tile >= 65536
 
 
+@torch.compiler.assume_constant_result  # (plain Python on launch constants: not for the tracer to look into)
 def work_queue_default(batch: int, heads: int, token_layout, kernel_size, stride, dilation, is_causal, q_tile_shape,
                        kv_tile_shape) -> bool:
     """The launch kind the ops pick when `run_persistent_kernel` is None, from the problem's tile counts."""
@@ -221,6 +228,7 @@ def _work_queue_default(batch, heads, token_layout, kernel_size, stride, dilatio
     return _use_work_queue(None, is_causal, tiles, visits)
 
 
+@torch.compiler.assume_constant_result
 def kv_splits_default(batch: int, heads: int, token_layout, kernel_size, stride, dilation, is_causal, q_tile_shape,
                       kv_tile_shape) -> int:
     """How many workgroups share the KV tiles of a Q tile when `kv_splits` is None: 4 or 2 when the

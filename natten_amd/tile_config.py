@@ -64,6 +64,17 @@ def _dim_cost(L: int, k: int, s: int, causal: bool, tq: int, tk: int, anchored: 
     return visited, full
 
 
+def visited_pairs(token_layout, kernel_size, stride, dilation, is_causal, q_tile_shape, kv_tile_shape,
+                  anchored: bool = True) -> int:
+    """(query, key) pairs per head the forward kernel multiplies with these tile shapes: every Q tile
+    (padding rows included) times the whole tiles of its KV box, over all dilation groups (counted
+    with the extent of the largest group).  `anchored` as in the one-launch forward."""
+    total = 1
+    for X, k, s, d, c, tq, tk in zip(token_layout, kernel_size, stride, dilation, is_causal, q_tile_shape, kv_tile_shape):
+        total *= d * _dim_cost(_ceil_div(int(X), int(d)), int(k), int(s), bool(c), int(tq), int(tk), bool(anchored))[0]
+    return total
+
+
 def _factorisations(total: int, n: int) -> List[DimensionType]:
     if n == 1:
         return [(total,)]
@@ -76,8 +87,17 @@ def _factorisations(total: int, n: int) -> List[DimensionType]:
     return out
 
 
-@functools.lru_cache(maxsize=1024)
+@torch.compiler.assume_constant_result  # (a search over launch constants: not for the tracer to look into)
 def choose_tile_shapes(
+    token_layout: DimensionType, kernel_size: DimensionType, stride: DimensionType, dilation: DimensionType,
+    is_causal: Tuple[bool, ...], q_size: int, kv_size: int, anchored: bool = False,
+) -> Tuple[DimensionType, DimensionType]:
+    return _choose_tile_shapes(tuple(token_layout), tuple(kernel_size), tuple(stride), tuple(dilation), tuple(is_causal),
+                               int(q_size), int(kv_size), bool(anchored))
+
+
+@functools.lru_cache(maxsize=1024)
+def _choose_tile_shapes(
     token_layout: DimensionType, kernel_size: DimensionType, stride: DimensionType, dilation: DimensionType,
     is_causal: Tuple[bool, ...], q_size: int, kv_size: int, anchored: bool = False,
 ) -> Tuple[DimensionType, DimensionType]:
@@ -171,8 +191,17 @@ def _half_tile(tile: DimensionType) -> DimensionType:
     return tuple(t)
 
 
-@functools.lru_cache(maxsize=1024)
+@torch.compiler.assume_constant_result
 def choose_backward_role_tile_shapes(
+    token_layout: DimensionType, kernel_size: DimensionType, stride: DimensionType, dilation: DimensionType,
+    is_causal: Tuple[bool, ...],
+) -> Optional[Tuple[Tuple[DimensionType, DimensionType], Tuple[DimensionType, DimensionType]]]:
+    return _choose_backward_role_tile_shapes(tuple(token_layout), tuple(kernel_size), tuple(stride), tuple(dilation),
+                                             tuple(is_causal))
+
+
+@functools.lru_cache(maxsize=1024)
+def _choose_backward_role_tile_shapes(
     token_layout: DimensionType, kernel_size: DimensionType, stride: DimensionType, dilation: DimensionType,
     is_causal: Tuple[bool, ...],
 ) -> Optional[Tuple[Tuple[DimensionType, DimensionType], Tuple[DimensionType, DimensionType]]]:

@@ -51,8 +51,14 @@ def run_case(B, H, Hkv, D, shape, k, s, d, causal, dtype, q_tile=None, kv_tile=N
                                          return_lse=True, fused=False)
         assert_routes_agree("output " + tag, out1, out2, shape, d, kt_used)
         assert_routes_agree("LSE " + tag, lse1, lse2, shape, d, kt_used)
-        assert_close("anchored against aligned tiles, output " + tag, to_np(out), to_np(out1), atol=4e-3, rtol=8e-3)
-        assert_close("anchored against aligned tiles, LSE " + tag, to_np(lse), to_np(lse1), atol=4e-3, rtol=8e-3)
+        # the aligned tiling sums in another order than the anchored one above: it meets the same bar
+        # against the oracle, not some tighter one against the other route
+        if samples is None:
+            assert_close("aligned tiles, output " + tag, to_np(out1), ref_o)
+            assert_close("aligned tiles, LSE " + tag, to_np(lse1), ref_l)
+        else:
+            sampled_check(q, kk, v, out1, lse1, k, s, d, causal, max(samples // 2, 100), seed=seed + 2000,
+                          tag="aligned tiles, " + tag)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])

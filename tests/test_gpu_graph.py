@@ -37,6 +37,36 @@ def test_forward_replays_from_a_graph(shape, kernel, causal):
             assert torch.equal(out, ref_out) and torch.equal(lse, ref_lse), f"replay {i} differs from the eager call"
 
 
+def test_static_entry_point_replays_from_a_graph():
+    # the entry point that allocates nothing, captured after one eager call on the device (which
+    # resolves the address of the library's static queue array outside any capture)
+    from natten_amd import _lib
+
+    shape, kernel, stride, dil, causal, qt, kt = (16, 32), (7, 5), (2, 1), (1, 2), (False, True), (8, 16), (8, 8)
+    gen = torch.Generator().manual_seed(5)
+    mk = lambda: torch.randn((2, *shape, 2, 64), generator=gen).to(torch.float16).cuda()
+    q, k, v = mk(), mk(), mk()
+    out = torch.empty_like(q)
+    lse = torch.empty(q.shape[:-1], dtype=torch.float32, device=q.device)
+    fn = lambda: _lib.fna_forward_fused_static(q, k, v, out, lse, kernel, stride, dil, causal, 0.125, qt, kt)
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        fn()  # eager warm-up: first call on this device
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        fn()
+    for i in range(3):
+        for t in (q, k, v):
+            t.copy_(mk())
+        out.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        ref_out, ref_lse = _lib.fna_forward_fused(q, k, v, kernel, stride, dil, causal, 0.125, qt, kt)  # eager work in between
+        torch.cuda.synchronize()
+        assert torch.equal(out, ref_out) and torch.equal(lse, ref_lse), f"replay {i} differs from the eager call"
+
+
 def test_split_forward_replays_from_a_graph():
     # a small grid with long windows: the op splits the KV tiles of every Q tile over several
     # workgroups and merges the partial results -- two launches and two allocations inside the capture

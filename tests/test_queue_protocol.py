@@ -1,0 +1,258 @@
+"""The work-queue launch protocol, walked through on the CPU.
+
+Two models, both exhaustive over every interleaving of a small launch:
+
+* the counters in device memory (natten_amd/csrc/work_queue.hpp, compiled here with g++ so that the
+  model runs the kernels' own decision functions): every launch position is handed out exactly once,
+  every workgroup ends after at most `nq * per_queue + nq` increments, nobody touches a counter once
+  the last workgroup out has begun to store zeros, and the block is all zero when the launch ends;
+* the hand-over of a position from thread 0 to the other waves of its workgroup through the two LDS
+  slots of fna_queue_loop (natten_amd/csrc/fna_fwd.hpp): every wave reads, for every tile, the value
+  thread 0 wrote for that tile.
+
+Each model is also run on a deliberately broken protocol, which it must reject.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+
+import pytest
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+@pytest.fixture(scope="module")
+def wq(tmp_path_factory):
+    out = tmp_path_factory.mktemp("queue_model") / "libqueue_model.so"
+    cmd = ["g++", "-O1", "-std=c++17", "-shared", "-fPIC", os.path.join(HERE, "queue_model.cpp"), "-o", str(out)]
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    assert proc.returncode == 0, proc.stdout
+    lib = ctypes.CDLL(str(out))
+    lib.wq_position.argtypes = [ctypes.c_int, ctypes.POINTER(ctypes.c_int), ctypes.c_uint32, ctypes.c_int, ctypes.c_int]
+    lib.wq_last_one_out.argtypes = [ctypes.c_uint32, ctypes.c_uint32]
+    lib.wq_max_increments.restype = ctypes.c_longlong
+    return lib
+
+
+class Violation(Exception):
+    pass
+
+
+# ---------------------------------------------------------------------------------------------
+# Model 1: the counters.  A workgroup is a small state machine; each of its steps is one atomic
+# operation on the shared block (an atomicAdd that returns the old value, or a plain store).
+# ---------------------------------------------------------------------------------------------
+TAKE, DONE, RESET, END = 0, 1, 2, 3
+
+
+def explore_counters(lib, nq, per_queue, workgroups, start=None, last_out=None, position=None):
+    """Walks every interleaving.  start: initial counter values (default zeros).  last_out /
+    position: replacements for the library's decisions (the broken protocols)."""
+    stride = lib.wq_stride()
+    last_out = last_out or (lambda left, n: bool(lib.wq_last_one_out(left, n)))
+
+    def lib_position(home, victim, ticket):
+        v = ctypes.c_int(victim)
+        pos = lib.wq_position(home, ctypes.byref(v), ticket, per_queue, nq)
+        return pos, v.value
+
+    position = position or lib_position
+    bound = lib.wq_max_increments(per_queue, nq)
+    total = nq * per_queue
+    # state: (counters tuple, done word, handed-out bitmask, per workgroup (pc, victim, increments, reset index))
+    init = (tuple(start or [0] * nq), 0, 0, tuple((TAKE, 0, 0, 0) for _ in range(workgroups)))
+    seen = {init}
+    stack = [init]
+    terminals = 0
+    while stack:
+        counters, done, handed, wgs = stack.pop()
+        # the last workgroup out is storing zeros, or has finished doing so
+        resetting = any(pc == RESET or (pc == END and ridx > 0) for pc, _, _, ridx in wgs)
+        live = [w for w, (pc, *_) in enumerate(wgs) if pc != END]
+        if not live:
+            terminals += 1
+            if handed != (1 << total) - 1:
+                raise Violation(f"positions handed out: {handed:b}, expected all {total}")
+            if any(counters) or done:
+                raise Violation(f"block not zero at exit: {counters} done={done}")
+            continue
+        for w in live:
+            pc, victim, incs, ridx = wgs[w]
+            home = w % nq
+            c, d, h = list(counters), done, handed
+            if pc == TAKE:
+                if resetting:
+                    raise Violation("a counter is incremented while the last workgroup out stores zeros")
+                q = lib.wq_counter_word(home, victim, nq) // stride
+                ticket = c[q]
+                c[q] += 1
+                incs += 1
+                if incs > bound:
+                    raise Violation(f"workgroup {w} made {incs} increments, bound {bound}")
+                pos, victim = position(home, victim, ticket)
+                if pos >= 0:
+                    if not 0 <= pos < total:
+                        raise Violation(f"position {pos} outside the launch")
+                    if h >> pos & 1:
+                        raise Violation(f"position {pos} handed out twice")
+                    h |= 1 << pos
+                elif victim == nq:
+                    pc = DONE
+            elif pc == DONE:
+                if resetting:
+                    raise Violation("the done word is incremented while the last workgroup out stores zeros")
+                left = d
+                d += 1
+                if last_out(left, workgroups):
+                    pc, ridx = RESET, 0
+                else:
+                    pc = END
+            else:  # RESET: nq counter stores, then the done word
+                if ridx < nq:
+                    c[ridx] = 0
+                    ridx += 1
+                else:
+                    d = 0
+                    pc = END
+            nxt = (tuple(c), d, h, wgs[:w] + ((pc, victim, incs, ridx),) + wgs[w + 1:])
+            if nxt not in seen:
+                seen.add(nxt)
+                stack.append(nxt)
+    return len(seen), terminals
+
+
+def test_layout_constants(wq):
+    nq, stride = wq.wq_num_xcd(), wq.wq_stride()
+    assert wq.wq_words() == nq * stride and stride * 4 == 64  # one counter per 64-byte line
+    assert 0 < wq.wq_done_word() < stride  # shares the first queue's line, not its counter
+    words = {wq.wq_counter_word(h, v, nq) for h in range(nq) for v in range(nq)}
+    assert words == {x * stride for x in range(nq)}
+    for h in range(nq):  # a workgroup visits every queue once, its own first
+        order = [wq.wq_counter_word(h, v, nq) // stride for v in range(nq)]
+        assert order[0] == h and sorted(order) == list(range(nq))
+
+
+@pytest.mark.parametrize("nq,per_queue,workgroups", [
+    (1, 3, 3), (2, 1, 2), (2, 2, 3), (2, 3, 2), (3, 1, 3), (3, 2, 3), (2, 0, 2), (4, 1, 2), (2, 2, 4),
+])
+def test_every_interleaving_small(wq, nq, per_queue, workgroups):
+    states, terminals = explore_counters(wq, nq, per_queue, workgroups)
+    assert terminals >= 1 and states > 0
+
+
+def test_every_interleaving_eight_queues(wq):
+    # the shipped queue count, two resident workgroups (homes 0 and 1) and three
+    explore_counters(wq, wq.wq_num_xcd(), 1, 2)
+    explore_counters(wq, wq.wq_num_xcd(), 2, 2)
+    explore_counters(wq, wq.wq_num_xcd(), 1, 3)
+
+
+def test_more_workgroups_than_positions(wq):
+    explore_counters(wq, 2, 1, 4)
+
+
+def test_model_rejects_reset_by_first_out(wq):
+    # zeros stored by the first workgroup to leave instead of the last: others still increment
+    with pytest.raises(Violation):
+        explore_counters(wq, 2, 2, 3, last_out=lambda left, n: left == 0)
+
+
+def test_model_rejects_returning_to_a_retired_queue(wq):
+    # a workgroup that does not move on from an empty queue never ends: the increment bound catches it
+    def stuck(home, victim, ticket):
+        return (int(ticket) * 2 + (home + victim) % 2, victim) if ticket < 1 else (-1, victim)
+
+    with pytest.raises(Violation):
+        explore_counters(wq, 2, 1, 2, position=stuck)
+
+
+def test_model_rejects_counters_that_do_not_start_at_zero(wq):
+    # what `run_persistent = 2` asks its caller to vouch for: a stale count skips positions
+    with pytest.raises(Violation):
+        explore_counters(wq, 2, 2, 2, start=[1, 0])
+
+
+# ---------------------------------------------------------------------------------------------
+# Model 2: the hand-over inside a workgroup.  Every wave runs the loop of fna_queue_loop:
+#   barrier; read s_pos[i]; leave if it is negative; the tile (some barriers; thread 0, in wave 0,
+#   writes s_pos[i ^ 1] after the last of them -- a tile that returns at once has none);  i ^= 1.
+# A step is a barrier arrival, an LDS read or an LDS write; a barrier releases when every wave has
+# arrived.  Waves are otherwise free to run at any relative speed.
+# ---------------------------------------------------------------------------------------------
+def wave_program(wave, tiles, barriers_per_tile, write_at):
+    ops = [("write", 0)] if wave == 0 else []
+    for n, pid in enumerate(tiles):
+        ops += [("bar",), ("read", n)]
+        if pid < 0:
+            break
+        if wave == 0 and write_at == "top":
+            ops.append(("write", n + 1))
+        ops += [("bar",)] * barriers_per_tile[n % len(barriers_per_tile)]
+        if wave == 0 and write_at == "end":
+            ops.append(("write", n + 1))
+    return ops
+
+
+def explore_handover(waves, tiles, slots=2, barriers_per_tile=(2, 0, 1), write_at="end"):
+    """tiles: the positions thread 0 obtains, in order, ending with a negative one."""
+    progs = [wave_program(w, tiles, barriers_per_tile, write_at) for w in range(waves)]
+    init = ((None,) * slots, (0,) * waves, frozenset())
+    seen = {init}
+    stack = [init]
+    while stack:
+        lds, pcs, waiting = stack.pop()
+        runnable = [w for w in range(waves) if pcs[w] < len(progs[w]) and w not in waiting]
+        if not runnable:
+            if waiting:
+                raise Violation("deadlock: some waves wait at a barrier the others never reach")
+            continue
+        for w in runnable:
+            op = progs[w][pcs[w]]
+            l, pc, wt = list(lds), list(pcs), set(waiting)
+            if op[0] == "bar":
+                wt.add(w)
+                if len(wt) == sum(1 for x in range(waves) if pcs[x] < len(progs[x])):
+                    for x in wt:
+                        pc[x] += 1
+                    wt = set()
+            elif op[0] == "read":
+                n = op[1]
+                got = l[n % slots]
+                if got != tiles[n]:
+                    raise Violation(f"wave {w} read {got} for its tile {n}; thread 0 wrote {tiles[n]} for it")
+                pc[w] += 1
+            else:
+                l[op[1] % slots] = tiles[op[1]]
+                pc[w] += 1
+            nxt = (tuple(l), tuple(pc), frozenset(wt))
+            if nxt not in seen:
+                seen.add(nxt)
+                stack.append(nxt)
+    return len(seen)
+
+
+TILES = [5, 9, 2, 7, -1]
+
+
+@pytest.mark.parametrize("waves", [2, 4])
+@pytest.mark.parametrize("barriers", [(2,), (0,), (2, 0, 1), (0, 3)])
+def test_handover_two_slots(waves, barriers):
+    # the shipped form: thread 0 stores the next position after the tile's last barrier
+    assert explore_handover(waves, TILES, slots=2, barriers_per_tile=barriers, write_at="end") > 0
+    # ... and the form that stores it right after reading the current one
+    assert explore_handover(waves, TILES, slots=2, barriers_per_tile=barriers, write_at="top") > 0
+
+
+def test_handover_single_tile_and_empty_queue():
+    explore_handover(4, [-1])
+    explore_handover(4, [3, -1])
+
+
+@pytest.mark.parametrize("write_at", ["end", "top"])
+def test_model_rejects_one_slot(write_at):
+    # with a single slot thread 0 may overwrite a position a slower wave has not read yet
+    with pytest.raises(Violation):
+        explore_handover(2, TILES, slots=1, barriers_per_tile=(0,), write_at=write_at)
