@@ -35,7 +35,8 @@ constexpr float kFp8LazyRescaleLog2 = 2.0f; // so that 2^6 * 2^2 = 256 stays bel
 // LDS tile: 64 rows of D bytes, 16-byte chunks XOR-swizzled by (row / rows-per-256-bytes); the
 // rows of a V tile are stored in the order the P fragment holds its keys (see v_key_of_lds_row).
 // `pid`: the launch position (the workgroup id of a launch with one workgroup per Q tile).
-template <bool E5M2, int D, int NWAVES, typename Hook>
+// NOMASK: fully block-sparse launch (see fna_fwd_tile): no mask code, tables or per-wave windows.
+template <bool E5M2, int D, int NWAVES, bool NOMASK = false, typename Hook>
 static __device__ __forceinline__ void fna_fwd_fp8_tile(const FnaParams& p, const uint32_t pid, Hook&& before_stores) {
   constexpr int KVT = 64;
   constexpr int NT = NWAVES * 64;
@@ -61,7 +62,7 @@ static __device__ __forceinline__ void fna_fwd_fp8_tile(const FnaParams& p, cons
   __shared__ __attribute__((aligned(1024))) char sV0[TILE_BYTES];
   __shared__ __attribute__((aligned(1024))) char sK1[TILE_BYTES];
   __shared__ __attribute__((aligned(1024))) char sV1[TILE_BYTES];
-  __shared__ __attribute__((aligned(16))) uint32_t sTab[KVT];
+  __shared__ __attribute__((aligned(16))) uint32_t sTab[NOMASK ? 1 : KVT];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -134,7 +135,7 @@ static __device__ __forceinline__ void fna_fwd_fp8_tile(const FnaParams& p, cons
   // dimension: a KV tile outside the union is skipped by this wave, one inside the
   // intersection needs no mask.
   int wave_lo[3], wave_hi[3], wave_full_lo[3], wave_full_hi[3];
-  {
+  if constexpr (!NOMASK) {
     const int i0 = wave * 32, i1 = i0 + 31;
     const int lg2 = p.q_tile_lg[2], lg12 = p.q_tile_lg[1] + p.q_tile_lg[2];
     int f[3], l[3];
@@ -169,7 +170,7 @@ static __device__ __forceinline__ void fna_fwd_fp8_tile(const FnaParams& p, cons
   }
 
   // in-tile coordinates of every KV position, packed in 10-bit fields
-  for (int i = tid; i < KVT; i += NT) {
+  for (int i = tid; i < (NOMASK ? 0 : KVT); i += NT) {
     const int t0 = i & (p.kv_tile[0] - 1);
     const int r1 = i >> p.kv_tile_lg[0];
     const int t1 = r1 & (p.kv_tile[1] - 1);
@@ -246,8 +247,10 @@ static __device__ __forceinline__ void fna_fwd_fp8_tile(const FnaParams& p, cons
     for (int a = 0; a < 3; ++a) {
       const int org = box_org[a] + (itc[a] << p.kv_tile_lg[a]);
       const int end = org + p.kv_tile[a];
-      t.full = t.full && (org >= wave_full_lo[a]) && (end <= wave_full_hi[a]);  // never when end > extent
-      t.skip = t.skip || (end <= wave_lo[a]) || (org >= wave_hi[a]);
+      if constexpr (!NOMASK) {
+        t.full = t.full && (org >= wave_full_lo[a]) && (end <= wave_full_hi[a]);  // never when end > extent
+        t.skip = t.skip || (end <= wave_lo[a]) || (org >= wave_hi[a]);
+      }
       // a tile that would reach past the group is moved back to end at the group's last position
       t.origin[a] = p.anchor ? na_min(org, extent[a] - p.kv_tile[a]) : org;
     }
@@ -294,8 +297,10 @@ static __device__ __forceinline__ void fna_fwd_fp8_tile(const FnaParams& p, cons
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
       const int c = q_first[a] + off[a];
-      wst[a] = na_window_start(c, p.ksize[a], p.stride[a], p.d_stride[a], extent[a], p.causal[a] != 0);
-      wen[a] = na_window_end(c, wst[a], p.ksize[a], extent[a], p.causal[a] != 0);
+      if constexpr (!NOMASK) {
+        wst[a] = na_window_start(c, p.ksize[a], p.stride[a], p.d_stride[a], extent[a], p.causal[a] != 0);
+        wen[a] = na_window_end(c, wst[a], p.ksize[a], extent[a], p.causal[a] != 0);
+      }
       if (p.fused) {
         valid = valid && (c < extent[a]);
         row += c * tok_step[a];
@@ -377,6 +382,7 @@ static __device__ __forceinline__ void fna_fwd_fp8_tile(const FnaParams& p, cons
   };
 
   auto apply_mask = [&](f32x16_t (&S)[NSB], const int (&origin)[3]) {
+    if constexpr (NOMASK) return;
     uint32_t addc = 0, subc = 0;
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
@@ -524,10 +530,11 @@ static __device__ __forceinline__ void fna_fwd_fp8_tile(const FnaParams& p, cons
       acc[t] = mfma8(vf[t], pf, acc[t], FmtIn{}, FmtP{});
       constexpr int NV = NSB * 16;
       constexpr int e_lo = (t * NV) / N_PV, e_hi = ((t + 1) * NV) / N_PV;
+      static_assert((e_hi - e_lo) % 4 == 0, "row maxima are taken two logits per instruction, on two chains");
 #pragma unroll
-      for (int e = e_lo; e < e_hi; ++e) {
-        if (e % 2 == 0) mx0 = fmaxf(mx0, S_nxt[e / 16][e % 16]);
-        else mx1 = fmaxf(mx1, S_nxt[e / 16][e % 16]);
+      for (int e = e_lo; e < e_hi; e += 4) {
+        mx0 = fmaxf(fmaxf(mx0, S_nxt[e / 16][e % 16]), S_nxt[(e + 1) / 16][(e + 1) % 16]);
+        mx1 = fmaxf(fmaxf(mx1, S_nxt[(e + 2) / 16][(e + 2) % 16]), S_nxt[(e + 3) / 16][(e + 3) % 16]);
       }
       pin(mx0);
       pin(mx1);
@@ -573,19 +580,19 @@ static __device__ __forceinline__ void fna_fwd_fp8_tile(const FnaParams& p, cons
   }
 }
 
-template <bool E5M2, int D, int NWAVES>
+template <bool E5M2, int D, int NWAVES, bool NOMASK = false>
 __global__ void __launch_bounds__(NWAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 fna_fwd_fp8_kernel(const FnaParams p) {
-  fna_fwd_fp8_tile<E5M2, D, NWAVES>(p, blockIdx.x, []() {});
+  fna_fwd_fp8_tile<E5M2, D, NWAVES, NOMASK>(p, blockIdx.x, []() {});
 }
 
 // Work-queue form (see fna_fwd_queue_kernel).
-template <bool E5M2, int D, int NWAVES>
+template <bool E5M2, int D, int NWAVES, bool NOMASK = false>
 __global__ void __launch_bounds__(NWAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 fna_fwd_fp8_queue_kernel(const FnaParams p, uint32_t* __restrict__ queues, const int per_xcd) {
   FnaKernargPtr args = fna_kernarg_params();
   fna_queue_loop(queues, per_xcd, [&](int pid, auto& fetch) __attribute__((always_inline)) {
-    fna_fwd_fp8_tile<E5M2, D, NWAVES>(fna_params_for_this_tile(args), uint32_t(pid), fetch);
+    fna_fwd_fp8_tile<E5M2, D, NWAVES, NOMASK>(fna_params_for_this_tile(args), uint32_t(pid), fetch);
   });
   (void)p;
 }

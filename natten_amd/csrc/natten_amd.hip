@@ -147,8 +147,8 @@ bool fully_block_sparse(const FnaParams& p) {
   return true;
 }
 
-template <bool E5M2, int D>
-int launch_fna_fp8(const FnaParams& p, hipStream_t stream, WorkQueue queues) {
+template <bool E5M2, int D, bool NOMASK>
+int launch_fna_fp8_instance(const FnaParams& p, hipStream_t stream, WorkQueue queues) {
   constexpr int QT = 128;
   if (!fna_tiles_are_powers_of_two(p)) return fail("fna_forward: tile extents must be powers of two");
   if ((p.seqlen_q + QT - 1) / QT != p.num_q_tiles) return fail("fna_forward: internal tile count mismatch");
@@ -157,12 +157,18 @@ int launch_fna_fp8(const FnaParams& p, hipStream_t stream, WorkQueue queues) {
   if (queues.counters != nullptr) {
     const long long resident = resident_workgroups();
     if (queues.clear_first) hipLaunchKernelGGL(fna_queue_clear_kernel, dim3(1), dim3(kQueueWords), 0, stream, queues.counters);
-    hipLaunchKernelGGL((fna_fwd_fp8_queue_kernel<E5M2, D, 4>), dim3((unsigned)(wgs < resident ? wgs : resident)), dim3(256), 0,
-                       stream, p, queues.counters, int(wgs / kNumXcd));
+    hipLaunchKernelGGL((fna_fwd_fp8_queue_kernel<E5M2, D, 4, NOMASK>), dim3((unsigned)(wgs < resident ? wgs : resident)),
+                       dim3(256), 0, stream, p, queues.counters, int(wgs / kNumXcd));
     return check_launch("fna_forward (work queue)");
   }
-  hipLaunchKernelGGL((fna_fwd_fp8_kernel<E5M2, D, 4>), dim3((unsigned)wgs), dim3(256), 0, stream, p);
+  hipLaunchKernelGGL((fna_fwd_fp8_kernel<E5M2, D, 4, NOMASK>), dim3((unsigned)wgs), dim3(256), 0, stream, p);
   return check_launch("fna_forward");
+}
+
+template <bool E5M2, int D>
+int launch_fna_fp8(const FnaParams& p, hipStream_t stream, WorkQueue queues) {
+  if (fully_block_sparse(p)) return launch_fna_fp8_instance<E5M2, D, true>(p, stream, queues);
+  return launch_fna_fp8_instance<E5M2, D, false>(p, stream, queues);
 }
 
 template <typename T, int D>
