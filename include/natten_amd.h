@@ -126,12 +126,12 @@ int natten_amd_fna_forward(const void* q, const void* k, const void* v, void* ou
  *   - every qkv_shape[a] a multiple of dilation[a] * kv_tile_shape[a] (no KV tile reaches past
  *     its dilation group): every dtype but float32 and every tile pair; with anchor_kv_tiles == 0
  *     the results are bit-identical to the permuted path with the same tile shapes;
- *   - any other extent with fp16 / bf16 operands: a tile that would reach past its dilation group
- *     is gathered from one tile extent before the group's end and its leading keys, which the tile
+ *   - any other extent whose dilation groups are all at least one KV tile wide in every dimension
+ *     (fp16 / bf16 and 8-bit float operands): a tile that would reach past its dilation group is
+ *     gathered from one tile extent before the group's end and its leading keys, which the tile
  *     before it delivered, are masked (sums then run in another order than on the permuted path);
- *     when some dilation group is narrower than the KV tile in a dimension, only tiles of 128 x 64
- *     tokens are taken (the instance that clamps its gathers);
- *   - 8-bit float operands take multiples only.
+ *   - a dilation group narrower than the KV tile in some dimension: fp16 / bf16 operands with tiles
+ *     of 128 x 64 tokens only (the instance that clamps its gathers).
  * Anything else returns an error that says which rule was missed, and the caller uses the
  * permuted path.  A KV tile must span less than 2^31 bytes of the input.  dtype, tiles, head_dim,
  * scales, run_persistent and workspace as in natten_amd_fna_forward.
@@ -319,9 +319,14 @@ int natten_amd_fna_backward(const void* q, const void* k, const void* v, const v
  * k, v, dk, dv [batch, *qkv_shape, heads_kv, head_dim], lse and delta head-major
  * [batch, heads_q, prod(qkv_shape)].  The kernels gather and scatter the rows of their tiles
  * themselves, which replaces the six token permutes and three unpermutes of the reference's
- * backward driver (src/natten/backends/blackwell_fna.py:205-297); results are bit-identical to
- * them.  Every extent must be a multiple of dilation x tile for both tile shapes (an error
- * otherwise: use natten_amd_fna_backward on permuted operands).
+ * backward driver (src/natten/backends/blackwell_fna.py:205-297).  Where every extent is a
+ * multiple of dilation x tile for both tile shapes the results are bit-identical to that
+ * sequence.  Other extents are taken as long as every dilation group is at least one tile wide
+ * (both tile shapes) in every dimension: rows of a tile past the end of its dilation group are
+ * computed on a clamped copy and not stored, a streamed tile that would reach past the group is
+ * gathered from one tile extent before its end and its leading rows, which the tile before it
+ * delivered, take no part (sums then run in another order than on permuted operands).  Narrower
+ * groups return an error: use natten_amd_fna_backward on permuted operands.
  *
  * roles: 3 makes both launches; 1 only the one that writes dq, 2 only the one that writes dk and
  * dv (the other results are left untouched).  With no permuted layout to share, the two launches

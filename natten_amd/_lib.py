@@ -310,16 +310,18 @@ def fused_layout_supported(qkv_shape, dilation, kv_tile_shape, row_bytes: int = 
     """Whether fna_forward_fused accepts this problem.  Always: (given `row_bytes` = heads_kv *
     head_dim * 2) a KV tile spans less than 2^31 bytes of the input.  When every extent is a multiple
     of dilation x KV tile no KV tile reaches past its dilation group.  Otherwise (`q_tile_shape`
-    and `dtype` given) the operands must be fp16 / bf16, and if some dilation group is narrower than
-    the KV tile in a dimension the tiles must be 128 x 64 tokens (the one instance that clamps)."""
+    and `dtype` given) every dilation group must be at least a KV tile wide in every dimension, or
+    the operands fp16 / bf16 with tiles of 128 x 64 tokens (the one instance that clamps)."""
     if not _tile_span_fits(qkv_shape, dilation, kv_tile_shape, row_bytes):
         return False
     if all(X % (d * t) == 0 for X, d, t in zip(qkv_shape, dilation, kv_tile_shape)):
         return True
-    if q_tile_shape is None or dtype not in (torch.float16, torch.bfloat16):
+    if q_tile_shape is None or dtype is None:
         return False
     if all(X // d >= t for X, d, t in zip(qkv_shape, dilation, kv_tile_shape)):
-        return True
+        return True  # (every kernel moves a tile that would reach past its group back to the group's end)
+    if dtype not in (torch.float16, torch.bfloat16):
+        return False
     q_tokens = kv_tokens = 1
     for tq, tk in zip(q_tile_shape, kv_tile_shape):
         q_tokens *= tq
@@ -553,10 +555,11 @@ def fna_backward(
 
 
 def backward_fused_layout_supported(token_layout, dilation, q_tile_shape, kv_tile_shape, row_bytes: int = 0) -> bool:
-    """Whether the backward kernels can work on the original tensors: no padding on either side,
-    and (given `row_bytes` = heads_q * head_dim * 2) tiles that span less than 2^31 bytes."""
+    """Whether the backward kernels can work on the original tensors: every dilation group at least
+    one tile wide (either side's) in every dimension, and (given `row_bytes` = heads_q * head_dim * 2)
+    tiles that span less than 2^31 bytes."""
     return (
-        all(X % (d * tq) == 0 and X % (d * tk) == 0
+        all(X // d >= tq and X // d >= tk
             for X, d, tq, tk in zip(token_layout, dilation, q_tile_shape, kv_tile_shape))
         and _tile_span_fits(token_layout, dilation, q_tile_shape, row_bytes)
         and _tile_span_fits(token_layout, dilation, kv_tile_shape, row_bytes)

@@ -56,9 +56,14 @@ struct FnaBwdParams {
   float scale;
   // Operand layout.  fused == 0: token-permuted sequences as described above.  fused == 1: the
   // original tensors [batch, X0, X1, X2, heads, D] (lse / delta [batch, heads, X0 * X1 * X2]);
-  // the kernel gathers and scatters the rows of a tile itself.  Every extent must then be a
-  // multiple of dilation x tile for both tile shapes (no padding rows exist).
+  // the kernel gathers and scatters the rows of a tile itself.
   int fused;
+  // fused == 1 only: some extent is not a multiple of dilation x tile, so tiles may reach past a
+  // dilation group (every group is at least a tile wide in every dimension).  Rows of the stationary
+  // tile past the group's end are computed on a clamped copy and not stored; a streamed tile that
+  // would reach past it is gathered from one tile extent before the end, and its leading rows,
+  // which the tile before it delivered, take no part (as in the forward kernel).
+  int edge;
   int tok_stride[3];  // tokens per unit step of an original coordinate: X1*X2, X2, 1
   int tokens;         // X0 * X1 * X2
   // Sequence-packed dense attention (VARLEN instances only; null otherwise).  `batch` sequences
@@ -276,8 +281,17 @@ fna_bwd_kernel(const FnaBwdParams p) {
   a_off[2] = r_in / (a_tile[0] * a_tile[1]);
   // Row of the tensors / index into lse and delta: position in the permuted sequence, or the
   // token of the lane's coordinate in the original layout.
-  const int a_tok = group_tok + (a_first[0] + a_off[0]) * tok_step[0] + (a_first[1] + a_off[1]) * tok_step[1] +
-                    (a_first[2] + a_off[2]) * tok_step[2];
+  // (original layout: a row past the end of its dilation group works on the group's last row and stores nothing)
+  int a_crd[3];
+  bool a_valid = true;
+#pragma unroll
+  for (int a = 0; a < 3; ++a) {
+    const int c = a_first[a] + a_off[a];
+    const int e = KV_STATIONARY ? extent[a] : q_extent[a];
+    a_valid = a_valid && (c < e || !p.fused);
+    a_crd[a] = p.fused ? na_min(c, e - 1) : c;
+  }
+  const int a_tok = group_tok + a_crd[0] * tok_step[0] + a_crd[1] * tok_step[1] + a_crd[2] * tok_step[2];
   const int64_t batch_row0 = p.fused ? int64_t(bg / p.num_groups) * p.tokens : 0;  // first row of the batch entry (original layout)
   const int64_t a_row = p.fused ? batch_row0 + a_tok : (seq_row_a + int64_t(at) * AT + r_in);
   const int64_t a_stride = int64_t(heads_a) * D;
@@ -286,6 +300,7 @@ fna_bwd_kernel(const FnaBwdParams p) {
 
   typedef T tx4 __attribute__((ext_vector_type(4)));
   auto store_rows = [&](void* dst, const f32x16_t (&acc)[DB], float mul) {
+    if (!a_valid) return;
     T* orow = reinterpret_cast<T*>(dst) + a_row * a_stride + int64_t(head_a) * D;
 #pragma unroll
     for (int db = 0; db < DB; ++db)
@@ -339,7 +354,7 @@ fna_bwd_kernel(const FnaBwdParams p) {
   if constexpr (!KV_STATIONARY) {
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
-      const int c = a_first[a] + a_off[a];
+      const int c = a_crd[a];
       wst[a] = na_window_start(c, ksz[a], p.stride[a], extent[a], p.causal[a] != 0);
       wen[a] = na_window_end(c, wst[a], ksz[a], extent[a], p.causal[a] != 0);
     }
@@ -379,7 +394,8 @@ fna_bwd_kernel(const FnaBwdParams p) {
   }
 
   struct Tile {
-    int origin[3];  // coordinate of the tile's first token
+    int origin[3];  // coordinate of the tile's first token (a tile moved back from the group's edge: of the first one gathered)
+    int lead[3];    // ... whose first lead[a] positions along dimension a belong to the tile before it
     int row0;       // its first row in the streamed side's permuted sequence
     int head_b;
   };
@@ -431,6 +447,12 @@ fna_bwd_kernel(const FnaBwdParams p) {
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
       t.origin[a] = wc[a] * b_sub[a];
+      t.lead[a] = 0;
+      if (p.edge) {
+        const int moved = na_min(t.origin[a], (KV_STATIONARY ? q_extent[a] : extent[a]) - b_sub[a]);
+        t.lead[a] = t.origin[a] - moved;
+        t.origin[a] = moved;
+      }
       const bool split = (a == split_dim);
       half |= split ? (wc[a] & 1) : 0;
       cc[a] = split ? (wc[a] >> 1) : wc[a];
@@ -464,7 +486,7 @@ fna_bwd_kernel(const FnaBwdParams p) {
 #pragma unroll
         for (int a = 0; a < 3; ++a) {
           const int qc = t.origin[a] + qo[a];
-          valid = valid && (qc < q_extent[a]);
+          valid = valid && (qc < q_extent[a]) && (qo[a] >= t.lead[a]);
           const int st = na_window_start(qc, ksz[a], p.stride[a], extent[a], p.causal[a] != 0);
           const int en = na_window_end(qc, st, ksz[a], extent[a], p.causal[a] != 0);
           const int lo = na_min(na_max(st - a_first[a], 0), a_tile[a]);
@@ -793,7 +815,7 @@ fna_bwd_kernel(const FnaBwdParams p) {
       } else {
         wait_vmcnt<0>();
       }
-      __syncthreads();
+      workgroup_sync();
       const int s2_ahead = s2 == 0 ? 2 : s2 - 1;  // (it + 2) % 3
       auto ahead = [&]() __attribute__((always_inline)) {
         if (it + 2 < n_iter) {
@@ -816,7 +838,7 @@ fna_bwd_kernel(const FnaBwdParams p) {
       s2 = s2 == 2 ? 0 : s2 + 1;
     }
     wait_vmcnt<0>();
-    __syncthreads();  // stages and probability buffers are free for the next pass
+    workgroup_sync();  // stages and probability buffers are free for the next pass
   };
 
   // ---- pipeline: tile `it` is multiplied while tiles it+1 .. it+NS-1 are in flight ----------------
@@ -829,12 +851,16 @@ fna_bwd_kernel(const FnaBwdParams p) {
     // origin of the tile being multiplied); og<k> = origin of tile it + k
     constexpr bool NEED_ORIGIN = MASKED && !KV_STATIONARY;
     int og0[3] = {0, 0, 0}, og1[3] = {0, 0, 0}, og2[3] = {0, 0, 0};
+    int ld0[3] = {0, 0, 0}, ld1[3] = {0, 0, 0}, ld2[3] = {0, 0, 0};  // ... and their leads
     if (0 < n_iter && NS > 1) {
       const Tile t = next_tile(std::integral_constant<bool, !MASKED>{}, 1 < n_iter);
       issue(t, 0, MASKED);
       if constexpr (NEED_ORIGIN) {
 #pragma unroll
-        for (int a = 0; a < 3; ++a) og0[a] = t.origin[a];
+        for (int a = 0; a < 3; ++a) {
+          og0[a] = t.origin[a];
+          ld0[a] = t.lead[a];
+        }
       }
     }
     if (1 < n_iter && NS > 2) {
@@ -842,7 +868,10 @@ fna_bwd_kernel(const FnaBwdParams p) {
       issue(t, 1, MASKED);
       if constexpr (NEED_ORIGIN) {
 #pragma unroll
-        for (int a = 0; a < 3; ++a) og1[a] = t.origin[a];
+        for (int a = 0; a < 3; ++a) {
+          og1[a] = t.origin[a];
+          ld1[a] = t.lead[a];
+        }
       }
     }
 
@@ -857,13 +886,16 @@ fna_bwd_kernel(const FnaBwdParams p) {
       } else {
         wait_vmcnt<0>();
       }
-      __syncthreads();  // tile `it` and its tables are in LDS; everyone is done with the stage of tile it - 1
+      workgroup_sync();  // tile `it` and its tables are in LDS; everyone is done with the stage of tile it - 1
       if (it + NS - 1 < n_iter) {
         const Tile t = next_tile(std::integral_constant<bool, !MASKED>{}, it + NS < n_iter);
         issue(t, (it + NS - 1) % NS, MASKED);
         if constexpr (NEED_ORIGIN) {
 #pragma unroll
-          for (int a = 0; a < 3; ++a) (NS == 3 ? og2[a] : og1[a]) = t.origin[a];
+          for (int a = 0; a < 3; ++a) {
+            (NS == 3 ? og2[a] : og1[a]) = t.origin[a];
+            (NS == 3 ? ld2[a] : ld1[a]) = t.lead[a];
+          }
         }
       }
 
@@ -871,7 +903,7 @@ fna_bwd_kernel(const FnaBwdParams p) {
       if constexpr (NEED_ORIGIN) {
 #pragma unroll
         for (int a = 0; a < 3; ++a) {
-          const int lo = na_min(na_max(wst[a] - og0[a], 0), b_sub[a]);
+          const int lo = na_min(na_max(wst[a] - og0[a], ld0[a]), b_sub[a]);
           const int hi = na_min(na_max(wen[a] - og0[a], 0), b_sub[a]);
           addc |= uint32_t(512 - lo) << (10 * a);
           subc |= uint32_t(511 + hi) << (10 * a);
@@ -883,11 +915,13 @@ fna_bwd_kernel(const FnaBwdParams p) {
         for (int a = 0; a < 3; ++a) {
           og0[a] = og1[a];
           og1[a] = og2[a];
+          ld0[a] = ld1[a];
+          ld1[a] = ld2[a];
         }
       }
     }
     wait_vmcnt<0>();
-    __syncthreads();  // the stages are free for the next pass
+    workgroup_sync();  // the stages are free for the next pass
   };
   const int heads_walked = KV_STATIONARY ? rep : 1;
   if constexpr (PAIR) {

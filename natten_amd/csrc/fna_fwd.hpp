@@ -244,6 +244,18 @@ static __device__ __forceinline__ void wait_vmcnt() {
   __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 0xF) | ((N >> 4) << 14));
 }
 
+// Workgroup barrier that every wave enters with its own LDS operations complete (s_waitcnt
+// lgkmcnt(0); vmcnt and expcnt are left alone).  __syncthreads() leaves that wait to the compiler's
+// bookkeeping of outstanding operations, and on one path of the work-queue loop -- thread 0 stores the
+// workgroup's next position to LDS, nothing else touches LDS, the loop returns to the barrier at
+// its top -- the generated code had no wait at all: a wave on another SIMD could then read the
+// word before the store had been performed and work on the position the slot held two tiles
+// earlier.  Written out, the wait costs nothing where nothing is outstanding.
+static __device__ __forceinline__ void workgroup_sync() {
+  __builtin_amdgcn_s_waitcnt(0xC07F);
+  __syncthreads();
+}
+
 // calls f(std::integral_constant<int, LO + i>{}) for i = 0 .. N-1, in order
 template <int LO, typename F, int... Is>
 static __device__ __forceinline__ void for_range_impl(F&& f, std::integer_sequence<int, Is...>) {
@@ -345,11 +357,11 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
   // out to spill lanes:
   //   sKeys[a][x]  the keys of a tile whose coordinate along dimension a is >= x, one bit per key
   //   sWin[row]    window of the Q tile's query `row` (row-major): start and end per dimension
-  //   sGeo[a]      KV tile extent, its log2, and the box origin along dimension a
+  //   sGeo[a]      KV tile extent along dimension a
   constexpr int MASK_ROWS = NOMASK ? 1 : KVT + 1;
   __shared__ __attribute__((aligned(16))) uint64_t sKeys[NOMASK ? 1 : 3][MASK_ROWS];
   __shared__ __attribute__((aligned(16))) int sWin[NOMASK ? 1 : NWAVES * MQ * 32][8];
-  __shared__ __attribute__((aligned(16))) int sGeo[3][4];
+  __shared__ __attribute__((aligned(16))) int sGeo[4];
   static_assert(NOMASK || KVT == 64, "the element mask holds one bit per key of a 64-key tile");
 
   const int tid = threadIdx.x;
@@ -510,13 +522,8 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
     }
   }
 
-  enum { kGeoKvTile, kGeoKvLog2, kGeoBoxOrg };
   if constexpr (!NOMASK) {
-    if (tid < 3) {
-      sGeo[tid][kGeoKvTile] = p.kv_tile[tid];
-      sGeo[tid][kGeoKvLog2] = p.kv_tile_lg[tid];
-      sGeo[tid][kGeoBoxOrg] = box_org[tid];
-    }
+    if (tid < 3) sGeo[tid] = p.kv_tile[tid];
     // one row per thread and dimension: keys are numbered with dimension 0 fastest
     int lg_stride = 0;
 #pragma unroll
@@ -667,6 +674,7 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
     int origin[3];  // coordinate of its first token (a tile moved back from the group's edge: of the first one gathered)
     bool full;      // every key of the tile is attended by every query of this wave
     bool skip;      // no key of the tile is attended by any query of this wave
+    int lead[3];    // a tile moved back from the group's edge: its first lead[a] positions belong to the tile before it
   };
   int itc[3] = {0, 0, 0};
   if constexpr (SPLIT) {
@@ -689,11 +697,14 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
       }
       // a tile that would reach past the group is moved back to end at the group's last position
       t.origin[a] = (p.edge == 1 || p.anchor) ? na_min(org, extent[a] - p.kv_tile[a]) : org;
+      t.lead[a] = org - t.origin[a];
     }
-    t.row0 = p.fused ? t.origin[0] * tok_step[0] + t.origin[1] * tok_step[1] + t.origin[2] * tok_step[2]
-                     : (((box_org[0] >> p.kv_tile_lg[0]) + itc[0]) +
-                        p.kv_tiled[0] * (((box_org[1] >> p.kv_tile_lg[1]) + itc[1]) +
-                                         p.kv_tiled[1] * ((box_org[2] >> p.kv_tile_lg[2]) + itc[2]))) * KVT;
+    // (both forms are a handful of scalar operations: computed side by side and selected, a branch costs more)
+    const int row0_fused = t.origin[0] * tok_step[0] + t.origin[1] * tok_step[1] + t.origin[2] * tok_step[2];
+    const int row0_permuted = (((box_org[0] >> p.kv_tile_lg[0]) + itc[0]) +
+                               p.kv_tiled[0] * (((box_org[1] >> p.kv_tile_lg[1]) + itc[1]) +
+                                                p.kv_tiled[1] * ((box_org[2] >> p.kv_tile_lg[2]) + itc[2]))) * KVT;
+    t.row0 = p.fused ? row0_fused : row0_permuted;
     if (++itc[2] == box_n[2]) {
       itc[2] = 0;
       if (++itc[1] == box_n[1]) {
@@ -888,7 +899,11 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
   // or after its end); the AND over the dimensions has one bit per key of the tile.  A tile moved back
   // from the group's edge starts before its place in the tiling (the box origin plus a multiple of the
   // tile extent): the keys up to there (`lead`) belong to the tile before it.
-  auto apply_mask = [&](f32x16_t (&S)[NSB], int mb, const int (&origin)[3]) __attribute__((always_inline)) {
+  // the keys of the tile at `origin` that the lane's query of row block mb attends, one bit per key,
+  // shifted so that bit 32 sb + 8 (r / 4) + r % 4 belongs to the lane's logit r of sub-block sb
+  // (which is key 32 sb + 8 (r / 4) + 4 g + r % 4 of the tile)
+  auto mask_keys = [&](int mb, const int (&origin)[3], const int (&lead)[3]) __attribute__((always_inline)) {
+    uint64_t keys = ~uint64_t(0);
     if constexpr (!NOMASK) {
       typedef int i32x4 __attribute__((ext_vector_type(4)));
       typedef int i32x2 __attribute__((ext_vector_type(2)));
@@ -896,31 +911,38 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
       const i32x4 w01 = *reinterpret_cast<const i32x4*>(&sWin[row][0]);
       const i32x2 w2 = *reinterpret_cast<const i32x2*>(&sWin[row][4]);
       const int ws[3] = {w01[0], w01[2], w2[0]}, we[3] = {w01[1], w01[3], w2[1]};
-      uint64_t keys = ~uint64_t(0);
 #pragma unroll
       for (int a = 0; a < 3; ++a) {
-        const i32x4 geo = *reinterpret_cast<const i32x4*>(&sGeo[a][0]);
-        const int kt = geo[kGeoKvTile], kt_lg = geo[kGeoKvLog2];
-        const int from_box = origin[a] - geo[kGeoBoxOrg];
-        const int lead = (((from_box + kt - 1) >> kt_lg) << kt_lg) - from_box;
-        const int lo = na_min(na_max(ws[a] - origin[a], lead), kt);
+        const int kt = sGeo[a];
+        const int lo = na_min(na_max(ws[a] - origin[a], lead[a]), kt);
         const int hi = na_min(na_max(we[a] - origin[a], 0), kt);
         keys &= sKeys[a][lo] & ~sKeys[a][hi];
       }
-      // the lane's logit r of sub-block sb belongs to key 32 sb + 8 (r / 4) + 4 g + r % 4
       keys >>= 4 * g;
+    }
+    return keys;
+  };
+  // logit r of sub-block sb: kept where its key's bit is set, else -inf; two instructions (the
+  // sign-extended bit, a bitwise select) and no condition codes
+  auto mask_elem = [&](f32x16_t (&S)[NSB], int sb, int r, const uint64_t keys) __attribute__((always_inline)) {
+    const uint32_t half = uint32_t(keys >> (32 * sb));
+    const uint32_t keep = uint32_t(__builtin_amdgcn_sbfe(int(half), 8 * (r / 4) + r % 4, 1));  // 0 or ~0
+    const float logit = S[sb][r];  // (a copy: a bit cast of the vector element itself reads element 0)
+    const uint32_t bits = __builtin_bit_cast(uint32_t, logit);
+    S[sb][r] = __builtin_bit_cast(float, (bits & keep) | (~keep & 0xff800000u));
+  };
+  // Element mask of a PARTIAL tile for row block mb.  Per dimension the lane's window, relative to the
+  // tile origin and clamped to the tile, selects two rows of sKeys (keys at or after its start, keys at
+  // or after its end); the AND over the dimensions has one bit per key of the tile.  A tile moved back
+  // from the group's edge starts before its place in the tiling (the box origin plus a multiple of the
+  // tile extent): the keys up to there (`lead`) belong to the tile before it.
+  auto apply_mask = [&](f32x16_t (&S)[NSB], int mb, const int (&origin)[3], const int (&lead)[3]) __attribute__((always_inline)) {
+    if constexpr (!NOMASK) {
+      const uint64_t keys = mask_keys(mb, origin, lead);
 #pragma unroll
-      for (int sb = 0; sb < NSB; ++sb) {
-        const uint32_t half = uint32_t(keys >> (32 * sb));
-        // two instructions per logit (sign-extended bit, bitwise select) and no condition codes
+      for (int sb = 0; sb < NSB; ++sb)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const uint32_t keep = uint32_t(__builtin_amdgcn_sbfe(int(half), 8 * (r / 4) + r % 4, 1));  // 0 or ~0
-          const float logit = S[sb][r];  // (a copy: a bit cast of the vector element itself reads element 0)
-          const uint32_t bits = __builtin_bit_cast(uint32_t, logit);
-          S[sb][r] = __builtin_bit_cast(float, (bits & keep) | (~keep & 0xff800000u));
-        }
-      }
+        for (int r = 0; r < 16; ++r) mask_elem(S, sb, r, keys);
     }
   };
 
@@ -956,7 +978,8 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
     asm volatile("" : "+v"(c_init[mb]));
   };
   // masks (PARTIAL tiles) and maxima of a whole tile of logits, outside the slots
-  auto finish_logits = [&](f32x16_t (&S)[MQ][NSB], const bool t_full, const bool t_skip, const int (&t_origin)[3], bool have_max, const float (&mx_in)[MQ]) __attribute__((always_inline)) {
+  auto finish_logits = [&](f32x16_t (&S)[MQ][NSB], const TileInfo& t, bool have_max, const float (&mx_in)[MQ]) __attribute__((always_inline)) {
+    const bool t_full = t.full, t_skip = t.skip;
 #pragma unroll
     for (int mb = 0; mb < MQ; ++mb) {
       float mx = mx_in[mb];
@@ -968,7 +991,7 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
 #pragma unroll
           for (int r = 0; r < 16; ++r) S[mb][sb][r] = -INFINITY;
       } else if (!t_full || !have_max) {
-        if (!t_full) apply_mask(S[mb], mb, t_origin);
+        if (!t_full) apply_mask(S[mb], mb, t.origin, t.lead);
         mx = -INFINITY;
 #pragma unroll
         for (int sb = 0; sb < NSB; ++sb)
@@ -986,7 +1009,7 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
   // LDS: K(j) and V(j) live in stage j % 2.
   TileInfo nxt = next_tile();  // tile 1 (a descriptor past the box is never used)
   wait_vmcnt<0>();
-  __syncthreads();  // K(0), V(0) and the coordinate table are in LDS
+  workgroup_sync();  // K(0), V(0), the mask tables and the queries' windows are in LDS
   if (1 < total_tiles) issue_tile_load(kbase, ld_koff, sK1, nxt.row0, nxt.origin, KLayout{});
 #pragma unroll
   for (int mb = 0; mb < MQ; ++mb)
@@ -1006,7 +1029,7 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
       for (int mb = 0; mb < MQ; ++mb) S_a[mb][s / KSTEPS] = M::run(kf, qf[mb][s % KSTEPS], S_a[mb][s / KSTEPS]);
     }
     const float none[MQ] = {};
-    finish_logits(S_a, cur.full, cur.skip, cur.origin, false, none);
+    finish_logits(S_a, cur, false, none);
   }
 
   // CUR / NXT: this wave attends keys of tile j / tile j + 1; an inactive tile only takes part
@@ -1024,7 +1047,7 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
 
     wait_vmcnt<0>();   // this thread's copies of K(j+1) and V(j) have landed
     if constexpr ((kAblate & kAblateBarrier) == 0)
-      __syncthreads();   // ... and everyone's; everyone is done reading K(j) and V(j-1)
+      workgroup_sync();   // ... and everyone's; everyone is done reading K(j) and V(j-1)
     const TileInfo t2 = next_tile();
     // Past the end of the box the spread copies re-read the current tile into the free stage
     // (never used), which keeps the slots below free of control flow.
@@ -1151,7 +1174,7 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
       float mxs[MQ];
 #pragma unroll
       for (int mb = 0; mb < MQ; ++mb) mxs[mb] = fmaxf(mx[mb][0], mx[mb][1]);
-      finish_logits(S_nxt, nxt.full, nxt.skip, nxt.origin, true, mxs);
+      finish_logits(S_nxt, nxt, true, mxs);
     }
     cur = nxt;
     nxt = t2;
@@ -1278,7 +1301,7 @@ static __device__ __forceinline__ void fna_queue_loop(uint32_t* __restrict__ que
   }
   for (int i = 0;; i ^= 1) {
     // s_pos[i] is written, everyone has read s_pos[i ^ 1] and is done with the LDS of the previous tile
-    __syncthreads();
+    workgroup_sync();
     const int pid = __builtin_amdgcn_readfirstlane(s_pos[i]);
     if (pid < 0) break;
     bool fetched = false;

@@ -118,7 +118,7 @@ __global__ void __launch_bounds__(256) fna_fwd_f32_kernel(const FnaParams p) {
       for (int t0 = t_lo[0]; t0 <= t_hi[0]; ++t0) {
         const int64_t row0 = int64_t(t0 + p.kv_tiled[0] * (t1 + p.kv_tiled[1] * t2)) * KVT;
         const int org[3] = {t0 * p.kv_tile[0], t1 * p.kv_tile[1], t2 * p.kv_tile[2]};
-        __syncthreads();  // everyone is done with the previous tile (and sCrd is written)
+        workgroup_sync();  // everyone is done with the previous tile (and sCrd is written)
 #pragma unroll
         for (int c = tid; c < KVT * (D / 4); c += NT) {
           const int r = c / (D / 4), c4 = c % (D / 4);
@@ -126,7 +126,7 @@ __global__ void __launch_bounds__(256) fna_fwd_f32_kernel(const FnaParams p) {
           *reinterpret_cast<f32x4_t*>(&sK[r * LDW + c4 * 4]) = *reinterpret_cast<const f32x4_t*>(kbase + off);
           *reinterpret_cast<f32x4_t*>(&sV[r * LDW + c4 * 4]) = *reinterpret_cast<const f32x4_t*>(vbase + off);
         }
-        __syncthreads();
+        workgroup_sync();
 
         // S^T = K Q^T (already in the exp2 domain), two blocks of 32 keys
         f32x16_t S[2];

@@ -252,7 +252,7 @@ static __device__ __forceinline__ void fna_fwd_fp8_tile(const FnaParams& p, cons
         t.skip = t.skip || (end <= wave_lo[a]) || (org >= wave_hi[a]);
       }
       // a tile that would reach past the group is moved back to end at the group's last position
-      t.origin[a] = p.anchor ? na_min(org, extent[a] - p.kv_tile[a]) : org;
+      t.origin[a] = (p.edge == 1 || p.anchor) ? na_min(org, extent[a] - p.kv_tile[a]) : org;
     }
     t.row0 = p.fused ? t.origin[0] * tok_step[0] + t.origin[1] * tok_step[1] + t.origin[2] * tok_step[2]
                      : (((box_org[0] >> p.kv_tile_lg[0]) + itc[0]) +
@@ -457,7 +457,7 @@ static __device__ __forceinline__ void fna_fwd_fp8_tile(const FnaParams& p, cons
   constexpr int N_ELEMS = NSB * 16;
   TileInfo nxt = next_tile();
   wait_vmcnt<0>();
-  __syncthreads();
+  workgroup_sync();
   if (1 < total_tiles) issue_tile_load(kbase, ld_koff, sK1, nxt.row0);
   msc = -kFp8ProbLog2Scale;
   {
@@ -481,7 +481,7 @@ static __device__ __forceinline__ void fna_fwd_fp8_tile(const FnaParams& p, cons
     char* sV_nxt = st ? sV0 : sV1;
 
     wait_vmcnt<0>();
-    __syncthreads();
+    workgroup_sync();
     const TileInfo t2 = next_tile();
     const TileCopy ck = make_copy(kbase, sK_cur, (j + 2 < total_tiles) ? t2.row0 : cur.row0);
     const TileCopy cv = make_copy(vbase, sV_nxt, (j + 1 < total_tiles) ? nxt.row0 : cur.row0);

@@ -484,9 +484,9 @@ int fused_geometry(const char* what, FnaParams& p, bool sixteen_bit, int na_dim,
       qt *= q_tile_shape[a];
       kvt *= kv_tile_shape[a];
     }
-    if (!sixteen_bit)
-      return fail("%s: an input extent that is not a multiple of dilation * KV tile in every dimension needs fp16 / bf16 "
-                  "operands; use the token-permuted entry point", what);
+    if (edge == 2 && !sixteen_bit)
+      return fail("%s: a dilation group narrower than the KV tile needs fp16 / bf16 operands; use the token-permuted "
+                  "entry point", what);
     if (edge == 2 && (qt != 128 || kvt != 64))
       return fail("%s: a dilation group narrower than the KV tile needs tiles of 128 x 64 tokens (got %lld x %lld); use "
                   "the token-permuted entry point", what, qt, kvt);
@@ -920,24 +920,30 @@ int natten_amd_fna_backward_fused(const void* q, const void* k, const void* v, c
   if (roles < 1 || roles > 3) return fail("%s: roles must be 1 (dq), 2 (dk and dv) or 3 (all), got %d", what, roles);
   if (!qkv_shape || !kernel_size || !stride || !dilation || !is_causal || !q_tile_shape || !kv_tile_shape)
     return fail("%s: null shape argument", what);
-  // per-group layouts: without padding, which needs every extent to be a multiple of dilation x tile
-  int group_shape[3] = {1, 1, 1};
+  // Per-group layouts, padded to whole tiles.  Extents that are not multiples of dilation x tile are
+  // taken as long as every dilation group is at least one tile wide (either side's) in every
+  // dimension: tiles that would reach past a group are then moved back or clamped by the kernels.
+  int q_group_shape[3] = {1, 1, 1}, kv_group_shape[3] = {1, 1, 1}, edge = 0;
   long long tokens = 1;
   for (int a = 0; a < na_dim; ++a) {
     if (qkv_shape[a] < 1 || dilation[a] < 1 || q_tile_shape[a] < 1 || kv_tile_shape[a] < 1)
       return fail("%s: invalid parameter along dimension %d", what, a);
-    if (qkv_shape[a] % (dilation[a] * q_tile_shape[a]) != 0 || qkv_shape[a] % (dilation[a] * kv_tile_shape[a]) != 0)
-      return fail("%s: extent %d along dimension %d is not a multiple of dilation x tile (%d x %d, %d x %d); use the "
-                  "token-permuted entry point",
-                  what, qkv_shape[a], a, dilation[a], q_tile_shape[a], dilation[a], kv_tile_shape[a]);
-    group_shape[a] = qkv_shape[a] / dilation[a];
+    if (qkv_shape[a] % (dilation[a] * q_tile_shape[a]) != 0 || qkv_shape[a] % (dilation[a] * kv_tile_shape[a]) != 0) edge = 1;
+    if (qkv_shape[a] / dilation[a] < q_tile_shape[a] || qkv_shape[a] / dilation[a] < kv_tile_shape[a])
+      return fail("%s: a dilation group of dimension %d (%d tokens / dilation %d) is narrower than a tile (%d, %d); use "
+                  "the token-permuted entry point",
+                  what, a, qkv_shape[a], dilation[a], q_tile_shape[a], kv_tile_shape[a]);
+    const int ext = na_ceil_div(qkv_shape[a], dilation[a]);
+    q_group_shape[a] = na_ceil_div(ext, q_tile_shape[a]) * q_tile_shape[a];
+    kv_group_shape[a] = na_ceil_div(ext, kv_tile_shape[a]) * kv_tile_shape[a];
     tokens *= qkv_shape[a];
   }
   if (tokens > 0x7fffffffLL) return fail("%s: more than 2^31 tokens", what);
   FnaParams f;
-  if (int rc = fill_fna_params(what, f, na_dim, group_shape, group_shape, qkv_shape, kernel_size, stride, dilation,
+  if (int rc = fill_fna_params(what, f, na_dim, q_group_shape, kv_group_shape, qkv_shape, kernel_size, stride, dilation,
                                is_causal, q_tile_shape, kv_tile_shape))
     return rc;
+  if (!fna_tiles_are_powers_of_two(f)) return fail("%s: tile extents must be powers of two", what);
   if (int rc = check_common(what, q, k, v, dq, lse, batch, int(tokens), int(tokens), heads_q, heads_kv, head_dim)) return rc;
   // per-lane byte offsets inside a tile are 32-bit
   long long span_q = 0, span_kv = 0;
@@ -987,6 +993,7 @@ int natten_amd_fna_backward_fused(const void* q, const void* k, const void* v, c
   p.q_extent0 = 0;
   p.scale = scale;
   p.fused = 1;
+  p.edge = edge;
   p.tokens = int(tokens);
   p.roles = roles;
   return dispatch_bwd(p, dtype, head_dim, static_cast<hipStream_t>(stream));

@@ -59,6 +59,11 @@ def run_backward(B, H, Hkv, D, shape, k, s, d, causal, dtype, bq=None, bkv=None,
         # both place the keys alike in their tiles; elsewhere they agree up to summation order)
         _, fwd_kt = check_fna_forward_config(q, k, s, d, causal, None, None)
         exact = routes_agree_bit_for_bit(shape, d, fwd_kt)
+        # ... and the backward on the original tensors sums in the permuted route's order only where its
+        # own tiles divide the extents (elsewhere it moves the last tile of a dimension back)
+        from natten_amd.tile_config import check_fna_backward_config
+        bwd_tiles = check_fna_backward_config(q, k, s, d, causal, bq, bkv)
+        exact = exact and all(X % (dd * t) == 0 for tile in bwd_tiles for X, dd, t in zip(shape, d, tile))
         for name, a, b, c in zip(("dq", "dk", "dv"), grads[0], grads[1], (q.grad, kk.grad, v.grad)):
             if exact:
                 assert torch.equal(a, b), f"original-layout and permuted backward differ in {name}: {tag}"
@@ -67,6 +72,26 @@ def run_backward(B, H, Hkv, D, shape, k, s, d, causal, dtype, bq=None, bkv=None,
             # and the default (KV tiles of the forward laid out from the window's first key): two
             # roundings of the same gradient, a unit of the last place apart at most
             assert_close(f"default route {name} {tag}", to_np(c), to_np(b), atol=1.5 * TOL[dtype], rtol=TOL[dtype])
+
+
+@pytest.mark.parametrize("case", [
+    # extents no tile shape divides, uneven dilation groups: the backward still runs on the original tensors
+    (1, 2, 2, 64, (57, 20, 88), (5, 7, 9), (1, 2, 3), (2, 1, 1), (False, False, False)),
+    (1, 4, 2, 128, (84, 69), (11, 9), (2, 1), (1, 1), (True, False)),
+    (2, 2, 1, 32, (301,), (33,), (4,), (2,), (False,)),
+    (1, 2, 2, 128, (11, 19, 37), (4, 6, 9), (1, 2, 4), (1, 1, 1), (True, False, True)),
+])
+def test_backward_odd_extents_on_the_original_tensors(case):
+    from natten_amd import _lib
+    from natten_amd.tile_config import check_fna_backward_config
+
+    B, H, Hkv, D, shape, k, s, d, causal = case
+    probe = torch.empty((B, *shape, H, D), dtype=torch.bfloat16, device="meta")
+    bq, bkv = check_fna_backward_config(probe, k, s, d, causal, None, None)
+    assert any(X % (dd * t) for tile in (bq, bkv) for X, dd, t in zip(shape, d, tile)), "the case is meant to need edge tiles"
+    assert _lib.backward_fused_layout_supported(shape, d, bq, bkv, row_bytes=H * D * 2)
+    run_backward(B, H, Hkv, D, shape, k, s, d, causal, torch.bfloat16, seed=31)
+    run_backward(B, H, Hkv, D, shape, k, s, d, causal, torch.float16, seed=32)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])

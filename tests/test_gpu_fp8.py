@@ -242,6 +242,20 @@ def test_fp8_odd_extents_work_queue_equals_per_tile(shape, kernel, stride, dilat
     ref_o, ref_l = c_oracle.na_forward(to_np(qd), to_np(kd), to_np(vd), kernel, stride, dilation, causal, None)
     check_out("out", True, to_np(out_q), ref_o, vd)
     assert_close("lse", to_np(lse_q), ref_l)
+    # where every dilation group is at least a KV tile wide the 8-bit kernel takes these extents in
+    # one launch on the original tensors (edge tiles moved back); the permuted route meets the same bar
+    from natten_amd import _lib
+    from natten_amd.tile_config import check_fna_forward_config
+
+    qt, kt = check_fna_forward_config(q8, kernel, stride, dilation, causal, None, None)
+    if all(X // d >= t for X, d, t in zip(shape, dilation, kt)):
+        assert _lib.fused_layout_supported(shape, dilation, kt, row_bytes=Hkv * D * 2, q_tile_shape=qt, dtype=q8.dtype)
+        with torch.no_grad():
+            out_f, lse_f = amd_fna_generic(q8, k8, v8, kernel, stride, dilation, causal, fused=True, **kw)
+            out_p, lse_p = amd_fna_generic(q8, k8, v8, kernel, stride, dilation, causal, fused=False, **kw)
+        assert torch.equal(out_f, out_q) and torch.equal(lse_f, lse_q)
+        check_out("out (permuted route)", True, to_np(out_p), ref_o, vd)
+        assert_close("lse (permuted route)", to_np(lse_p), ref_l)
 
 
 def test_fp8_matmul_rejects_unsupported_shapes():

@@ -58,7 +58,9 @@ def test_fused_rejects_what_no_kernel_instance_gathers():
     assert not _lib.fused_layout_supported((20, 6), (1, 1), (8, 8), q_tile_shape=(8, 8), dtype=torch.bfloat16)
     assert _lib.fused_layout_supported((20, 6), (1, 1), (8, 8), q_tile_shape=(16, 8), dtype=torch.bfloat16)
     assert _lib.fused_layout_supported((20, 24), (1, 1), (8, 8), q_tile_shape=(8, 8), dtype=torch.bfloat16)
-    assert not _lib.fused_layout_supported((20, 24), (1, 1), (8, 8), q_tile_shape=(8, 8), dtype=torch.float8_e4m3fn)
+    # 8-bit operands: taken while every dilation group is at least a KV tile wide, never by the clamping instance
+    assert _lib.fused_layout_supported((20, 24), (1, 1), (8, 8), q_tile_shape=(8, 8), dtype=torch.float8_e4m3fn)
+    assert not _lib.fused_layout_supported((20, 6), (1, 1), (8, 8), q_tile_shape=(16, 8), dtype=torch.float8_e4m3fn)
     with pytest.raises(ValueError):
         amd_fna_generic(q, kk, v, *args, q_tile_shape=(8, 8), kv_tile_shape=(8, 8), fused=True)
     with pytest.raises(RuntimeError):

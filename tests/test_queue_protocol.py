@@ -179,40 +179,50 @@ def test_model_rejects_counters_that_do_not_start_at_zero(wq):
 # Model 2: the hand-over inside a workgroup.  Every wave runs the loop of fna_queue_loop:
 #   barrier; read s_pos[i]; leave if it is negative; the tile (some barriers; thread 0, in wave 0,
 #   writes s_pos[i ^ 1] after the last of them -- a tile that returns at once has none);  i ^= 1.
-# A step is a barrier arrival, an LDS read or an LDS write; a barrier releases when every wave has
-# arrived.  Waves are otherwise free to run at any relative speed.
+# A step is a barrier arrival, an LDS read, the issue of an LDS write, or the LDS unit performing
+# the oldest write a wave has issued: a write is not visible to the other waves before that, and
+# only a wait for the wave's own LDS operations (what workgroup_sync() puts in front of every
+# barrier) holds the wave until it has happened.  A barrier releases when every wave has arrived.
+# Waves are otherwise free to run at any relative speed.
 # ---------------------------------------------------------------------------------------------
-def wave_program(wave, tiles, barriers_per_tile, write_at):
+def wave_program(wave, tiles, barriers_per_tile, write_at, wait_before_barrier):
+    bar = [("wait",), ("bar",)] if wait_before_barrier else [("bar",)]
     ops = [("write", 0)] if wave == 0 else []
     for n, pid in enumerate(tiles):
-        ops += [("bar",), ("read", n)]
+        ops += bar + [("read", n)]
         if pid < 0:
             break
         if wave == 0 and write_at == "top":
             ops.append(("write", n + 1))
-        ops += [("bar",)] * barriers_per_tile[n % len(barriers_per_tile)]
+        ops += bar * barriers_per_tile[n % len(barriers_per_tile)]
         if wave == 0 and write_at == "end":
             ops.append(("write", n + 1))
     return ops
 
 
-def explore_handover(waves, tiles, slots=2, barriers_per_tile=(2, 0, 1), write_at="end"):
+def explore_handover(waves, tiles, slots=2, barriers_per_tile=(2, 0, 1), write_at="end", wait_before_barrier=True):
     """tiles: the positions thread 0 obtains, in order, ending with a negative one."""
-    progs = [wave_program(w, tiles, barriers_per_tile, write_at) for w in range(waves)]
-    init = ((None,) * slots, (0,) * waves, frozenset())
+    progs = [wave_program(w, tiles, barriers_per_tile, write_at, wait_before_barrier) for w in range(waves)]
+    # state: LDS slots, program counters, waves waiting at the barrier, writes issued by wave 0 and not yet performed
+    init = ((None,) * slots, (0,) * waves, frozenset(), ())
     seen = {init}
     stack = [init]
     while stack:
-        lds, pcs, waiting = stack.pop()
+        lds, pcs, waiting, pending = stack.pop()
+        succ = []
+        if pending:  # the LDS unit performs wave 0's oldest outstanding write
+            l = list(lds)
+            l[pending[0] % slots] = tiles[pending[0]]
+            succ.append((tuple(l), pcs, waiting, pending[1:]))
         runnable = [w for w in range(waves) if pcs[w] < len(progs[w]) and w not in waiting]
-        if not runnable:
-            if waiting:
-                raise Violation("deadlock: some waves wait at a barrier the others never reach")
-            continue
         for w in runnable:
             op = progs[w][pcs[w]]
-            l, pc, wt = list(lds), list(pcs), set(waiting)
-            if op[0] == "bar":
+            pc, wt, pend = list(pcs), set(waiting), pending
+            if op[0] == "wait":
+                if w == 0 and pending:
+                    continue  # held until its writes have been performed
+                pc[w] += 1
+            elif op[0] == "bar":
                 wt.add(w)
                 if len(wt) == sum(1 for x in range(waves) if pcs[x] < len(progs[x])):
                     for x in wt:
@@ -220,14 +230,23 @@ def explore_handover(waves, tiles, slots=2, barriers_per_tile=(2, 0, 1), write_a
                     wt = set()
             elif op[0] == "read":
                 n = op[1]
-                got = l[n % slots]
+                got = lds[n % slots]
+                if w == 0:  # a wave sees its own writes in program order
+                    for m in pending:
+                        if m % slots == n % slots:
+                            got = tiles[m]
                 if got != tiles[n]:
                     raise Violation(f"wave {w} read {got} for its tile {n}; thread 0 wrote {tiles[n]} for it")
                 pc[w] += 1
             else:
-                l[op[1] % slots] = tiles[op[1]]
+                pend = pending + (op[1],)
                 pc[w] += 1
-            nxt = (tuple(l), tuple(pc), frozenset(wt))
+            succ.append((lds, tuple(pc), frozenset(wt), pend))
+        if not succ:
+            if waiting:
+                raise Violation("deadlock: some waves wait at a barrier the others never reach")
+            continue
+        for nxt in succ:
             if nxt not in seen:
                 seen.add(nxt)
                 stack.append(nxt)
@@ -256,3 +275,13 @@ def test_model_rejects_one_slot(write_at):
     # with a single slot thread 0 may overwrite a position a slower wave has not read yet
     with pytest.raises(Violation):
         explore_handover(2, TILES, slots=1, barriers_per_tile=(0,), write_at=write_at)
+
+
+@pytest.mark.parametrize("barriers", [(0,), (2, 0, 1)])
+def test_model_rejects_a_barrier_without_the_wait_for_the_store(barriers):
+    # The fault the work-queue launch had: on the path of a tile that returns at once nothing held
+    # thread 0's wave between its store of the next position and the barrier at the top of the loop,
+    # so another wave could read the slot before the store had been performed and work on the
+    # position it held two tiles earlier.
+    with pytest.raises(Violation):
+        explore_handover(2, TILES, slots=2, barriers_per_tile=barriers, write_at="end", wait_before_barrier=False)
