@@ -953,7 +953,7 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
     mx = cross_half_max(mx);
     const bool first = (m_run[mb] == -INFINITY) && (mx != -INFINITY);
     const bool grow = first || (mx > kLazyRescaleLog2);
-    if (__any(grow)) {
+    if (__builtin_expect(__any(grow), 0)) {
       // rows still at -inf take their first maximum as it is (it may be negative) and have
       // nothing accumulated yet; the others only grow
       const bool was_inf = m_run[mb] == -INFINITY;
@@ -979,24 +979,29 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
   };
   // masks (PARTIAL tiles) and maxima of a whole tile of logits, outside the slots
   auto finish_logits = [&](f32x16_t (&S)[MQ][NSB], const TileInfo& t, bool have_max, const float (&mx_in)[MQ]) __attribute__((always_inline)) {
+    // One test on the way of a tile that needs nothing (attended in full, maxima at hand): every
+    // wave-uniform branch in the tile loop costs about a hundredth of its time.
     const bool t_full = t.full, t_skip = t.skip;
+    const bool plain = t_full && !t_skip && have_max;
 #pragma unroll
     for (int mb = 0; mb < MQ; ++mb) {
       float mx = mx_in[mb];
-      if (t_skip) {
-        // none of this wave's queries attends the tile: every logit is masked
-        mx = -INFINITY;
+      if (__builtin_expect(!plain, 0)) {
+        if (t_skip) {
+          // none of this wave's queries attends the tile: every logit is masked
+          mx = -INFINITY;
 #pragma unroll
-        for (int sb = 0; sb < NSB; ++sb)
+          for (int sb = 0; sb < NSB; ++sb)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) S[mb][sb][r] = -INFINITY;
-      } else if (!t_full || !have_max) {
-        if (!t_full) apply_mask(S[mb], mb, t.origin, t.lead);
-        mx = -INFINITY;
+            for (int r = 0; r < 16; ++r) S[mb][sb][r] = -INFINITY;
+        } else {
+          if (!t_full) apply_mask(S[mb], mb, t.origin, t.lead);
+          mx = -INFINITY;
 #pragma unroll
-        for (int sb = 0; sb < NSB; ++sb)
+          for (int sb = 0; sb < NSB; ++sb)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) mx = fmaxf(mx, S[mb][sb][r]);
+            for (int r = 0; r < 16; ++r) mx = fmaxf(mx, S[mb][sb][r]);
+        }
       }
       update_max(mb, mx, S[mb]);
     }
