@@ -303,10 +303,20 @@ int natten_amd_compute_delta(const void* out, const void* d_out, float* delta, i
  * dq, dk, dv are written completely (padding rows get zeros); nothing is accumulated through
  * memory, results are deterministic.  The gradient of the LSE output is not propagated (as in
  * the reference).  16-bit float operands, head_dim 32 / 64 / 128.
+ *
+ * q_scaled (all four backward entry points): workspace of q's shape and type.  The forward
+ * kernel multiplies the keys with q' = round(q * scale * log2(e)) (rounded to the operand type
+ * once), so that its logits need no further scaling; the backward forms its logits from the same
+ * q', which makes its probabilities exp(logit - LSE) those the forward normalised (they sum to
+ * one over a query's window).  The launch that writes dq scales the query rows it holds in
+ * registers; the launch that writes dk and dv streams q' and first writes it to q_scaled with
+ * one pass over q.  The call makes the dk / dv launch first and the dq launch last, so q_scaled
+ * may be the dq buffer itself (for a call that only makes the dk / dv launch: if dq is written
+ * afterwards); it must not be q.  May be null for a call that only makes the dq launch.
  */
 int natten_amd_fna_backward(const void* q, const void* k, const void* v, const void* d_out,
                             const float* lse, const float* delta, void* dq, void* dk, void* dv,
-                            int dtype, int na_dim, int batch, int seqlen_q, int seqlen_kv,
+                            void* q_scaled, int dtype, int na_dim, int batch, int seqlen_q, int seqlen_kv,
                             int heads_q, int heads_kv, int head_dim, const int32_t* q_shape,
                             const int32_t* kv_shape, const int32_t* qkv_shape,
                             const int32_t* kernel_size, const int32_t* stride,
@@ -336,7 +346,7 @@ int natten_amd_fna_backward(const void* q, const void* k, const void* v, const v
  */
 int natten_amd_fna_backward_fused(const void* q, const void* k, const void* v, const void* d_out,
                                   const float* lse, const float* delta, void* dq, void* dk,
-                                  void* dv, int dtype, int na_dim, int batch, int heads_q,
+                                  void* dv, void* q_scaled, int dtype, int na_dim, int batch, int heads_q,
                                   int heads_kv, int head_dim, const int32_t* qkv_shape,
                                   const int32_t* kernel_size, const int32_t* stride,
                                   const int32_t* dilation, const int32_t* is_causal,
@@ -350,7 +360,7 @@ int natten_amd_fna_backward_fused(const void* q, const void* k, const void* v, c
  */
 int natten_amd_attention_backward(const void* q, const void* k, const void* v, const void* d_out,
                                   const float* lse, const float* delta, void* dq, void* dk,
-                                  void* dv, int dtype, int batch, int seqlen_q, int seqlen_kv,
+                                  void* dv, void* q_scaled, int dtype, int batch, int seqlen_q, int seqlen_kv,
                                   int padded_seqlen_q, int padded_seqlen_kv, int heads_q,
                                   int heads_kv, int head_dim, int is_causal, float scale,
                                   void* stream);
@@ -370,7 +380,7 @@ int natten_amd_attention_backward(const void* q, const void* k, const void* v, c
  */
 int natten_amd_attention_backward_varlen(const void* q, const void* k, const void* v,
                                          const void* d_out, const float* lse, const float* delta,
-                                         void* dq, void* dk, void* dv, int dtype, int num_seqs,
+                                         void* dq, void* dk, void* dv, void* q_scaled, int dtype, int num_seqs,
                                          int rows_q, int rows_kv, const int32_t* cu_seqlens_q,
                                          const int32_t* cu_seqlens_kv,
                                          const int32_t* padded_cu_seqlens_q,

@@ -22,7 +22,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 # NATTEN_AMD_LIBRARY: another build of the library (the timing-only ones of natten_amd.build --ablate)
 LIB_PATH = os.environ.get("NATTEN_AMD_LIBRARY") or os.path.join(_HERE, "libnatten_amd.so")
 
-ABI_VERSION = 14
+ABI_VERSION = 15
 
 DTYPE_CODES = {
     torch.float16: 0,
@@ -86,20 +86,20 @@ _SIGNATURES = {
     ),
     "natten_amd_fna_backward": (
         ctypes.c_int,
-        [ctypes.c_void_p] * 9 + [ctypes.c_int] * 8 + [ctypes.c_void_p] * 9 + [ctypes.c_float, ctypes.c_void_p],
+        [ctypes.c_void_p] * 10 + [ctypes.c_int] * 8 + [ctypes.c_void_p] * 9 + [ctypes.c_float, ctypes.c_void_p],
     ),
     "natten_amd_fna_backward_fused": (
         ctypes.c_int,
-        [ctypes.c_void_p] * 9 + [ctypes.c_int] * 6 + [ctypes.c_void_p] * 7
+        [ctypes.c_void_p] * 10 + [ctypes.c_int] * 6 + [ctypes.c_void_p] * 7
         + [ctypes.c_float, ctypes.c_int, ctypes.c_void_p],
     ),
     "natten_amd_attention_backward": (
         ctypes.c_int,
-        [ctypes.c_void_p] * 9 + [ctypes.c_int] * 10 + [ctypes.c_float, ctypes.c_void_p],
+        [ctypes.c_void_p] * 10 + [ctypes.c_int] * 10 + [ctypes.c_float, ctypes.c_void_p],
     ),
     "natten_amd_attention_backward_varlen": (
         ctypes.c_int,
-        [ctypes.c_void_p] * 9 + [ctypes.c_int] * 4 + [ctypes.c_void_p] * 4 + [ctypes.c_int] * 6
+        [ctypes.c_void_p] * 10 + [ctypes.c_int] * 4 + [ctypes.c_void_p] * 4 + [ctypes.c_int] * 6
         + [ctypes.c_float, ctypes.c_void_p],
     ),
     "natten_amd_token_permute_widen": (
@@ -545,7 +545,7 @@ def fna_backward(
     with _on_device(q):
         rc = L.natten_amd_fna_backward(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), d_out.data_ptr(), lse.data_ptr(), delta.data_ptr(),
-            dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), DTYPE_CODES[q.dtype], na_dim, q.shape[0], q.shape[1],
+            dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), dq.data_ptr(), DTYPE_CODES[q.dtype], na_dim, q.shape[0], q.shape[1],
             k.shape[1], q.shape[2], k.shape[2], q.shape[3], _i32(q_shape), _i32(kv_shape), _i32(qkv_shape),
             _i32(kernel_size), _i32(stride), _i32(dilation), _i32([1 if c else 0 for c in is_causal]),
             _i32(q_tile_shape), _i32(kv_tile_shape), float(scale), _stream(q),
@@ -588,13 +588,16 @@ def fna_backward_fused(
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     same = kv_role_q_tile_shape is None or (
         tuple(kv_role_q_tile_shape) == tuple(q_tile_shape) and tuple(kv_role_kv_tile_shape) == tuple(kv_tile_shape))
+    # The dk / dv launch streams the queries as the forward kernel multiplied them (scaled, rounded
+    # once) from a workspace of q's size that the call fills first; dq serves as that workspace, so
+    # the launch that writes dq comes last.
     launches = [(3, q_tile_shape, kv_tile_shape)] if same else [
-        (1, q_tile_shape, kv_tile_shape), (2, kv_role_q_tile_shape, kv_role_kv_tile_shape)]
+        (2, kv_role_q_tile_shape, kv_role_kv_tile_shape), (1, q_tile_shape, kv_tile_shape)]
     with _on_device(q):
         for roles, qt, kt in launches:
             rc = L.natten_amd_fna_backward_fused(
                 q.data_ptr(), k.data_ptr(), v.data_ptr(), d_out.data_ptr(), lse.data_ptr(), delta.data_ptr(),
-                dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), DTYPE_CODES[q.dtype], na_dim, B, H, k.shape[-2],
+                dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), dq.data_ptr(), DTYPE_CODES[q.dtype], na_dim, B, H, k.shape[-2],
                 q.shape[-1], _i32(q.shape[1 : 1 + na_dim]), _i32(kernel_size), _i32(stride), _i32(dilation),
                 _i32([1 if c else 0 for c in is_causal]), _i32(qt), _i32(kt), float(scale), roles, _stream(q),
             )
@@ -617,7 +620,7 @@ def attention_backward(
     with _on_device(q):
         rc = L.natten_amd_attention_backward(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), d_out.data_ptr(), lse.data_ptr(), delta.data_ptr(),
-            dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), DTYPE_CODES[q.dtype], q.shape[0], int(seqlen_q),
+            dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), dq.data_ptr(), DTYPE_CODES[q.dtype], q.shape[0], int(seqlen_q),
             int(seqlen_kv), q.shape[1], k.shape[1], q.shape[2], k.shape[2], q.shape[3], 1 if is_causal else 0,
             float(scale), _stream(q),
         )
@@ -648,7 +651,7 @@ def attention_backward_varlen(
     with _on_device(q):
         rc = L.natten_amd_attention_backward_varlen(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), d_out.data_ptr(), lse.data_ptr(), delta.data_ptr(),
-            dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), DTYPE_CODES[q.dtype], cu_q.numel() - 1, q.shape[1], k.shape[1],
+            dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), dq.data_ptr(), DTYPE_CODES[q.dtype], cu_q.numel() - 1, q.shape[1], k.shape[1],
             cu_q.data_ptr(), cu_kv.data_ptr(), padded_cu_q.data_ptr(), padded_cu_kv.data_ptr(), int(max_seqlen_q),
             int(max_seqlen_kv), q.shape[2], k.shape[2], q.shape[3], 1 if is_causal else 0, float(scale), _stream(q),
         )

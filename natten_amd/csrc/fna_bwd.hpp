@@ -7,8 +7,14 @@
 //   dKV, paired role : stationary = keys    (operands K, V; results dK and dV), streamed = queries (Q, dO)
 // Per streamed tile, with Y1/Y2 the streamed and X1/X2 the stationary operands:
 //   S^T  = Y1 X1^T,  dP^T = Y2 X2^T                     (32x32x16 MFMA, the lane owns a stationary row)
-//   P    = exp2(c S - log2e LSE) on unmasked pairs, 0 elsewhere;  dS = P (dP - delta)
-//   acc1^T += Y1^T dS^T   (dQ = scale * sum_k dS k  /  dK = scale * sum_q dS q)
+//   P    = exp2(S - log2e LSE) on unmasked pairs, 0 elsewhere;  dS = P (dP - delta)
+//   acc1^T += Y1^T dS^T   (dQ = scale * sum_k dS k  /  dK = ln 2 * sum_q dS q')
+// The logits are formed from the same operand as in the forward kernel, q' = round(q * scale *
+// log2(e)) in the operand type, so that S is the forward's logit to the last bit of its operands
+// and P the probability its LSE normalises (the rows of P sum to one); with the unscaled queries
+// the two passes' logits differ by the rounding of q', and a probability of a one-key window
+// comes out as 1 +- 0.5 % instead of 1.  The dQ role scales its stationary query fragments as it
+// loads them; the key-stationary roles stream q' from a copy (qs) that a pass over q writes first.
 //   acc2^T += Y2^T P^T    (dV = sum_q P dO)
 // In the dKV role one wave forms all of this for its 32 key rows.  At head dim 128 the
 // accumulators, stationary fragments and both products of that no longer fit the 256 vector
@@ -35,6 +41,7 @@ namespace natten_amd {
 
 struct FnaBwdParams {
   const void* q;      // [batch, seqlen_q, heads_q, D]   (batch counts dilation groups)
+  const void* qs;     // like q: round(q * scale * log2(e)), the forward kernel's logit operand (key-stationary roles)
   const void* k;      // [batch, seqlen_kv, heads_kv, D]
   const void* v;
   const void* d_out;  // like q
@@ -344,6 +351,7 @@ fna_bwd_kernel(const FnaBwdParams p) {
 #pragma unroll
   for (int ks = 0; ks < KSTEPS; ++ks) {
     x1f[ks] = *reinterpret_cast<const vec8*>(x1 + ks * 16);
+    if constexpr (!KV_STATIONARY) x1f[ks] = scale_query_fragment<T>(x1f[ks], p.scale * kLog2e);
     if constexpr (HAS_DS) x2f[ks] = *reinterpret_cast<const vec8*>(x2 + ks * 16);
   }
 
@@ -374,7 +382,7 @@ fna_bwd_kernel(const FnaBwdParams p) {
   }
 
   // ---- streamed tiles ---------------------------------------------------------------------------
-  const T* y1_all = reinterpret_cast<const T*>(KV_STATIONARY ? p.q : p.k);
+  const T* y1_all = reinterpret_cast<const T*>(KV_STATIONARY ? p.qs : p.k);
   const T* y2_all = reinterpret_cast<const T*>(KV_STATIONARY ? p.d_out : p.v);
 
   // row (permuted) or token offset (original layout) of position r (dimension 0 fastest) of a streamed tile
@@ -548,8 +556,6 @@ fna_bwd_kernel(const FnaBwdParams p) {
     return __builtin_bit_cast(vec8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
   };
 
-  const float c_log2 = p.scale * kLog2e;
-
   // One streamed tile: its two 32-row sub-blocks one after the other, each as products (S, dP),
   // probabilities, accumulations.  Only one sub-block's products are live at a time, which keeps
   // the kernel within 256 registers: two workgroups share a CU, and the other wave of a SIMD
@@ -631,8 +637,8 @@ fna_bwd_kernel(const FnaBwdParams p) {
       constexpr int i = r % 4;
       if constexpr (i == 0) load_group(std::integral_constant<int, sb * 4 + r / 4>{});
       float x;
-      if constexpr (KV_STATIONARY) x = fast_exp2(S[sb][r] * c_log2 - ls4[i]);
-      else x = fast_exp2(S[sb][r] * c_log2 - lse_l);
+      if constexpr (KV_STATIONARY) x = fast_exp2(S[sb][r] - ls4[i]);
+      else x = fast_exp2(S[sb][r] - lse_l);
       if constexpr (MASKED) {
         uint32_t ok;
         if constexpr (KV_STATIONARY) ok = (key_packed + ta[i]) & (tb[i] - key_packed) & kGuardBits;
@@ -939,7 +945,18 @@ fna_bwd_kernel(const FnaBwdParams p) {
     run_pass(std::false_type{}, n_whole * heads_walked);
   }
 
-  store_results(acc1, acc2, p.scale);
+  // dQ = scale * sum_k dS k;  dK = scale * sum_q dS q = ln 2 * sum_q dS q'
+  store_results(acc1, acc2, KV_STATIONARY ? 0.6931471805599453f : p.scale);
+}
+
+// qs = round(q * scale * log2(e)) for `chunks` runs of 8 elements: the logit operand of the
+// key-stationary roles (see scale_query_fragment).
+template <typename T>
+__global__ void __launch_bounds__(256) scale_queries_kernel(const T* q, T* qs, int64_t chunks, float c_log2) {
+  using vec8 = typename Mma<T>::vec8;
+  const int64_t i = int64_t(blockIdx.x) * 256 + threadIdx.x;
+  if (i < chunks)
+    *reinterpret_cast<vec8*>(qs + i * 8) = scale_query_fragment<T>(*reinterpret_cast<const vec8*>(q + i * 8), c_log2);
 }
 
 // delta[item] = sum_d out[item, d] * d_out[item, d] over `items` rows of D contiguous elements

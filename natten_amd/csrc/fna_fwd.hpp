@@ -163,6 +163,22 @@ struct Mma<_Float16> {
   }
 };
 
+// The logit operand of a query row: q' = round(q * scale * log2(e)) in the operand type (the
+// factor is formed in float, one multiplication per element, one rounding), clamped to the type's
+// finite range (only fp16 has one that a finite product can leave).  The forward kernel and every
+// role of the backward form their logits from q', so that they agree to the last bit of the operand.
+template <typename T>
+static __device__ __forceinline__ typename Mma<T>::vec8 scale_query_fragment(typename Mma<T>::vec8 raw, float c_log2) {
+  typename Mma<T>::vec8 out;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    float x = float(raw[e]) * c_log2;
+    if constexpr (std::is_same<T, _Float16>::value) x = fminf(fmaxf(x, -65504.f), 65504.f);
+    out[e] = static_cast<T>(x);
+  }
+  return out;
+}
+
 // LDS transpose read: the 16 lanes of a group each point at 4 consecutive 16-bit elements of
 // a row (lane 4e+j -> row e, columns 4j..4j+3 of a 4x16 block); lane c of the group receives
 // column c of the block (rows 0..3).
@@ -780,14 +796,8 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
       // The query row carries the softmax scale (in the exp2 domain) into the matrix product, so
       // that the logits leave the matrix pipe ready for exp2: q' = round(q * scale * log2(e)).
       // Rounding q' to the operand type moves a logit by about 2^-9 (bf16) / 2^-12 (fp16) of
-      // |q||k| scale / sqrt(D) -- the size of the operands' own rounding; values are clamped to
-      // the type's finite range (only fp16 has one that a finite product can leave).
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        float x = float(raw[e]) * c_log2;
-        if constexpr (std::is_same<T, _Float16>::value) x = fminf(fmaxf(x, -65504.f), 65504.f);
-        qf[mb][ks][e] = static_cast<T>(x);
-      }
+      // |q||k| scale / sqrt(D) -- the size of the operands' own rounding.
+      qf[mb][ks] = scale_query_fragment<T>(raw, c_log2);
     }
   }
 

@@ -320,7 +320,7 @@ int fused_geometry(const char* what, FnaParams& p, bool sixteen_bit, int na_dim,
 
 extern "C" {
 
-int natten_amd_abi_version(void) { return 14; }
+int natten_amd_abi_version(void) { return 15; }
 
 uint64_t natten_amd_fna_forward_workspace_bytes(void) { return uint64_t(kQueueWords) * 4; }
 
@@ -790,19 +790,32 @@ static int launch_bwd(const FnaBwdParams& params, hipStream_t stream) {
   }
   if (wg_q > 0x7fffffffLL || wg_kv > 0x7fffffffLL) return fail("fna_backward: problem needs more than 2^31 workgroups");
   const int roles = p.roles ? p.roles : 3;
+  if (roles & 2) {
+    // The key-stationary launch streams the queries as the forward kernel multiplied them: scaled
+    // and rounded once, into the workspace.  It runs before the dQ launch, so that the workspace
+    // may be the dq buffer.
+    const long long q_rows = p.cu_q ? (long long)p.seqlen_q
+                                    : p.fused ? (long long)(p.batch / p.num_groups) * p.tokens : (long long)p.batch * p.seqlen_q;
+    const long long chunks = q_rows * p.heads_q * (D / 8);
+    const long long blocks = (chunks + 255) / 256;
+    if (blocks > 0x7fffffffLL) return fail("fna_backward: problem needs more than 2^31 workgroups");
+    hipLaunchKernelGGL((scale_queries_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, stream, static_cast<const T*>(p.q),
+                       static_cast<T*>(const_cast<void*>(p.qs)), (int64_t)chunks, p.scale * 1.4426950408889634f);
+    if (int rc = check_launch("fna_backward (scaled queries)")) return rc;
+    if constexpr (D == 128) {
+      // dK and dV by wave pairs (eight waves per workgroup): one wave's registers cannot hold the
+      // accumulators, fragments and products of both
+      hipLaunchKernelGGL((fna_bwd_kernel<T, D, kBwdPair, VARLEN>), dim3((unsigned)wg_kv), dim3(512), 0, stream, p);
+    } else {
+      hipLaunchKernelGGL((fna_bwd_kernel<T, D, kBwdDKV, VARLEN>), dim3((unsigned)wg_kv), dim3(256), 0, stream, p);
+    }
+    if (int rc = check_launch("fna_backward (dK, dV)")) return rc;
+  }
   if (roles & 1) {
     hipLaunchKernelGGL((fna_bwd_kernel<T, D, kBwdDQ, VARLEN>), dim3((unsigned)wg_q), dim3(256), 0, stream, p);
     if (int rc = check_launch("fna_backward (dQ)")) return rc;
   }
-  if (!(roles & 2)) return 0;
-  if constexpr (D == 128) {
-    // dK and dV by wave pairs (eight waves per workgroup): one wave's registers cannot hold the
-    // accumulators, fragments and products of both
-    hipLaunchKernelGGL((fna_bwd_kernel<T, D, kBwdPair, VARLEN>), dim3((unsigned)wg_kv), dim3(512), 0, stream, p);
-  } else {
-    hipLaunchKernelGGL((fna_bwd_kernel<T, D, kBwdDKV, VARLEN>), dim3((unsigned)wg_kv), dim3(256), 0, stream, p);
-  }
-  return check_launch("fna_backward (dK, dV)");
+  return 0;
 }
 
 template <typename T>
@@ -834,8 +847,12 @@ static int split_dim_of(const int* tile) {
 }
 
 static int check_bwd_pointers(const char* what, const void* q, const void* k, const void* v, const void* d_out,
-                              const float* lse, const float* delta, void* dq, void* dk, void* dv) {
+                              const float* lse, const float* delta, void* dq, void* dk, void* dv, void* q_scaled,
+                              int roles) {
   if (!q || !k || !v || !d_out || !lse || !delta || !dq || !dk || !dv) return fail("%s: null pointer argument", what);
+  if ((roles & 2) && !q_scaled) return fail("%s: the dk / dv launch needs the q_scaled workspace", what);
+  if (q_scaled == q) return fail("%s: q_scaled must not be q itself (the dq launch reads the unscaled queries)", what);
+  if (reinterpret_cast<uintptr_t>(q_scaled) & 15) return fail("%s: q_scaled must be 16-byte aligned", what);
   const uintptr_t all = reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v) |
                         reinterpret_cast<uintptr_t>(d_out) | reinterpret_cast<uintptr_t>(dq) |
                         reinterpret_cast<uintptr_t>(dk) | reinterpret_cast<uintptr_t>(dv);
@@ -844,15 +861,15 @@ static int check_bwd_pointers(const char* what, const void* q, const void* k, co
 }
 
 int natten_amd_fna_backward(const void* q, const void* k, const void* v, const void* d_out, const float* lse,
-                            const float* delta, void* dq, void* dk, void* dv, int dtype, int na_dim, int batch,
-                            int seqlen_q, int seqlen_kv, int heads_q, int heads_kv, int head_dim,
+                            const float* delta, void* dq, void* dk, void* dv, void* q_scaled, int dtype, int na_dim,
+                            int batch, int seqlen_q, int seqlen_kv, int heads_q, int heads_kv, int head_dim,
                             const int32_t* q_shape, const int32_t* kv_shape, const int32_t* qkv_shape,
                             const int32_t* kernel_size, const int32_t* stride, const int32_t* dilation,
                             const int32_t* is_causal, const int32_t* q_tile_shape, const int32_t* kv_tile_shape,
                             float scale, void* stream) {
   g_error[0] = 0;
   const char* what = "fna_backward";
-  if (int rc = check_bwd_pointers(what, q, k, v, d_out, lse, delta, dq, dk, dv)) return rc;
+  if (int rc = check_bwd_pointers(what, q, k, v, d_out, lse, delta, dq, dk, dv, q_scaled, 3)) return rc;
   if (int rc = check_common(what, q, k, v, dq, lse, batch, seqlen_q, seqlen_kv, heads_q, heads_kv, head_dim)) return rc;
   if (na_dim < 1 || na_dim > 3) return fail("%s: na_dim must be 1, 2 or 3, got %d", what, na_dim);
   if (!q_shape || !kv_shape || !qkv_shape || !kernel_size || !stride || !dilation || !is_causal || !q_tile_shape ||
@@ -888,6 +905,7 @@ int natten_amd_fna_backward(const void* q, const void* k, const void* v, const v
     return fail("%s: sequence lengths (%d, %d) do not match the padded layouts (%d, %d)", what, seqlen_q, seqlen_kv,
                 prod3(p.q_tiled) * 128, prod3(p.kv_tiled) * 128);
   p.q = q;
+  p.qs = q_scaled;
   p.k = k;
   p.v = v;
   p.d_out = d_out;
@@ -908,16 +926,16 @@ int natten_amd_fna_backward(const void* q, const void* k, const void* v, const v
 }
 
 int natten_amd_fna_backward_fused(const void* q, const void* k, const void* v, const void* d_out, const float* lse,
-                                  const float* delta, void* dq, void* dk, void* dv, int dtype, int na_dim, int batch,
-                                  int heads_q, int heads_kv, int head_dim, const int32_t* qkv_shape,
+                                  const float* delta, void* dq, void* dk, void* dv, void* q_scaled, int dtype, int na_dim,
+                                  int batch, int heads_q, int heads_kv, int head_dim, const int32_t* qkv_shape,
                                   const int32_t* kernel_size, const int32_t* stride, const int32_t* dilation,
                                   const int32_t* is_causal, const int32_t* q_tile_shape, const int32_t* kv_tile_shape,
                                   float scale, int roles, void* stream) {
   g_error[0] = 0;
   const char* what = "fna_backward_fused";
-  if (int rc = check_bwd_pointers(what, q, k, v, d_out, lse, delta, dq, dk, dv)) return rc;
-  if (na_dim < 1 || na_dim > 3) return fail("%s: na_dim must be 1, 2 or 3, got %d", what, na_dim);
   if (roles < 1 || roles > 3) return fail("%s: roles must be 1 (dq), 2 (dk and dv) or 3 (all), got %d", what, roles);
+  if (int rc = check_bwd_pointers(what, q, k, v, d_out, lse, delta, dq, dk, dv, q_scaled, roles)) return rc;
+  if (na_dim < 1 || na_dim > 3) return fail("%s: na_dim must be 1, 2 or 3, got %d", what, na_dim);
   if (!qkv_shape || !kernel_size || !stride || !dilation || !is_causal || !q_tile_shape || !kv_tile_shape)
     return fail("%s: null shape argument", what);
   // Per-group layouts, padded to whole tiles.  Extents that are not multiples of dilation x tile are
@@ -976,6 +994,7 @@ int natten_amd_fna_backward_fused(const void* q, const void* k, const void* v, c
     groups *= f.dil[a];
   }
   p.q = q;
+  p.qs = q_scaled;
   p.k = k;
   p.v = v;
   p.d_out = d_out;
@@ -1000,12 +1019,12 @@ int natten_amd_fna_backward_fused(const void* q, const void* k, const void* v, c
 }
 
 int natten_amd_attention_backward(const void* q, const void* k, const void* v, const void* d_out, const float* lse,
-                                  const float* delta, void* dq, void* dk, void* dv, int dtype, int batch,
+                                  const float* delta, void* dq, void* dk, void* dv, void* q_scaled, int dtype, int batch,
                                   int seqlen_q, int seqlen_kv, int padded_seqlen_q, int padded_seqlen_kv, int heads_q,
                                   int heads_kv, int head_dim, int is_causal, float scale, void* stream) {
   g_error[0] = 0;
   const char* what = "attention_backward";
-  if (int rc = check_bwd_pointers(what, q, k, v, d_out, lse, delta, dq, dk, dv)) return rc;
+  if (int rc = check_bwd_pointers(what, q, k, v, d_out, lse, delta, dq, dk, dv, q_scaled, 3)) return rc;
   if (int rc = check_common(what, q, k, v, dq, lse, batch, seqlen_q, seqlen_kv, heads_q, heads_kv, head_dim)) return rc;
   if (padded_seqlen_q % 128 != 0 || padded_seqlen_kv % 128 != 0 || padded_seqlen_q < seqlen_q ||
       padded_seqlen_kv < seqlen_kv)
@@ -1025,6 +1044,7 @@ int natten_amd_attention_backward(const void* q, const void* k, const void* v, c
   p.kv_tiled[0] = padded_seqlen_kv / 128;
   p.q_extent0 = seqlen_q;
   p.q = q;
+  p.qs = q_scaled;
   p.k = k;
   p.v = v;
   p.d_out = d_out;
@@ -1044,15 +1064,15 @@ int natten_amd_attention_backward(const void* q, const void* k, const void* v, c
 }
 
 int natten_amd_attention_backward_varlen(const void* q, const void* k, const void* v, const void* d_out,
-                                         const float* lse, const float* delta, void* dq, void* dk, void* dv, int dtype,
-                                         int num_seqs, int rows_q, int rows_kv, const int32_t* cu_seqlens_q,
+                                         const float* lse, const float* delta, void* dq, void* dk, void* dv,
+                                         void* q_scaled, int dtype, int num_seqs, int rows_q, int rows_kv, const int32_t* cu_seqlens_q,
                                          const int32_t* cu_seqlens_kv, const int32_t* padded_cu_seqlens_q,
                                          const int32_t* padded_cu_seqlens_kv, int max_seqlen_q, int max_seqlen_kv,
                                          int heads_q, int heads_kv, int head_dim, int is_causal, float scale,
                                          void* stream) {
   g_error[0] = 0;
   const char* what = "attention_backward_varlen";
-  if (int rc = check_bwd_pointers(what, q, k, v, d_out, lse, delta, dq, dk, dv)) return rc;
+  if (int rc = check_bwd_pointers(what, q, k, v, d_out, lse, delta, dq, dk, dv, q_scaled, 3)) return rc;
   if (int rc = check_common(what, q, k, v, dq, lse, num_seqs, rows_q, rows_kv, heads_q, heads_kv, head_dim)) return rc;
   if (!cu_seqlens_q || !cu_seqlens_kv || !padded_cu_seqlens_q || !padded_cu_seqlens_kv)
     return fail("%s: null cumulative length argument", what);
@@ -1074,6 +1094,7 @@ int natten_amd_attention_backward_varlen(const void* q, const void* k, const voi
   p.q_tiled[0] = (max_seqlen_q + 127) / 128;
   p.kv_tiled[0] = (max_seqlen_kv + 127) / 128;
   p.q = q;
+  p.qs = q_scaled;
   p.k = k;
   p.v = v;
   p.d_out = d_out;

@@ -162,18 +162,26 @@ def test_backward_entry_point_rejects_tiles_beyond_32_bit_offsets():
     i32 = lambda xs: (C.c_int32 * 3)(*xs)
     ptr = 0x10000
     rc = L.natten_amd_fna_backward_fused(
-        ptr, ptr, ptr, ptr, ptr, ptr, ptr, ptr, ptr, _lib.DTYPE_CODES[__import__("torch").bfloat16], 3, 1, 24, 24, 128,
+        ptr, ptr, ptr, ptr, ptr, ptr, ptr, ptr, ptr, 2 * ptr, _lib.DTYPE_CODES[__import__("torch").bfloat16], 3, 1, 24, 24, 128,
         i32((128, 512, 512)), i32((3, 3, 3)), i32((1, 1, 1)), i32((1, 1, 1)), i32((0, 0, 0)), i32((128, 1, 1)),
         i32((2, 8, 8)), C.c_float(0.1), 3, None,
     )
     assert rc != 0 and b"2^31 bytes" in L.natten_amd_last_error()
     # `roles` names the launches to make: 1 (dq), 2 (dk and dv) or 3
     rc = L.natten_amd_fna_backward_fused(
-        ptr, ptr, ptr, ptr, ptr, ptr, ptr, ptr, ptr, _lib.DTYPE_CODES[__import__("torch").bfloat16], 3, 1, 24, 24, 128,
+        ptr, ptr, ptr, ptr, ptr, ptr, ptr, ptr, ptr, 2 * ptr, _lib.DTYPE_CODES[__import__("torch").bfloat16], 3, 1, 24, 24, 128,
         i32((16, 16, 16)), i32((3, 3, 3)), i32((1, 1, 1)), i32((1, 1, 1)), i32((0, 0, 0)), i32((2, 8, 8)),
         i32((2, 8, 8)), C.c_float(0.1), 0, None,
     )
     assert rc != 0 and b"roles" in L.natten_amd_last_error()
+    # the dk / dv launch needs the workspace of the scaled queries, which cannot be q itself
+    for q_scaled, roles, message in ((None, 2, b"q_scaled workspace"), (None, 3, b"q_scaled workspace"), (ptr, 3, b"must not be q")):
+        rc = L.natten_amd_fna_backward_fused(
+            ptr, 3 * ptr, 3 * ptr, 3 * ptr, 3 * ptr, 3 * ptr, 3 * ptr, 3 * ptr, 3 * ptr, q_scaled,
+            _lib.DTYPE_CODES[__import__("torch").bfloat16], 3, 1, 24, 24, 128, i32((16, 16, 16)), i32((3, 3, 3)),
+            i32((1, 1, 1)), i32((1, 1, 1)), i32((0, 0, 0)), i32((2, 8, 8)), i32((2, 8, 8)), C.c_float(0.1), roles, None,
+        )
+        assert rc != 0 and message in L.natten_amd_last_error(), L.natten_amd_last_error()
 
 
 def test_every_entry_point_rejects_null_arguments_before_touching_a_device():
