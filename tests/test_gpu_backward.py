@@ -151,6 +151,22 @@ def test_backward_random_sweep():
         done += 1
 
 
+@pytest.mark.parametrize("case", [
+    # (H, Hkv, D, shape, k, s, d, causal, seed): windows of one or two keys, where a probability is 1
+    # or close to it.  Formed from other logits than the forward's (queries scaled after the matrix
+    # product instead of before it), such a probability came out as 1 +- 0.5 % and dv missed the
+    # tolerance by up to a factor of two; formed from the forward's own operand it is exact.
+    (4, 2, 64, (24,), (3,), (1,), (3,), (True,), 27693),
+    (2, 1, 64, (55,), (2,), (2,), (13,), (True,), 27895),
+    (2, 1, 128, (230,), (10,), (5,), (16,), (True,), 27897),
+    (4, 2, 64, (34, 28), (2, 3), (2, 2), (7, 5), (True, True), 28641),
+    (2, 1, 32, (7, 10, 10), (2, 10, 2), (2, 1, 2), (1, 1, 1), (True, True, True), 27707),
+])
+def test_backward_uses_the_forward_logits(case):
+    H, Hkv, D, shape, k, s, d, causal, seed = case
+    run_backward(1, H, Hkv, D, shape, k, s, d, causal, torch.bfloat16, seed=seed)
+
+
 ATTN_CASES = [
     # B, Sq, Skv, H, Hkv, D, causal
     (2, 128, 128, 2, 2, 64, False),

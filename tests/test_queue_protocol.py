@@ -8,9 +8,17 @@ Two models, both exhaustive over every interleaving of a small launch:
   the last workgroup out has begun to store zeros, and the block is all zero when the launch ends;
 * the hand-over of a position from thread 0 to the other waves of its workgroup through the two LDS
   slots of fna_queue_loop (natten_amd/csrc/fna_fwd.hpp): every wave reads, for every tile, the value
-  thread 0 wrote for that tile.
+  thread 0 wrote for that tile.  LDS stores are modelled as the hardware performs them: issued by the
+  wave, performed at some later point unless the wave waits for its LDS operations (`s_waitcnt
+  lgkmcnt(0)`), and a barrier by itself does not wait for them.  The kernels therefore enter every
+  barrier through workgroup_sync(), which waits first; without that wait a wave released by the barrier
+  can read the slot before thread 0's store has been performed and gets the position of two tiles
+  earlier -- the fault the work-queue launch had on launch positions past the end of a problem, where
+  the compiler had placed no wait between the store and the barrier.
 
-Each model is also run on a deliberately broken protocol, which it must reject.
+Each model is also run on deliberately broken protocols (zeros stored by the first workgroup out, a
+return to a retired queue, counters that do not start at zero; one slot instead of two, a barrier
+without the wait), which it must reject.
 """
 
 from __future__ import annotations
