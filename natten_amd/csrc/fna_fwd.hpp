@@ -371,11 +371,12 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
   // What the element mask of a PARTIAL tile needs (absent from NOMASK instances), kept in LDS and read
   // where such a tile is met -- in registers for the whole loop these values would push the loop's own
   // out to spill lanes:
-  //   sKeys[a][x]  the keys of a tile whose coordinate along dimension a is >= x, one bit per key
+  //   sKeys[a][g][x]  the keys of a tile whose coordinate along dimension a is >= x, one bit per key:
+  //                   the 32 bits that the lanes of wave half g hold logits for (na_lane_half_bits)
   //   sWin[row]    window of the Q tile's query `row` (row-major): start and end per dimension
   //   sGeo[a]      KV tile extent along dimension a
   constexpr int MASK_ROWS = NOMASK ? 1 : KVT + 1;
-  __shared__ __attribute__((aligned(16))) uint64_t sKeys[NOMASK ? 1 : 3][MASK_ROWS];
+  __shared__ __attribute__((aligned(16))) uint32_t sKeys[NOMASK ? 1 : 3][2][MASK_ROWS];
   __shared__ __attribute__((aligned(16))) int sWin[NOMASK ? 1 : NWAVES * MQ * 32][8];
   __shared__ __attribute__((aligned(16))) int sGeo[4];
   static_assert(NOMASK || KVT == 64, "the element mask holds one bit per key of a 64-key tile");
@@ -544,7 +545,11 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
     int lg_stride = 0;
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
-      if (tid <= p.kv_tile[a]) sKeys[a][tid] = na_keys_at_or_after(tid, lg_stride, p.kv_tile_lg[a]);
+      if (tid <= p.kv_tile[a]) {
+        const uint64_t keys = na_keys_at_or_after(tid, lg_stride, p.kv_tile_lg[a]);
+        sKeys[a][0][tid] = na_lane_half_bits(keys, 0);
+        sKeys[a][1][tid] = na_lane_half_bits(keys, 1);
+      }
       lg_stride += p.kv_tile_lg[a];
     }
   }
@@ -906,14 +911,13 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
 
   // Element mask of a PARTIAL tile for row block mb.  Per dimension the lane's window, relative to the
   // tile origin and clamped to the tile, selects two rows of sKeys (keys at or after its start, keys at
-  // or after its end); the AND over the dimensions has one bit per key of the tile.  A tile moved back
-  // from the group's edge starts before its place in the tiling (the box origin plus a multiple of the
-  // tile extent): the keys up to there (`lead`) belong to the tile before it.
-  // the keys of the tile at `origin` that the lane's query of row block mb attends, one bit per key,
-  // shifted so that bit 32 sb + 8 (r / 4) + r % 4 belongs to the lane's logit r of sub-block sb
-  // (which is key 32 sb + 8 (r / 4) + 4 g + r % 4 of the tile)
-  auto mask_keys = [&](int mb, const int (&origin)[3], const int (&lead)[3]) __attribute__((always_inline)) {
-    uint64_t keys = ~uint64_t(0);
+  // or after its end); the AND over the dimensions has one bit per logit of the lane: bit 16 sb + r
+  // for logit r of sub-block sb.  A tile moved back from the group's edge starts before its place in
+  // the tiling (the box origin plus a multiple of the tile extent): the keys up to there (`lead`)
+  // belong to the tile before it.  All six rows are read at once (one register each), so that a
+  // masked tile waits for LDS twice -- the windows, then the rows -- and not once per dimension.
+  auto mask_bits = [&](int mb, const int (&origin)[3], const int (&lead)[3]) __attribute__((always_inline)) {
+    uint32_t bits = ~uint32_t(0);
     if constexpr (!NOMASK) {
       typedef int i32x4 __attribute__((ext_vector_type(4)));
       typedef int i32x2 __attribute__((ext_vector_type(2)));
@@ -921,38 +925,39 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
       const i32x4 w01 = *reinterpret_cast<const i32x4*>(&sWin[row][0]);
       const i32x2 w2 = *reinterpret_cast<const i32x2*>(&sWin[row][4]);
       const int ws[3] = {w01[0], w01[2], w2[0]}, we[3] = {w01[1], w01[3], w2[1]};
+      int lo[3], hi[3];
 #pragma unroll
       for (int a = 0; a < 3; ++a) {
         const int kt = sGeo[a];
-        const int lo = na_min(na_max(ws[a] - origin[a], lead[a]), kt);
-        const int hi = na_min(na_max(we[a] - origin[a], 0), kt);
-        keys &= sKeys[a][lo] & ~sKeys[a][hi];
+        lo[a] = na_min(na_max(ws[a] - origin[a], lead[a]), kt);
+        hi[a] = na_min(na_max(we[a] - origin[a], 0), kt);
       }
-      keys >>= 4 * g;
+      uint32_t from[3], upto[3];
+#pragma unroll
+      for (int a = 0; a < 3; ++a) {
+        from[a] = sKeys[a][g][lo[a]];
+        upto[a] = sKeys[a][g][hi[a]];
+      }
+#pragma unroll
+      for (int a = 0; a < 3; ++a) bits &= from[a] & ~upto[a];
     }
-    return keys;
+    return bits;
   };
-  // logit r of sub-block sb: kept where its key's bit is set, else -inf; two instructions (the
+  // logit r of sub-block sb: kept where its bit is set, else -inf; two instructions (the
   // sign-extended bit, a bitwise select) and no condition codes
-  auto mask_elem = [&](f32x16_t (&S)[NSB], int sb, int r, const uint64_t keys) __attribute__((always_inline)) {
-    const uint32_t half = uint32_t(keys >> (32 * sb));
-    const uint32_t keep = uint32_t(__builtin_amdgcn_sbfe(int(half), 8 * (r / 4) + r % 4, 1));  // 0 or ~0
+  auto mask_elem = [&](f32x16_t (&S)[NSB], int sb, int r, const uint32_t lane_bits) __attribute__((always_inline)) {
+    const uint32_t keep = uint32_t(__builtin_amdgcn_sbfe(int(lane_bits), 16 * sb + r, 1));  // 0 or ~0
     const float logit = S[sb][r];  // (a copy: a bit cast of the vector element itself reads element 0)
     const uint32_t bits = __builtin_bit_cast(uint32_t, logit);
     S[sb][r] = __builtin_bit_cast(float, (bits & keep) | (~keep & 0xff800000u));
   };
-  // Element mask of a PARTIAL tile for row block mb.  Per dimension the lane's window, relative to the
-  // tile origin and clamped to the tile, selects two rows of sKeys (keys at or after its start, keys at
-  // or after its end); the AND over the dimensions has one bit per key of the tile.  A tile moved back
-  // from the group's edge starts before its place in the tiling (the box origin plus a multiple of the
-  // tile extent): the keys up to there (`lead`) belong to the tile before it.
   auto apply_mask = [&](f32x16_t (&S)[NSB], int mb, const int (&origin)[3], const int (&lead)[3]) __attribute__((always_inline)) {
     if constexpr (!NOMASK) {
-      const uint64_t keys = mask_keys(mb, origin, lead);
+      const uint32_t lane_bits = mask_bits(mb, origin, lead);
 #pragma unroll
       for (int sb = 0; sb < NSB; ++sb)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) mask_elem(S, sb, r, keys);
+        for (int r = 0; r < 16; ++r) mask_elem(S, sb, r, lane_bits);
     }
   };
 

@@ -84,6 +84,31 @@ NA_HD uint64_t na_keys_at_or_after(int x, int lg_stride, int lg_extent) {
   return m;
 }
 
+// A lane of the forward kernels holds 32 of a tile's 64 logits: logit r (0..15) of sub-block sb
+// (0..1) belongs to key 32 sb + 8 (r / 4) + 4 g + r % 4, where g is the lane's half of the wave.
+// The bits of a key set that a lane of half g needs, bit 16 sb + r for its logit (sb, r): of every
+// byte of the set the nibble at 4 g, the eight nibbles packed into one word.
+NA_HD uint32_t na_lane_half_bits(uint64_t keys, int g) {
+  uint32_t out = 0;
+  for (int sb = 0; sb < 2; ++sb) {
+    uint32_t w = uint32_t(keys >> (32 * sb + 4 * g)) & 0x0f0f0f0fu;  // nibbles of keys 8 m + 4 g .. + 3 at bits 8 m
+    w = (w | (w >> 4)) & 0x00ff00ffu;
+    w = (w | (w >> 8)) & 0x0000ffffu;
+    out |= w << (16 * sb);
+  }
+  return out;
+}
+// ... and back: the key set whose bits for both halves are `half0` and `half1` (host-side checks).
+NA_HD uint64_t na_keys_of_lane_halves(uint32_t half0, uint32_t half1) {
+  uint64_t keys = 0;
+  for (int g = 0; g < 2; ++g)
+    for (int b = 0; b < 32; ++b) {
+      const int sb = b >> 4, r = b & 15;
+      if (((g ? half1 : half0) >> b) & 1u) keys |= uint64_t(1) << (32 * sb + 8 * (r / 4) + 4 * g + r % 4);
+    }
+  return keys;
+}
+
 // Number of tokens of dilation group g along a dimension of extent X.
 NA_HD int na_group_extent(int X, int d, int g) { return X / d + 1 - ((g + (d - X % d)) / d); }
 

@@ -351,14 +351,17 @@ int natten_amd_tile_key_mask(const int32_t* kv_tile_shape, const int32_t* lo, co
     keys *= kv_tile_shape[a];
   }
   if (keys != 64) return fail("tile_key_mask: the tile must hold 64 keys, got %d", keys);
-  // the rows the kernels keep in LDS and how their element mask combines them
-  uint64_t m = ~uint64_t(0);
+  // the rows the kernels keep in LDS (per half of the wave: the bits its lanes hold logits for) and
+  // how their element mask combines them
+  uint32_t half[2] = {~uint32_t(0), ~uint32_t(0)};
   int lg_stride = 0;
   for (int a = 0; a < 3; ++a) {
-    m &= na_keys_at_or_after(lo[a], lg_stride, lg[a]) & ~na_keys_at_or_after(hi[a], lg_stride, lg[a]);
+    for (int g = 0; g < 2; ++g)
+      half[g] &= na_lane_half_bits(na_keys_at_or_after(lo[a], lg_stride, lg[a]), g) &
+                 ~na_lane_half_bits(na_keys_at_or_after(hi[a], lg_stride, lg[a]), g);
     lg_stride += lg[a];
   }
-  *mask = m;
+  *mask = na_keys_of_lane_halves(half[0], half[1]);
   return 0;
 }
 
