@@ -235,6 +235,19 @@ int natten_amd_fna_fully_block_sparse(int na_dim, const int32_t* qkv_shape,
                                       int anchor_kv_tiles, int32_t* result);
 
 /*
+ * Host arithmetic only: the box of 32 queries (extents per dimension, product 32) that one wave of
+ * the 16-bit forward kernels holds for this problem.  A Q tile is a grid of such boxes; a (wave, KV
+ * tile) pair needs the element mask unless the tile lies inside the windows of all of the wave's
+ * queries or outside all of them, and the launch takes the box with the fewest pairs that do (the
+ * row-major box on ties).  No counterpart in the reference, whose threads own rows of a fixed
+ * layout.
+ */
+int natten_amd_fna_wave_box(int na_dim, const int32_t* qkv_shape, const int32_t* kernel_size,
+                            const int32_t* stride, const int32_t* dilation,
+                            const int32_t* is_causal, const int32_t* q_tile_shape,
+                            const int32_t* kv_tile_shape, int anchor_kv_tiles, int32_t* box);
+
+/*
  * Supported tile sizes (tokens per tile).  Writes up to `capacity` pairs
  * (q_tile_size, kv_tile_size) for the given dtype / head_dim and returns how many exist.
  */

@@ -22,7 +22,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 # NATTEN_AMD_LIBRARY: another build of the library (the timing-only ones of natten_amd.build --ablate)
 LIB_PATH = os.environ.get("NATTEN_AMD_LIBRARY") or os.path.join(_HERE, "libnatten_amd.so")
 
-ABI_VERSION = 15
+ABI_VERSION = 16
 
 DTYPE_CODES = {
     torch.float16: 0,
@@ -42,6 +42,7 @@ _SIGNATURES = {
     "natten_amd_window": (ctypes.c_int, [ctypes.c_int] * 5 + [ctypes.c_void_p] * 2),
     "natten_amd_tile_key_mask": (ctypes.c_int, [ctypes.c_void_p] * 4),
     "natten_amd_fna_fully_block_sparse": (ctypes.c_int, [ctypes.c_int] + [ctypes.c_void_p] * 7 + [ctypes.c_int, ctypes.c_void_p]),
+    "natten_amd_fna_wave_box": (ctypes.c_int, [ctypes.c_int] + [ctypes.c_void_p] * 7 + [ctypes.c_int, ctypes.c_void_p]),
     "natten_amd_fna_supported_tiles": (
         ctypes.c_int,
         [ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int],
@@ -501,6 +502,18 @@ def fully_block_sparse(qkv_shape, kernel_size, stride, dilation, is_causal, q_ti
         _i32([1 if c else 0 for c in is_causal]), _i32(q_tile_shape), _i32(kv_tile_shape), 1 if anchored_tiles else 0,
         ctypes.addressof(r)))
     return bool(r.value)
+
+
+def wave_box(qkv_shape, kernel_size, stride, dilation, is_causal, q_tile_shape, kv_tile_shape,
+             anchored_tiles: bool = True) -> Tuple[int, ...]:
+    """The box of 32 queries that one wave of the 16-bit forward kernels holds for this problem
+    (host arithmetic only)."""
+    box = (ctypes.c_int32 * len(qkv_shape))()
+    _check(lib().natten_amd_fna_wave_box(
+        len(qkv_shape), _i32(qkv_shape), _i32(kernel_size), _i32(stride), _i32(dilation),
+        _i32([1 if c else 0 for c in is_causal]), _i32(q_tile_shape), _i32(kv_tile_shape), 1 if anchored_tiles else 0,
+        ctypes.addressof(box)))
+    return tuple(int(x) for x in box)
 
 
 def query_range(key_first: int, key_last: int, kernel_size: int, stride: int, extent: int, num_queries: int,

@@ -80,6 +80,10 @@ struct FnaParams {
   // Derived by set_wg_layout(): what the per-workgroup set-up would otherwise divide for.
   // Tile extents are powers of two (log2 below); the other divisors get multiply-shift pairs.
   int q_tile_lg[3], kv_tile_lg[3];
+  // log2 extents of the box of 32 queries that a wave's lanes hold (sum 5, each <= q_tile_lg): the Q
+  // tile is a grid of such boxes, one per wave and row block.  Chosen per launch (choose_wave_box) so
+  // that as many (wave, KV tile) pairs as possible need no element mask.
+  int wave_box_lg[3];
   int ext_base[3], ext_rem[3];  // qkv_shape / dil and qkv_shape % dil: extent of dilation group g = base + (g < rem)
   NaDiv d_stride[3], d_dil[3], d_q_tiled[3];
   NaDiv d_wg_group, d_groups_per_bh, d_heads_q, d_q_per_kv, d_num_groups;
@@ -497,31 +501,36 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
   }
 
   // ---- this wave's share of the Q tile ------------------------------------------------------------
-  // Lanes take the tile's tokens in row-major order (dimension 0 slowest), MQ * 32 consecutive
-  // ones per wave, so that a wave covers a compact box of queries; the token's row inside the
-  // permuted tile (dimension 0 fastest) follows from its coordinates.  Window starts and ends
+  // The Q tile is a grid of boxes of 32 queries (extents 2^wave_box_lg, dimension 2 fastest inside a
+  // box and across the grid); row block mb of wave w holds box w * MQ + mb, one query per lane of each
+  // half of the wave.  With the default box (as much of dimension 2 as fits, then of dimension 1, ...)
+  // the lanes take the tile's tokens in row-major order.  The token's row inside the permuted tile
+  // (dimension 0 fastest) follows from its coordinates.  Window starts and ends
   // are monotone in the query coordinate, hence over the wave's bounding box the union of the
   // windows is [start(min), end(max)) and their intersection [start(max), end(min)) per
   // dimension: a KV tile outside the union is skipped by this wave, one inside the
   // intersection needs no mask.
+  auto box_origin = [&](int block, int (&o)[3]) {
+#pragma unroll
+    for (int a = 2; a >= 0; --a) {
+      const int nb = p.q_tile_lg[a] - p.wave_box_lg[a];  // log2 boxes along this dimension
+      o[a] = (block & ((1 << nb) - 1)) << p.wave_box_lg[a];
+      block >>= nb;
+    }
+  };
   int wave_lo[3], wave_hi[3], wave_full_lo[3], wave_full_hi[3];
   if constexpr (!NOMASK) {
-    const int i0 = wave * (MQ * 32), i1 = i0 + MQ * 32 - 1;
-    const int lg2 = p.q_tile_lg[2], lg12 = p.q_tile_lg[1] + p.q_tile_lg[2];
     int f[3], l[3];
-    f[0] = i0 >> lg12;
-    f[1] = (i0 >> lg2) & (p.q_tile[1] - 1);
-    f[2] = i0 & (p.q_tile[2] - 1);
-    l[0] = i1 >> lg12;
-    l[1] = (i1 >> lg2) & (p.q_tile[1] - 1);
-    l[2] = i1 & (p.q_tile[2] - 1);
-    if (f[0] != l[0]) {
-      f[1] = 0;
-      l[1] = p.q_tile[1] - 1;
-    }
-    if (f[0] != l[0] || f[1] != l[1]) {
-      f[2] = 0;
-      l[2] = p.q_tile[2] - 1;
+#pragma unroll
+    for (int mb = 0; mb < MQ; ++mb) {
+      int o[3];
+      box_origin(wave * MQ + mb, o);
+#pragma unroll
+      for (int a = 0; a < 3; ++a) {
+        const int last = o[a] + (1 << p.wave_box_lg[a]) - 1;
+        f[a] = mb == 0 ? o[a] : na_min(f[a], o[a]);
+        l[a] = mb == 0 ? last : na_max(l[a], last);
+      }
     }
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
@@ -759,12 +768,16 @@ static __device__ __forceinline__ void fna_fwd_tile(const FnaParams& p, const in
   vec8 qf[MQ][KSTEPS];
 #pragma unroll
   for (int mb = 0; mb < MQ; ++mb) {
-    int r = (wave * MQ + mb) * 32 + l32;  // row-major index inside the tile
-    int off[3];
-    off[2] = r & (p.q_tile[2] - 1);
-    r >>= p.q_tile_lg[2];
-    off[1] = r & (p.q_tile[1] - 1);
-    off[0] = r >> p.q_tile_lg[1];
+    int off[3];  // the lane's query inside the tile: its box's origin plus its place in the box
+    box_origin(wave * MQ + mb, off);
+    {
+      int r = l32;
+#pragma unroll
+      for (int a = 2; a >= 0; --a) {
+        off[a] += r & ((1 << p.wave_box_lg[a]) - 1);
+        r >>= p.wave_box_lg[a];
+      }
+    }
     int row = qtile_idx * QT + off[0] + p.q_tile[0] * (off[1] + p.q_tile[1] * off[2]);
     bool valid = row < seqlen_q;
     int row_c = na_min(row, seqlen_q - 1);
@@ -1366,6 +1379,71 @@ __global__ void fna_queue_clear_kernel(uint32_t* queues) {
 // dimension-0 slabs when possible, so that the tiles resident on an XCD overlap in their KV boxes.
 // `tiles_per_wg` Q tiles share a workgroup (consecutive tiles of the enumeration) and an XCD keeps
 // about 64 Q tiles resident either way (32 CUs x 2 single-tile workgroups or x 1 two-tile workgroup).
+// The box of 32 queries that a wave holds (FnaParams::wave_box_lg).  A (wave, KV tile) pair needs
+// the element mask unless the tile lies inside the windows of all of the wave's queries or outside
+// all of them, and both conditions factor over the dimensions: the number of pairs that need none is
+// a product of per-dimension sums over Q tiles, boxes and KV tiles, cheap to count on the host with
+// the kernels' own window and box arithmetic.  Of the boxes that fit the Q tile the one with the
+// fewest pairs that need the mask is taken; the row-major box (as much of dimension 2 as fits, then
+// dimension 1, then 0) on ties, and for sequence-packed launches, whose extents only the device knows.
+inline void choose_wave_box(FnaParams& p) {
+  int best[3], left = 5;
+  for (int a = 2; a >= 0; --a) {
+    best[a] = p.q_tile_lg[a] < left ? p.q_tile_lg[a] : left;
+    left -= best[a];
+  }
+  for (int a = 0; a < 3; ++a) p.wave_box_lg[a] = best[a];
+  if (p.cu_q) return;
+  // per dimension and box extent: (wave box, KV tile) pairs attended in full / attended at all,
+  // summed over the Q tiles
+  double full[3][6], some[3][6];
+  for (int a = 0; a < 3; ++a) {
+    const int L = p.ext_base[a] + (p.ext_rem[a] ? 1 : 0), kt = p.kv_tile[a], qt = p.q_tile[a];
+    const bool causal = p.causal[a] != 0;
+    for (int wb = 0; wb <= 5; ++wb) {
+      full[a][wb] = some[a][wb] = 0;
+      if (wb > p.q_tile_lg[a]) continue;
+      const int box = 1 << wb;
+      for (int q0 = 0; q0 < L; q0 += qt) {
+        const int q_last = na_min(q0 + qt - 1, L - 1);
+        const int st_f = na_window_start(q0, p.ksize[a], p.stride[a], L, causal);
+        const int st_l = na_window_start(q_last, p.ksize[a], p.stride[a], L, causal);
+        const int en_l = na_window_end(q_last, st_l, p.ksize[a], L, causal);
+        const int org = (p.anchor && L >= kt) ? st_f : (st_f / kt) * kt;
+        const int tiles = (en_l - org + kt - 1) / kt;
+        for (int b0 = 0; b0 < qt; b0 += box) {
+          const int qmin = na_min(q0 + b0, L - 1), qmax = na_min(q0 + b0 + box - 1, L - 1);
+          const int st_min = na_window_start(qmin, p.ksize[a], p.stride[a], L, causal);
+          const int st_max = na_window_start(qmax, p.ksize[a], p.stride[a], L, causal);
+          const int en_min = na_window_end(qmin, st_min, p.ksize[a], L, causal);
+          const int en_max = na_window_end(qmax, st_max, p.ksize[a], L, causal);
+          for (int t = 0; t < tiles; ++t) {
+            const int o = org + t * kt, e = o + kt;
+            if (o >= st_max && e <= en_min && e <= L) full[a][wb] += 1;
+            if (!(e <= st_min || o >= en_max)) some[a][wb] += 1;
+          }
+        }
+      }
+    }
+  }
+  auto masked = [&](int w0, int w1, int w2) {
+    return some[0][w0] * some[1][w1] * some[2][w2] - full[0][w0] * full[1][w1] * full[2][w2];
+  };
+  double best_masked = masked(best[0], best[1], best[2]);
+  for (int w0 = 0; w0 <= 5 && w0 <= p.q_tile_lg[0]; ++w0)
+    for (int w1 = 0; w0 + w1 <= 5 && w1 <= p.q_tile_lg[1]; ++w1) {
+      const int w2 = 5 - w0 - w1;
+      if (w2 > p.q_tile_lg[2]) continue;
+      const double m = masked(w0, w1, w2);
+      if (m < best_masked * 0.9999999 - 0.5) {
+        best_masked = m;
+        p.wave_box_lg[0] = w0;
+        p.wave_box_lg[1] = w1;
+        p.wave_box_lg[2] = w2;
+      }
+    }
+}
+
 inline void set_wg_layout(FnaParams& p, int tiles_per_wg = 1) {
   p.num_q_tiles = p.q_tiled[0] * p.q_tiled[1] * p.q_tiled[2];
   const int slab = p.q_tiled[1] * p.q_tiled[2];
@@ -1396,6 +1474,7 @@ inline void set_wg_layout(FnaParams& p, int tiles_per_wg = 1) {
     p.d_dil[a] = na_make_div(p.dil[a]);
     p.d_q_tiled[a] = na_make_div(p.q_tiled[a]);
   }
+  choose_wave_box(p);
   p.d_wg_group = na_make_div(p.wg_group);
   p.d_groups_per_bh = na_make_div(p.groups_per_bh);
   p.d_heads_q = na_make_div(p.heads_q);

@@ -320,7 +320,7 @@ int fused_geometry(const char* what, FnaParams& p, bool sixteen_bit, int na_dim,
 
 extern "C" {
 
-int natten_amd_abi_version(void) { return 15; }
+int natten_amd_abi_version(void) { return 16; }
 
 uint64_t natten_amd_fna_forward_workspace_bytes(void) { return uint64_t(kQueueWords) * 4; }
 
@@ -381,6 +381,24 @@ int natten_amd_fna_fully_block_sparse(int na_dim, const int32_t* qkv_shape, cons
   p.heads_q = p.heads_kv = 1;
   set_wg_layout(p, 1);
   *result = fully_block_sparse(p) ? 1 : 0;
+  return 0;
+}
+
+int natten_amd_fna_wave_box(int na_dim, const int32_t* qkv_shape, const int32_t* kernel_size, const int32_t* stride,
+                            const int32_t* dilation, const int32_t* is_causal, const int32_t* q_tile_shape,
+                            const int32_t* kv_tile_shape, int anchor_kv_tiles, int32_t* box) {
+  g_error[0] = 0;
+  if (na_dim < 1 || na_dim > 3) return fail("fna_wave_box: na_dim must be 1, 2 or 3, got %d", na_dim);
+  if (!box) return fail("fna_wave_box: null pointer argument");
+  FnaParams p;
+  long long tokens = 0;
+  if (int rc = fused_geometry("fna_wave_box", p, true, na_dim, 1, 32, qkv_shape, kernel_size, stride, dilation, is_causal,
+                              q_tile_shape, kv_tile_shape, anchor_kv_tiles, &tokens))
+    return rc;
+  p.batch = p.num_groups;
+  p.heads_q = p.heads_kv = 1;
+  set_wg_layout(p, 1);
+  for (int a = 0; a < na_dim; ++a) box[a] = 1 << p.wave_box_lg[a];
   return 0;
 }
 

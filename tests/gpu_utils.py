@@ -113,13 +113,16 @@ def routes_agree_bit_for_bit(shape, dilation, kv_tile) -> bool:
     return not all(X // d >= t for X, d, t in zip(shape, dilation, kv_tile))
 
 
-def assert_routes_agree(tag, a, b, shape, dilation, kv_tile):
-    """Outputs / LSEs of the two routes: bit-equal where the key placement is the same, else equal up
-    to the order of summation (a few units in the last place of the 16-bit result)."""
+def assert_routes_agree(tag, a, b, shape, dilation, kv_tile) -> bool:
+    """Outputs / LSEs of the two routes: bit-equal where the key placement is the same (returns
+    True).  Elsewhere they sum in different orders and round their probabilities against different
+    stale maxima: two results that each meet the oracle's bar, which is all that is asserted of their
+    difference here (returns False: the caller checks each against the oracle)."""
     if routes_agree_bit_for_bit(shape, dilation, kv_tile):
         assert torch.equal(a, b), "the two routes differ: " + tag
-    else:
-        assert_close("routes " + tag, to_np(a), to_np(b), atol=4e-3, rtol=8e-3)
+        return True
+    assert_close("routes " + tag, to_np(a), to_np(b), atol=1e-2, rtol=1e-2)
+    return False
 
 
 def _dim_windows(X, k, s, d, causal):

@@ -49,8 +49,16 @@ def run_case(B, H, Hkv, D, shape, k, s, d, causal, dtype, q_tile=None, kv_tile=N
                                          return_lse=True, anchored_tiles=False)
             out2, lse2 = amd_fna_generic(q, kk, v, k, s, d, causal, q_tile_shape=q_tile, kv_tile_shape=kv_tile,
                                          return_lse=True, fused=False)
-        assert_routes_agree("output " + tag, out1, out2, shape, d, kt_used)
+        exact = assert_routes_agree("output " + tag, out1, out2, shape, d, kt_used)
         assert_routes_agree("LSE " + tag, lse1, lse2, shape, d, kt_used)
+        if not exact:
+            # the permuted route then stands on its own against the oracle
+            if samples is None:
+                assert_close("permuted route, output " + tag, to_np(out2), ref_o)
+                assert_close("permuted route, LSE " + tag, to_np(lse2), ref_l)
+            else:
+                sampled_check(q, kk, v, out2, lse2, k, s, d, causal, max(samples // 2, 100), seed=seed + 3000,
+                              tag="permuted route, " + tag)
         # the aligned tiling sums in another order than the anchored one above: it meets the same bar
         # against the oracle, not some tighter one against the other route
         if samples is None:

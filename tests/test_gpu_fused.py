@@ -115,16 +115,21 @@ def test_fused_on_extents_that_tiles_do_not_divide(case):
             out_a, lse_a = amd_fna_generic(q, kk, v, k, s, d, causal, q_tile_shape=qt, kv_tile_shape=kt,
                                            return_lse=True, fused=True, anchored_tiles=True)
         tag = f"{shape} k={k} s={s} d={d} c={causal}"
-        assert_close("anchored tiles, output " + tag, to_np(out_a), to_np(out_f), atol=4e-3, rtol=8e-3)
-        assert_close("anchored tiles, LSE " + tag, to_np(lse_a), to_np(lse_f), atol=4e-3, rtol=8e-3)
-        assert_routes_agree("output " + tag, out_f, out_p, shape, d, kt)
+        exact = assert_routes_agree("output " + tag, out_f, out_p, shape, d, kt)
         assert_routes_agree("LSE " + tag, lse_f, lse_p, shape, d, kt)
-        if int(torch.tensor(shape).prod()) <= 40000:
-            ref_o, ref_l = oracle_full(q, kk, v, k, s, d, causal)
-            assert_close("out " + tag, to_np(out_f), ref_o)
-            assert_close("lse " + tag, to_np(lse_f), ref_l)
-        else:
-            sampled_check(q, kk, v, out_f, lse_f, k, s, d, causal, 400, seed=ci, tag=tag)
+        # both tilings of the one-launch route against the oracle (they sum in different orders: each
+        # meets the oracle's bar, not some tighter one against the other), and the permuted route
+        # too where it is not bit-equal to the aligned tiling
+        routes = [("aligned tiles", out_f, lse_f), ("anchored tiles", out_a, lse_a)]
+        if not exact:
+            routes.append(("permuted route", out_p, lse_p))
+        for name, o, l in routes:
+            if int(torch.tensor(shape).prod()) <= 40000:
+                ref_o, ref_l = oracle_full(q, kk, v, k, s, d, causal)
+                assert_close(f"{name}, out {tag}", to_np(o), ref_o)
+                assert_close(f"{name}, lse {tag}", to_np(l), ref_l)
+            else:
+                sampled_check(q, kk, v, o, l, k, s, d, causal, 400, seed=ci, tag=f"{name}, {tag}")
 
 
 def test_fused_with_dequantisation_scales():

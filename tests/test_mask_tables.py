@@ -145,3 +145,57 @@ def test_predicate_never_claims_full_when_the_mask_has_a_hole():
             agree += got == want
             claimed += got
     assert claimed > 5 and agree > 300
+
+
+def _masked_pairs(shape, k, s, c, q_tile, kv_tile, box):
+    """(wave box, KV tile) pairs that need the element mask, counted pair by pair from the dense
+    per-dimension windows: a tile needs none when every query of the box attends all of it (and it
+    lies inside the extent) or no query of the box attends any of it.  Dilation 1, KV tiles laid out
+    from the first key of each Q tile's window."""
+    n = len(shape)
+    start = [[int(O.window_start(i, k[a], s[a], shape[a], c[a])) for i in range(shape[a])] for a in range(n)]
+    end = [[int(O.window_end(i, start[a][i], k[a], shape[a], c[a])) for i in range(shape[a])] for a in range(n)]
+    count = 0
+    for qt in itertools.product(*[range(0, shape[a], q_tile[a]) for a in range(n)]):
+        org, tiles = [], []
+        for a in range(n):
+            last = min(qt[a] + q_tile[a] - 1, shape[a] - 1)
+            o = start[a][qt[a]] if shape[a] >= kv_tile[a] else (start[a][qt[a]] // kv_tile[a]) * kv_tile[a]
+            org.append(o)
+            tiles.append(-(-(end[a][last] - o) // kv_tile[a]))
+        for b in itertools.product(*[range(0, q_tile[a], box[a]) for a in range(n)]):
+            qs = [range(min(qt[a] + b[a], shape[a] - 1), min(qt[a] + b[a] + box[a] - 1, shape[a] - 1) + 1) for a in range(n)]
+            for t in itertools.product(*[range(x) for x in tiles]):
+                full, some = True, True
+                for a in range(n):
+                    o, e = org[a] + t[a] * kv_tile[a], org[a] + (t[a] + 1) * kv_tile[a]
+                    inside = all(start[a][i] <= o and e <= end[a][i] for i in qs[a]) and e <= shape[a]
+                    touched = any(start[a][i] < e and o < end[a][i] for i in qs[a])
+                    full, some = full and inside, some and touched
+                count += int(some and not full)
+    return count
+
+
+@pytest.mark.parametrize("case", [
+    # shape, kernel, stride, causal, Q tile, KV tile
+    ((48, 64), (20, 20), (1, 1), (False, False), (8, 16), (8, 8)),
+    ((40, 48), (9, 17), (1, 1), (True, False), (16, 8), (4, 16)),
+    ((12, 24, 32), (6, 8, 12), (1, 1, 1), (False, False, False), (2, 8, 8), (2, 4, 8)),
+    ((10, 16, 24), (4, 8, 8), (1, 8, 8), (True, False, False), (2, 8, 8), (1, 8, 8)),
+    ((16, 16, 16), (5, 5, 5), (1, 2, 1), (False, True, False), (4, 4, 8), (4, 4, 4)),
+])
+def test_wave_box_has_the_fewest_masked_pairs(case):
+    shape, k, s, c, q_tile, kv_tile = case
+    n = len(shape)
+    got = _lib.wave_box(shape, k, s, (1,) * n, c, q_tile, kv_tile)
+    assert int(np.prod(got)) == 32 and all(q % b == 0 for q, b in zip(q_tile, got)), got
+    candidates = [b for b in itertools.product(*[[1 << i for i in range(6) if (1 << i) <= q] for q in q_tile])
+                  if int(np.prod(b)) == 32]
+    counts = {b: _masked_pairs(shape, k, s, c, q_tile, kv_tile, b) for b in candidates}
+    assert counts[got] == min(counts.values()), (got, counts)
+
+
+def test_wave_box_defaults():
+    # sequence order (as much of the last dimension as fits) where nothing is gained, e.g. block-sparse shapes
+    assert _lib.wave_box((128, 128), (32, 32), (16, 16), (1, 1), (False, False), (8, 16), (8, 8)) == (2, 16)
+    assert _lib.wave_box((32768,), (2048,), (1,), (1,), (False,), (128,), (64,)) == (32,)
