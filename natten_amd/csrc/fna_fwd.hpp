@@ -20,6 +20,7 @@
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <string.h>
 
 #include <type_traits>
 #include <utility>
@@ -1394,8 +1395,39 @@ inline void choose_wave_box(FnaParams& p) {
   }
   for (int a = 0; a < 3; ++a) p.wave_box_lg[a] = best[a];
   if (p.cu_q) return;
+  // the boxes that fit the Q tile; with one (every 1-D problem) there is nothing to choose
+  int cand[21][3], n_cand = 0;
+  for (int w0 = 0; w0 <= 5 && w0 <= p.q_tile_lg[0]; ++w0)
+    for (int w1 = 0; w0 + w1 <= 5 && w1 <= p.q_tile_lg[1]; ++w1) {
+      const int w2 = 5 - w0 - w1;
+      if (w2 > p.q_tile_lg[2]) continue;
+      cand[n_cand][0] = w0;
+      cand[n_cand][1] = w1;
+      cand[n_cand][2] = w2;
+      ++n_cand;
+    }
+  if (n_cand <= 1) return;
+  // the same geometry as the call before (a model calls a layer over and over): the same answer
+  struct Key {
+    int v[3][7];
+    int anchor;
+    bool operator==(const Key& o) const { return memcmp(this, &o, sizeof(Key)) == 0; }
+  };
+  Key key;
+  memset(&key, 0, sizeof(key));
+  for (int a = 0; a < 3; ++a) {
+    const int vals[7] = {p.ext_base[a], p.ext_rem[a], p.ksize[a], p.stride[a], p.causal[a], p.q_tile[a], p.kv_tile[a]};
+    for (int i = 0; i < 7; ++i) key.v[a][i] = vals[i];
+  }
+  key.anchor = p.anchor;
+  thread_local Key last_key;
+  thread_local int last_box[3] = {-1, -1, -1};
+  if (last_box[0] >= 0 && key == last_key) {
+    for (int a = 0; a < 3; ++a) p.wave_box_lg[a] = last_box[a];
+    return;
+  }
   // per dimension and box extent: (wave box, KV tile) pairs attended in full / attended at all,
-  // summed over the Q tiles
+  // summed over the Q tiles (tile counts in closed form: the cost is Q tiles x boxes per dimension)
   double full[3][6], some[3][6];
   for (int a = 0; a < 3; ++a) {
     const int L = p.ext_base[a] + (p.ext_rem[a] ? 1 : 0), kt = p.kv_tile[a], qt = p.q_tile[a];
@@ -1417,31 +1449,30 @@ inline void choose_wave_box(FnaParams& p) {
           const int st_max = na_window_start(qmax, p.ksize[a], p.stride[a], L, causal);
           const int en_min = na_window_end(qmin, st_min, p.ksize[a], L, causal);
           const int en_max = na_window_end(qmax, st_max, p.ksize[a], L, causal);
-          for (int t = 0; t < tiles; ++t) {
-            const int o = org + t * kt, e = o + kt;
-            if (o >= st_max && e <= en_min && e <= L) full[a][wb] += 1;
-            if (!(e <= st_min || o >= en_max)) some[a][wb] += 1;
-          }
+          // tile t covers [org + t kt, org + (t + 1) kt).  Attended in full: it starts at or after
+          // st_max and ends at or before min(en_min, L).  Attended at all: it ends after st_min and
+          // starts before en_max.  (org <= st_min: the box starts at or before every window.)
+          const int f_lo = (st_max - org + kt - 1) / kt, f_hi = na_min((na_min(en_min, L) - org) / kt, tiles);
+          const int s_lo = (st_min - org) / kt, s_hi = na_min((en_max - org + kt - 1) / kt, tiles);
+          full[a][wb] += na_max(f_hi - f_lo, 0);
+          some[a][wb] += na_max(s_hi - s_lo, 0);
         }
       }
     }
   }
-  auto masked = [&](int w0, int w1, int w2) {
-    return some[0][w0] * some[1][w1] * some[2][w2] - full[0][w0] * full[1][w1] * full[2][w2];
+  auto masked = [&](const int* w) {
+    return some[0][w[0]] * some[1][w[1]] * some[2][w[2]] - full[0][w[0]] * full[1][w[1]] * full[2][w[2]];
   };
-  double best_masked = masked(best[0], best[1], best[2]);
-  for (int w0 = 0; w0 <= 5 && w0 <= p.q_tile_lg[0]; ++w0)
-    for (int w1 = 0; w0 + w1 <= 5 && w1 <= p.q_tile_lg[1]; ++w1) {
-      const int w2 = 5 - w0 - w1;
-      if (w2 > p.q_tile_lg[2]) continue;
-      const double m = masked(w0, w1, w2);
-      if (m < best_masked * 0.9999999 - 0.5) {
-        best_masked = m;
-        p.wave_box_lg[0] = w0;
-        p.wave_box_lg[1] = w1;
-        p.wave_box_lg[2] = w2;
-      }
+  double best_masked = masked(best);
+  for (int c = 0; c < n_cand; ++c) {
+    const double m = masked(cand[c]);
+    if (m < best_masked * 0.9999999 - 0.5) {
+      best_masked = m;
+      for (int a = 0; a < 3; ++a) p.wave_box_lg[a] = cand[c][a];
     }
+  }
+  last_key = key;
+  for (int a = 0; a < 3; ++a) last_box[a] = p.wave_box_lg[a];
 }
 
 inline void set_wg_layout(FnaParams& p, int tiles_per_wg = 1) {

@@ -199,3 +199,15 @@ def test_wave_box_defaults():
     # sequence order (as much of the last dimension as fits) where nothing is gained, e.g. block-sparse shapes
     assert _lib.wave_box((128, 128), (32, 32), (16, 16), (1, 1), (False, False), (8, 16), (8, 8)) == (2, 16)
     assert _lib.wave_box((32768,), (2048,), (1,), (1,), (False,), (128,), (64,)) == (32,)
+
+
+def test_wave_box_choice_is_cheap_on_the_host():
+    # the choice runs inside every forward call: a long sequence (one candidate box: nothing to
+    # count) and a large image (counted in closed form per Q tile and box) must cost microseconds
+    import time
+
+    t0 = time.perf_counter()
+    assert _lib.wave_box((1 << 20,), (1 << 19,), (1,), (1,), (False,), (128,), (64,)) == (32,)
+    box = _lib.wave_box((4096, 4096), (255, 255), (1, 1), (1, 1), (False, True), (8, 16), (8, 8))
+    assert int(np.prod(box)) == 32
+    assert time.perf_counter() - t0 < 0.05
