@@ -28,9 +28,9 @@
  *   natten_amd_fna_backward_fused <- the reference driver's permutes + backward + unpermutes,
  *                                  src/natten/backends/blackwell_fna.py:205-297, without the copies
  *   natten_amd_attention_backward <- blackwell_fmha_backward csrc/include/natten/blackwell_fmha.h:52-73
+ *                                  (fixed-length batches)
  *   natten_amd_attention_backward_varlen <- the same function with cumulative_seqlen_Q / _KV,
  *                                  max_seqlen_Q / _KV (csrc/include/natten/blackwell_fmha.h:52-73)
- *                                  (fixed-length batches)
  *   natten_amd_compute_delta    <- compute_delta            csrc/include/natten/compute_delta.h:33-36
  *   natten_amd_merge_attentions <- the elementwise merge of src/natten/attn_merge.py:48-105
  *                                  (the reference runs it as framework ops; here it is one kernel)
@@ -99,8 +99,10 @@ const char* natten_amd_last_error(void);
  * so the call may be captured in a graph): any memory will do.  run_persistent == 2: the caller
  * vouches that they are zero, which is how every work-queue launch leaves them (its last workgroup
  * resets them): a workspace zeroed once and then only handed to these launches, one at a time,
- * needs no clearing again, and the call is a single kernel launch.  Two calls must not use one
- * workspace concurrently.  Tile
+ * needs no clearing again, and the call is a single kernel launch.  (A launch that did not run to
+ * completion leaves counts behind; a later call in this mode on that workspace would then skip Q
+ * tiles without any error: after a failed or aborted launch, clear the workspace or use mode 1.)
+ * Two calls must not use one workspace concurrently.  Tile
  * pairs other than 128 x 64 tokens and float32 operands ignore the flag.  run_persistent == 0:
  * workspace may be NULL.
  */
