@@ -401,7 +401,7 @@ def bench_backward(args, q, k, v, kernel, stride, dilation, causal, dt_name):
             "backward_kv_tile_shape": list(kv_tile_dq),
             "dk_dv_launch_tile_shapes": [list(t) for t in kv_role] if kv_role[0] is not None else None,
             "permuted_route_tile_shapes": [list(q_tile), list(kv_tile)],
-            "path": ("forward (one launch) + delta + dQ kernel + dK/dV kernel on the original tensors" if fused else
+            "path": ("forward (one launch) + delta + scaled queries + dK/dV kernel + dQ kernel on the original tensors" if fused else
                      "forward + delta + token permutes + dQ and dK/dV kernels + unpermutes"),
         },
         "na_flop_per_step": 3.5 * fwd_flops,
