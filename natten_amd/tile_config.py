@@ -209,14 +209,16 @@ def _choose_backward_role_tile_shapes(
     the two launches together: ((q_tile, kv_tile) of the dq launch, (q_tile, kv_tile) of the dk / dv
     launch).  The dq launch streams half KV tiles past every Q tile, the dk / dv launch half Q tiles
     past every KV tile; each gets the shapes that visit the fewest (query, key) pairs, counted like
-    choose_tile_shapes does (partially masked pairs weigh more).  Only shapes that divide every
-    extent (times the dilation) qualify; None when there are none."""
+    choose_tile_shapes does (partially masked pairs weigh more).  Only shapes that fit every dilation
+    group (at least one tile wide in every dimension: what the kernels need on the original tensors)
+    qualify; None when there are none."""
     n = len(token_layout)
     shapes = [t for t in _factorisations(BACKWARD_TILE_SIZE, n)
-              if all(x % (d * e) == 0 for x, d, e in zip(token_layout, dilation, t))]
+              if all(x // d >= e for x, d, e in zip(token_layout, dilation, t))
+              and [e for e in t if e > 1][-1] % 2 == 0]
     if not shapes:
         return None
-    ext = tuple(x // d for x, d in zip(token_layout, dilation))
+    ext = tuple(_ceil_div(x, d) for x, d in zip(token_layout, dilation))
 
     def cost(q_ext: DimensionType, kv_ext: DimensionType) -> float:
         visited = full = 1

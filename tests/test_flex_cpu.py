@@ -179,8 +179,11 @@ def test_backward_tile_shapes_per_launch():
     # c4: a causal dimension 0 with one-frame half tiles on the streamed side
     dq, kv = choose_backward_role_tile_shapes((30, 48, 80), (18, 24, 24), (1, 8, 8), (1, 1, 1), (True, False, False))
     assert dq == ((2, 8, 8), (1, 8, 16)) and kv == ((1, 8, 16), (2, 8, 8))
-    # shapes must divide every extent (times the dilation): none does here
-    assert choose_backward_role_tile_shapes((29, 46, 78), (9, 24, 24), (1, 8, 8), (2, 1, 1), (False,) * 3) is None
+    # shapes need not divide the extents (the kernels move or clamp the tiles at a group's end) ...
+    dq, kv = choose_backward_role_tile_shapes((29, 46, 78), (9, 24, 24), (1, 8, 8), (2, 1, 1), (False,) * 3)
+    assert dq == ((2, 8, 8), (1, 8, 16)) and kv == ((1, 8, 16), (2, 8, 8))
+    # ... but every dilation group must be at least a tile wide in every dimension: none fits here
+    assert choose_backward_role_tile_shapes((6, 6), (3, 3), (1, 1), (1, 1), (False, False)) is None
     # 1-D: one factorisation, the same for both launches
     assert choose_backward_role_tile_shapes((4096,), (512,), (1,), (1,), (True,)) == (((128,), (128,)),) * 2
     # whatever is chosen holds 128 tokens and divides the extents
